@@ -1,0 +1,10 @@
+"""arle_amd: a small, whole inference engine for one AMD MI355X (gfx950).
+
+Model folder (config.json + safetensors) or a configuration and a seed -> generated tokens:
+typed configuration and architecture registry (`config`), weights (`weights`), layers put
+together from parts (`parts`, `models`), a paged cache with state slots (`cache`), one step
+function and a scheduler above it (`engine`), sampling (`sampling`), hand-written HIP
+kernels (`csrc`, `kernels`).
+"""
+
+__version__ = "0.1.0"

@@ -1,0 +1,65 @@
+// Embedding gather and the SiLU-gated product.
+//
+// embed_gather: out[t, :] = float(table[ids[t], :])      (residual stream is 32-bit)
+//   reference counterpart: crates/cuda-kernels/csrc/misc/elementwise_basic.cu:186-211
+// silu_mul:     out[t, j] = silu(gate[t, j]) * up[t, j], silu(z) = z / (1 + exp(-z))
+//   reference counterpart: crates/cuda-kernels/csrc/misc/elementwise_basic.cu:18-24,34-95
+#include "common.h"
+
+namespace arle {
+
+template <typename TT>
+__global__ void embed_gather_kernel(const TT* __restrict__ table, const int* __restrict__ ids,
+                                    float* __restrict__ out, int hidden) {
+  const int t = blockIdx.x;
+  const TT* src = table + static_cast<int64_t>(ids[t]) * hidden;
+  float* dst = out + static_cast<int64_t>(t) * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
+}
+
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict__ up,
+                                int64_t in_stride, T* __restrict__ out, int width) {
+  const int t = blockIdx.x;
+  const int j = blockIdx.y * blockDim.x + threadIdx.x;
+  if (j >= width) return;
+  const float g = to_float(gate[static_cast<int64_t>(t) * in_stride + j]);
+  const float u = to_float(up[static_cast<int64_t>(t) * in_stride + j]);
+  const float act = g / (1.0f + expf(-g));
+  out[static_cast<int64_t>(t) * width + j] = from_float<T>(act * u);
+}
+
+}  // namespace arle
+
+using namespace arle;
+
+extern "C" int arle_embed_gather(const void* table, int table_dtype, const int* ids, float* out,
+                                 int tokens, int hidden, void* stream) {
+  if (tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (table_dtype == kF32) {
+    embed_gather_kernel<float><<<tokens, 256, 0, s>>>(static_cast<const float*>(table), ids, out, hidden);
+  } else {
+    embed_gather_kernel<bf16><<<tokens, 256, 0, s>>>(static_cast<const bf16*>(table), ids, out, hidden);
+  }
+  return launch_status();
+}
+
+// gate and up are two columns blocks of rows with a common row stride (in
+// elements), so one fused [T, 2I] buffer and two separate buffers both fit.
+extern "C" int arle_silu_mul(const void* gate, const void* up, long long in_stride, void* out,
+                             int dtype, int tokens, int width, void* stream) {
+  if (tokens == 0 || width == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(tokens, (width + 255) / 256);
+  if (dtype == kF32) {
+    silu_mul_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(gate),
+                                                static_cast<const float*>(up), in_stride,
+                                                static_cast<float*>(out), width);
+  } else {
+    silu_mul_kernel<bf16><<<grid, 256, 0, s>>>(static_cast<const bf16*>(gate),
+                                               static_cast<const bf16*>(up), in_stride,
+                                               static_cast<bf16*>(out), width);
+  }
+  return launch_status();
+}

@@ -1,0 +1,146 @@
+// Per-head RMSNorm of q and k, rotary position encoding, and the write of k and v
+// into the paged cache, in one pass over the projections of a packed batch.
+//
+// For every token t and head h (q heads, then k heads, then v heads):
+//   x  = head vector [D]
+//   x  = x * 1/sqrt(mean(x^2) + eps) * w          (q and k only, if a weight is given)
+//   for d < rot/2:  y_d = x_d cos_d - x_{d+rot/2} sin_d ;  y_{d+rot/2} = x_d sin_d + x_{d+rot/2} cos_d
+//   (dims >= rot pass through; rot == 0 means no rotation)
+//   q -> written back in place; k, v -> cache row of (slot, position), or k in place
+//   when no cache is given.
+// cos/sin are 32-bit tables [positions, rot/2]; all arithmetic is 32-bit and the
+// result is rounded once at the store.
+// reference counterparts: crates/cuda-kernels/csrc/attention/prefill_attention_paged_prep.cu:8-106,
+// crates/cuda-kernels/csrc/attention/decode_prep_paged.cu:73-160 (head_dim fixed to 128 there).
+//
+// Cache layout per layer: [page, kv_head, slot_in_page, D].
+#include "common.h"
+
+namespace arle {
+
+constexpr int kPrepWaves = 4;
+constexpr int kMaxHeadDim = 512;
+
+template <typename T, typename TW>
+__global__ __launch_bounds__(kPrepWaves* kWave) void qk_prep_kernel(
+    T* __restrict__ q, int64_t q_stride, T* __restrict__ k, int64_t k_stride,
+    const T* __restrict__ v, int64_t v_stride, const TW* __restrict__ q_w,
+    const TW* __restrict__ k_w, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    int rot, const int* __restrict__ positions, const int* __restrict__ slot_of_token,
+    const int* __restrict__ block_table, int table_stride, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int nq, int nkv, int D, int page_size, float eps) {
+  extern __shared__ float lds[];  // [kPrepWaves][D]
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int head = blockIdx.y * kPrepWaves + wave;  // same for all lanes of a wave
+  const bool valid = head < nq + 2 * nkv;
+  const bool is_v = valid && head >= nq + nkv;
+  const bool is_qk = valid && !is_v;
+  const bool is_q = head < nq;
+  float* x = lds + wave * D;
+
+  const int pos = positions[t];
+  int64_t cache_row = 0;  // element offset of [page, kv head 0, slot_in_page, 0]
+  if (valid && !is_q && (k_pages || v_pages)) {
+    const int slot = slot_of_token[t];
+    const int page = block_table[static_cast<int64_t>(slot) * table_stride + pos / page_size];
+    cache_row = (static_cast<int64_t>(page) * nkv * page_size + (pos % page_size)) * D;
+  }
+
+  if (is_v && v_pages) {  // v head: copy into the cache
+    const int kvh = head - nq - nkv;
+    const T* vsrc = v + static_cast<int64_t>(t) * v_stride + kvh * D;
+    T* vdst = v_pages + cache_row + static_cast<int64_t>(kvh) * page_size * D;
+    for (int d = lane; d < D; d += kWave) vdst[d] = vsrc[d];
+  }
+
+  const int local = is_q ? head : head - nq;
+  T* src = is_q ? q + static_cast<int64_t>(t) * q_stride + local * D
+                : k + static_cast<int64_t>(t) * k_stride + local * D;
+  if (is_qk) {
+    const TW* w = is_q ? q_w : k_w;
+    float ss = 0.f;
+    for (int d = lane; d < D; d += kWave) {
+      const float val = to_float(src[d]);
+      x[d] = val;
+      ss += val * val;
+    }
+    if (w) {
+      ss = wave_sum(ss);
+      const float inv = 1.0f / sqrtf(ss / static_cast<float>(D) + eps);
+      for (int d = lane; d < D; d += kWave) x[d] = x[d] * inv * to_float(w[d]);
+    }
+  }
+  __syncthreads();  // every thread of the block arrives: the LDS rows are complete
+  if (!is_qk) return;
+
+  T* dst = src;
+  if (!is_q && k_pages) dst = k_pages + cache_row + static_cast<int64_t>(local) * page_size * D;
+  const int half = rot / 2;
+  const float* cs = cos_t + static_cast<int64_t>(pos) * half;
+  const float* sn = sin_t + static_cast<int64_t>(pos) * half;
+  for (int d = lane; d < D; d += kWave) {
+    float y;
+    if (d < half) {
+      y = x[d] * cs[d] - x[d + half] * sn[d];
+    } else if (d < rot) {
+      const int p = d - half;
+      y = x[p] * sn[p] + x[d] * cs[p];
+    } else {
+      y = x[d];
+    }
+    dst[d] = from_float<T>(y);
+  }
+}
+
+template <typename T>
+int launch_prep(void* q, long long q_stride, void* k, long long k_stride, const void* v,
+                long long v_stride, const void* q_w, const void* k_w, int w_dtype,
+                const float* cos_t, const float* sin_t, int rot, const int* positions,
+                const int* slot_of_token, const int* block_table, int table_stride, void* k_pages,
+                void* v_pages, int tokens, int nq, int nkv, int D, int page_size, float eps,
+                hipStream_t s) {
+  dim3 grid(tokens, (nq + 2 * nkv + kPrepWaves - 1) / kPrepWaves);
+  const size_t lds = static_cast<size_t>(kPrepWaves) * D * sizeof(float);
+  if (w_dtype == kF32) {
+    qk_prep_kernel<T, float><<<grid, kPrepWaves * kWave, lds, s>>>(
+        static_cast<T*>(q), q_stride, static_cast<T*>(k), k_stride, static_cast<const T*>(v),
+        v_stride, static_cast<const float*>(q_w), static_cast<const float*>(k_w), cos_t, sin_t, rot,
+        positions, slot_of_token, block_table, table_stride, static_cast<T*>(k_pages),
+        static_cast<T*>(v_pages), nq, nkv, D, page_size, eps);
+  } else {
+    qk_prep_kernel<T, bf16><<<grid, kPrepWaves * kWave, lds, s>>>(
+        static_cast<T*>(q), q_stride, static_cast<T*>(k), k_stride, static_cast<const T*>(v),
+        v_stride, static_cast<const bf16*>(q_w), static_cast<const bf16*>(k_w), cos_t, sin_t, rot,
+        positions, slot_of_token, block_table, table_stride, static_cast<T*>(k_pages),
+        static_cast<T*>(v_pages), nq, nkv, D, page_size, eps);
+  }
+  return launch_status();
+}
+
+}  // namespace arle
+
+using namespace arle;
+
+// q [T, nq*D], k [T, nkv*D], v [T, nkv*D] with row strides in elements (so three
+// buffers or three column blocks of one fused buffer both fit).  q_w/k_w may be
+// null (no per-head norm); rot may be 0 (no rotation; cos/sin unused); k_pages /
+// v_pages may be null (no cache write; k is then rewritten in place).
+extern "C" int arle_qk_prep(void* q, long long q_stride, void* k, long long k_stride, const void* v,
+                            long long v_stride, int dtype, const void* q_w, const void* k_w,
+                            int w_dtype, const float* cos_t, const float* sin_t, int rot,
+                            const int* positions, const int* slot_of_token, const int* block_table,
+                            int table_stride, void* k_pages, void* v_pages, int tokens, int nq,
+                            int nkv, int D, int page_size, float eps, void* stream) {
+  if (tokens == 0) return 0;
+  if (D > kMaxHeadDim || rot > D || (rot & 1)) return static_cast<int>(hipErrorInvalidValue);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == kF32)
+    return launch_prep<float>(q, q_stride, k, k_stride, v, v_stride, q_w, k_w, w_dtype, cos_t, sin_t,
+                              rot, positions, slot_of_token, block_table, table_stride, k_pages,
+                              v_pages, tokens, nq, nkv, D, page_size, eps, s);
+  return launch_prep<bf16>(q, q_stride, k, k_stride, v, v_stride, q_w, k_w, w_dtype, cos_t, sin_t,
+                           rot, positions, slot_of_token, block_table, table_stride, k_pages,
+                           v_pages, tokens, nq, nkv, D, page_size, eps, s);
+}

@@ -1,0 +1,138 @@
+"""The engine: a model, its cache, and the one step function everything else is built on.
+
+`step(entries)` takes a batch of (request, its next tokens, wanted places): portions of
+prompts beside single decoded tokens, cut anywhere.  It makes room in the cache for all of
+them or for none, runs only the rows it is given against the cache earlier steps left,
+and returns float32 logits at the wanted places, in the order of the entries and of their
+`want` lists.  The reference splits this over three calls (prefill batch, decode batch,
+mixed batch: infer/src/model/qwen3/forward.rs:376-400,605-637,650-665); here a decoded token
+is an entry of one token and there is one call.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import models  # noqa: F401  (registers the architectures)
+from ..cache.manager import CacheManager
+from ..config.registry import detect_architecture, load_model_config
+from ..models.decoder import build_model, expected_checkpoint_tensors
+from ..parts.base import Runtime
+from ..weights.loader import load_weights
+from ..weights.random_init import random_weights
+from .batch import StepEntry, build_step_batch
+
+DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
+          "fp32": torch.float32}
+DEFAULT_PAGE_SIZE = 16  # tokens per page, as the reference's bf16 pool (crates/cuda-kernels/src/kv_types.rs:53-59)
+
+
+class EngineError(RuntimeError):
+    pass
+
+
+def _device(device=None) -> torch.device:
+    if not torch.cuda.is_available():
+        raise EngineError("arle_amd needs a GPU: torch.cuda.is_available() is False and there is "
+                          "no CPU path")
+    return torch.device(device or "cuda:0")
+
+
+def parse_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        return name
+    try:
+        return DTYPES[str(name)]
+    except KeyError:
+        raise EngineError(f"unknown dtype {name!r}; use bfloat16 or float32") from None
+
+
+class Engine:
+    def __init__(self, spec, tensors: dict, *, dtype=torch.bfloat16, device=None,
+                 page_size: int = DEFAULT_PAGE_SIZE, max_tokens: int | None = None,
+                 num_pages: int | None = None, max_slots: int = 4,
+                 max_request_tokens: int | None = None):
+        """
+        max_tokens: tokens the cache holds over all live requests (num_pages = ceil(max_tokens / page_size)
+            unless num_pages is given).
+        max_request_tokens: longest single request (default: min(model's positions, cache capacity)).
+        """
+        self.device = _device(device)
+        self.dtype = parse_dtype(dtype)
+        self.spec = spec
+        self.rt = Runtime(device=self.device, act_dtype=self.dtype)
+        self.model = build_model(spec, tensors, self.rt)
+        if num_pages is None:
+            if max_tokens is None:
+                raise EngineError("give max_tokens or num_pages to size the cache")
+            num_pages = -(-int(max_tokens) // page_size)
+        capacity = num_pages * page_size
+        if max_request_tokens is None:
+            max_request_tokens = min(spec.max_positions, capacity)
+        needs, readers = self.model.cache_needs()
+        self.cache = CacheManager(needs, page_size=page_size, num_pages=num_pages,
+                                  max_slots=max_slots, max_request_tokens=max_request_tokens,
+                                  device=self.device, dtype=self.dtype, readers=readers)
+        self.page_size = page_size
+        self.max_request_tokens = max_request_tokens
+        self.steps_run = 0
+
+    # -- construction -----------------------------------------------------------------
+    @classmethod
+    def from_folder(cls, model_dir: str, *, dtype="bfloat16", device=None, **cache_args) -> "Engine":
+        """A model folder (config.json + safetensors); the model class comes from config.json."""
+        arch, config, stops = load_model_config(model_dir)
+        spec = arch.recipe(config, stops)
+        dev = _device(device)
+        tensors = load_weights(model_dir, expected_checkpoint_tensors(spec), dev, parse_dtype(dtype))
+        engine = cls(spec, tensors, dtype=dtype, device=dev, **cache_args)
+        engine.config, engine.architecture = config, arch.name
+        return engine
+
+    @classmethod
+    def from_config(cls, arch_name: str, config, *, seed: int = 0, std: float = 0.02,
+                    norm_std: float = 0.0, dtype="bfloat16", device=None, **cache_args) -> "Engine":
+        """Random weights drawn on the GPU from a configuration and a seed (no files)."""
+        arch = detect_architecture({"architectures": [arch_name]})
+        spec = arch.recipe(config, ())
+        dev = _device(device)
+        tensors = random_weights(spec, seed, std, norm_std, parse_dtype(dtype), device=dev)
+        engine = cls(spec, tensors, dtype=dtype, device=dev, **cache_args)
+        engine.config, engine.architecture = config, arch.name
+        return engine
+
+    # -- requests -----------------------------------------------------------------------
+    def add_request(self, key) -> int:
+        return self.cache.admit(key)
+
+    def end_request(self, key) -> None:
+        self.cache.release(key)
+
+    def length(self, key) -> int:
+        return self.cache.length(key)
+
+    # -- the step -------------------------------------------------------------------------
+    @torch.no_grad()
+    def step(self, entries) -> torch.Tensor:
+        """Run one packed step; returns float32 logits [wanted, vocab] on the GPU.
+
+        Raises `OutOfPages` (nothing changed) if the cache cannot take all entries.
+        """
+        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        for e in entries:
+            if not self.cache.is_live(e.request):
+                raise EngineError(f"request {e.request!r} is not live; add_request it first")
+        batch = build_step_batch(entries, self.cache.slot_of.__getitem__, self.cache.length,
+                                 self.spec.vocab_size, self.device)
+        before = {e.request: self.cache.length(e.request) for e in entries}
+        self.cache.append([(e.request, len(e.tokens)) for e in entries])
+        try:
+            self.cache.sync_tables()
+            logits = self.model.forward(batch, self.cache)
+        except Exception:
+            for key, n in before.items():
+                self.cache.truncate(key, n)
+            raise
+        for e in entries:
+            self.cache.trim_windows(e.request)
+        self.steps_run += 1
+        return logits

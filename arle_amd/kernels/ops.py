@@ -1,0 +1,346 @@
+"""Typed Python entry points of the HIP kernels.
+
+Each function checks on the host that the operands have the shapes, dtypes and
+layout its kernel assumes (a kernel never sees a shape it was not written for),
+then launches on torch's current HIP stream.  There is no CPU path: tensors must
+live on the GPU.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import lib
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+MAX_HEAD_DIM = 512
+_GRID_Y_MAX = 65535
+
+
+class ShapeError(ValueError):
+    """Operands that a kernel was not written for."""
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _CODES[t.dtype]
+    except KeyError:
+        raise ShapeError(f"unsupported element type {t.dtype}; kernels take float32 and bfloat16")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ShapeError(msg)
+
+
+def _gpu(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise ShapeError("arle_amd kernels run on the GPU only; got a CPU tensor")
+
+
+def _rows(t: torch.Tensor, name: str) -> None:
+    _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-D with contiguous rows")
+
+
+def _i32(t, name: str, n: int | None = None) -> None:
+    _need(t.dtype == torch.int32 and t.dim() == 1 and t.is_contiguous(), f"{name} must be int32 1-D")
+    if n is not None:
+        _need(t.numel() == n, f"{name} must have {n} entries, has {t.numel()}")
+
+
+def _ptr(t) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+# ------------------------------------------------------------------ embedding
+
+
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None):
+    """out[t, :] = float32(table[ids[t], :]).  ids must already be checked to lie in range."""
+    _gpu(table, ids, out)
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [V, H]")
+    _i32(ids, "ids")
+    tokens, hidden = ids.numel(), table.shape[1]
+    if out is None:
+        out = torch.empty((tokens, hidden), dtype=torch.float32, device=table.device)
+    _need(out.dtype == torch.float32 and out.shape == (tokens, hidden) and out.is_contiguous(),
+          "embed_gather output must be contiguous float32 [T, H]")
+    lib.call("arle_embed_gather", table.data_ptr(), _code(table), ids.data_ptr(), out.data_ptr(),
+             tokens, hidden, _stream())
+    return out
+
+
+def silu_mul(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor | None = None):
+    """out = silu(gate) * up for two [T, I] views with the same row stride."""
+    _gpu(gate, up, out)
+    _rows(gate, "gate")
+    _rows(up, "up")
+    _need(gate.shape == up.shape and gate.dtype == up.dtype and gate.stride(0) == up.stride(0),
+          "gate and up must agree in shape, dtype and row stride")
+    tokens, width = gate.shape
+    _need(math.ceil(width / 256) <= _GRID_Y_MAX, "silu_mul: width too large")
+    if out is None:
+        out = torch.empty((tokens, width), dtype=gate.dtype, device=gate.device)
+    _need(out.shape == (tokens, width) and out.dtype == gate.dtype and out.is_contiguous(),
+          "silu_mul output must be contiguous [T, I] of the input type")
+    lib.call("arle_silu_mul", gate.data_ptr(), up.data_ptr(), gate.stride(0), out.data_ptr(),
+             _code(gate), tokens, width, _stream())
+    return out
+
+
+# ----------------------------------------------------------------------- norms
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+            rows: torch.Tensor | None = None, out: torch.Tensor | None = None):
+    """out[r] = x[src(r)] / sqrt(mean(x^2) + eps) * weight;  src(r) = rows[r] or r."""
+    _gpu(x, weight, rows, out)
+    _rows(x, "x")
+    width = x.shape[1]
+    _need(weight.shape == (width,) and weight.is_contiguous(), "norm weight must be [width]")
+    n_rows = x.shape[0]
+    if rows is not None:
+        _i32(rows, "rows")
+        n_rows = rows.numel()
+    if out is None:
+        out = torch.empty((n_rows, width), dtype=out_dtype, device=x.device)
+    _need(out.shape == (n_rows, width) and out.dtype == out_dtype and out.is_contiguous(),
+          "rmsnorm output must be contiguous [rows, width]")
+    lib.call("arle_rmsnorm", x.data_ptr(), _code(x), x.stride(0), weight.data_ptr(), _code(weight),
+             out.data_ptr(), _code(out), _ptr(rows), n_rows, width, float(eps), _stream())
+    return out
+
+
+def add_rmsnorm(residual: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, rows: torch.Tensor | None = None,
+                out: torch.Tensor | None = None):
+    """residual += delta (float32, in place unless `rows` is given); out = rmsnorm(residual)."""
+    _gpu(residual, delta, weight, rows, out)
+    _need(residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous(),
+          "residual must be contiguous float32 [T, H]")
+    _need(delta.shape == residual.shape and delta.is_contiguous(), "delta must match the residual")
+    width = residual.shape[1]
+    _need(weight.shape == (width,) and weight.is_contiguous(), "norm weight must be [width]")
+    n_rows = residual.shape[0]
+    if rows is not None:
+        _i32(rows, "rows")
+        n_rows = rows.numel()
+    if out is None:
+        out = torch.empty((n_rows, width), dtype=out_dtype, device=residual.device)
+    _need(out.shape == (n_rows, width) and out.dtype == out_dtype and out.is_contiguous(),
+          "add_rmsnorm output must be contiguous [rows, width]")
+    lib.call("arle_add_rmsnorm", residual.data_ptr(), delta.data_ptr(), _code(delta),
+             weight.data_ptr(), _code(weight), out.data_ptr(), _code(out), _ptr(rows), n_rows, width,
+             float(eps), _stream())
+    return out
+
+
+# ------------------------------------------------------------------- products
+
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None):
+    """out[M, N] = a[M, K] . w[N, K]^T in true float32, fixed k order."""
+    _gpu(a, w, out)
+    _rows(a, "a")
+    _rows(w, "w")
+    _need(a.dtype == torch.float32 and w.dtype == torch.float32, "gemm_f32 takes float32 operands")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(w.shape[1] == K, f"gemm_f32: inner sizes differ ({K} vs {w.shape[1]})")
+    _need(math.ceil(M / 64) <= _GRID_Y_MAX, "gemm_f32: too many rows for one launch")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+    _rows(out, "out")
+    _need(out.shape == (M, N) and out.dtype == torch.float32, "gemm_f32 output must be float32 [M, N]")
+    lib.call("arle_gemm_f32", a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(),
+             out.stride(0), M, N, K, _stream())
+    return out
+
+
+# ------------------------------------------------------ q/k preparation + cache
+
+
+def qk_prep(q, k, v, *, num_q_heads: int, num_kv_heads: int, head_dim: int, eps: float,
+            q_weight=None, k_weight=None, cos=None, sin=None, rotary_dim: int = 0,
+            positions=None, slot_of_token=None, block_table=None, k_pages=None, v_pages=None,
+            page_size: int = 0):
+    """Per-head norm + rotation of q and k in place; k and v written to the paged cache.
+
+    q [T, nq*D], k, v [T, nkv*D] (row views of one fused buffer are fine).  With no
+    cache given k is rewritten in place and v is left alone.
+    """
+    _gpu(q, k, v, q_weight, k_weight, cos, sin, positions, slot_of_token, block_table, k_pages, v_pages)
+    tokens = q.shape[0]
+    D = head_dim
+    _need(0 < D <= MAX_HEAD_DIM, f"head_dim {D} is outside the supported range 1..{MAX_HEAD_DIM}")
+    for name, t, heads in (("q", q, num_q_heads), ("k", k, num_kv_heads), ("v", v, num_kv_heads)):
+        _rows(t, name)
+        _need(t.shape == (tokens, heads * D), f"{name} must be [T, heads*D]")
+        _need(t.dtype == q.dtype, "q, k and v must share one element type")
+    _need((q_weight is None) == (k_weight is None), "give both q and k norm weights or neither")
+    w_code = F32
+    if q_weight is not None:
+        _need(q_weight.shape == (D,) and k_weight.shape == (D,) and q_weight.dtype == k_weight.dtype
+              and q_weight.is_contiguous() and k_weight.is_contiguous(),
+              "q/k norm weights must be [head_dim] of one type")
+        w_code = _code(q_weight)
+    _i32(positions, "positions", tokens)
+    if rotary_dim:
+        _need(rotary_dim % 2 == 0 and rotary_dim <= D, "rotary_dim must be even and <= head_dim")
+        _need(cos is not None and sin is not None and cos.dtype == torch.float32
+              and sin.dtype == torch.float32 and cos.dim() == 2 and cos.shape == sin.shape
+              and cos.shape[1] == rotary_dim // 2 and cos.is_contiguous() and sin.is_contiguous(),
+              "cos/sin must be contiguous float32 [positions, rotary_dim/2]")
+    table_stride = 0
+    if k_pages is not None or v_pages is not None:
+        _need(k_pages is not None and v_pages is not None, "give both k and v pages or neither")
+        _need(page_size > 0, "page_size must be positive")
+        for name, t in (("k_pages", k_pages), ("v_pages", v_pages)):
+            _need(t.dim() == 4 and t.shape[1:] == (num_kv_heads, page_size, D) and t.is_contiguous()
+                  and t.dtype == q.dtype, f"{name} must be contiguous [pages, nkv, page_size, D]")
+        _i32(slot_of_token, "slot_of_token", tokens)
+        _need(block_table is not None and block_table.dtype == torch.int32 and block_table.dim() == 2
+              and block_table.is_contiguous(), "block_table must be contiguous int32 [slots, pages]")
+        table_stride = block_table.shape[1]
+    heads = num_q_heads + 2 * num_kv_heads
+    _need(math.ceil(heads / 4) <= _GRID_Y_MAX, "too many heads")
+    lib.call("arle_qk_prep", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(),
+             v.stride(0), _code(q), _ptr(q_weight), _ptr(k_weight), w_code, _ptr(cos), _ptr(sin),
+             int(rotary_dim), positions.data_ptr(), _ptr(slot_of_token), _ptr(block_table),
+             table_stride, _ptr(k_pages), _ptr(v_pages), tokens, num_q_heads, num_kv_heads, D,
+             int(page_size), float(eps), _stream())
+
+
+# ------------------------------------------------------------------ attention
+
+
+def _check_paged(q, out, k_pages, v_pages, block_table, positions, slot_of_token, nq, nkv, D,
+                 page_size):
+    _gpu(q, out, k_pages, v_pages, block_table, positions, slot_of_token)
+    tokens = q.shape[0]
+    _rows(q, "q")
+    _rows(out, "out")
+    _need(q.shape == (tokens, nq * D) and out.shape == (tokens, nq * D) and out.dtype == q.dtype,
+          "q and out must be [T, nq*D] of one type")
+    _need(nkv > 0 and nq % nkv == 0, "number of q heads must be a multiple of the kv heads")
+    for name, t in (("k_pages", k_pages), ("v_pages", v_pages)):
+        _need(t.dim() == 4 and t.shape[1:] == (nkv, page_size, D) and t.is_contiguous()
+              and t.dtype == q.dtype, f"{name} must be contiguous [pages, nkv, page_size, D]")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "block_table must be contiguous int32 [slots, pages]")
+    _i32(positions, "positions", tokens)
+    _i32(slot_of_token, "slot_of_token", tokens)
+
+
+def attn_paged_simt(q, out, k_pages, v_pages, block_table, positions, slot_of_token, *,
+                    num_q_heads: int, num_kv_heads: int, head_dim: int, page_size: int,
+                    scale: float, window: int = 0, row_list=None):
+    """Causal attention of every token row (or of `row_list`) over its request's cached keys."""
+    _check_paged(q, out, k_pages, v_pages, block_table, positions, slot_of_token, num_q_heads,
+                 num_kv_heads, head_dim, page_size)
+    _need(0 < head_dim <= MAX_HEAD_DIM, f"head_dim {head_dim} outside 1..{MAX_HEAD_DIM}")
+    _need(num_q_heads <= _GRID_Y_MAX, "too many heads")
+    n_rows = q.shape[0]
+    if row_list is not None:
+        _gpu(row_list)
+        _i32(row_list, "row_list")
+        n_rows = row_list.numel()
+    lib.call("arle_attn_paged_simt", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
+             k_pages.data_ptr(), v_pages.data_ptr(), _code(q), block_table.data_ptr(),
+             block_table.shape[1], positions.data_ptr(), slot_of_token.data_ptr(), _ptr(row_list),
+             n_rows, num_q_heads, num_kv_heads, head_dim, page_size, float(scale), int(window),
+             _stream())
+    return out
+
+
+# ------------------------------------------------------------------- sampling
+
+
+def _logits(logits):
+    _gpu(logits)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.is_contiguous(),
+          "logits must be contiguous float32 [rows, vocab]")
+    return logits.shape
+
+
+def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
+    rows, vocab = _logits(logits)
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    lib.call("arle_argmax_rows", logits.data_ptr(), rows, vocab, out.data_ptr(), _stream())
+    return out
+
+
+def sample_rows(logits, temperature, top_k, top_p, min_p, u) -> torch.Tensor:
+    """One token id per row; per-row float32 temperature/top_p/min_p/u and int32 top_k."""
+    rows, vocab = _logits(logits)
+    for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+                        ("top_p", top_p, torch.float32), ("min_p", min_p, torch.float32),
+                        ("u", u, torch.float32)):
+        _gpu(t)
+        _need(t.dtype == dt and t.shape == (rows,) and t.is_contiguous(), f"{name} must be {dt} [rows]")
+    probs = torch.empty((rows, vocab), dtype=torch.float32, device=logits.device)
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    lib.call("arle_sample_rows", logits.data_ptr(), rows, vocab, probs.data_ptr(),
+             temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), min_p.data_ptr(),
+             u.data_ptr(), out.data_ptr(), _stream())
+    return out
+
+
+def apply_penalties(logits, indptr, tokens, counts, repetition, frequency, presence) -> None:
+    """In place: repetition, frequency and presence penalties on the listed (row, token, count)."""
+    rows, vocab = _logits(logits)
+    _gpu(indptr, tokens, counts, repetition, frequency, presence)
+    _i32(indptr, "indptr", rows + 1)
+    _i32(tokens, "tokens")
+    _i32(counts, "counts", tokens.numel())
+    for name, t in (("repetition", repetition), ("frequency", frequency), ("presence", presence)):
+        _need(t.dtype == torch.float32 and t.shape == (rows,) and t.is_contiguous(),
+              f"{name} must be float32 [rows]")
+    lib.call("arle_apply_penalties", logits.data_ptr(), rows, vocab, indptr.data_ptr(),
+             tokens.data_ptr(), counts.data_ptr(), repetition.data_ptr(), frequency.data_ptr(),
+             presence.data_ptr(), _stream())
+
+
+# ------------------------------------------------------------ bfloat16 products
+
+
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16):
+    """out[M, N] = x[M, K] . w[N, K]^T, bfloat16 operands, float32 accumulation.
+
+    Many rows go to the vendor library (hipBLASLt through torch.matmul), the matrix
+    product the reference also leaves to a library (crates/cuda-kernels/csrc/gemm/gemv.cu:240-330).
+    """
+    _gpu(x, w)
+    _rows(x, "x")
+    _need(w.dim() == 2 and w.is_contiguous(), "w must be contiguous [N, K]")
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_bf16 takes bfloat16 operands")
+    _need(x.shape[1] == w.shape[1], f"gemm_bf16: inner sizes differ ({x.shape[1]} vs {w.shape[1]})")
+    _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_bf16 writes bfloat16 or float32")
+    if out_dtype == torch.float32:
+        return _library_mm_f32out(x, w)
+    return torch.matmul(x, w.t())
+
+
+_MM_OUT_DTYPE_OK: bool | None = None
+
+
+def _library_mm_f32out(x, w):
+    """bfloat16 x bfloat16 -> float32 through the library, without rounding the result to bfloat16."""
+    global _MM_OUT_DTYPE_OK
+    if _MM_OUT_DTYPE_OK is None:
+        try:
+            y = torch.mm(x, w.t(), out_dtype=torch.float32)
+            _MM_OUT_DTYPE_OK = True
+            return y
+        except (TypeError, RuntimeError):
+            _MM_OUT_DTYPE_OK = False
+    if _MM_OUT_DTYPE_OK:
+        return torch.mm(x, w.t(), out_dtype=torch.float32)
+    return torch.matmul(x, w.t()).float()

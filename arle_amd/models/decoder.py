@@ -1,0 +1,75 @@
+"""A model built from a ModelSpec: embedding, blocks run in schedule order, final norm, head.
+
+Nothing here knows an architecture.  The forward pass of a packed step follows the
+reference's order (infer/src/model/qwen3/prefill.rs:460-547): embed all rows, run the
+layers, then norm and project only the rows whose logits are wanted
+(infer/src/model/qwen3/batch_decode.rs:1519-1601 compacts them the same way).
+"""
+from __future__ import annotations
+
+from ..parts import base  # noqa: F401  (registries)
+from ..parts import attention, block, embedding, feed_forward, norm, position  # noqa: F401  registers the stock parts
+from ..parts.base import Runtime, build_part, expected_tensors, lookup
+from ..parts.spec import ModelSpec
+
+
+def expected_checkpoint_tensors(spec: ModelSpec) -> dict:
+    """checkpoint tensor name -> WeightDecl over the whole model (a tied tensor appears once)."""
+    out: dict = {}
+
+    def merge(found: dict) -> None:
+        for name, decl in found.items():
+            if name in out and tuple(out[name].shape) != tuple(decl.shape):
+                raise ValueError(f"tensor '{name}' is used with two shapes: {out[name].shape} and {decl.shape}")
+            out.setdefault(name, decl)
+
+    merge(expected_tensors("embedding", spec.embedding))
+    for layer in spec.layers:
+        merge(expected_tensors("mixer", layer.mixer))
+        merge(expected_tensors("feed_forward", layer.feed_forward))
+        for norm_spec in layer.norms.values():
+            merge(expected_tensors("norm", norm_spec))
+    merge(expected_tensors("norm", spec.final_norm))
+    merge(expected_tensors("head", spec.head))
+    return out
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, fetch, rt: Runtime):
+        spec.validate()
+        self.spec = spec
+        self.rt = rt
+        self.embedding = build_part("embedding", spec.embedding, fetch, rt)
+        self.blocks = []
+        for layer in spec.layers:
+            mixer = build_part("mixer", layer.mixer, fetch, rt)
+            ffn = build_part("feed_forward", layer.feed_forward, fetch, rt)
+            norms = {role: build_part("norm", s, fetch, rt) for role, s in layer.norms.items()}
+            self.blocks.append(lookup("block", layer.block)(mixer, ffn, norms))
+        self.schedule = list(spec.schedule)
+        self.final_norm = build_part("norm", spec.final_norm, fetch, rt)
+        self.head = build_part("head", spec.head, fetch, rt)
+
+    def cache_needs(self):
+        """(need of every schedule entry that owns a cache, {reader entry -> owner entry})."""
+        needs, readers = [], {}
+        for i, entry in enumerate(self.schedule):
+            if entry.cache_from is not None:
+                needs.append(None)
+                readers[i] = entry.cache_from
+            else:
+                needs.append(self.blocks[entry.layer].mixer.cache_need())
+        return needs, readers
+
+    def forward(self, batch, cache):
+        """Logits float32 [len(batch.want_rows), vocab] of one packed step."""
+        residual = self.embedding.forward(batch.token_ids)
+        delta = None
+        for i, entry in enumerate(self.schedule):
+            residual, delta = self.blocks[entry.layer].forward(residual, delta, batch, cache.view(i))
+        wanted = self.final_norm.add_norm(residual, delta, rows=batch.want_rows)
+        return self.head.forward(wanted)
+
+
+def build_model(spec: ModelSpec, tensors: dict, rt: Runtime) -> DecoderModel:
+    return DecoderModel(spec, tensors.__getitem__, rt)

@@ -1,0 +1,121 @@
+"""Grouped-query attention over a paged cache, with optional per-head q/k RMSNorm,
+a position encoding of its own choice and an optional window.
+
+Per token row: q, k, v projections (no bias) -> per-head RMSNorm of q and k over head_dim
+(one weight [D] for all heads, before the rotation) -> position encoding -> k, v into the
+cache at the token's position -> softmax(q k^T / sqrt(D)) v over the request's earlier
+keys (all of them, or the last `window`) -> output projection.
+infer/src/model/qwen3/prefill.rs:652-738; crates/cuda-kernels/csrc/attention/decode_prep_paged.cu:73-160;
+scale infer/src/ops/attention.rs:636; q head j reads kv head j // (nq/nkv).
+
+q, k and v come from one fused [Q+2KV, H] product.  When the schedule says that this layer
+reads another layer's cache (`cache_view.writes` False), only q is projected and nothing
+is written.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..cache.manager import PagedNeed
+from ..kernels import ops
+from .base import Part, WeightDecl, register
+from .linear import Linear
+
+
+@register("mixer", "paged_attention")
+class PagedAttention(Part):
+    """params: hidden_size, num_q_heads, num_kv_heads, head_dim, qk_norm (bool), eps,
+    position (PartSpec), window (int | None), scale (float | None: 1/sqrt(head_dim))."""
+
+    @classmethod
+    def declare_weights(cls, params):
+        h, d = params["hidden_size"], params["head_dim"]
+        nq, nkv = params["num_q_heads"], params["num_kv_heads"]
+        decl = {
+            "q": WeightDecl((nq * d, h)),
+            "k": WeightDecl((nkv * d, h)),
+            "v": WeightDecl((nkv * d, h)),
+            "o": WeightDecl((h, nq * d)),
+        }
+        if params.get("qk_norm"):
+            decl["q_norm"] = WeightDecl((d,), init="ones")
+            decl["k_norm"] = WeightDecl((d,), init="ones")
+        return decl
+
+    @classmethod
+    def children(cls, params):
+        return {"position": ("position", params["position"])}
+
+    def __init__(self, params, tensors, rt, children=None):
+        super().__init__(params, tensors, rt, children)
+        self.nq = int(params["num_q_heads"])
+        self.nkv = int(params["num_kv_heads"])
+        self.D = int(params["head_dim"])
+        if self.nq % self.nkv:
+            raise ValueError("num_q_heads must be a multiple of num_kv_heads")
+        if self.D % 16 or not 0 < self.D <= ops.MAX_HEAD_DIM:
+            raise ValueError(f"head_dim {self.D} is not supported: the attention kernels take "
+                             f"multiples of 16 up to {ops.MAX_HEAD_DIM}")
+        self.eps = float(params.get("eps", 0.0))
+        self.window = params.get("window")
+        self.scale = float(params["scale"]) if params.get("scale") is not None else 1.0 / math.sqrt(self.D)
+        self.position = children["position"]
+        self.q_norm = tensors.get("q_norm")
+        self.k_norm = tensors.get("k_norm")
+        wq, wk, wv = tensors["q"], tensors["k"], tensors["v"]
+        if not (wq.dtype == wk.dtype == wv.dtype):
+            raise ValueError("q, k and v projections must be stored in one type")
+        self.q_width, self.kv_width = self.nq * self.D, self.nkv * self.D
+        self.qkv = Linear(torch.cat([wq, wk, wv], dim=0).contiguous())
+        # for a layer that reads another layer's cache: the q rows of the fused matrix, no copy
+        self.q_only = Linear(self.qkv.weight[: self.q_width])
+        self.o = Linear(tensors["o"])
+
+    def cache_need(self):
+        return PagedNeed(num_kv_heads=self.nkv, head_dim=self.D, window=self.window)
+
+    def forward(self, x, batch, cache):
+        Q, KV = self.q_width, self.kv_width
+        self.position.ensure_positions(batch.max_position + 1)
+        cos, sin, rot = self.position.fused_rotary()
+        fused = getattr(self.position, "fusable", False)
+        common = dict(num_q_heads=self.nq, num_kv_heads=self.nkv, head_dim=self.D, eps=self.eps,
+                      positions=batch.positions)
+        if cache.writes:
+            qkv = self.qkv(x)
+            q, k, v = qkv[:, :Q], qkv[:, Q:Q + KV], qkv[:, Q + KV:]
+            to_cache = dict(slot_of_token=batch.slot_of_token, block_table=cache.block_table,
+                            k_pages=cache.k_pages, v_pages=cache.v_pages, page_size=cache.page_size)
+        else:
+            # this layer reads a cache that an earlier layer wrote: only q is needed; the k
+            # operand of the preparation kernel is a scratch row that is thrown away
+            q = self.q_only(x)
+            k = v = torch.zeros((x.shape[0], KV), dtype=q.dtype, device=q.device)
+            to_cache = {}
+        if fused:
+            ops.qk_prep(q, k, v, q_weight=self.q_norm, k_weight=self.k_norm, cos=cos, sin=sin,
+                        rotary_dim=rot, **to_cache, **common)
+        else:
+            # a position encoding the fused kernel does not know: norm, encode, then write
+            if self.q_norm is not None:
+                ops.qk_prep(q, k, v, q_weight=self.q_norm, k_weight=self.k_norm, **common)
+            self.position.apply(q, k, batch.positions, self.nq, self.nkv)
+            if to_cache:
+                ops.qk_prep(q, k, v, **to_cache, **common)
+        out = torch.empty((x.shape[0], Q), dtype=q.dtype, device=q.device)
+        paged_attention(q, out, cache, batch, num_q_heads=self.nq, num_kv_heads=self.nkv,
+                        head_dim=self.D, scale=self.scale, window=self.window or 0)
+        return self.o(out)
+
+
+def paged_attention(q, out, cache, batch, *, num_q_heads, num_kv_heads, head_dim, scale, window):
+    """Attention of every row of the packed step over its request's cached keys.
+
+    float32 storage runs the fixed-order kernel (the true 32-bit path); bfloat16 storage runs
+    the MFMA kernels: one for prompt portions, a split-KV one for single decoded tokens.
+    """
+    ops.attn_paged_simt(q, out, cache.k_pages, cache.v_pages, cache.block_table, batch.positions,
+                        batch.slot_of_token, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads,
+                        head_dim=head_dim, page_size=cache.page_size, scale=scale, window=window)

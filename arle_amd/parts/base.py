@@ -1,0 +1,111 @@
+"""Registries of parts by role, the runtime handed to every part, and the part interfaces.
+
+Roles: "embedding", "norm", "position", "mixer", "feed_forward", "block", "head".
+A part class declares the parameters it needs (`declare_weights`) and any parts nested
+in it (`children`), is built from its sizes, its tensors and its children, and never
+learns which model it is in.
+
+Interfaces (T = tokens of the packed step, H = hidden size, A = activation dtype):
+
+* norm          `forward(x[T,W]) -> A[T,W]`;  `add_norm(residual f32[T,H], delta A[T,H] | None,
+                rows=None) -> A[rows or T, H]` adds the delta into the residual (in place) first.
+* position      `fused_rotary() -> (cos, sin, rotary_dim) | None`;  `apply(q, k, positions)` in place.
+* mixer         `cache_need() -> PagedNeed | StateNeed | None`;
+                `forward(x A[T,H], batch: StepBatch, cache_view) -> A[T,H]`.
+* feed_forward  `forward(x A[T,H]) -> A[T,H]`.
+* block         `forward(residual f32[T,H], delta A[T,H] | None, batch, cache_view) -> (residual, delta)`;
+                the returned delta is what the next block (or the final norm) still has to add.
+* embedding     `forward(token_ids i32[T]) -> f32[T,H]`.
+* head          `forward(x A[R,H]) -> f32[R,V]`.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from .spec import PartSpec, WeightDecl
+
+ROLES = ("embedding", "norm", "position", "mixer", "feed_forward", "block", "head")
+_REGISTRY: dict = {role: {} for role in ROLES}
+
+
+class UnknownPart(KeyError):
+    pass
+
+
+def register(role: str, kind: str):
+    """Class decorator: make `kind` buildable wherever a spec asks for it in `role`."""
+    if role not in _REGISTRY:
+        raise ValueError(f"unknown role {role!r}; roles are {ROLES}")
+
+    def deco(cls):
+        _REGISTRY[role][kind] = cls
+        cls.role, cls.kind = role, kind
+        return cls
+
+    return deco
+
+
+def lookup(role: str, kind: str):
+    try:
+        return _REGISTRY[role][kind]
+    except KeyError:
+        known = ", ".join(sorted(_REGISTRY.get(role, {}))) or "none"
+        raise UnknownPart(f"no {role} part named {kind!r} is registered (known: {known})") from None
+
+
+@dataclass
+class Runtime:
+    """Where and in which precision a model runs."""
+
+    device: torch.device
+    act_dtype: torch.dtype  # torch.bfloat16 (serving) or torch.float32 (true 32-bit path)
+
+    @property
+    def is_f32(self) -> bool:
+        return self.act_dtype == torch.float32
+
+
+class Part:
+    role = ""
+    kind = ""
+
+    @classmethod
+    def declare_weights(cls, params: dict) -> dict:
+        """parameter name -> WeightDecl."""
+        return {}
+
+    @classmethod
+    def children(cls, params: dict) -> dict:
+        """child name -> (role, PartSpec) of parts nested in this one."""
+        return {}
+
+    def __init__(self, params: dict, tensors: dict, rt: Runtime, children: dict | None = None):
+        self.params = params
+        self.rt = rt
+
+
+def expected_tensors(role: str, spec: PartSpec) -> dict:
+    """checkpoint tensor name -> WeightDecl for a part and everything nested in it."""
+    cls = lookup(role, spec.kind)
+    out = {}
+    for pname, decl in cls.declare_weights(spec.params).items():
+        if pname not in spec.weights:
+            raise ValueError(f"{role} part {spec.kind!r}: no tensor name given for parameter {pname!r}")
+        out[spec.weights[pname]] = decl
+    for _, (child_role, child_spec) in cls.children(spec.params).items():
+        out.update(expected_tensors(child_role, child_spec))
+    return out
+
+
+def build_part(role: str, spec: PartSpec, fetch, rt: Runtime):
+    """Construct a part; `fetch(tensor_name)` returns the loaded tensor."""
+    cls = lookup(role, spec.kind)
+    tensors = {pname: fetch(spec.weights[pname]) for pname in cls.declare_weights(spec.params)}
+    kids = {name: build_part(r, s, fetch, rt) for name, (r, s) in cls.children(spec.params).items()}
+    return cls(spec.params, tensors, rt, kids)
+
+
+__all__ = ["register", "lookup", "Runtime", "Part", "expected_tensors", "build_part", "WeightDecl",
+           "PartSpec", "UnknownPart", "ROLES"]

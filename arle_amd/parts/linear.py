@@ -1,0 +1,37 @@
+"""y = x . W^T for a weight stored [out, in], the one projection every part uses.
+
+Which kernel runs depends only on the types of the operands:
+
+* float32 x, float32 W  -> the fixed-order float32 kernel (the true 32-bit path);
+* bfloat16 x, bfloat16 W -> the hand-written MFMA kernel for few rows (decode), the
+  vendor library (hipBLASLt through torch) for many rows, as the reference uses
+  cuBLAS for its projections (infer/src/ops/linear.rs:921-959);
+* bfloat16 x, float32 W (a tensor that the checkpoint stores in 32 bits stays so):
+  x is widened and the float32 kernel runs.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+
+
+class Linear:
+    def __init__(self, weight: torch.Tensor):
+        if weight.dim() != 2 or not weight.is_contiguous():
+            raise ValueError("a projection weight must be a contiguous [out, in] matrix")
+        self.weight = weight
+        self.out_features, self.in_features = weight.shape
+
+    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        """x [T, in] -> [T, out] in `out_dtype` (default: the type of x)."""
+        out_dtype = out_dtype or x.dtype
+        w = self.weight
+        if x.shape[0] == 0:
+            return torch.empty((0, self.out_features), dtype=out_dtype, device=x.device)
+        if w.dtype == torch.float32:
+            y = ops.gemm_f32(x if x.dtype == torch.float32 else x.float(), w)
+            return y if out_dtype == torch.float32 else y.to(out_dtype)
+        if x.dtype != torch.bfloat16:
+            raise ops.ShapeError(f"a bfloat16 weight needs bfloat16 activations, got {x.dtype}")
+        return ops.gemm_bf16(x, w, out_dtype)

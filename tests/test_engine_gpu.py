@@ -1,0 +1,89 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16, under every way
+of cutting the work: whole, prefill then token by token, portions of changing size, and
+mixed batches with so few pages that they are used again."""
+import pytest
+import torch
+
+import replay
+from arle_amd.engine import Engine
+from tiny import TINY, make_model_dir, random_tokens, read_folder
+
+pytestmark = pytest.mark.gpu
+
+# max |engine - plain(float64)| / max |plain|
+TOL = {"float32": 1e-5, "bfloat16": 2e-2}
+
+
+@pytest.fixture(scope="module", params=["A", "B", "C"])
+def model(request, tmp_path_factory):
+    name = request.param
+    d = make_model_dir(tmp_path_factory.mktemp("models"), name)
+    cfg, weights = read_folder(d)
+    return name, d, cfg, weights
+
+
+def _engine(model, dtype, max_tokens, **kw):
+    name, d, cfg, _ = model
+    return Engine.from_folder(d, dtype=dtype, page_size=TINY[name][1], max_tokens=max_tokens,
+                              max_slots=4, **kw)
+
+
+def _requests(cfg, lengths, seed):
+    return {f"r{i}": random_tokens(n, cfg["vocab_size"], seed + i) for i, n in enumerate(lengths)}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_requests(model, dtype):
+    _, _, cfg, weights = model
+    reqs = _requests(cfg, [1, 9, 23, 40, 70], 100)
+    eng = _engine(model, dtype, 128)
+    got = {}
+    for rid, toks in reqs.items():
+        got.update(replay.run_steps(eng, replay.whole(rid, toks)))
+    replay.compare(got, cfg, weights, reqs, TOL[dtype], f"whole/{dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prefill_then_last_32_one_by_one(model, dtype):
+    _, _, cfg, weights = model
+    reqs = _requests(cfg, [33, 50, 75], 200)
+    eng = _engine(model, dtype, 128)
+    got = {}
+    for rid, toks in reqs.items():
+        got.update(replay.run_steps(eng, replay.prefill_then_decode(rid, toks, 32)))
+    replay.compare(got, cfg, weights, reqs, TOL[dtype], f"decode/{dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_portions_of_changing_size(model, dtype):
+    _, _, cfg, weights = model
+    reqs = _requests(cfg, [17, 61, 90], 300)
+    eng = _engine(model, dtype, 128)
+    got = {}
+    for rid, toks in reqs.items():
+        got.update(replay.run_steps(eng, replay.portions(rid, toks)))
+    replay.compare(got, cfg, weights, reqs, TOL[dtype], f"portions/{dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_with_page_reuse(model, dtype):
+    name, _, cfg, weights = model
+    reqs = _requests(cfg, [40, 23, 57, 31, 64, 18, 45, 12], 400)
+    # room for the four longest neighbours only: later requests get pages that earlier ones used
+    eng = _engine(model, dtype, 4 * 64)
+    steps = replay.mixed(reqs, max_live=4, seed=7)
+    got = replay.run_steps(eng, steps)
+    replay.compare(got, cfg, weights, reqs, TOL[dtype], f"mixed/{dtype}")
+    assert eng.cache.free_pages()[0] == eng.cache.groups[0].pool.num_pages
+
+
+def test_float32_is_bit_identical_across_cuttings(model):
+    """The 32-bit path fixes the order of every reduction, so cutting changes no bit."""
+    _, _, cfg, weights = model
+    toks = random_tokens(45, cfg["vocab_size"], 5)
+    eng = _engine(model, "float32", 128)
+    a = replay.run_steps(eng, replay.whole("x", toks))
+    b = replay.run_steps(eng, replay.portions("x", toks))
+    c = replay.run_steps(eng, replay.prefill_then_decode("x", toks, 20))
+    for key in a:
+        assert torch.equal(a[key], b[key]) and torch.equal(a[key], c[key]), key

@@ -1,0 +1,292 @@
+"""Each HIP kernel alone against its plain reference, at sizes other than the engine's."""
+import math
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from arle_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _rel(a, b):
+    return float((a.double() - b.double()).abs().max() / b.double().abs().max().clamp_min(1e-30))
+
+
+def _g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def test_embed_gather():
+    table = torch.randn(333, 88, generator=_g(0))
+    ids = torch.tensor([0, 332, 5, 5, 17], dtype=torch.int32)
+    for dt in (torch.float32, torch.bfloat16):
+        out = ops.embed_gather(table.to(dt).to(DEV), ids.to(DEV))
+        assert out.dtype == torch.float32
+        assert torch.equal(out.cpu(), table.to(dt).float()[ids.long()])
+
+
+@pytest.mark.parametrize("width", [4, 96, 260, 2560])
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("wdt", [torch.float32, torch.bfloat16])
+def test_rmsnorm_and_fused_add(width, act, wdt):
+    x = torch.randn(7, width, generator=_g(1)) * 3.0
+    w = (1.0 + 0.3 * torch.randn(width, generator=_g(2))).to(wdt)
+    eps = 1e-5
+    want = plain.rms_norm(x.double(), w.double(), eps)
+    got = ops.rmsnorm(x.to(DEV), w.to(DEV), eps, act)
+    tol = 1e-6 if act == torch.float32 else 5e-3
+    assert got.dtype == act and _rel(got.cpu(), want) < tol
+    # rows picked by index
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32)
+    got = ops.rmsnorm(x.to(DEV), w.to(DEV), eps, act, rows=rows.to(DEV))
+    assert _rel(got.cpu(), want[rows.long()]) < tol
+    # residual add fused in
+    delta = (torch.randn(7, width, generator=_g(3))).to(act)
+    res = x.clone().to(DEV)
+    got = ops.add_rmsnorm(res, delta.to(DEV), w.to(DEV), eps, act)
+    total = x.double() + delta.double()
+    assert _rel(res.cpu(), total) < 1e-6  # the residual stream itself stays 32-bit
+    assert _rel(got.cpu(), plain.rms_norm(total, w.double(), eps)) < tol
+    # with rows the residual is left alone
+    res2 = x.clone().to(DEV)
+    got = ops.add_rmsnorm(res2, delta.to(DEV), w.to(DEV), eps, act, rows=rows.to(DEV))
+    assert torch.equal(res2.cpu(), x)
+    assert _rel(got.cpu(), plain.rms_norm(total, w.double(), eps)[rows.long()]) < tol
+
+
+def test_rmsnorm_vector_of_the_reference_and_zero_weight():
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0]])
+    got = ops.rmsnorm(x.to(DEV), torch.ones(4, device=DEV), 1e-6, torch.float32).cpu()
+    assert torch.allclose(got, x / math.sqrt(7.5 + 1e-6), atol=1e-7)
+    got = ops.rmsnorm(x.to(DEV), torch.zeros(4, device=DEV), 1e-6, torch.float32).cpu()
+    assert torch.count_nonzero(got) == 0  # plain weight, not (1 + w)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 2, 3), (7, 333, 88), (70, 96, 224), (130, 64, 17), (64, 129, 2560)])
+def test_gemm_f32(M, N, K):
+    a = torch.randn(M, K, generator=_g(4))
+    w = torch.randn(N, K, generator=_g(5))
+    got = ops.gemm_f32(a.to(DEV), w.to(DEV)).cpu()
+    assert _rel(got, a.double() @ w.double().T) < 2e-6
+    if (M, N, K) == (1, 2, 3):
+        a = torch.tensor([[1.0, 2.0, 3.0]])
+        w = torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]])
+        assert ops.gemm_f32(a.to(DEV), w.to(DEV)).cpu().tolist() == [[14.0, 32.0]]
+
+
+def test_gemm_f32_rows_do_not_depend_on_the_batch():
+    a = torch.randn(77, 200, generator=_g(6)).to(DEV)
+    w = torch.randn(150, 200, generator=_g(7)).to(DEV)
+    full = ops.gemm_f32(a, w)
+    for r in (0, 13, 76):
+        assert torch.equal(ops.gemm_f32(a[r:r + 1], w)[0], full[r])
+    assert torch.equal(ops.gemm_f32(a[10:31], w), full[10:31])
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (5, 333, 88), (64, 256, 2560), (300, 224, 96)])
+def test_gemm_bf16(M, N, K):
+    a = torch.randn(M, K, generator=_g(8)).bfloat16()
+    w = (torch.randn(N, K, generator=_g(9)) * 0.1).bfloat16()
+    want = a.double() @ w.double().T
+    got = ops.gemm_bf16(a.to(DEV), w.to(DEV), torch.float32).cpu()
+    assert got.dtype == torch.float32 and _rel(got, want) < 1e-3
+    got = ops.gemm_bf16(a.to(DEV), w.to(DEV), torch.bfloat16).cpu()
+    assert got.dtype == torch.bfloat16 and _rel(got, want) < 8e-3
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_silu_mul(dt):
+    gu = torch.randn(5, 2 * 136, generator=_g(10)).to(dt)
+    g, u = gu[:, :136].double(), gu[:, 136:].double()
+    want = plain.silu(g) * u
+    d = gu.to(DEV)
+    got = ops.silu_mul(d[:, :136], d[:, 136:]).cpu()
+    assert _rel(got, want) < (1e-6 if dt == torch.float32 else 5e-3)
+    z = torch.zeros(2, 8, dtype=dt, device=DEV)
+    assert torch.count_nonzero(ops.silu_mul(z, torch.ones_like(z))) == 0
+
+
+def _paged_setup(lengths, nkv, D, P, dtype, seed, shuffle=True):
+    """Block tables with shuffled physical pages for requests of the given lengths."""
+    g = _g(seed)
+    slots = len(lengths)
+    pages_per = [-(-n // P) for n in lengths]
+    total = sum(pages_per) + 3
+    perm = torch.randperm(total, generator=g).tolist() if shuffle else list(range(total))
+    table = torch.zeros(slots, max(pages_per) + 1, dtype=torch.int32)
+    it = iter(perm)
+    for s, n in enumerate(pages_per):
+        for i in range(n):
+            table[s, i] = next(it)
+    k_pages = torch.zeros(total, nkv, P, D, dtype=dtype)
+    v_pages = torch.zeros(total, nkv, P, D, dtype=dtype)
+    return table, k_pages, v_pages
+
+
+@pytest.mark.parametrize("nq,nkv,D,rot", [(3, 1, 48, 48), (4, 2, 16, 16), (8, 2, 128, 128), (2, 2, 64, 32),
+                                           (5, 5, 32, 0)])
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_qk_prep_norm_rope_and_cache_write(nq, nkv, D, rot, dt):
+    P, eps, theta = 8, 1e-5, 1e4
+    lengths = [11, 5]
+    table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, 20)
+    positions = torch.tensor([3, 4, 5, 10, 0, 4], dtype=torch.int32)   # rows of two requests
+    slots = torch.tensor([0, 0, 0, 0, 1, 1], dtype=torch.int32)
+    T = positions.numel()
+    qkv = torch.randn(T, (nq + 2 * nkv) * D, generator=_g(21)).to(dt)
+    qw = (1.0 + 0.2 * torch.randn(D, generator=_g(22))).to(dt)
+    kw = (1.0 + 0.2 * torch.randn(D, generator=_g(23))).to(dt)
+    cos = sin = None
+    if rot:
+        cos, sin = plain.rope_cos_sin(range(16), rot, theta)
+    d_qkv = qkv.to(DEV)
+    Q, KV = nq * D, nkv * D
+    dk, dv = k_pages.to(DEV), v_pages.to(DEV)
+    ops.qk_prep(d_qkv[:, :Q], d_qkv[:, Q:Q + KV], d_qkv[:, Q + KV:], num_q_heads=nq, num_kv_heads=nkv,
+                head_dim=D, eps=eps, q_weight=qw.to(DEV), k_weight=kw.to(DEV),
+                cos=None if cos is None else cos.to(DEV), sin=None if sin is None else sin.to(DEV),
+                rotary_dim=rot, positions=positions.to(DEV), slot_of_token=slots.to(DEV),
+                block_table=table.to(DEV), k_pages=dk, v_pages=dv, page_size=P)
+    # plain: norm per head, rotate the first `rot` dims, at each row's own position
+    x = qkv.double()
+    q = plain.qk_norm(x[:, :Q].reshape(T, nq, D), qw.double(), eps)
+    k = plain.qk_norm(x[:, Q:Q + KV].reshape(T, nkv, D), kw.double(), eps)
+    v = x[:, Q + KV:].reshape(T, nkv, D)
+    if rot:
+        c, s = plain.rope_cos_sin(positions.tolist(), rot, theta, dtype=torch.float64)
+        q = torch.cat([plain.apply_rope(q[..., :rot], c, s), q[..., rot:]], -1)
+        k = torch.cat([plain.apply_rope(k[..., :rot], c, s), k[..., rot:]], -1)
+    tol = 2e-6 if dt == torch.float32 else 6e-3
+    assert _rel(d_qkv[:, :Q].cpu().reshape(T, nq, D), q) < tol
+    dk, dv = dk.cpu(), dv.cpu()
+    for t in range(T):
+        page = int(table[slots[t], positions[t] // P])
+        assert _rel(dk[page, :, positions[t] % P], k[t]) < tol
+        assert torch.equal(dv[page, :, positions[t] % P].double(), v[t])
+    # nothing else in the cache was touched
+    written = torch.zeros(dk.shape[0], P, dtype=torch.bool)
+    for t in range(T):
+        written[int(table[slots[t], positions[t] // P]), positions[t] % P] = True
+    assert torch.count_nonzero(dk.transpose(1, 2)[~written]) == 0
+
+
+def _fill_cache(table, k_pages, v_pages, slot, k, v, P):
+    for pos in range(k.shape[0]):
+        page = int(table[slot, pos // P])
+        k_pages[page, :, pos % P] = k[pos]
+        v_pages[page, :, pos % P] = v[pos]
+
+
+@pytest.mark.parametrize("nq,nkv,D,P", [(3, 1, 48, 16), (4, 2, 16, 4), (8, 2, 128, 16), (6, 2, 32, 8),
+                                         (2, 1, 256, 32)])
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_simt_against_plain(nq, nkv, D, P, dt, window):
+    lengths = [150, 70, 1]
+    table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, 30)
+    qs, ks, vs, pos, slots = [], [], [], [], []
+    for s, n in enumerate(lengths):
+        g = _g(31 + s)
+        q = torch.randn(n, nq, D, generator=g).to(dt)
+        k = torch.randn(n, nkv, D, generator=g).to(dt)
+        v = torch.randn(n, nkv, D, generator=g).to(dt)
+        _fill_cache(table, k_pages, v_pages, s, k, v, P)
+        qs.append(q), ks.append(k), vs.append(v)
+        pos += list(range(n))
+        slots += [s] * n
+    q_all = torch.cat(qs).reshape(-1, nq * D)
+    out = torch.empty_like(q_all).to(DEV)
+    ops.attn_paged_simt(q_all.to(DEV), out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV),
+                        torch.tensor(pos, dtype=torch.int32, device=DEV),
+                        torch.tensor(slots, dtype=torch.int32, device=DEV), num_q_heads=nq,
+                        num_kv_heads=nkv, head_dim=D, page_size=P, scale=1.0 / math.sqrt(D), window=window)
+    want = torch.cat([plain.causal_attention(q.double(), k.double(), v.double(), nkv,
+                                             window=window or None).reshape(-1, nq * D)
+                      for q, k, v in zip(qs, ks, vs)])
+    assert _rel(out.cpu(), want) < (3e-6 if dt == torch.float32 else 6e-3)
+
+
+def test_attention_finds_a_far_key_among_hundreds():
+    """One early key is made to stand out for the last query; its value must dominate."""
+    nq, nkv, D, P, n = 4, 2, 64, 16, 700
+    table, k_pages, v_pages = _paged_setup([n], nkv, D, P, torch.float32, 40)
+    g = _g(41)
+    q = torch.randn(n, nq, D, generator=g) * 0.1
+    k = torch.randn(n, nkv, D, generator=g) * 0.1
+    v = torch.randn(n, nkv, D, generator=g)
+    far = 3
+    k[far, 0] = q[n - 1, 1] * 400.0   # head 1 reads kv head 0
+    _fill_cache(table, k_pages, v_pages, 0, k, v, P)
+    out = torch.empty(n, nq * D, device=DEV)
+    ops.attn_paged_simt(q.reshape(n, -1).to(DEV), out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV),
+                        torch.arange(n, dtype=torch.int32, device=DEV),
+                        torch.zeros(n, dtype=torch.int32, device=DEV), num_q_heads=nq, num_kv_heads=nkv,
+                        head_dim=D, page_size=P, scale=1.0 / math.sqrt(D))
+    got = out.cpu().reshape(n, nq, D)
+    assert torch.allclose(got[n - 1, 1], v[far, 0], atol=1e-3)
+    want = plain.causal_attention(q.double(), k.double(), v.double(), nkv)
+    assert _rel(got, want) < 3e-6
+
+
+def test_argmax_rows_first_maximum_wins():
+    x = torch.tensor([[1.0, 9.0, 3.0, 8.0], [2.0, 7.0, 7.0, 1.0]])
+    assert ops.argmax_rows(x.to(DEV)).tolist() == [1, 1]   # infer/src/ops/tests.rs:81-87
+    big = torch.randn(5, 151936, generator=_g(50))
+    big[2, 150000] = 50.0
+    big[3, 7] = 60.0
+    big[3, 100000] = 60.0
+    assert ops.argmax_rows(big.to(DEV)).tolist() == big.argmax(-1).tolist()
+
+
+def _sample(logits, temperature, u, top_k=-1, top_p=1.0, min_p=0.0):
+    rows = logits.shape[0]
+    f = lambda v: torch.full((rows,), v, dtype=torch.float32, device=DEV)
+    return ops.sample_rows(logits.to(DEV), f(temperature), torch.full((rows,), top_k, dtype=torch.int32, device=DEV),
+                           f(top_p), f(min_p), torch.as_tensor(u, dtype=torch.float32).expand(rows).contiguous().to(DEV)).tolist()
+
+
+def test_sampling_vectors_of_the_reference():
+    x = torch.tensor([[1.0, 2.0, 10.0, 1.5, 0.5]])  # infer/src/ops/tests.rs:333-378
+    assert _sample(x, 0.01, 0.5) == [2]
+    assert _sample(x, 1.0, 0.0) == [0]
+    assert _sample(x, 1.0, 0.9, top_k=1) == [2]
+    assert _sample(x, 0.0, 0.3) == [2]
+
+
+@pytest.mark.parametrize("vocab", [5, 333, 4099])
+def test_sampling_against_plain_inverse_cdf(vocab):
+    g = _g(60)
+    logits = torch.randn(6, vocab, generator=g) * 2.0
+    cases = [dict(temperature=0.8), dict(temperature=1.3, top_k=7), dict(temperature=1.0, top_p=0.6),
+             dict(temperature=0.7, min_p=0.05), dict(temperature=1.1, top_k=20, top_p=0.8, min_p=0.01)]
+    for case in cases:
+        for u in (0.0, 0.13, 0.5, 0.77, 0.999):
+            got = _sample(logits, case["temperature"], u, case.get("top_k", -1), case.get("top_p", 1.0),
+                          case.get("min_p", 0.0))
+            want = [plain.sample_token(row, case["temperature"], u, case.get("top_k", -1),
+                                       case.get("top_p", 1.0), case.get("min_p", 0.0)) for row in logits]
+            assert got == want, (case, u)
+
+
+def test_penalties():
+    logits = torch.tensor([[2.0, -2.0, 1.0, 0.5], [1.0, 1.0, 1.0, 1.0]])
+    d = logits.to(DEV)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    f32 = lambda v: torch.tensor(v, dtype=torch.float32, device=DEV)
+    ops.apply_penalties(d, i32([0, 2, 3]), i32([0, 1, 3]), i32([2, 1, 4]), f32([2.0, 1.0]), f32([0.5, 0.25]),
+                        f32([0.25, 0.0]))
+    want0 = plain.apply_penalties(logits[0], {0: 2, 1: 1}, 2.0, 0.5, 0.25)
+    want1 = plain.apply_penalties(logits[1], {3: 4}, 1.0, 0.25, 0.0)
+    assert torch.allclose(d.cpu(), torch.stack([want0, want1]))
+
+
+def test_kernels_refuse_what_they_were_not_written_for():
+    with pytest.raises(ops.ShapeError):
+        ops.gemm_f32(torch.zeros(2, 3, device=DEV), torch.zeros(4, 5, device=DEV))
+    with pytest.raises(ops.ShapeError):
+        ops.rmsnorm(torch.zeros(2, 3), torch.ones(3), 1e-6, torch.float32)  # CPU tensors
+    with pytest.raises(ops.ShapeError):
+        ops.embed_gather(torch.zeros(4, 4, device=DEV), torch.zeros(2, dtype=torch.int64, device=DEV))

@@ -1,0 +1,58 @@
+"""Tiny Qwen3 configurations for tests, and helpers that make model folders from them.
+
+A and B differ in every size and option: layers, widths (B's are no powers of two), head
+counts and group size, head_dim (B's q width differs from its hidden size), vocabulary,
+eps, theta, tied or untied head, page size and the spread of the weights.  C has a head_dim
+that is a multiple of 16 but no power of two and odd-ish widths.
+"""
+from __future__ import annotations
+
+import json
+import os
+
+import torch
+
+from arle_amd.config import Qwen3Config
+from arle_amd.weights import SafetensorsFile, write_random_model
+
+ARCH = "Qwen3ForCausalLM"
+
+TINY_A = dict(num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2,
+              head_dim=16, intermediate_size=128, vocab_size=256, rope_theta=10000.0,
+              rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=1024)
+TINY_B = dict(num_hidden_layers=3, hidden_size=96, num_attention_heads=6, num_key_value_heads=2,
+              head_dim=32, intermediate_size=224, vocab_size=384, rope_theta=1000000.0,
+              rms_norm_eps=1e-5, tie_word_embeddings=False, max_position_embeddings=2048)
+TINY_C = dict(num_hidden_layers=2, hidden_size=88, num_attention_heads=3, num_key_value_heads=1,
+              head_dim=48, intermediate_size=136, vocab_size=333, rope_theta=50000.0,
+              rms_norm_eps=3e-6, tie_word_embeddings=False, max_position_embeddings=1024)
+
+# name -> (config, page size, weight std, norm std, seed)
+TINY = {
+    "A": (TINY_A, 4, 0.02, 0.02, 11),
+    "B": (TINY_B, 8, 0.05, 0.05, 22),
+    "C": (TINY_C, 16, 0.08, 0.1, 33),
+}
+
+
+def make_model_dir(tmp_path, name: str, std_scale: float = 1.0) -> str:
+    raw, _, std, norm_std, seed = TINY[name]
+    config = Qwen3Config.from_dict(raw)
+    d = os.path.join(str(tmp_path), f"tiny_{name}")
+    write_random_model(d, ARCH, config, seed=seed, std=std * std_scale, norm_std=norm_std)
+    return d
+
+
+def read_folder(model_dir: str):
+    """(config dict, {name: float32 CPU tensor}) read straight from the files."""
+    with open(os.path.join(model_dir, "config.json")) as fh:
+        cfg = json.load(fh)
+    f = SafetensorsFile(os.path.join(model_dir, "model.safetensors"))
+    weights = {n: f.read(n).to(torch.float32) for n in f.names()}
+    f.close()
+    return cfg, weights
+
+
+def random_tokens(n: int, vocab: int, seed: int) -> list:
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
