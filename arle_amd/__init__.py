@@ -8,3 +8,17 @@ kernels (`csrc`, `kernels`).
 """
 
 __version__ = "0.1.0"
+
+
+def __getattr__(name):
+    # heavy imports (torch) happen only when the entry points are asked for
+    if name in ("LLM", "generate", "CompletionOutput"):
+        from .engine import api
+        return getattr(api, name)
+    if name in ("Engine", "StepEntry"):
+        from . import engine
+        return getattr(engine, name)
+    if name == "SamplingParams":
+        from .sampling import SamplingParams
+        return SamplingParams
+    raise AttributeError(name)

@@ -1,0 +1,130 @@
+"""The Python entry point: load a model, generate for a list of prompts.
+
+    from arle_amd import LLM
+    llm = LLM("path/to/model")                       # config.json + safetensors
+    outs = llm.generate([[1, 2, 3]], max_tokens=16)  # greedy
+    outs[0].response_token_ids, outs[0].finish_reason, outs[0].usage
+
+Request and result follow the reference's engine facade: `CompletionRequest{prompt,
+max_tokens, sampling, ...}` -> `CompletionOutput{text, finish_reason, usage,
+prompt_token_ids, response_token_ids}` (infer/src/server_engine/types.rs:10-60,147-185).
+Prompts are token ids; text goes through the folder's tokenizer.json when the `tokenizers`
+package and the file are there.
+"""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass, field
+
+from ..sampling import Sampler, SamplingParams
+from .engine import Engine
+from .scheduler import Scheduler, SchedulerConfig
+
+
+@dataclass
+class TokenUsage:
+    prompt_tokens: int
+    completion_tokens: int
+
+    @property
+    def total_tokens(self) -> int:
+        return self.prompt_tokens + self.completion_tokens
+
+
+@dataclass
+class CompletionOutput:
+    text: str | None
+    finish_reason: str            # "length" | "stop"
+    usage: TokenUsage
+    prompt_token_ids: list
+    response_token_ids: list
+    ttft_s: float | None = None   # submit -> first token
+    token_logprobs: list = field(default_factory=list)
+
+
+class LLM:
+    def __init__(self, model, *, dtype="bfloat16", device=None, page_size: int | None = None,
+                 kv_cache_tokens: int | None = None, num_slots: int = 4, max_seq_len: int | None = None,
+                 chunked_prefill_size: int = 512, max_num_batched_tokens: int = 16384,
+                 max_prefill_tokens: int = 16384, prefill_max_requests: int | None = None, seed: int = 42):
+        """model: a model folder, or an Engine that is already built.
+
+        kv_cache_tokens: tokens the paged cache holds over all live requests
+        (default: num_slots * max_seq_len, max_seq_len defaulting to min(model's positions, 4096)).
+        """
+        if isinstance(model, Engine):
+            self.engine = model
+        else:
+            from ..config.registry import load_model_config
+            from .engine import DEFAULT_PAGE_SIZE
+            from .. import models  # noqa: F401
+
+            _, config, _ = load_model_config(model)
+            positions = getattr(config, "max_position_embeddings", 4096)
+            max_seq_len = max_seq_len or min(positions, 4096)
+            kv_cache_tokens = kv_cache_tokens or num_slots * max_seq_len
+            self.engine = Engine.from_folder(model, dtype=dtype, device=device,
+                                             page_size=page_size or DEFAULT_PAGE_SIZE,
+                                             max_tokens=kv_cache_tokens, max_slots=num_slots,
+                                             max_request_tokens=min(max_seq_len, positions))
+        self.model_dir = model if isinstance(model, str) else None
+        self.seed = seed
+        self.sched_config = SchedulerConfig(
+            num_slots=self.engine.cache.max_slots, chunked_prefill_size=chunked_prefill_size,
+            max_num_batched_tokens=max_num_batched_tokens, max_prefill_tokens=max_prefill_tokens,
+            prefill_max_requests=prefill_max_requests, max_seq_len=max_seq_len)
+        self.sampler = Sampler(self.engine.device)
+        self.tokenizer = self._load_tokenizer()
+        self.last_stats: dict = {}
+
+    def _load_tokenizer(self):
+        if not self.model_dir:
+            return None
+        path = os.path.join(self.model_dir, "tokenizer.json")
+        if not os.path.exists(path):
+            return None
+        try:
+            from tokenizers import Tokenizer
+        except ImportError:
+            return None
+        return Tokenizer.from_file(path)
+
+    def tokenize(self, text: str) -> list:
+        if self.tokenizer is None:
+            raise RuntimeError("this model folder has no tokenizer.json (or the `tokenizers` package is "
+                               "missing): give prompts as token ids")
+        return self.tokenizer.encode(text).ids
+
+    def generate(self, prompts, max_tokens: int = 16, temperature: float = 0.0, seed: int | None = None,
+                 ignore_eos: bool = False, sampling: SamplingParams | None = None) -> list:
+        """prompts: a list of token-id lists (or strings, with a tokenizer).  One CompletionOutput each,
+        in order.  `sampling` overrides temperature / seed / ignore_eos when given."""
+        sched = Scheduler(self.engine, self.sampler, self.sched_config, seed=self.seed,
+                          stop_token_ids=self.engine.spec.stop_token_ids)
+        ids = []
+        for p in prompts:
+            toks = self.tokenize(p) if isinstance(p, str) else list(p)
+            params = sampling or SamplingParams(temperature=temperature, seed=seed, ignore_eos=ignore_eos)
+            ids.append(sched.submit(toks, params, max_tokens))
+        sched.run_until_done()
+        self.last_stats = sched.stats
+        outs = []
+        for rid in ids:
+            r = sched.finished[rid]
+            text = self.tokenizer.decode(r.generated) if self.tokenizer is not None else None
+            ttft = (r.t_first_token - r.t_submit) if r.t_first_token is not None else None
+            outs.append(CompletionOutput(text=text, finish_reason=r.finish_reason,
+                                         usage=TokenUsage(len(r.prompt), len(r.generated)),
+                                         prompt_token_ids=list(r.prompt),
+                                         response_token_ids=list(r.generated), ttft_s=ttft))
+        return outs
+
+
+def generate(model, prompts, max_tokens: int = 16, temperature: float = 0.0, seed: int | None = None,
+             ignore_eos: bool = False, **engine_args) -> list:
+    """One-shot helper: `LLM(model, **engine_args).generate(...)` as plain dictionaries."""
+    llm = model if isinstance(model, LLM) else LLM(model, **engine_args)
+    return [{"token_ids": o.response_token_ids, "finish_reason": o.finish_reason,
+             "usage": {"prompt_tokens": o.usage.prompt_tokens, "completion_tokens": o.usage.completion_tokens,
+                       "total_tokens": o.usage.total_tokens}, "text": o.text}
+            for o in llm.generate(prompts, max_tokens, temperature, seed, ignore_eos)]

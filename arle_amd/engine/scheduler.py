@@ -1,0 +1,342 @@
+"""Continuous batching above the step function: admit, cut prompts into portions under a
+token budget, decode, finish and free -- and what happens when pages run out.
+
+One `iteration()` does, in the reference's order (infer/src/scheduler/cuda/runtime/scheduler_loop.rs:116-199,
+infer/src/scheduler/cuda/execution.rs:385-425,669-800):
+
+1. admission: a waiting request enters when a slot is free and the pool has pages for its
+   prompt + 1 token after the same target of every running request is set aside; decode
+   growth is not reserved (scheduler_loop.rs:202-315, budget.rs:17-33).  A request that does
+   not fit stays in the queue, in order; later ones may still enter.
+2. decode rows: every decoding request brings its last token.  If the pool cannot take one
+   more token of each, the request with the fewest generated tokens (ties: the longest
+   prompt) is preempted until it can (decode.rs:16-21,82-116); a lone request that still
+   does not fit finishes with `length`.
+3. prompt portions under the token budget min(max_num_batched_tokens - decode rows,
+   max_prefill_tokens): per request min(remaining, chunked_prefill_size), also capped by
+   long_prefill_token_threshold while rows are decoding; a portion that does not fit the
+   remaining budget is skipped whole, not shrunk; queue order is the only priority
+   (execution.rs:117-215,265-317, budget.rs:229-264).  Pages: each running decode's remaining
+   growth min(max_tokens - generated, 4096) is set aside first (execution.rs:160-168).
+4. one `Engine.step` with the decode rows first, then the portions; logits are asked only
+   where a token is sampled (the reference computes them for every portion and discards them).
+5. sampling and transitions: a stop token ends the request without being emitted
+   (prefill.rs:426-479, decode.rs:784-808); `max_tokens` ends it with `length`.
+6. finished requests give their pages and slot back.
+
+Kept differently on purpose: a preempted request keeps the tokens it has generated and
+feeds prompt + generated again when it re-enters (the reference drops them and generates
+anew); and decode rows and prompt portions always share one step (the reference's default
+runs two forwards, `Split`).
+"""
+from __future__ import annotations
+
+import time
+from collections import deque
+from dataclasses import dataclass, field
+
+from ..cache.pages import OutOfPages
+from ..sampling.params import SamplingParams
+from .batch import StepEntry
+
+LENGTH, STOP = "length", "stop"
+REQUEST_INPUT_SLACK_TOKENS = 5      # infer/src/scheduler/types.rs:499
+DECODE_RESERVATION_CLIP = 4096      # infer/src/scheduler/cuda/budget.rs:3
+
+
+class SchedulerFull(RuntimeError):
+    pass
+
+
+@dataclass
+class SchedulerConfig:
+    """Names and defaults of infer/src/scheduler/types.rs:63-238 (the flags of `infer`)."""
+
+    num_slots: int = 4
+    chunked_prefill_size: int = 512
+    max_num_batched_tokens: int = 16384
+    max_prefill_tokens: int = 16384
+    prefill_max_requests: int | None = None
+    long_prefill_token_threshold: int = 512
+    max_waiting_requests: int = 256
+    max_seq_len: int | None = None
+
+    def validate(self) -> None:
+        for name in ("num_slots", "chunked_prefill_size", "max_num_batched_tokens",
+                     "max_prefill_tokens", "long_prefill_token_threshold", "max_waiting_requests"):
+            if getattr(self, name) <= 0:
+                raise ValueError(f"{name} must be positive")
+        if self.prefill_max_requests is not None and self.prefill_max_requests <= 0:
+            raise ValueError("prefill_max_requests must be positive when set")
+        if self.max_num_batched_tokens < self.num_slots:
+            raise ValueError("max_num_batched_tokens must hold one decode row per slot")
+
+
+@dataclass
+class Request:
+    id: int
+    prompt: list
+    sampling: SamplingParams
+    max_tokens: int
+    seed: int
+    feed: list = field(default_factory=list)       # tokens that have to pass through the model
+    fed: int = 0                                   # how many of them have
+    generated: list = field(default_factory=list)
+    phase: str = "waiting"                         # waiting | prefilling | decoding | finished
+    finish_reason: str | None = None
+    preemptions: int = 0
+    t_submit: float = 0.0
+    t_first_token: float | None = None
+    t_finish: float | None = None
+
+    @property
+    def remaining_prompt(self) -> int:
+        return len(self.feed) - self.fed
+
+
+@dataclass
+class StepPlan:
+    decode: list          # requests that bring one token
+    prefill: list         # (request, tokens of this portion)
+
+    @property
+    def kind(self) -> str:
+        if self.decode and self.prefill:
+            return "mixed"
+        return "decode" if self.decode else ("prefill" if self.prefill else "idle")
+
+
+def retract_victim(decoding: list):
+    """Fewest generated tokens first; ties: the longest prompt (decode.rs:16-21)."""
+    return min(decoding, key=lambda r: (len(r.generated), -len(r.prompt)))
+
+
+def plan_prefill(queue, decode_rows: int, cfg: SchedulerConfig, fits) -> list:
+    """Pick portions of queued prompts for this step: [(request, tokens)].
+
+    queue: prefilling requests in queue order.  fits(reserved, request, page_tokens) says whether
+    the pool can take `page_tokens` more tokens of `request` on top of `reserved`, the
+    [(request, page_tokens)] of the portions picked before it.
+    """
+    tokens_left = min(max(cfg.max_num_batched_tokens - decode_rows, 0), cfg.max_prefill_tokens)
+    requests_left = cfg.prefill_max_requests if cfg.prefill_max_requests is not None else len(queue)
+    cap = cfg.chunked_prefill_size
+    if decode_rows > 0:
+        cap = min(cap, cfg.long_prefill_token_threshold)
+    picked, reserved = [], []
+    for req in queue:
+        remaining = req.remaining_prompt
+        if remaining <= 0:
+            continue
+        n = min(remaining, max(cap, 1))
+        if n > tokens_left or requests_left <= 0:
+            continue  # skipped whole, never shrunk; a later, smaller one may still fit
+        completes = n == remaining
+        first_decode = 1 if completes and req.max_tokens - len(req.generated) > 0 else 0
+        if not fits(reserved, req, n + first_decode):
+            continue
+        picked.append((req, n))
+        reserved.append((req, n + first_decode))
+        tokens_left -= n
+        requests_left -= 1
+    return picked
+
+
+class Scheduler:
+    def __init__(self, engine, sampler, config: SchedulerConfig | None = None, seed: int = 42,
+                 stop_token_ids=()):
+        self.cfg = config or SchedulerConfig()
+        self.cfg.validate()
+        self.engine = engine
+        self.cache = engine.cache
+        self.sampler = sampler
+        self.seed = seed
+        self.stop_token_ids = set(stop_token_ids)
+        self.waiting: deque = deque()
+        self.prefilling: list = []
+        self.decoding: list = []
+        self.finished: dict = {}
+        self._next_id = 0
+        pool_tokens = min((g.pool.num_pages for g in self.cache.groups), default=1 << 30) * self.cache.page_size
+        context = self.cfg.max_seq_len or pool_tokens
+        context = min(context, self.cache.max_pages_per_request * self.cache.page_size)
+        # infer/src/scheduler/types.rs:511-553
+        self.max_request_len = min(max(context - 1, 0), max(pool_tokens - 1, 0))
+        self.max_request_input_len = max(self.max_request_len - REQUEST_INPUT_SLACK_TOKENS, 0)
+        self.stats = {"steps": {"decode": 0, "prefill": 0, "mixed": 0}, "tokens_prefilled": 0,
+                      "tokens_decoded": 0, "preemptions": 0, "rejected": 0, "pages_high_water": 0}
+
+    # -- intake ---------------------------------------------------------------------------
+    def submit(self, prompt_tokens, sampling: SamplingParams | None = None,
+               max_tokens: int | None = None) -> int:
+        """Queue a request; returns its id.  Rejections finish at once with `length` and no tokens
+        (infer/src/scheduler/cuda/runtime/admission.rs:71-120)."""
+        sampling = sampling or SamplingParams()
+        if len(self.waiting) >= self.cfg.max_waiting_requests:
+            raise SchedulerFull(f"{len(self.waiting)} requests are waiting already")
+        rid = self._next_id
+        self._next_id += 1
+        prompt = [int(t) for t in prompt_tokens]
+        if max_tokens is None:
+            max_tokens = sampling.max_new_tokens if sampling.max_new_tokens is not None else self.max_request_len
+        seed = sampling.seed if sampling.seed is not None else (self.seed * 0x9E3779B1 + rid) & ((1 << 63) - 1)
+        req = Request(rid, prompt, sampling, int(max_tokens), seed, feed=list(prompt), t_submit=time.perf_counter())
+        if not prompt or len(prompt) >= self.max_request_input_len or req.max_tokens <= 0:
+            self.stats["rejected"] += 1
+            self._finish(req, LENGTH)
+            self.finished[rid] = req
+            return rid
+        req.max_tokens = min(req.max_tokens, max(self.max_request_len - len(prompt) - 1, 0))
+        self.waiting.append(req)
+        return rid
+
+    # -- one iteration ------------------------------------------------------------------------
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.prefilling or self.decoding)
+
+    def iteration(self) -> StepPlan:
+        self._admit()
+        plan = self._plan()
+        if plan.kind != "idle":
+            self._run(plan)
+        self._cleanup()
+        return plan
+
+    def run_until_done(self, max_iterations: int = 1 << 30) -> None:
+        idle = 0
+        for _ in range(max_iterations):
+            if not self.has_work():
+                return
+            plan = self.iteration()
+            idle = idle + 1 if plan.kind == "idle" else 0
+            if idle > 2:
+                raise RuntimeError("scheduler makes no progress: a waiting request can never be admitted")
+
+    # -- admission ------------------------------------------------------------------------------
+    def _pages(self, tokens: int) -> int:
+        return -(-tokens // self.cache.page_size)
+
+    def _admit(self) -> None:
+        if not self.waiting:
+            return
+        free = min(self.cache.free_pages(), default=1 << 30)
+        # pages that running requests still need to reach prompt + 1
+        for r in self.prefilling + self.decoding:
+            target = len(r.feed) + 1
+            free -= max(0, self._pages(target) - self._pages(self.cache.length(r.id)))
+        deferred = deque()
+        while self.waiting:
+            req = self.waiting.popleft()
+            need = self._pages(len(req.feed) + 1)
+            if self.cache.free_slot_count == 0 or need > free:
+                deferred.append(req)
+                continue
+            free -= need
+            self.engine.add_request(req.id)
+            req.phase = "prefilling"
+            req.fed = 0
+            self.prefilling.append(req)
+        self.waiting = deferred
+
+    # -- planning -------------------------------------------------------------------------------
+    def _plan(self) -> StepPlan:
+        decode = list(self.decoding)
+        # pages run out while decoding: preempt until one more token of each fits
+        while decode and not self.cache.can_append([(r.id, 1) for r in decode]):
+            if len(decode) == 1:
+                self._finish(decode.pop(), LENGTH)
+                break
+            victim = retract_victim(decode)
+            decode.remove(victim)
+            self._preempt(victim)
+        growth = [(r.id, min(max(r.max_tokens - len(r.generated), 0), DECODE_RESERVATION_CLIP))
+                  for r in decode]
+        growth = [(k, n) for k, n in growth if n > 0]
+
+        def fits(reserved, req, page_tokens):
+            return self.cache.can_append(growth + [(r.id, n) for r, n in reserved] + [(req.id, page_tokens)])
+
+        prefill = plan_prefill(self.prefilling, len(decode), self.cfg, fits)
+        if not decode and not prefill and self.prefilling:
+            # nothing is decoding and no portion fits beside the reservations: the pool is
+            # simply too small for the queue's head portion; try it alone against the free pages
+            req = self.prefilling[0]
+            n = min(req.remaining_prompt, self.cfg.chunked_prefill_size, self.cfg.max_prefill_tokens,
+                    self.cfg.max_num_batched_tokens)
+            if n > 0 and self.cache.can_append([(req.id, n)]):
+                prefill = [(req, n)]
+        return StepPlan(decode, prefill)
+
+    # -- execution --------------------------------------------------------------------------------
+    def _run(self, plan: StepPlan) -> None:
+        entries, sampled = [], []
+        for r in plan.decode:
+            entries.append(StepEntry(r.id, [r.generated[-1]], [0]))
+            sampled.append(r)
+        for r, n in plan.prefill:
+            completes = n == r.remaining_prompt
+            entries.append(StepEntry(r.id, r.feed[r.fed:r.fed + n], [n - 1] if completes else []))
+            if completes:
+                sampled.append(r)
+        try:
+            logits = self.engine.step(entries)
+        except OutOfPages:
+            # planning said it fits; if the pool disagrees, nothing was changed: skip the portions
+            if not plan.prefill:
+                raise
+            return self._run(StepPlan(plan.decode, []))
+        self.stats["steps"][plan.kind] += 1
+        self.stats["tokens_decoded"] += len(plan.decode)
+        self.stats["tokens_prefilled"] += sum(n for _, n in plan.prefill)
+        held = max((g.pool.num_pages - g.pool.free_count for g in self.cache.groups), default=0)
+        self.stats["pages_high_water"] = max(self.stats["pages_high_water"], held)
+        for r, n in plan.prefill:
+            r.fed += n
+        if not sampled:
+            return
+        rows = [(r.sampling, r.seed, len(r.generated), r.generated) for r in sampled]
+        tokens = self.sampler.sample(logits, rows)
+        now = time.perf_counter()
+        for r, tok in zip(sampled, tokens):
+            self._apply_token(r, int(tok), now)
+
+    def _apply_token(self, r: Request, tok: int, now: float) -> None:
+        if r.phase == "prefilling":
+            self.prefilling.remove(r)
+            r.phase = "decoding"
+            self.decoding.append(r)
+        if r.t_first_token is None:
+            r.t_first_token = now
+        stops = self.stop_token_ids | set(r.sampling.stop_token_ids)
+        if tok in stops and not r.sampling.ignore_eos:
+            self._finish(r, STOP)  # the stop token is not emitted
+            return
+        r.generated.append(tok)
+        r.feed.append(tok)
+        r.fed = len(r.feed) - 1  # the new token is fed by the next decode row
+        if len(r.generated) >= r.max_tokens:
+            self._finish(r, LENGTH)
+
+    # -- transitions ------------------------------------------------------------------------------
+    def _finish(self, r: Request, reason: str) -> None:
+        r.phase = "finished"
+        r.finish_reason = reason
+        r.t_finish = time.perf_counter()
+
+    def _preempt(self, r: Request) -> None:
+        """Give a decoding request's pages back and queue it again, at the front."""
+        self.decoding.remove(r)
+        self.engine.end_request(r.id)
+        r.phase = "waiting"
+        r.fed = 0
+        r.preemptions += 1
+        self.stats["preemptions"] += 1
+        self.waiting.appendleft(r)
+
+    def _cleanup(self) -> None:
+        for group in (self.prefilling, self.decoding):
+            for r in [r for r in group if r.phase == "finished"]:
+                group.remove(r)
+                if self.cache.is_live(r.id):
+                    self.engine.end_request(r.id)
+                self.finished[r.id] = r

@@ -28,8 +28,6 @@ SOURCES = {
     "gemm_f32": "gemm_f32.hip",
     "rope_kv": "rope_kv.hip",
     "attention_simt": "attention_simt.hip",
-    "attention_mfma": "attention_mfma.hip",
-    "gemm_bf16": "gemm_bf16.hip",
     "sampling": "sampling.hip",
 }
 HEADERS = ("common.h",)
@@ -61,8 +59,20 @@ def find_hipcc() -> str:
     raise BuildError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin/hipcc)")
 
 
+_lib_dir_lock = threading.Lock()
+_lib_dir_cache: dict = {}
+
+
 def lib_dir() -> str:
     """Folder that holds the built libraries; created if it does not exist."""
+    key = os.environ.get("ARLE_AMD_LIB_DIR", "")
+    with _lib_dir_lock:
+        if key not in _lib_dir_cache:
+            _lib_dir_cache[key] = _find_lib_dir()
+        return _lib_dir_cache[key]
+
+
+def _find_lib_dir() -> str:
     override = os.environ.get("ARLE_AMD_LIB_DIR")
     primary = override or os.path.join(PACKAGE_DIR, "_lib")
     try:

@@ -1,0 +1,246 @@
+"""The scheduler's decisions, on the CPU, against a fake engine that keeps the real cache
+bookkeeping but computes nothing (the reference tests its scheduling logic the same way:
+infer/src/scheduler/cuda/execution.rs:829-1075, budget.rs:330-545, decode.rs:940-960)."""
+from types import SimpleNamespace
+
+import pytest
+
+from arle_amd.cache import CacheManager, OutOfPages, PagedNeed
+from arle_amd.engine.scheduler import (LENGTH, STOP, Request, Scheduler, SchedulerConfig, plan_prefill,
+                                       retract_victim)
+from arle_amd.sampling import SamplingParams
+
+VOCAB = 97
+
+
+def next_token(history):
+    """The fake model: the next token is a function of the whole history, so any token fed
+    wrongly, twice or out of order changes everything after it."""
+    h = 0
+    for t in history:
+        h = (h * 31 + t + 1) % 1000003
+    return h % VOCAB
+
+
+class FakeEngine:
+    def __init__(self, num_pages=64, page_size=4, slots=4, max_request_tokens=256):
+        self.cache = CacheManager([PagedNeed(1, 16)], page_size=page_size, num_pages=num_pages,
+                                  max_slots=slots, max_request_tokens=max_request_tokens)
+        self.spec = SimpleNamespace(vocab_size=VOCAB, stop_token_ids=())
+        self.history = {}
+        self.steps = []
+
+    def add_request(self, key):
+        self.history[key] = []
+        return self.cache.admit(key)
+
+    def end_request(self, key):
+        self.cache.release(key)
+        del self.history[key]
+
+    def step(self, entries):
+        self.cache.append([(e.request, len(e.tokens)) for e in entries])
+        self.cache.check()
+        rows = []
+        for e in entries:
+            assert len(self.history[e.request]) + len(e.tokens) == self.cache.length(e.request)
+            for i, t in enumerate(e.tokens):
+                self.history[e.request].append(t)
+                if i in e.want:
+                    rows.append(next_token(self.history[e.request]))
+        self.steps.append([(e.request, len(e.tokens), list(e.want)) for e in entries])
+        return rows
+
+
+class FakeSampler:
+    def sample(self, logits, rows):
+        assert len(logits) == len(rows)
+        return list(logits)
+
+
+def expected_output(prompt, n):
+    hist, out = list(prompt), []
+    for _ in range(n):
+        out.append(next_token(hist))
+        hist.append(out[-1])
+    return out
+
+
+def make(num_pages=64, page_size=4, slots=4, **cfg):
+    eng = FakeEngine(num_pages, page_size, slots)
+    return eng, Scheduler(eng, FakeSampler(), SchedulerConfig(num_slots=slots, **cfg))
+
+
+def prompt(n, k=0):
+    return [(7 * i + k) % VOCAB for i in range(n)]
+
+
+def test_one_request_prefill_then_decode():
+    eng, s = make()
+    rid = s.submit(prompt(10), max_tokens=5)
+    s.run_until_done()
+    r = s.finished[rid]
+    assert r.generated == expected_output(prompt(10), 5) and r.finish_reason == LENGTH
+    assert eng.steps[0] == [(rid, 10, [9])]
+    assert all(step == [(rid, 1, [0])] for step in eng.steps[1:]) and len(eng.steps) == 5
+    assert not eng.cache.slot_of and eng.cache.free_pages() == [64]
+
+
+def test_prompts_are_cut_into_portions_and_logits_asked_only_at_the_end():
+    eng, s = make(chunked_prefill_size=4)
+    rid = s.submit(prompt(10), max_tokens=2)
+    s.run_until_done()
+    assert eng.steps[:3] == [[(rid, 4, [])], [(rid, 4, [])], [(rid, 2, [1])]]
+    assert s.finished[rid].generated == expected_output(prompt(10), 2)
+
+
+def test_continuous_batching_mixes_decode_rows_and_portions_in_one_step():
+    eng, s = make(chunked_prefill_size=8)
+    a = s.submit(prompt(6, 1), max_tokens=6)
+    s.iteration()                       # a's whole prompt
+    b = s.submit(prompt(20, 2), max_tokens=3)
+    plan = s.iteration()
+    assert plan.kind == "mixed"
+    assert eng.steps[-1] == [(a, 1, [0]), (b, 8, [])]   # decode rows first, then the portion
+    s.run_until_done()
+    assert s.finished[a].generated == expected_output(prompt(6, 1), 6)
+    assert s.finished[b].generated == expected_output(prompt(20, 2), 3)
+    assert s.stats["steps"]["mixed"] >= 2
+
+
+def test_token_budget_is_never_exceeded_and_decode_rows_come_first():
+    eng, s = make(num_pages=400, slots=4, max_num_batched_tokens=12, max_prefill_tokens=10,
+                  chunked_prefill_size=6)
+    ids = [s.submit(prompt(25, k), max_tokens=8) for k in range(4)]
+    s.run_until_done()
+    for step in eng.steps:
+        decode = sum(n for _, n, _ in step if n == 1)
+        assert sum(n for _, n, _ in step) <= 12
+        assert sum(n for _, n, _ in step if n > 1) <= min(12 - decode, 10)
+    for k, rid in enumerate(ids):
+        assert s.finished[rid].generated == expected_output(prompt(25, k), 8)
+
+
+def _req(i, remaining, generated=0, max_tokens=16, prompt_len=None):
+    r = Request(i, prompt(prompt_len or remaining), SamplingParams(), max_tokens, 0)
+    r.feed = list(r.prompt)
+    r.generated = [1] * generated
+    return r
+
+
+def test_a_portion_that_does_not_fit_is_skipped_whole_not_shrunk():
+    cfg = SchedulerConfig(max_num_batched_tokens=100, max_prefill_tokens=10, chunked_prefill_size=8)
+    queue = [_req(0, 8), _req(1, 5), _req(2, 2), _req(3, 1)]
+    picked = plan_prefill(queue, 0, cfg, lambda reserved, r, n: True)
+    # 8 fits (2 left); 5 does not and is skipped; 2 fits exactly; nothing left for the last
+    assert [(r.id, n) for r, n in picked] == [(0, 8), (2, 2)]
+    # FCFS among equals: queue order is the only priority
+    picked = plan_prefill([_req(5, 4), _req(4, 4), _req(6, 4)], 0, cfg, lambda reserved, r, n: True)
+    assert [r.id for r, _ in picked] == [5, 4]
+    # decode rows shrink the budget first, and cap portions by the long-prefill threshold
+    cfg = SchedulerConfig(max_num_batched_tokens=10, max_prefill_tokens=10, chunked_prefill_size=8,
+                          long_prefill_token_threshold=3)
+    picked = plan_prefill([_req(0, 8), _req(1, 8)], 4, cfg, lambda reserved, r, n: True)
+    assert [(r.id, n) for r, n in picked] == [(0, 3), (1, 3)]
+    # prefill_max_requests
+    cfg = SchedulerConfig(prefill_max_requests=1)
+    assert len(plan_prefill([_req(0, 8), _req(1, 8)], 0, cfg, lambda reserved, r, n: True)) == 1
+    # pages: the finishing portion asks for one token more (the first decoded token)
+    asked = []
+    plan_prefill([_req(0, 8), _req(1, 600)], 0, SchedulerConfig(), lambda res, r, n: asked.append((r.id, n)) or True)
+    assert asked == [(0, 9), (1, 512)]
+
+
+def test_retract_victim_is_least_progress_then_longest_prompt():
+    a, b, c = _req(0, 1, generated=5, prompt_len=10), _req(1, 1, generated=2, prompt_len=10), _req(2, 1, generated=2, prompt_len=30)
+    assert retract_victim([a, b, c]) is c
+    assert retract_victim([a, b]) is b
+
+
+def test_stop_token_is_not_emitted_and_max_tokens_is_exact():
+    eng, s = make()
+    p = prompt(9)
+    out = expected_output(p, 6)
+    stop = out[3]
+    first = out.index(stop)
+    rid = s.submit(p, SamplingParams(stop_token_ids=[stop]), max_tokens=6)
+    rid2 = s.submit(p, SamplingParams(stop_token_ids=[stop], ignore_eos=True), max_tokens=6)
+    s.run_until_done()
+    assert s.finished[rid].generated == out[:first] and s.finished[rid].finish_reason == STOP
+    assert s.finished[rid2].generated == out and s.finished[rid2].finish_reason == LENGTH
+    # stop ids of the model itself
+    eng, s = make()
+    s.stop_token_ids = {out[0]}
+    rid = s.submit(p, max_tokens=6)
+    s.run_until_done()
+    assert s.finished[rid].generated == [] and s.finished[rid].finish_reason == STOP
+
+
+def test_rejections_and_the_length_contract():
+    eng, s = make(num_pages=8, page_size=4)           # pool of 32 tokens
+    assert s.max_request_len == 31 and s.max_request_input_len == 26
+    empty = s.submit([], max_tokens=4)
+    long = s.submit(prompt(26), max_tokens=4)
+    assert s.finished[empty].finish_reason == LENGTH and s.finished[empty].generated == []
+    assert s.finished[long].finish_reason == LENGTH and s.stats["rejected"] == 2
+    ok = s.submit(prompt(25), max_tokens=100)          # clamped to 31 - 25 - 1 = 5
+    s.run_until_done()
+    assert len(s.finished[ok].generated) == 5
+    assert not s.has_work() and eng.cache.free_pages() == [8]
+
+
+def test_admission_needs_a_slot_and_pages_for_prompt_plus_one():
+    eng, s = make(num_pages=10, page_size=4, slots=2)  # 40 tokens
+    a = s.submit(prompt(20, 1), max_tokens=3)          # 21 tokens -> 6 pages
+    b = s.submit(prompt(19, 2), max_tokens=3)          # 20 tokens -> 5 pages: does not fit beside a
+    c = s.submit(prompt(10, 3), max_tokens=3)          # 11 tokens -> 3 pages: fits beside a
+    s.iteration()
+    live = set(eng.cache.slot_of)
+    assert live == {a, c} and [r.id for r in s.waiting] == [b]   # b keeps its place in the queue
+    s.run_until_done()
+    for rid, (n, k) in zip((a, b, c), ((20, 1), (19, 2), (10, 3))):
+        assert s.finished[rid].generated == expected_output(prompt(n, k), 3)
+
+
+def test_when_pages_run_out_a_decoding_request_is_preempted_and_everything_still_finishes():
+    # 4 requests of 10-token prompts are admitted against 4 * 11 = 44 tokens, then each wants to
+    # grow by 24 more: the pool of 52 tokens cannot hold that
+    eng, s = make(num_pages=13, page_size=4, slots=4)
+    ids = [s.submit(prompt(10, k), max_tokens=24) for k in range(4)]
+    s.run_until_done()
+    assert s.stats["preemptions"] > 0
+    for k, rid in enumerate(ids):
+        r = s.finished[rid]
+        # a preempted request keeps what it generated and feeds prompt + generated again
+        assert r.generated == expected_output(prompt(10, k), 24) and r.finish_reason == LENGTH
+    assert any(s.finished[rid].preemptions for rid in ids)
+    assert not s.has_work() and not eng.cache.slot_of and eng.cache.free_pages() == [13]
+    eng.cache.check()
+
+
+def test_a_lone_request_that_cannot_grow_finishes_with_length():
+    eng, s = make(num_pages=4, page_size=4, slots=2)    # 16 tokens; contract allows 15
+    s.max_request_len, s.max_request_input_len = 100, 95  # lift the contract to reach the pool's edge
+    rid = s.submit(prompt(12), max_tokens=50)
+    s.run_until_done()
+    r = s.finished[rid]
+    assert r.finish_reason == LENGTH and len(r.generated) == 5   # 12 + 4 fed tokens fill the 16; the 5th is sampled, not fed
+    assert r.generated == expected_output(prompt(12), 5)
+    assert eng.cache.free_pages() == [4]
+
+
+def test_config_is_validated():
+    with pytest.raises(ValueError):
+        SchedulerConfig(chunked_prefill_size=0).validate()
+    with pytest.raises(ValueError):
+        SchedulerConfig(num_slots=8, max_num_batched_tokens=4).validate()
+
+
+def test_sampling_params_greedy_rule():
+    # infer/src/sampler.rs:82-84,178-
+    assert SamplingParams().is_greedy()
+    assert SamplingParams(temperature=0.7, top_k=1).is_greedy()
+    assert not SamplingParams(temperature=0.7).is_greedy()
+    assert not SamplingParams(temperature=0.0, top_p=0.9).is_greedy()
+    assert not SamplingParams(temperature=0.0, min_p=0.1).is_greedy()
+    assert SamplingParams(repetition_penalty=1.1).has_penalties() and not SamplingParams().has_penalties()
