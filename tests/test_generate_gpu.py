@@ -1,0 +1,168 @@
+"""Generation through the entry point, the scheduler on the real engine, and bin/trace_run."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import replay
+from arle_amd import LLM, SamplingParams
+from arle_amd.sampling import uniform
+from tiny import TINY, make_model_dir, random_tokens, read_folder
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..")
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    base = tmp_path_factory.mktemp("gen")
+    # a larger weight spread than the default separates the logits, so greedy ties are no issue
+    return {name: make_model_dir(base, name, std_scale=6.0) for name in ("A", "B")}
+
+
+def _plain_greedy(cfg, weights, prompt, n):
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(plain.forward_logits(weights, cfg, toks, dtype=torch.float64)[-1].argmax()))
+    return toks[len(prompt):]
+
+
+def test_greedy_generation_equals_the_plain_implementation(folders):
+    # configuration A of the task: prompts of 5 / 11 / 17 tokens, 8 greedy tokens each
+    cfg, weights = read_folder(folders["A"])
+    prompts = [random_tokens(n, cfg["vocab_size"], 70 + n) for n in (5, 11, 17)]
+    want = [_plain_greedy(cfg, weights, p, 8) for p in prompts]
+    llm = LLM(folders["A"], dtype="float32", page_size=TINY["A"][1], kv_cache_tokens=256, max_seq_len=64)
+    outs = llm.generate(prompts, max_tokens=8)
+    assert [o.response_token_ids for o in outs] == want
+    assert all(o.finish_reason == "length" and o.usage.completion_tokens == 8 for o in outs)
+    assert [o.usage.prompt_tokens for o in outs] == [5, 11, 17]
+    assert llm.last_stats["steps"]["decode"] > 0
+
+
+def test_bfloat16_greedy_picks_near_best_tokens(folders):
+    cfg, weights = read_folder(folders["A"])
+    prompts = [random_tokens(n, cfg["vocab_size"], 80 + n) for n in (5, 11, 17)]
+    llm = LLM(folders["A"], dtype="bfloat16", page_size=TINY["A"][1], kv_cache_tokens=256, max_seq_len=64)
+    for p, o in zip(prompts, llm.generate(prompts, max_tokens=8)):
+        hist = list(p)
+        for t in o.response_token_ids:
+            logits = plain.forward_logits(weights, cfg, hist, dtype=torch.float64)[-1]
+            assert float(logits.max() - logits[t]) <= 0.03 * float(logits.abs().max())
+            hist.append(t)
+
+
+def test_temperature_sampling_with_portions_equals_plain_inverse_cdf(folders):
+    # configuration B of the task: prompts of 1 / 9 / 23 / 40, portions of 16, temperature 0.8, 6 tokens
+    cfg, weights = read_folder(folders["B"])
+    prompts = [random_tokens(n, cfg["vocab_size"], 90 + n) for n in (1, 9, 23, 40)]
+    llm = LLM(folders["B"], dtype="float32", page_size=TINY["B"][1], kv_cache_tokens=512, max_seq_len=128,
+              chunked_prefill_size=16, seed=7)
+    params = SamplingParams(temperature=0.8, seed=1234)
+    outs = llm.generate(prompts, max_tokens=6, sampling=params)
+    assert llm.last_stats["steps"]["mixed"] > 0          # portions ran beside decoded tokens
+    for p, o in zip(prompts, outs):
+        hist = list(p)
+        for i, t in enumerate(o.response_token_ids):
+            logits = plain.forward_logits(weights, cfg, hist, dtype=torch.float64)[-1]
+            assert t == plain.sample_token(logits, 0.8, uniform(1234, i)), (len(p), i)
+            hist.append(t)
+        assert len(o.response_token_ids) == 6
+    # the same seed gives the same tokens whatever else is in the batch
+    alone = llm.generate([prompts[2]], max_tokens=6, sampling=params)[0]
+    assert alone.response_token_ids == outs[2].response_token_ids
+
+
+def test_generation_survives_a_pool_that_runs_out(folders):
+    cfg, weights = read_folder(folders["A"])
+    prompts = [random_tokens(10, cfg["vocab_size"], 60 + k) for k in range(4)]
+    want = [_plain_greedy(cfg, weights, p, 24) for p in prompts]
+    llm = LLM(folders["A"], dtype="float32", page_size=4, kv_cache_tokens=52, max_seq_len=64)
+    outs = llm.generate(prompts, max_tokens=24)
+    assert llm.last_stats["preemptions"] > 0
+    assert [o.response_token_ids for o in outs] == want
+    assert llm.engine.cache.free_pages() == [13] and not llm.engine.cache.slot_of
+
+
+def test_stop_token_from_generation_config(folders, tmp_path):
+    cfg, weights = read_folder(folders["A"])
+    prompt = random_tokens(9, cfg["vocab_size"], 5)
+    free_run = _plain_greedy(cfg, weights, prompt, 8)
+    stop = free_run[4]
+    with open(os.path.join(folders["A"], "generation_config.json"), "w") as fh:
+        json.dump({"eos_token_id": [stop]}, fh)
+    try:
+        llm = LLM(folders["A"], dtype="float32", page_size=4, kv_cache_tokens=256, max_seq_len=64)
+        out = llm.generate([prompt], max_tokens=8)[0]
+        assert out.response_token_ids == free_run[:free_run.index(stop)] and out.finish_reason == "stop"
+        out = llm.generate([prompt], max_tokens=8, ignore_eos=True)[0]
+        assert out.response_token_ids == free_run and out.finish_reason == "length"
+    finally:
+        os.remove(os.path.join(folders["A"], "generation_config.json"))
+
+
+def test_command_line_run(folders):
+    cfg, weights = read_folder(folders["A"])
+    prompt = random_tokens(7, cfg["vocab_size"], 3)
+    want = _plain_greedy(cfg, weights, prompt, 5)
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "arle-amd"), "--model-path", folders["A"], "--max-tokens", "5",
+           "--dtype", "float32", "--max-seq-len", "64", "run", "--prompt-ids", ",".join(map(str, prompt)), "--json"]
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr[-2000:]
+    doc = json.loads(res.stdout.strip().splitlines()[-1])
+    assert doc["token_ids"] == want and doc["usage"] == {"prompt_tokens": 7, "completion_tokens": 5, "total_tokens": 12}
+    assert "tok/s" in res.stderr and "TTFT" in res.stderr
+
+
+class TraceRun:
+    """bin/trace_run as a child process: one JSON line in, `done <step>` out."""
+
+    def __init__(self, model, dtype, out, max_tokens):
+        self.out = out
+        self.proc = subprocess.Popen(
+            [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model, "--dtype", dtype,
+             "--out", out, "--max-tokens", str(max_tokens)],
+            stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, bufsize=1)
+
+    def step(self, rec):
+        self.proc.stdin.write(json.dumps(rec) + "\n")
+        self.proc.stdin.flush()
+        line = self.proc.stdout.readline().strip()
+        assert line == f"done {rec['step']}", f"trace_run said {line!r}"
+        path = os.path.join(self.out, f"{rec['step']}.f32")
+        return np.fromfile(path, dtype="<f4") if os.path.exists(path) else None
+
+    def close(self):
+        self.proc.stdin.close()
+        assert self.proc.wait(timeout=120) == 0
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-5), ("bfloat16", 2e-2)])
+def test_trace_run_program(folders, tmp_path, dtype, tol):
+    cfg, weights = read_folder(folders["B"])
+    vocab = cfg["vocab_size"]
+    reqs = {f"q{i}": random_tokens(n, vocab, 500 + i) for i, n in enumerate([37, 64, 20, 51, 45])}
+    steps = replay.mixed(reqs, max_live=4, seed=3)
+    tr = TraceRun(folders["B"], dtype, str(tmp_path / f"out_{dtype}"), max_tokens=4 * 64)
+    got, fed = {}, {r: 0 for r in reqs}
+    try:
+        for i, st in enumerate(steps):
+            rec = {"step": i, "entries": [{"id": r, "tokens": t, "want": w} for r, t, w in st["entries"]],
+                   "end": st["end"]}
+            flat = tr.step(rec)
+            where = [(r, fed[r] + k) for r, t, w in st["entries"] for k in w]
+            for r, t, _ in st["entries"]:
+                fed[r] += len(t)
+            if where:
+                rows = torch.from_numpy(flat.reshape(len(where), vocab).copy())
+                got.update(dict(zip(where, rows)))
+        # a step that wants nothing writes no file
+        assert tr.step({"step": 9999, "entries": [{"id": "z", "tokens": [1, 2, 3], "want": []}], "end": ["z"]}) is None
+    finally:
+        tr.close()
+    replay.compare(got, cfg, weights, reqs, tol, f"trace_run/{dtype}")
