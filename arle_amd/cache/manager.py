@@ -40,7 +40,7 @@ class PagedView:
     """What a mixer sees of its paged cache during a step."""
 
     k_pages: torch.Tensor | None   # [pages, kv_heads, page_size, head_dim]
-    v_pages: torch.Tensor | None
+    v_pages: torch.Tensor | None   # [pages, kv_heads, head_dim, page_size]  (d-major inside a page)
     block_table: torch.Tensor | None  # int32 [slots, max_pages_per_request], shared by the group
     page_size: int
     window: int | None
@@ -102,10 +102,12 @@ class CacheManager:
         self.k_buffers, self.v_buffers, self.tables_dev, self.state_buffers = [], [], [], {}
         if device is not None:
             for g, need in enumerate(self._group_needs):
-                shape = (len(self._group_entries[g]), num_pages, need.num_kv_heads, page_size,
-                         need.head_dim)
-                self.k_buffers.append(torch.zeros(shape, dtype=dtype, device=device))
-                self.v_buffers.append(torch.zeros(shape, dtype=dtype, device=device))
+                n = len(self._group_entries[g])
+                # keys [.., slot in page, d]; values d-major inside a page [.., d, slot in page]
+                self.k_buffers.append(torch.zeros((n, num_pages, need.num_kv_heads, page_size, need.head_dim),
+                                                  dtype=dtype, device=device))
+                self.v_buffers.append(torch.zeros((n, num_pages, need.num_kv_heads, need.head_dim, page_size),
+                                                  dtype=dtype, device=device))
                 self.tables_dev.append(torch.zeros((max_slots, self.max_pages_per_request),
                                                    dtype=torch.int32, device=device))
             for entry, need in enumerate(self.needs):

@@ -71,11 +71,11 @@ __global__ __launch_bounds__(kWave) void attn_paged_simt_kernel(
       const float pj = __shfl(p, j, kWave);
       const int cj = tile * kWave + j;
       const int page = table[cj / page_size];
-      const T* vr = v_pages + page * page_elems + head_off + static_cast<int64_t>(cj % page_size) * D;
+      const T* vr = v_pages + page * page_elems + head_off + (cj % page_size);  // [d][slot in page]
 #pragma unroll
       for (int i = 0; i < kSimtMaxD / kWave; ++i) {
         const int d = lane + i * kWave;
-        if (d < D) acc[i] = fmaf(pj, to_float(vr[d]), acc[i]);
+        if (d < D) acc[i] = fmaf(pj, to_float(vr[static_cast<int64_t>(d) * page_size]), acc[i]);
       }
     }
     m = m_new;
@@ -94,8 +94,8 @@ __global__ __launch_bounds__(kWave) void attn_paged_simt_kernel(
 
 using namespace arle;
 
-// q, out: [tokens, nq*D] with row strides in elements.  k_pages, v_pages:
-// [pages, nkv, page_size, D].  block_table: [slots, table_stride].  row_list
+// q, out: [tokens, nq*D] with row strides in elements.  k_pages [pages, nkv, page_size, D];
+// v_pages [pages, nkv, D, page_size].  block_table: [slots, table_stride].  row_list
 // (may be null) names the token rows to process; n_rows is its length, or the
 // number of tokens when it is null.  window == 0 means all earlier keys.
 extern "C" int arle_attn_paged_simt(const void* q, long long q_stride, void* out,

@@ -13,7 +13,8 @@
 // reference counterparts: crates/cuda-kernels/csrc/attention/prefill_attention_paged_prep.cu:8-106,
 // crates/cuda-kernels/csrc/attention/decode_prep_paged.cu:73-160 (head_dim fixed to 128 there).
 //
-// Cache layout per layer: [page, kv_head, slot_in_page, D].
+// Cache layout per layer: keys [page, kv_head, slot_in_page, D]; values [page, kv_head, D, slot_in_page]
+// (d-major, so that a matrix-core operand of 4 consecutive keys at one d is one 8-byte load).
 #include "common.h"
 
 namespace arle {
@@ -41,18 +42,19 @@ __global__ __launch_bounds__(kPrepWaves* kWave) void qk_prep_kernel(
   float* x = lds + wave * D;
 
   const int pos = positions[t];
-  int64_t cache_row = 0;  // element offset of [page, kv head 0, slot_in_page, 0]
+  int64_t page_base = 0;  // element offset of the token's page, [page, kv head 0, 0, 0]
+  const int in_page = pos % page_size;
   if (valid && !is_q && (k_pages || v_pages)) {
     const int slot = slot_of_token[t];
     const int page = block_table[static_cast<int64_t>(slot) * table_stride + pos / page_size];
-    cache_row = (static_cast<int64_t>(page) * nkv * page_size + (pos % page_size)) * D;
+    page_base = static_cast<int64_t>(page) * nkv * page_size * D;
   }
 
-  if (is_v && v_pages) {  // v head: copy into the cache
+  if (is_v && v_pages) {  // v head: copy into the cache, d-major inside the page
     const int kvh = head - nq - nkv;
     const T* vsrc = v + static_cast<int64_t>(t) * v_stride + kvh * D;
-    T* vdst = v_pages + cache_row + static_cast<int64_t>(kvh) * page_size * D;
-    for (int d = lane; d < D; d += kWave) vdst[d] = vsrc[d];
+    T* vdst = v_pages + page_base + static_cast<int64_t>(kvh) * page_size * D + in_page;
+    for (int d = lane; d < D; d += kWave) vdst[static_cast<int64_t>(d) * page_size] = vsrc[d];
   }
 
   const int local = is_q ? head : head - nq;
@@ -76,7 +78,8 @@ __global__ __launch_bounds__(kPrepWaves* kWave) void qk_prep_kernel(
   if (!is_qk) return;
 
   T* dst = src;
-  if (!is_q && k_pages) dst = k_pages + cache_row + static_cast<int64_t>(local) * page_size * D;
+  if (!is_q && k_pages)
+    dst = k_pages + page_base + (static_cast<int64_t>(local) * page_size + in_page) * D;
   const int half = rot / 2;
   const float* cs = cos_t + static_cast<int64_t>(pos) * half;
   const float* sn = sin_t + static_cast<int64_t>(pos) * half;

@@ -35,6 +35,7 @@ class StepBatch:
     num_tokens: int
     segments: list
     max_position: int
+    max_qlen: int                # longest segment
     token_ids: torch.Tensor      # int32 [T]
     positions: torch.Tensor      # int32 [T]  absolute position of each row in its request
     slot_of_token: torch.Tensor  # int32 [T]  row of the block tables / state buffers
@@ -93,4 +94,5 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device) -> St
     for k, n in zip(order, sizes):
         dev[k] = packed[off:off + n]
         off += n
-    return StepBatch(num_tokens=row, segments=segments, max_position=max(pos), host=host, **dev)
+    return StepBatch(num_tokens=row, segments=segments, max_position=max(pos),
+                     max_qlen=max(s.length for s in segments), host=host, **dev)

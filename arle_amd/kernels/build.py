@@ -28,6 +28,7 @@ SOURCES = {
     "gemm_f32": "gemm_f32.hip",
     "rope_kv": "rope_kv.hip",
     "attention_simt": "attention_simt.hip",
+    "attention_mfma": "attention_mfma.hip",
     "sampling": "sampling.hip",
 }
 HEADERS = ("common.h",)

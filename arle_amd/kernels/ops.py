@@ -202,9 +202,7 @@ def qk_prep(q, k, v, *, num_q_heads: int, num_kv_heads: int, head_dim: int, eps:
     if k_pages is not None or v_pages is not None:
         _need(k_pages is not None and v_pages is not None, "give both k and v pages or neither")
         _need(page_size > 0, "page_size must be positive")
-        for name, t in (("k_pages", k_pages), ("v_pages", v_pages)):
-            _need(t.dim() == 4 and t.shape[1:] == (num_kv_heads, page_size, D) and t.is_contiguous()
-                  and t.dtype == q.dtype, f"{name} must be contiguous [pages, nkv, page_size, D]")
+        _check_pages(k_pages, v_pages, num_kv_heads, page_size, D, q.dtype)
         _i32(slot_of_token, "slot_of_token", tokens)
         _need(block_table is not None and block_table.dtype == torch.int32 and block_table.dim() == 2
               and block_table.is_contiguous(), "block_table must be contiguous int32 [slots, pages]")
@@ -221,6 +219,15 @@ def qk_prep(q, k, v, *, num_q_heads: int, num_kv_heads: int, head_dim: int, eps:
 # ------------------------------------------------------------------ attention
 
 
+def _check_pages(k_pages, v_pages, nkv, page_size, D, dtype):
+    """Keys [pages, nkv, page_size, D]; values d-major inside a page [pages, nkv, D, page_size]."""
+    _need(k_pages.dim() == 4 and tuple(k_pages.shape[1:]) == (nkv, page_size, D) and k_pages.is_contiguous()
+          and k_pages.dtype == dtype, "k_pages must be contiguous [pages, nkv, page_size, D]")
+    _need(v_pages.dim() == 4 and tuple(v_pages.shape[1:]) == (nkv, D, page_size) and v_pages.is_contiguous()
+          and v_pages.dtype == dtype and v_pages.shape[0] == k_pages.shape[0],
+          "v_pages must be contiguous [pages, nkv, D, page_size]")
+
+
 def _check_paged(q, out, k_pages, v_pages, block_table, positions, slot_of_token, nq, nkv, D,
                  page_size):
     _gpu(q, out, k_pages, v_pages, block_table, positions, slot_of_token)
@@ -230,9 +237,7 @@ def _check_paged(q, out, k_pages, v_pages, block_table, positions, slot_of_token
     _need(q.shape == (tokens, nq * D) and out.shape == (tokens, nq * D) and out.dtype == q.dtype,
           "q and out must be [T, nq*D] of one type")
     _need(nkv > 0 and nq % nkv == 0, "number of q heads must be a multiple of the kv heads")
-    for name, t in (("k_pages", k_pages), ("v_pages", v_pages)):
-        _need(t.dim() == 4 and t.shape[1:] == (nkv, page_size, D) and t.is_contiguous()
-              and t.dtype == q.dtype, f"{name} must be contiguous [pages, nkv, page_size, D]")
+    _check_pages(k_pages, v_pages, nkv, page_size, D, q.dtype)
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
           "block_table must be contiguous int32 [slots, pages]")
     _i32(positions, "positions", tokens)
@@ -257,6 +262,61 @@ def attn_paged_simt(q, out, k_pages, v_pages, block_table, positions, slot_of_to
              block_table.shape[1], positions.data_ptr(), slot_of_token.data_ptr(), _ptr(row_list),
              n_rows, num_q_heads, num_kv_heads, head_dim, page_size, float(scale), int(window),
              _stream())
+    return out
+
+
+MFMA_MAX_HEAD_DIM = 256
+_MFMA_TARGET_WAVES = 4096   # waves wanted in flight for a decode launch (256 CUs x 16)
+
+
+def attn_mfma_supported(dtype, head_dim: int, page_size: int) -> bool:
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 0 < head_dim <= MFMA_MAX_HEAD_DIM
+            and page_size % 4 == 0)
+
+
+def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *,
+                    max_qlen: int, max_kv_len: int, num_q_heads: int, num_kv_heads: int, head_dim: int,
+                    page_size: int, scale: float, window: int = 0, splits: int | None = None):
+    """Causal attention of a packed step on the matrix cores (bfloat16).
+
+    Segments: rows seg_row0[s]..seg_row0[s+1] belong to block-table row seg_slot[s] and start at
+    position seg_start[s].  A step of single decoded tokens is split over the keys (split-KV).
+    """
+    _gpu(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start)
+    tokens = q.shape[0]
+    _rows(q, "q")
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "the MFMA attention takes bfloat16")
+    _need(q.shape == (tokens, num_q_heads * head_dim) and out.shape == q.shape and out.is_contiguous(),
+          "q must be [T, nq*D] and out contiguous [T, nq*D]")
+    _need(attn_mfma_supported(q.dtype, head_dim, page_size),
+          f"the MFMA attention needs head_dim % 16 == 0, head_dim <= {MFMA_MAX_HEAD_DIM} and page_size % 4 == 0 "
+          f"(got head_dim {head_dim}, page_size {page_size})")
+    _need(q.data_ptr() % 16 == 0 and (q.stride(0) * 2) % 16 == 0, "q rows must be 16-byte aligned")
+    _need(num_kv_heads > 0 and num_q_heads % num_kv_heads == 0, "q heads must be a multiple of kv heads")
+    _check_pages(k_pages, v_pages, num_kv_heads, page_size, head_dim, q.dtype)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "block_table must be contiguous int32 [slots, pages]")
+    segments = seg_slot.numel()
+    _i32(seg_row0, "seg_row0", segments + 1)
+    _i32(seg_slot, "seg_slot")
+    _i32(seg_start, "seg_start", segments)
+    _need(1 <= max_qlen <= tokens, "max_qlen must lie in 1..tokens")
+    if splits is None:
+        splits = 1
+        if max_qlen == 1:
+            blocks = max(1, -(-max_kv_len // 32))
+            splits = max(1, min(-(-_MFMA_TARGET_WAVES // (segments * num_kv_heads)), blocks // 2, 32))
+    _need(splits == 1 or max_qlen == 1, "split-KV is for steps of single decoded tokens")
+    _need(segments * splits <= _GRID_Y_MAX and num_kv_heads <= _GRID_Y_MAX, "too many segments for one launch")
+    ws_o = ws_ml = None
+    if splits > 1:
+        ws_o = torch.empty((tokens, num_q_heads, splits, head_dim), dtype=torch.float32, device=q.device)
+        ws_ml = torch.empty((tokens, num_q_heads, splits, 2), dtype=torch.float32, device=q.device)
+    lib.call("arle_attn_paged_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
+             k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+             seg_row0.data_ptr(), seg_slot.data_ptr(), seg_start.data_ptr(), segments, int(max_qlen), tokens,
+             num_q_heads, num_kv_heads, head_dim, page_size, float(scale), int(window), int(splits),
+             _ptr(ws_o), _ptr(ws_ml), _stream())
     return out
 
 

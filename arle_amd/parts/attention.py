@@ -113,9 +113,17 @@ class PagedAttention(Part):
 def paged_attention(q, out, cache, batch, *, num_q_heads, num_kv_heads, head_dim, scale, window):
     """Attention of every row of the packed step over its request's cached keys.
 
-    float32 storage runs the fixed-order kernel (the true 32-bit path); bfloat16 storage runs
-    the MFMA kernels: one for prompt portions, a split-KV one for single decoded tokens.
+    bfloat16 storage runs the matrix-core kernel (split over the keys when the step holds only
+    single decoded tokens); float32 storage, and shapes the matrix-core kernel does not take,
+    run the fixed-order kernel, which is also the true 32-bit path.
     """
-    ops.attn_paged_simt(q, out, cache.k_pages, cache.v_pages, cache.block_table, batch.positions,
-                        batch.slot_of_token, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads,
-                        head_dim=head_dim, page_size=cache.page_size, scale=scale, window=window)
+    if ops.attn_mfma_supported(q.dtype, head_dim, cache.page_size):
+        ops.attn_paged_mfma(q, out, cache.k_pages, cache.v_pages, cache.block_table, batch.seg_row0,
+                            batch.seg_slot, batch.seg_start, max_qlen=batch.max_qlen,
+                            max_kv_len=batch.max_position + 1, num_q_heads=num_q_heads,
+                            num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=cache.page_size,
+                            scale=scale, window=window)
+    else:
+        ops.attn_paged_simt(q, out, cache.k_pages, cache.v_pages, cache.block_table, batch.positions,
+                            batch.slot_of_token, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads,
+                            head_dim=head_dim, page_size=cache.page_size, scale=scale, window=window)

@@ -122,7 +122,7 @@ def _paged_setup(lengths, nkv, D, P, dtype, seed, shuffle=True):
         for i in range(n):
             table[s, i] = next(it)
     k_pages = torch.zeros(total, nkv, P, D, dtype=dtype)
-    v_pages = torch.zeros(total, nkv, P, D, dtype=dtype)
+    v_pages = torch.zeros(total, nkv, D, P, dtype=dtype)   # values are d-major inside a page
     return table, k_pages, v_pages
 
 
@@ -165,7 +165,7 @@ def test_qk_prep_norm_rope_and_cache_write(nq, nkv, D, rot, dt):
     for t in range(T):
         page = int(table[slots[t], positions[t] // P])
         assert _rel(dk[page, :, positions[t] % P], k[t]) < tol
-        assert torch.equal(dv[page, :, positions[t] % P].double(), v[t])
+        assert torch.equal(dv[page, :, :, positions[t] % P].double(), v[t])
     # nothing else in the cache was touched
     written = torch.zeros(dk.shape[0], P, dtype=torch.bool)
     for t in range(T):
@@ -177,7 +177,7 @@ def _fill_cache(table, k_pages, v_pages, slot, k, v, P):
     for pos in range(k.shape[0]):
         page = int(table[slot, pos // P])
         k_pages[page, :, pos % P] = k[pos]
-        v_pages[page, :, pos % P] = v[pos]
+        v_pages[page, :, :, pos % P] = v[pos]
 
 
 @pytest.mark.parametrize("nq,nkv,D,P", [(3, 1, 48, 16), (4, 2, 16, 4), (8, 2, 128, 16), (6, 2, 32, 8),
@@ -290,3 +290,117 @@ def test_kernels_refuse_what_they_were_not_written_for():
         ops.rmsnorm(torch.zeros(2, 3), torch.ones(3), 1e-6, torch.float32)  # CPU tensors
     with pytest.raises(ops.ShapeError):
         ops.embed_gather(torch.zeros(4, 4, device=DEV), torch.zeros(2, dtype=torch.int64, device=DEV))
+
+
+def _mfma_case(nq, nkv, D, P, segs, window, splits, seed):
+    """segs: [(cached length before the step, rows in the step)].  Returns (got, want) [T, nq*D]."""
+    dt = torch.bfloat16
+    lengths = [a + b for a, b in segs]
+    table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, seed)
+    qs, wants, row0, seg_start = [], [], [0], []
+    for s, (cached, n) in enumerate(segs):
+        g = _g(seed + 1 + s)
+        total = cached + n
+        q = torch.randn(total, nq, D, generator=g).to(dt)
+        k = torch.randn(total, nkv, D, generator=g).to(dt)
+        v = torch.randn(total, nkv, D, generator=g).to(dt)
+        _fill_cache(table, k_pages, v_pages, s, k, v, P)
+        full = plain.causal_attention(q.double(), k.double(), v.double(), nkv, window=window or None)
+        qs.append(q[cached:].reshape(n, nq * D))
+        wants.append(full[cached:].reshape(n, nq * D))
+        row0.append(row0[-1] + n)
+        seg_start.append(cached)
+    q_all = torch.cat(qs).to(DEV)
+    out = torch.full_like(q_all, float("nan"))
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    ops.attn_paged_mfma(q_all, out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0),
+                        i32(list(range(len(segs)))), i32(seg_start), max_qlen=max(n for _, n in segs),
+                        max_kv_len=max(lengths), num_q_heads=nq, num_kv_heads=nkv, head_dim=D, page_size=P,
+                        scale=1.0 / math.sqrt(D), window=window, splits=splits)
+    return out.cpu(), torch.cat(wants)
+
+
+@pytest.mark.parametrize("nq,nkv,D,P", [(4, 2, 16, 4), (6, 2, 32, 8), (3, 1, 48, 16), (32, 8, 128, 16),
+                                         (5, 1, 64, 16), (8, 1, 128, 32), (2, 2, 256, 16), (16, 1, 80, 64)])
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_mfma_prompt_portions(nq, nkv, D, P, window):
+    # portions that start mid-page after a cached prefix, a whole prompt, and a single first token
+    got, want = _mfma_case(nq, nkv, D, P, [(0, 70), (45, 39), (0, 1), (130, 2)], window, 1, 70)
+    assert torch.isfinite(got).all()
+    assert _rel(got, want) < 8e-3
+
+
+@pytest.mark.parametrize("nq,nkv,D,P", [(4, 2, 16, 4), (6, 2, 32, 8), (3, 1, 48, 16), (32, 8, 128, 16),
+                                         (40, 8, 128, 16), (64, 2, 64, 16)])
+@pytest.mark.parametrize("splits", [None, 1, 3, 7])
+@pytest.mark.parametrize("window", [0, 50])
+def test_attention_mfma_decoded_tokens_split_over_the_keys(nq, nkv, D, P, splits, window):
+    got, want = _mfma_case(nq, nkv, D, P, [(299, 1), (0, 1), (31, 1), (32, 1), (95, 1)], window, splits, 80)
+    assert torch.isfinite(got).all()
+    assert _rel(got, want) < 8e-3
+
+
+def test_attention_mfma_mixed_step_and_stale_pages():
+    """Decoded tokens beside portions in one launch; pages hold NaN bits beyond each request's length."""
+    nq, nkv, D, P = 8, 2, 128, 16
+    dt = torch.bfloat16
+    segs = [(200, 1), (17, 30), (63, 1), (0, 5)]
+    lengths = [a + b for a, b in segs]
+    table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, 90)
+    k_pages.fill_(float("nan"))
+    v_pages.fill_(float("nan"))
+    qs, wants, row0, starts = [], [], [0], []
+    for s, (cached, n) in enumerate(segs):
+        g = _g(91 + s)
+        q, k, v = (torch.randn(cached + n, h, D, generator=g).to(dt) for h in (nq, nkv, nkv))
+        _fill_cache(table, k_pages, v_pages, s, k, v, P)
+        qs.append(q[cached:].reshape(n, -1))
+        wants.append(plain.causal_attention(q.double(), k.double(), v.double(), nkv)[cached:].reshape(n, -1))
+        row0.append(row0[-1] + n)
+        starts.append(cached)
+    q_all = torch.cat(qs).to(DEV)
+    out = torch.empty_like(q_all)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    ops.attn_paged_mfma(q_all, out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0), i32([0, 1, 2, 3]),
+                        i32(starts), max_qlen=30, max_kv_len=max(lengths), num_q_heads=nq, num_kv_heads=nkv,
+                        head_dim=D, page_size=P, scale=1.0 / math.sqrt(D))
+    assert torch.isfinite(out).all()
+    assert _rel(out.cpu(), torch.cat(wants)) < 8e-3
+
+
+def test_attention_mfma_finds_a_far_key():
+    nq, nkv, D, P, n = 4, 2, 64, 16, 900
+    dt = torch.bfloat16
+    table, k_pages, v_pages = _paged_setup([n], nkv, D, P, dt, 95)
+    g = _g(96)
+    q = (torch.randn(n, nq, D, generator=g) * 0.1).to(dt)
+    k = (torch.randn(n, nkv, D, generator=g) * 0.1).to(dt)
+    v = torch.randn(n, nkv, D, generator=g).to(dt)
+    far = 5
+    k[far, 0] = (q[n - 1, 1].float() * 400.0).to(dt)
+    _fill_cache(table, k_pages, v_pages, 0, k, v, P)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    for splits in (1, 6):   # as the last row of a portion, and as a decoded token split over the keys
+        rows = 40 if splits == 1 else 1
+        qq = q[n - rows:].reshape(rows, -1).to(DEV).contiguous()
+        out = torch.empty_like(qq)
+        ops.attn_paged_mfma(qq, out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32([0, rows]), i32([0]),
+                            i32([n - rows]), max_qlen=rows, max_kv_len=n, num_q_heads=nq, num_kv_heads=nkv,
+                            head_dim=D, page_size=P, scale=1.0 / math.sqrt(D), splits=splits)
+        got = out.cpu().reshape(rows, nq, D)
+        assert torch.allclose(got[-1, 1].float(), v[far, 0].float(), atol=2e-2)
+
+
+def test_attention_mfma_refuses_shapes_it_was_not_written_for():
+    assert not ops.attn_mfma_supported(torch.bfloat16, 24, 16)
+    assert not ops.attn_mfma_supported(torch.bfloat16, 128, 6)
+    assert not ops.attn_mfma_supported(torch.float32, 128, 16)
+    assert not ops.attn_mfma_supported(torch.bfloat16, 272, 16)
+    q = torch.zeros(2, 2 * 24, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ops.ShapeError, match="head_dim % 16"):
+        ops.attn_paged_mfma(q, torch.empty_like(q), torch.zeros(1, 1, 16, 24, dtype=torch.bfloat16, device=DEV),
+                            torch.zeros(1, 1, 24, 16, dtype=torch.bfloat16, device=DEV),
+                            torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+                            torch.tensor([0, 2], dtype=torch.int32, device=DEV),
+                            torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
+                            max_qlen=2, max_kv_len=2, num_q_heads=2, num_kv_heads=1, head_dim=24, page_size=16, scale=1.0)
