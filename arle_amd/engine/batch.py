@@ -44,12 +44,20 @@ class StepBatch:
     seg_slot: torch.Tensor       # int32 [S]
     seg_start: torch.Tensor      # int32 [S]  position of a segment's first row
     host: dict                   # the same arrays as numpy, for parts that plan on the host
+    kv_splits: int | None = None  # split-KV factor fixed by the caller (a captured graph), else chosen per call
 
 
-def build_step_batch(entries, slot_of, length_of, vocab_size: int, device) -> StepBatch:
+def packed_size(num_tokens: int, num_segments: int, num_wanted: int) -> int:
+    """int32 elements that the device arrays of a step take together."""
+    return 3 * num_tokens + num_wanted + (num_segments + 1) + 2 * num_segments
+
+
+def build_step_batch(entries, slot_of, length_of, vocab_size: int, device, into=None) -> StepBatch:
     """Check a step's entries and lay them out.
 
     slot_of(request) -> slot;  length_of(request) -> tokens cached before this step.
+    into: an int32 device buffer of exactly `packed_size(...)` elements to fill instead of a
+    fresh one (a captured graph reads its inputs from fixed addresses).
     """
     if not entries:
         raise ValueError("a step needs at least one entry")
@@ -89,7 +97,14 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device) -> St
     # one host->device copy for all arrays
     order = list(host)
     sizes = [host[k].size for k in order]
-    packed = torch.from_numpy(np.concatenate([host[k] for k in order])).to(device, non_blocking=False)
+    flat = torch.from_numpy(np.concatenate([host[k] for k in order]))
+    if into is None:
+        packed = flat.to(device, non_blocking=False)
+    else:
+        if into.numel() != flat.numel():
+            raise ValueError("the fixed step buffer does not fit this step")
+        into.copy_(flat)
+        packed = into
     dev, off = {}, 0
     for k, n in zip(order, sizes):
         dev[k] = packed[off:off + n]

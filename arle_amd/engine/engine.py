@@ -19,7 +19,8 @@ from ..models.decoder import build_model, expected_checkpoint_tensors
 from ..parts.base import Runtime
 from ..weights.loader import load_weights
 from ..weights.random_init import random_weights
-from .batch import StepEntry, build_step_batch
+from ..kernels import ops
+from .batch import StepEntry, build_step_batch, packed_size
 
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
           "fp32": torch.float32}
@@ -50,11 +51,13 @@ class Engine:
     def __init__(self, spec, tensors: dict, *, dtype=torch.bfloat16, device=None,
                  page_size: int = DEFAULT_PAGE_SIZE, max_tokens: int | None = None,
                  num_pages: int | None = None, max_slots: int = 4,
-                 max_request_tokens: int | None = None):
+                 max_request_tokens: int | None = None, cuda_graph: bool = True):
         """
         max_tokens: tokens the cache holds over all live requests (num_pages = ceil(max_tokens / page_size)
             unless num_pages is given).
         max_request_tokens: longest single request (default: min(model's positions, cache capacity)).
+        cuda_graph: replay steps of single decoded tokens from captured HIP graphs (the reference captures
+            its decode path per batch size: infer/src/model/qwen3/batch_decode.rs:1691-1730).
         """
         self.device = _device(device)
         self.dtype = parse_dtype(dtype)
@@ -75,6 +78,10 @@ class Engine:
         self.page_size = page_size
         self.max_request_tokens = max_request_tokens
         self.steps_run = 0
+        self.use_graphs = bool(cuda_graph) and self.model.graph_safe
+        self._graphs: dict = {}       # (rows, split cap) -> _DecodeGraph
+        self._graph_pool = None
+        self.graph_replays = 0
 
     # -- construction -----------------------------------------------------------------
     @classmethod
@@ -121,13 +128,22 @@ class Engine:
         for e in entries:
             if not self.cache.is_live(e.request):
                 raise EngineError(f"request {e.request!r} is not live; add_request it first")
-        batch = build_step_batch(entries, self.cache.slot_of.__getitem__, self.cache.length,
-                                 self.spec.vocab_size, self.device)
         before = {e.request: self.cache.length(e.request) for e in entries}
+        decode_only = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
+        batch = None
+        if not decode_only:
+            batch = build_step_batch(entries, self.cache.slot_of.__getitem__, self.cache.length,
+                                     self.spec.vocab_size, self.device)
+        else:   # check the entries before anything is changed
+            build_step_batch(entries, self.cache.slot_of.__getitem__, self.cache.length,
+                             self.spec.vocab_size, "cpu")
         self.cache.append([(e.request, len(e.tokens)) for e in entries])
         try:
             self.cache.sync_tables()
-            logits = self.model.forward(batch, self.cache)
+            if decode_only:
+                logits = self._decode_step_graphed(entries, before)
+            else:
+                logits = self.model.forward(batch, self.cache)
         except Exception:
             for key, n in before.items():
                 self.cache.truncate(key, n)
@@ -136,3 +152,52 @@ class Engine:
             self.cache.trim_windows(e.request)
         self.steps_run += 1
         return logits
+
+    # -- captured decode steps ----------------------------------------------------------------
+    def _decode_step_graphed(self, entries, before) -> torch.Tensor:
+        """A step of single decoded tokens through a HIP graph captured for its number of rows.
+
+        The graph computes the logits of every row; the wanted ones are picked afterwards.  What
+        varies from step to step (token ids, positions, slots) is copied into the graph's fixed
+        input buffer; block tables are device tensors at fixed addresses already.  The launch
+        shape of the split-KV attention is part of the graph, so a graph is keyed by the number
+        of rows and by the cap that the longest context puts on the number of splits.
+        """
+        rows = len(entries)
+        max_kv = max(before[e.request] for e in entries) + 1
+        key = (rows, ops.decode_split_cap(max_kv))
+        all_rows = [StepEntry(e.request, e.tokens, [0]) for e in entries]
+        length_before = before.__getitem__
+        rec = self._graphs.get(key)
+        if rec is None:
+            static = torch.empty(packed_size(rows, rows, rows), dtype=torch.int32, device=self.device)
+            batch = build_step_batch(all_rows, self.cache.slot_of.__getitem__, length_before,
+                                     self.spec.vocab_size, self.device, into=static)
+            batch.kv_splits = None
+            self._prepare_for_positions(self.max_request_tokens)
+            logits = self.model.forward(batch, self.cache)   # this step's result, and the warm-up
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                static_logits = self.model.forward(batch, self.cache)
+            self._graphs[key] = (graph, static, static_logits)
+        else:
+            graph, static, static_logits = rec
+            build_step_batch(all_rows, self.cache.slot_of.__getitem__, length_before,
+                             self.spec.vocab_size, self.device, into=static)
+            graph.replay()
+            self.graph_replays += 1
+            logits = static_logits.clone()
+        wanted = [i for i, e in enumerate(entries) for _ in e.want]
+        if wanted == list(range(rows)):
+            return logits
+        return logits[torch.tensor(wanted, dtype=torch.long, device=self.device)]
+
+    def _prepare_for_positions(self, n: int) -> None:
+        """Grow every position table to n positions now, so that no captured step has to."""
+        for block in self.model.blocks:
+            position = getattr(block.mixer, "position", None)
+            if position is not None:
+                position.ensure_positions(n)

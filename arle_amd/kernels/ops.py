@@ -274,6 +274,16 @@ def attn_mfma_supported(dtype, head_dim: int, page_size: int) -> bool:
             and page_size % 4 == 0)
 
 
+def decode_split_cap(max_kv_len: int) -> int:
+    """Most splits worth making for keys up to max_kv_len: at least two 32-key blocks each, at most 32."""
+    return max(1, min(-(-max_kv_len // 32) // 2, 32))
+
+
+def decode_splits(segments: int, num_kv_heads: int, max_kv_len: int) -> int:
+    """Split-KV factor of a step of single decoded tokens: enough waves to fill the chip."""
+    return max(1, min(-(-_MFMA_TARGET_WAVES // (segments * num_kv_heads)), decode_split_cap(max_kv_len)))
+
+
 def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *,
                     max_qlen: int, max_kv_len: int, num_q_heads: int, num_kv_heads: int, head_dim: int,
                     page_size: int, scale: float, window: int = 0, splits: int | None = None):
@@ -302,10 +312,7 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
     _i32(seg_start, "seg_start", segments)
     _need(1 <= max_qlen <= tokens, "max_qlen must lie in 1..tokens")
     if splits is None:
-        splits = 1
-        if max_qlen == 1:
-            blocks = max(1, -(-max_kv_len // 32))
-            splits = max(1, min(-(-_MFMA_TARGET_WAVES // (segments * num_kv_heads)), blocks // 2, 32))
+        splits = decode_splits(segments, num_kv_heads, max_kv_len) if max_qlen == 1 else 1
     _need(splits == 1 or max_qlen == 1, "split-KV is for steps of single decoded tokens")
     _need(segments * splits <= _GRID_Y_MAX and num_kv_heads <= _GRID_Y_MAX, "too many segments for one launch")
     ws_o = ws_ml = None

@@ -49,6 +49,10 @@ class DecoderModel:
         self.schedule = list(spec.schedule)
         self.final_norm = build_part("norm", spec.final_norm, fetch, rt)
         self.head = build_part("head", spec.head, fetch, rt)
+        parts = [self.embedding, self.final_norm, self.head]
+        for b in self.blocks:
+            parts += [b.mixer, b.feed_forward, *getattr(b, "norms", {}).values()]
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in parts)
 
     def cache_needs(self):
         """(need of every schedule entry that owns a cache, {reader entry -> owner entry})."""

@@ -29,6 +29,8 @@ class PagedAttention(Part):
     """params: hidden_size, num_q_heads, num_kv_heads, head_dim, qk_norm (bool), eps,
     position (PartSpec), window (int | None), scale (float | None: 1/sqrt(head_dim))."""
 
+    graph_safe = True  # positions, slots and lengths are read on the GPU; launches depend on shapes only
+
     @classmethod
     def declare_weights(cls, params):
         h, d = params["hidden_size"], params["head_dim"]
@@ -122,7 +124,7 @@ def paged_attention(q, out, cache, batch, *, num_q_heads, num_kv_heads, head_dim
                             batch.seg_slot, batch.seg_start, max_qlen=batch.max_qlen,
                             max_kv_len=batch.max_position + 1, num_q_heads=num_q_heads,
                             num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=cache.page_size,
-                            scale=scale, window=window)
+                            scale=scale, window=window, splits=getattr(batch, "kv_splits", None))
     else:
         ops.attn_paged_simt(q, out, cache.k_pages, cache.v_pages, cache.block_table, batch.positions,
                             batch.slot_of_token, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads,

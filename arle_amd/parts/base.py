@@ -70,6 +70,10 @@ class Runtime:
 class Part:
     role = ""
     kind = ""
+    # True if forward() launches the same kernels with the same arguments for every step of a given
+    # shape, reading whatever varies (positions, slots, lengths) from GPU memory: only then may the
+    # engine replay the part from a captured graph.
+    graph_safe = False
 
     @classmethod
     def declare_weights(cls, params: dict) -> dict:

@@ -19,6 +19,7 @@ class PreNormBlock:
     def __init__(self, mixer, feed_forward, norms: dict):
         self.mixer = mixer
         self.feed_forward = feed_forward
+        self.norms = norms
         self.norm_mixer = norms["mixer_in"]
         self.norm_ffn = norms["ffn_in"]
 

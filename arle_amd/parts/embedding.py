@@ -16,6 +16,8 @@ from .linear import Linear
 class TokenEmbedding(Part):
     """params: vocab_size, hidden_size."""
 
+    graph_safe = True  # launches depend on shapes only, never on the values of a step
+
     @classmethod
     def declare_weights(cls, params):
         return {"table": WeightDecl((params["vocab_size"], params["hidden_size"]))}
@@ -31,6 +33,8 @@ class TokenEmbedding(Part):
 @register("head", "linear")
 class LinearHead(Part):
     """params: vocab_size, hidden_size.  Logits are float32."""
+
+    graph_safe = True  # launches depend on shapes only, never on the values of a step
 
     @classmethod
     def declare_weights(cls, params):

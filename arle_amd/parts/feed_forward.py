@@ -17,6 +17,8 @@ from .linear import Linear
 class SwiGLU(Part):
     """params: hidden_size, intermediate_size."""
 
+    graph_safe = True  # launches depend on shapes only, never on the values of a step
+
     @classmethod
     def declare_weights(cls, params):
         h, i = params["hidden_size"], params["intermediate_size"]

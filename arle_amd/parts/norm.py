@@ -13,6 +13,8 @@ from .base import Part, WeightDecl, register
 class RMSNorm(Part):
     """params: width, eps."""
 
+    graph_safe = True  # launches depend on shapes only, never on the values of a step
+
     @classmethod
     def declare_weights(cls, params):
         return {"weight": WeightDecl((params["width"],), init="ones")}

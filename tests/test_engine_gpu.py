@@ -87,3 +87,32 @@ def test_float32_is_bit_identical_across_cuttings(model):
     c = replay.run_steps(eng, replay.prefill_then_decode("x", toks, 20))
     for key in a:
         assert torch.equal(a[key], b[key]) and torch.equal(a[key], c[key]), key
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_decode_steps_equal_eager_ones_on_every_replay(model, dtype):
+    """Steps of single decoded tokens are replayed from a HIP graph.  Every replay, with eager
+    steps (prompt portions, other batch sizes) and synchronisations in between, must give the
+    bits the eager engine gives."""
+    name, d, cfg, _ = model
+    reqs = _requests(cfg, [70, 41, 55], 900)
+    eager = Engine.from_folder(d, dtype=dtype, page_size=TINY[name][1], max_tokens=256, max_slots=4, cuda_graph=False)
+    graphed = Engine.from_folder(d, dtype=dtype, page_size=TINY[name][1], max_tokens=256, max_slots=4, cuda_graph=True)
+    assert graphed.use_graphs and not eager.use_graphs
+    steps = []
+    for rid, toks in reqs.items():                       # prompts first, all but the last 20 tokens
+        steps.append({"entries": [(rid, toks[:-20], [len(toks) - 21])], "end": []})
+    for i in range(20):                                  # then three decoded tokens a step ...
+        entries = [(rid, [toks[len(toks) - 20 + i]], [0]) for rid, toks in reqs.items()]
+        if i % 6 == 5:
+            entries = entries[:2]                        # ... sometimes two (another graph), the third catches up
+            steps.append({"entries": entries, "end": []})
+            rid, toks = list(reqs.items())[2]
+            steps.append({"entries": [(rid, [toks[len(toks) - 20 + i]], [0])], "end": []})
+        else:
+            steps.append({"entries": entries, "end": []})
+    a = replay.run_steps(eager, steps)
+    b = replay.run_steps(graphed, steps)
+    assert graphed.graph_replays >= 10
+    for key in a:
+        assert torch.equal(a[key], b[key]), f"graph replay differs from the eager step at {key}"
