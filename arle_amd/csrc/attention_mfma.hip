@@ -135,12 +135,28 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
   const int64_t k_head = static_cast<int64_t>(kvh) * P * D;
   const int64_t page_elems = static_cast<int64_t>(a.nkv) * P * D;
 
+  // Page ids of 64 consecutive logical pages sit in one register across the wave (lane i holds
+  // page pg_base + i) and are fetched with a cross-lane read, so that the address of a key or value
+  // load does not wait for a block-table load first.  Refilled when the walk leaves the window.
+  const int pg_last = (kv_hi - 1) / P;
+  int pg_base = 0, pg_reg = 0;
+  auto refill_pages = [&](int first_page) {
+    pg_base = first_page;
+    pg_reg = table[min(first_page + lane, pg_last)];
+  };
+  auto page_of = [&](int key) { return __shfl(pg_reg, key / P - pg_base, kWave); };
+  auto clamp_key = [&](int key) { return min(max(key, kv_lo), kv_hi - 1); };
+  // the blocks blk and blk + 1 are in use at any time: make sure the register covers both
+  auto cover = [&](int blk) {
+    const int first = clamp_key(blk * 32) / P, last = clamp_key(blk * 32 + 63) / P;
+    if (first < pg_base || last >= pg_base + kWave) refill_pages(first);
+  };
+
   auto load_k = [&](int blk, bf16x8 (&kreg)[2][DCH]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      int key = blk * 32 + 16 * t + li;
-      key = min(max(key, kv_lo), kv_hi - 1);  // a held, written key; out-of-range ones are masked below
-      const int page = table[key / P];
+      const int key = clamp_key(blk * 32 + 16 * t + li);  // a held, written key; out-of-range ones are masked below
+      const int page = page_of(key);
       const uint16_t* kp = a.k_pages + page * page_elems + k_head + static_cast<int64_t>(key % P) * D;
 #pragma unroll
       for (int c = 0; c < DCH; ++c) {
@@ -150,27 +166,33 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
     }
   };
 
-  bf16x8 kcur[2][DCH];
-  if (b0 < b1) load_k(b0, kcur);
-
-  for (int blk = b0; blk < b1; ++blk) {
-    const int key_base = blk * 32;
-    // values of this block: for each 16-key tile the 4 keys 4g..4g+3, at d = 16*dt + li
-    uint2 vraw[2][DTL];
+  // values of a block: for each 16-key tile the 4 keys 4g..4g+3, at d = 16*dt + li
+  auto load_v = [&](int blk, uint2 (&vreg)[2][DTL]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      int key4 = key_base + 16 * t + 4 * g;
+      int key4 = blk * 32 + 16 * t + 4 * g;
       key4 = min(max(key4, kv_lo & ~3), (kv_hi - 1) & ~3);
-      const int page = table[key4 / P];
+      const int page = page_of(key4);
       const uint16_t* vp = a.v_pages + page * page_elems + k_head + (key4 % P);
 #pragma unroll
       for (int dt = 0; dt < DTL; ++dt) {
-        if (dt < n_dt) vraw[t][dt] = *reinterpret_cast<const uint2*>(vp + static_cast<int64_t>(16 * dt + li) * P);
+        if (dt < n_dt) vreg[t][dt] = *reinterpret_cast<const uint2*>(vp + static_cast<int64_t>(16 * dt + li) * P);
       }
     }
-    // keys of the next block, while this one is computed
-    bf16x8 knext[2][DCH];
-    if (blk + 1 < b1) load_k(blk + 1, knext);
+  };
+
+  bf16x8 kcur[2][DCH];
+  uint2 vraw[2][DTL];
+  if (b0 < b1) {
+    refill_pages(clamp_key(b0 * 32) / P);
+    load_k(b0, kcur);
+    load_v(b0, vraw);
+  }
+
+  for (int blk = b0; blk < b1; ++blk) {
+    const int key_base = blk * 32;
+    const bool more = blk + 1 < b1;
+    if (more) cover(blk + 1);
 
     // scores S^T: s[n][t][r] belongs to key key_base + 16t + 4g + r and row (n, li)
     f32x4 s[NT][2];
@@ -184,6 +206,8 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
           if (c < n_dch) z = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[t][c], qreg[n][c], z, 0, 0, 0);
         s[n][t] = z;
       }
+    // the key registers are free again: fetch the next block's keys while this block goes on
+    if (more) load_k(blk + 1, kcur);
 
     // a key beyond what the request holds may carry stale bits: its value must be 0, not 0 * garbage
     if (key_base + 32 > kv_total) {
@@ -192,6 +216,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
         const int key4 = key_base + 16 * t + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DTL; ++dt) {
+          if (dt >= n_dt) continue;
           if (key4 + 0 >= kv_total) vraw[t][dt].x &= 0xffff0000u;
           if (key4 + 1 >= kv_total) vraw[t][dt].x &= 0x0000ffffu;
           if (key4 + 2 >= kv_total) vraw[t][dt].y &= 0xffff0000u;
@@ -254,12 +279,8 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
           acc[n][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pb[n], acc[n][dt], 0, 0, 0);
       }
     }
-    if (blk + 1 < b1) {
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int c = 0; c < DCH; ++c) kcur[t][c] = knext[t][c];
-    }
+    // and the value registers after the second product
+    if (more) load_v(blk + 1, vraw);
   }
 
   // acc[n][dt][r] is O^T[d = 16dt + 4g + r][row (n, li)]
@@ -299,27 +320,29 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
   }
 }
 
-// out[row][head][:] = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m)
+// out[row][head][:] = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).   One wave per (row, head);
+// lane s holds the statistics of split s (splits <= 64), the weights travel by cross-lane reads, and
+// the partial outputs are read with independent loads.
 __global__ __launch_bounds__(kWave) void attn_merge_kernel(const float* __restrict__ ws_o,
                                                            const float* __restrict__ ws_ml,
                                                            uint16_t* __restrict__ out, int64_t o_stride,
                                                            int nq, int D, int splits) {
-  const int row = blockIdx.x, head = blockIdx.y;
+  const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int64_t base = (static_cast<int64_t>(row) * nq + head) * splits;
-  float mx = -INFINITY;
-  for (int s = 0; s < splits; ++s) mx = fmaxf(mx, ws_ml[(base + s) * 2]);
-  float denom = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float ms = ws_ml[(base + s) * 2];
-    if (ms > -INFINITY) denom += ws_ml[(base + s) * 2 + 1] * exp2f(ms - mx);
+  float ms = -INFINITY, ls = 0.f;
+  if (lane < splits) {
+    const float2 ml = *reinterpret_cast<const float2*>(ws_ml + (base + lane) * 2);
+    ms = ml.x;
+    ls = ml.y;
   }
+  const float mx = wave_max(ms);
+  const float wgt = ms > -INFINITY ? exp2f(ms - mx) : 0.f;  // an empty split weighs nothing
+  const float denom = wave_sum(ls * wgt);
   const float inv = denom > 0.f ? 1.0f / denom : 0.f;
-  for (int d = threadIdx.x; d < D; d += kWave) {
+  for (int d = lane; d < D; d += kWave) {
     float o = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float ms = ws_ml[(base + s) * 2];
-      if (ms > -INFINITY) o += ws_o[(base + s) * D + d] * exp2f(ms - mx);
-    }
+#pragma unroll 4
+    for (int s = 0; s < splits; ++s) o += ws_o[(base + s) * D + d] * __shfl(wgt, s, kWave);
     out[static_cast<int64_t>(row) * o_stride + head * D + d] = f32_to_bf16_bits(o * inv);
   }
 }
@@ -352,7 +375,7 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
                                     int nq, int nkv, int D, int page_size, float scale, int window,
                                     int splits, float* ws_o, float* ws_ml, void* stream) {
   if (segments == 0 || token_rows == 0) return 0;
-  if (D % 16 != 0 || D > 256 || D <= 0 || page_size % 4 != 0 || nq % nkv != 0 || splits < 1)
+  if (D % 16 != 0 || D > 256 || D <= 0 || page_size % 4 != 0 || nq % nkv != 0 || splits < 1 || splits > 64)
     return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   AttnArgs a;

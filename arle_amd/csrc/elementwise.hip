@@ -17,14 +17,18 @@ __global__ void embed_gather_kernel(const TT* __restrict__ table, const int* __r
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
 }
 
+// block == 0: gate and up are two [T, width] views.  block > 0: one buffer whose columns alternate
+// between `block` gate columns and the `block` matching up columns (gate is its first column).
 template <typename T>
 __global__ void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict__ up,
-                                int64_t in_stride, T* __restrict__ out, int width) {
+                                int64_t in_stride, T* __restrict__ out, int width, int block) {
   const int t = blockIdx.x;
   const int j = blockIdx.y * blockDim.x + threadIdx.x;
   if (j >= width) return;
-  const float g = to_float(gate[static_cast<int64_t>(t) * in_stride + j]);
-  const float u = to_float(up[static_cast<int64_t>(t) * in_stride + j]);
+  const int64_t row = static_cast<int64_t>(t) * in_stride;
+  const int64_t gi = block > 0 ? row + (j / block) * 2 * block + j % block : row + j;
+  const float g = to_float(gate[gi]);
+  const float u = to_float(block > 0 ? gate[gi + block] : up[gi]);
   const float act = g / (1.0f + expf(-g));
   out[static_cast<int64_t>(t) * width + j] = from_float<T>(act * u);
 }
@@ -48,18 +52,18 @@ extern "C" int arle_embed_gather(const void* table, int table_dtype, const int* 
 // gate and up are two columns blocks of rows with a common row stride (in
 // elements), so one fused [T, 2I] buffer and two separate buffers both fit.
 extern "C" int arle_silu_mul(const void* gate, const void* up, long long in_stride, void* out,
-                             int dtype, int tokens, int width, void* stream) {
+                             int dtype, int tokens, int width, int block, void* stream) {
   if (tokens == 0 || width == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(tokens, (width + 255) / 256);
   if (dtype == kF32) {
     silu_mul_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(gate),
                                                 static_cast<const float*>(up), in_stride,
-                                                static_cast<float*>(out), width);
+                                                static_cast<float*>(out), width, block);
   } else {
     silu_mul_kernel<bf16><<<grid, 256, 0, s>>>(static_cast<const bf16*>(gate),
                                                static_cast<const bf16*>(up), in_stride,
-                                               static_cast<bf16*>(out), width);
+                                               static_cast<bf16*>(out), width, block);
   }
   return launch_status();
 }

@@ -20,9 +20,10 @@ _f = ctypes.c_float
 # function name -> (library, argument types); every function returns a hipError_t as int
 SIGNATURES = {
     "arle_embed_gather": ("elementwise", [_p, _i, _p, _p, _i, _i, _p]),
-    "arle_silu_mul": ("elementwise", [_p, _p, _ll, _p, _i, _i, _i, _p]),
+    "arle_silu_mul": ("elementwise", [_p, _p, _ll, _p, _i, _i, _i, _i, _p]),
     "arle_rmsnorm": ("norm", [_p, _i, _ll, _p, _i, _p, _i, _p, _i, _i, _f, _p]),
     "arle_add_rmsnorm": ("norm", [_p, _p, _i, _p, _i, _p, _i, _p, _i, _i, _f, _p]),
+    "arle_gemm_bf16_skinny": ("gemm_bf16", [_p, _ll, _p, _ll, _p, _ll, _i, _i, _i, _i, _i, _i, _p]),
     "arle_gemm_f32": ("gemm_f32", [_p, _ll, _p, _ll, _p, _ll, _i, _i, _i, _p]),
     "arle_qk_prep": ("rope_kv", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _p, _i, _p, _p, _i, _p, _p, _p,
                                  _i, _p, _p, _i, _i, _i, _i, _i, _f, _p]),

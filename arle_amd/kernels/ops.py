@@ -77,6 +77,21 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | Non
     return out
 
 
+def silu_mul_interleaved(gate_up: torch.Tensor, block: int = 16):
+    """out[:, j] = silu(g_j) * u_j for a [T, 2I] buffer whose columns alternate between `block` gate
+    columns and the `block` matching up columns."""
+    _gpu(gate_up)
+    _rows(gate_up, "gate_up")
+    tokens, two_i = gate_up.shape
+    _need(block > 0 and two_i % (2 * block) == 0, "interleaved gate/up width must be a multiple of 2*block")
+    width = two_i // 2
+    _need(math.ceil(width / 256) <= _GRID_Y_MAX, "silu_mul: width too large")
+    out = torch.empty((tokens, width), dtype=gate_up.dtype, device=gate_up.device)
+    lib.call("arle_silu_mul", gate_up.data_ptr(), gate_up.data_ptr(), gate_up.stride(0), out.data_ptr(),
+             _code(gate_up), tokens, width, int(block), _stream())
+    return out
+
+
 def silu_mul(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor | None = None):
     """out = silu(gate) * up for two [T, I] views with the same row stride."""
     _gpu(gate, up, out)
@@ -91,7 +106,7 @@ def silu_mul(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor | None = No
     _need(out.shape == (tokens, width) and out.dtype == gate.dtype and out.is_contiguous(),
           "silu_mul output must be contiguous [T, I] of the input type")
     lib.call("arle_silu_mul", gate.data_ptr(), up.data_ptr(), gate.stride(0), out.data_ptr(),
-             _code(gate), tokens, width, _stream())
+             _code(gate), tokens, width, 0, _stream())
     return out
 
 
@@ -378,11 +393,62 @@ def apply_penalties(logits, indptr, tokens, counts, repetition, frequency, prese
 # ------------------------------------------------------------ bfloat16 products
 
 
+SKINNY_MAX_ROWS = 64
+SKINNY_PREFERRED_ROWS = 16   # up to here the kernel beats the library on MI355X; beyond, the library is used
+EPI_NONE, EPI_SILU_MUL = 0, 1
+_SKINNY_TARGET_WAVES = 2048
+
+
+def gemm_skinny_supported(rows: int, k: int, x_stride: int) -> bool:
+    return 0 < rows <= SKINNY_MAX_ROWS and k % 8 == 0 and x_stride % 8 == 0
+
+
+def gemm_skinny_preferred(rows: int, k: int, x_stride: int) -> bool:
+    return rows <= SKINNY_PREFERRED_ROWS and gemm_skinny_supported(rows, k, x_stride)
+
+
+def _skinny_waves(M: int, N: int, K: int, fused: bool) -> int:
+    """Waves of a workgroup that split K: enough waves in flight to fill the chip, each with at least
+    four 32-wide steps of its own, within what the reduction's LDS allows."""
+    nt = 1 if (M <= 16 and not fused) else 2
+    tiles = -(-N // (16 * nt))
+    steps = -(-K // 32)
+    cap = 8 if M > 16 else 16
+    want = max(1, -(-_SKINNY_TARGET_WAVES // tiles))
+    return max(1, min(want, cap, max(1, steps // 4)))
+
+
+def gemm_bf16_skinny(x, w, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE):
+    """out = x . w^T for 1..64 rows of x on the matrix cores, streaming w once from HBM.
+
+    EPI_SILU_MUL: w holds gate and up rows interleaved in blocks of 16; out[m, j] = silu(gate_j) * up_j.
+    """
+    _gpu(x, w)
+    _rows(x, "x")
+    _need(w.dim() == 2 and w.is_contiguous(), "w must be contiguous [N, K]")
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_bf16_skinny takes bfloat16 operands")
+    M, K = x.shape
+    N = w.shape[0]
+    _need(w.shape[1] == K, f"gemm_bf16_skinny: inner sizes differ ({K} vs {w.shape[1]})")
+    _need(gemm_skinny_supported(M, K, x.stride(0)),
+          f"gemm_bf16_skinny takes 1..{SKINNY_MAX_ROWS} rows and K % 8 == 0 (got {M} rows, K = {K})")
+    _need(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
+    _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_bf16_skinny writes bfloat16 or float32")
+    fused = epilogue == EPI_SILU_MUL
+    if fused:
+        _need(N % 32 == 0, "the fused activation needs gate/up interleaved in blocks of 16")
+    out = torch.empty((M, N // 2 if fused else N), dtype=out_dtype, device=x.device)
+    lib.call("arle_gemm_bf16_skinny", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(),
+             out.stride(0), _CODES[out_dtype], M, N, K, int(epilogue), _skinny_waves(M, N, K, fused), _stream())
+    return out
+
+
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16):
     """out[M, N] = x[M, K] . w[N, K]^T, bfloat16 operands, float32 accumulation.
 
-    Many rows go to the vendor library (hipBLASLt through torch.matmul), the matrix
-    product the reference also leaves to a library (crates/cuda-kernels/csrc/gemm/gemv.cu:240-330).
+    Up to 64 rows (decode steps) run the hand-written weight-streaming kernel.  More rows go to the
+    vendor library (hipBLASLt through torch.matmul), the matrix product the reference also leaves to
+    a library (crates/cuda-kernels/csrc/gemm/gemv.cu:240-330).
     """
     _gpu(x, w)
     _rows(x, "x")
@@ -390,6 +456,8 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_bf16 takes bfloat16 operands")
     _need(x.shape[1] == w.shape[1], f"gemm_bf16: inner sizes differ ({x.shape[1]} vs {w.shape[1]})")
     _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_bf16 writes bfloat16 or float32")
+    if gemm_skinny_preferred(x.shape[0], x.shape[1], x.stride(0)) and x.data_ptr() % 16 == 0:
+        return gemm_bf16_skinny(x, w, out_dtype)
     if out_dtype == torch.float32:
         return _library_mm_f32out(x, w)
     return torch.matmul(x, w.t())

@@ -30,10 +30,25 @@ class SwiGLU(Part):
         gate, up = tensors["gate"], tensors["up"]
         if gate.dtype != up.dtype:
             raise ValueError("gate and up projections must be stored in one type")
-        self.gate_up = Linear(torch.cat([gate, up], dim=0).contiguous())
+        # bfloat16: rows interleaved in blocks of 16 (16 gate rows, the 16 matching up rows, ...), so
+        # that one tile of the decode kernel holds both halves of 16 outputs and applies the activation
+        # itself.  Otherwise gate rows first, then up rows.
+        self.block = 16 if (gate.dtype == torch.bfloat16 and self.inter % 16 == 0) else 0
+        if self.block:
+            h = gate.shape[1]
+            fused = torch.stack([gate.view(-1, 16, h), up.view(-1, 16, h)], dim=1).reshape(2 * self.inter, h)
+        else:
+            fused = torch.cat([gate, up], dim=0)
+        self.gate_up = Linear(fused.contiguous())
         self.down = Linear(tensors["down"])
 
     def forward(self, x):
-        gu = self.gate_up(x)
-        act = ops.silu_mul(gu[:, : self.inter], gu[:, self.inter:])
+        if self.block:
+            if ops.gemm_skinny_preferred(x.shape[0], x.shape[1], x.stride(0)):
+                act = ops.gemm_bf16_skinny(x, self.gate_up.weight, x.dtype, ops.EPI_SILU_MUL)
+            else:
+                act = ops.silu_mul_interleaved(self.gate_up(x), self.block)
+        else:
+            gu = self.gate_up(x)
+            act = ops.silu_mul(gu[:, : self.inter], gu[:, self.inter:])
         return self.down(act)
