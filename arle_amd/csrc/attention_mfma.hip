@@ -50,9 +50,11 @@ struct AttnArgs {
   const int* seg_slot;   // [segments]
   const int* seg_start;  // [segments] position of a segment's first token
   int nq, nkv, D, P;
+  int p_shift;  // log2(P): page sizes are powers of two, so / and % by P are a shift and a mask
   float scale_log2;
   int window;  // 0: all earlier keys
   int splits;
+  int rows_max;  // the streaming kernel skips segments with more rows than this (0: takes all)
 };
 
 __device__ __forceinline__ bf16x8 load_bf16x8(const uint16_t* p) {
@@ -73,7 +75,9 @@ __device__ __forceinline__ float group_sum4(float v) {
   return v + __shfl_xor(v, 32, kWave);
 }
 
-template <int NT, int DMAX>
+// EXACT: head_dim == DMAX, known at compile time, so every "is this chunk inside the head" test and
+// every multiplication by head_dim folds away; otherwise head_dim is any multiple of 16 up to DMAX.
+template <int NT, int DMAX, bool EXACT>
 __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
   constexpr int DCH = DMAX / 32;  // contraction chunks of the first product
   constexpr int DTL = DMAX / 16;  // d tiles of the output
@@ -86,10 +90,11 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
   const int rows = qlen * G;
   const int row_begin = blockIdx.x * (16 * NT);
   if (row_begin >= rows) return;  // the whole wave leaves
+  if (a.rows_max > 0 && rows > a.rows_max) return;  // long segments belong to the LDS kernel
   const int start = a.seg_start[seg];
   const int* table = a.block_table + static_cast<int64_t>(a.seg_slot[seg]) * a.table_stride;
-  const int D = a.D, P = a.P;
-  const int n_dch = (D + 31) / 32, n_dt = D / 16;
+  const int D = EXACT ? DMAX : a.D, P = a.P;
+  const int n_dch = EXACT ? DCH : (D + 31) / 32, n_dt = EXACT ? DTL : D / 16;
 
   const int tok_min = row_begin / G;
   const int tok_max = (min(row_begin + 16 * NT, rows) - 1) / G;
@@ -118,7 +123,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
 #pragma unroll
     for (int c = 0; c < DCH; ++c) {
       const int d = 32 * c + 8 * g;
-      qreg[n][c] = (c < n_dch && d < D) ? load_bf16x8(qp + d) : zero_bf16x8();
+      qreg[n][c] = (EXACT || (c < n_dch && d < D)) ? load_bf16x8(qp + d) : zero_bf16x8();
     }
   }
 
@@ -138,17 +143,18 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
   // Page ids of 64 consecutive logical pages sit in one register across the wave (lane i holds
   // page pg_base + i) and are fetched with a cross-lane read, so that the address of a key or value
   // load does not wait for a block-table load first.  Refilled when the walk leaves the window.
-  const int pg_last = (kv_hi - 1) / P;
+  const int pg_last = (kv_hi - 1) >> a.p_shift;
   int pg_base = 0, pg_reg = 0;
   auto refill_pages = [&](int first_page) {
     pg_base = first_page;
     pg_reg = table[min(first_page + lane, pg_last)];
   };
-  auto page_of = [&](int key) { return __shfl(pg_reg, key / P - pg_base, kWave); };
+  const int ps = a.p_shift, pm = P - 1;
+  auto page_of = [&](int key) { return __shfl(pg_reg, (key >> ps) - pg_base, kWave); };
   auto clamp_key = [&](int key) { return min(max(key, kv_lo), kv_hi - 1); };
   // the blocks blk and blk + 1 are in use at any time: make sure the register covers both
   auto cover = [&](int blk) {
-    const int first = clamp_key(blk * 32) / P, last = clamp_key(blk * 32 + 63) / P;
+    const int first = clamp_key(blk * 32) >> ps, last = clamp_key(blk * 32 + 63) >> ps;
     if (first < pg_base || last >= pg_base + kWave) refill_pages(first);
   };
 
@@ -157,11 +163,11 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
     for (int t = 0; t < 2; ++t) {
       const int key = clamp_key(blk * 32 + 16 * t + li);  // a held, written key; out-of-range ones are masked below
       const int page = page_of(key);
-      const uint16_t* kp = a.k_pages + page * page_elems + k_head + static_cast<int64_t>(key % P) * D;
+      const uint16_t* kp = a.k_pages + page * page_elems + k_head + static_cast<int64_t>(key & pm) * D;
 #pragma unroll
       for (int c = 0; c < DCH; ++c) {
         const int d = 32 * c + 8 * g;
-        kreg[t][c] = (c < n_dch && d < D) ? load_bf16x8(kp + d) : zero_bf16x8();
+        kreg[t][c] = (EXACT || (c < n_dch && d < D)) ? load_bf16x8(kp + d) : zero_bf16x8();
       }
     }
   };
@@ -173,10 +179,10 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
       int key4 = blk * 32 + 16 * t + 4 * g;
       key4 = min(max(key4, kv_lo & ~3), (kv_hi - 1) & ~3);
       const int page = page_of(key4);
-      const uint16_t* vp = a.v_pages + page * page_elems + k_head + (key4 % P);
+      const uint16_t* vp = a.v_pages + page * page_elems + k_head + (key4 & pm);
 #pragma unroll
       for (int dt = 0; dt < DTL; ++dt) {
-        if (dt < n_dt) vreg[t][dt] = *reinterpret_cast<const uint2*>(vp + static_cast<int64_t>(16 * dt + li) * P);
+        if (EXACT || dt < n_dt) vreg[t][dt] = *reinterpret_cast<const uint2*>(vp + static_cast<int64_t>(16 * dt + li) * P);
       }
     }
   };
@@ -184,7 +190,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
   bf16x8 kcur[2][DCH];
   uint2 vraw[2][DTL];
   if (b0 < b1) {
-    refill_pages(clamp_key(b0 * 32) / P);
+    refill_pages(clamp_key(b0 * 32) >> ps);
     load_k(b0, kcur);
     load_v(b0, vraw);
   }
@@ -203,7 +209,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
         f32x4 z = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int c = 0; c < DCH; ++c)
-          if (c < n_dch) z = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[t][c], qreg[n][c], z, 0, 0, 0);
+          if (EXACT || c < n_dch) z = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[t][c], qreg[n][c], z, 0, 0, 0);
         s[n][t] = z;
       }
     // the key registers are free again: fetch the next block's keys while this block goes on
@@ -216,7 +222,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
         const int key4 = key_base + 16 * t + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DTL; ++dt) {
-          if (dt >= n_dt) continue;
+          if (!EXACT && dt >= n_dt) continue;
           if (key4 + 0 >= kv_total) vraw[t][dt].x &= 0xffff0000u;
           if (key4 + 1 >= kv_total) vraw[t][dt].x &= 0x0000ffffu;
           if (key4 + 2 >= kv_total) vraw[t][dt].y &= 0xffff0000u;
@@ -252,8 +258,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
         for (int r = 0; r < 4; r += 2) {
           const float p0 = exp2f(sv[t][r] - m_use), p1 = exp2f(sv[t][r + 1] - m_use);
           psum += p0 + p1;
-          packed[2 * t + r / 2] = static_cast<uint32_t>(f32_to_bf16_bits(p0)) |
-                                  (static_cast<uint32_t>(f32_to_bf16_bits(p1)) << 16);
+          packed[2 * t + r / 2] = pack_bf16x2(p0, p1);
         }
       psum = group_sum4(psum);
       l[n] = l[n] * alpha + psum;
@@ -271,7 +276,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
 
 #pragma unroll
     for (int dt = 0; dt < DTL; ++dt) {
-      if (dt < n_dt) {
+      if (EXACT || dt < n_dt) {
         uint4 vv = {vraw[0][dt].x, vraw[0][dt].y, vraw[1][dt].x, vraw[1][dt].y};
         const bf16x8 vop = __builtin_bit_cast(bf16x8, vv);
 #pragma unroll
@@ -293,7 +298,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
       uint16_t* op = a.out + tok_row * a.o_stride + my_head[n] * D;
 #pragma unroll
       for (int dt = 0; dt < DTL; ++dt) {
-        if (dt < n_dt) {
+        if (EXACT || dt < n_dt) {
           uint2 w;
           w.x = static_cast<uint32_t>(f32_to_bf16_bits(acc[n][dt][0] * inv_l)) |
                 (static_cast<uint32_t>(f32_to_bf16_bits(acc[n][dt][1] * inv_l)) << 16);
@@ -307,7 +312,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
       float* wo = a.ws_o + slot * D;
 #pragma unroll
       for (int dt = 0; dt < DTL; ++dt) {
-        if (dt < n_dt) {
+        if (EXACT || dt < n_dt) {
           float4 w = {acc[n][dt][0], acc[n][dt][1], acc[n][dt][2], acc[n][dt][3]};
           *reinterpret_cast<float4*>(wo + 16 * dt + 4 * g) = w;
         }
@@ -320,14 +325,18 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
   }
 }
 
-// out[row][head][:] = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).   One wave per (row, head);
-// lane s holds the statistics of split s (splits <= 64), the weights travel by cross-lane reads, and
-// the partial outputs are read with independent loads.
-__global__ __launch_bounds__(kWave) void attn_merge_kernel(const float* __restrict__ ws_o,
-                                                           const float* __restrict__ ws_ml,
-                                                           uint16_t* __restrict__ out, int64_t o_stride,
-                                                           int nq, int D, int splits) {
-  const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+// out[row][head][:] = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).   One workgroup of four waves
+// per (row, head).  Lane s of every wave holds the statistics of split s (splits <= 64) and the
+// weights travel by cross-lane reads; wave w adds the splits s = w, w+4, ... with all its loads
+// independent of one another, and the four partial sums meet in LDS in wave order.
+constexpr int kMergeWaves = 4;
+constexpr int kMergeMaxD = 256;
+__global__ __launch_bounds__(kMergeWaves* kWave) void attn_merge_kernel(
+    const float* __restrict__ ws_o, const float* __restrict__ ws_ml, uint16_t* __restrict__ out,
+    int64_t o_stride, int nq, int D, int splits) {
+  __shared__ float part[kMergeWaves][kMergeMaxD];
+  const int row = blockIdx.x, head = blockIdx.y;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int64_t base = (static_cast<int64_t>(row) * nq + head) * splits;
   float ms = -INFINITY, ls = 0.f;
   if (lane < splits) {
@@ -339,22 +348,361 @@ __global__ __launch_bounds__(kWave) void attn_merge_kernel(const float* __restri
   const float wgt = ms > -INFINITY ? exp2f(ms - mx) : 0.f;  // an empty split weighs nothing
   const float denom = wave_sum(ls * wgt);
   const float inv = denom > 0.f ? 1.0f / denom : 0.f;
-  for (int d = lane; d < D; d += kWave) {
-    float o = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < splits; ++s) o += ws_o[(base + s) * D + d] * __shfl(wgt, s, kWave);
-    out[static_cast<int64_t>(row) * o_stride + head * D + d] = f32_to_bf16_bits(o * inv);
+  // each lane owns d = 4*lane .. 4*lane+3 (D <= 256)
+  const int d0 = 4 * lane;
+  float4 o = {0.f, 0.f, 0.f, 0.f};
+  const bool mine = d0 < D;
+  const float* src = ws_o + base * D + (mine ? d0 : 0);
+#pragma unroll 8
+  for (int s = wave; s < splits; s += kMergeWaves) {
+    const float w = __shfl(wgt, s, kWave);  // every lane takes part in the cross-lane read
+    const float4 v = *reinterpret_cast<const float4*>(src + static_cast<int64_t>(s) * D);
+    o.x += v.x * w;
+    o.y += v.y * w;
+    o.z += v.z * w;
+    o.w += v.w * w;
+  }
+  if (mine) *reinterpret_cast<float4*>(&part[wave][d0]) = o;
+  __syncthreads();
+  if (wave == 0 && d0 < D) {
+#pragma unroll
+    for (int v = 1; v < kMergeWaves; ++v) {
+      const float4 p = *reinterpret_cast<const float4*>(&part[v][d0]);
+      o.x += p.x;
+      o.y += p.y;
+      o.z += p.z;
+      o.w += p.w;
+    }
+    uint2 w;
+    w.x = static_cast<uint32_t>(f32_to_bf16_bits(o.x * inv)) | (static_cast<uint32_t>(f32_to_bf16_bits(o.y * inv)) << 16);
+    w.y = static_cast<uint32_t>(f32_to_bf16_bits(o.z * inv)) | (static_cast<uint32_t>(f32_to_bf16_bits(o.w * inv)) << 16);
+    *reinterpret_cast<uint2*>(out + static_cast<int64_t>(row) * o_stride + head * D + d0) = w;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Prompt portions: the same products, with keys and values staged through LDS.
+//
+// A workgroup of four waves owns 128 rows (32 per wave, two row tiles) of one segment and kv head
+// and walks the keys in tiles of 64.  All 256 threads fetch a tile with coalesced loads (a key page
+// [slot][d] and a value page [d][slot] are contiguous in memory), park it in LDS, and every wave
+// reads its MFMA operands from there, so a key or value is read from L2 once per 128 rows instead
+// of once per 32.  Two LDS stages: tile i+1 is on its way from memory while tile i is computed.
+constexpr int kPfWaves = 4;
+constexpr int kPfRows = 32 * kPfWaves;  // rows of a workgroup
+constexpr int kPfKeys = 64;             // keys of a tile
+
+template <int DMAX, bool EXACT>
+__global__ __launch_bounds__(kPfWaves* kWave) void attn_prefill_lds_kernel(const AttnArgs a, int min_rows) {
+  constexpr int NT = 2;
+  constexpr int DCH = DMAX / 32, DTL = DMAX / 16;
+  constexpr int kKPieces = (kPfKeys * (DMAX / 8) + kPfWaves * kWave - 1) / (kPfWaves * kWave);  // 16-byte pieces per thread
+  constexpr int kVPieces = (kPfKeys / 4 * DMAX + kPfWaves * kWave - 1) / (kPfWaves * kWave);    // 8-byte pieces per thread
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, g = lane >> 4;
+  const int seg = blockIdx.z, kvh = blockIdx.y;
+  const int G = a.nq / a.nkv;
+  const int row0 = a.seg_row0[seg];
+  const int qlen = a.seg_row0[seg + 1] - row0;
+  const int rows = qlen * G;
+  if (rows < min_rows) return;  // short segments (decoded tokens) belong to the other kernel
+  const int wg_row = blockIdx.x * kPfRows;
+  if (wg_row >= rows) return;
+  const int start = a.seg_start[seg];
+  const int* table = a.block_table + static_cast<int64_t>(a.seg_slot[seg]) * a.table_stride;
+  const int D = EXACT ? DMAX : a.D, P = a.P;
+  const int n_dch = EXACT ? DCH : (D + 31) / 32, n_dt = EXACT ? DTL : D / 16;
+
+  // LDS: two stages of [64 keys][D + 8] keys and [D][64 + 8] values (bfloat16; rows padded by 16 bytes)
+  const int k_pitch = D + 8, v_pitch = kPfKeys + 8;
+  const int stage_elems = kPfKeys * k_pitch + D * v_pitch;
+  uint16_t* lds = reinterpret_cast<uint16_t*>(lds_raw);
+
+  // keys this workgroup needs
+  const int tok_min = wg_row / G;
+  const int tok_max = (min(wg_row + kPfRows, rows) - 1) / G;
+  const int kv_total = start + qlen;
+  const int kv_hi = start + tok_max + 1;
+  const int kv_lo = a.window > 0 ? max(0, start + tok_min - a.window + 1) : 0;
+  const int t0 = kv_lo / kPfKeys, t1 = (kv_hi + kPfKeys - 1) / kPfKeys;
+
+  // this wave's rows
+  const int row_begin = wg_row + 32 * wave;
+  const bool wave_has_rows = row_begin < rows;
+  const int wave_tok_max = wave_has_rows ? (min(row_begin + 32, rows) - 1) / G : 0;
+  const int wave_kv_hi = start + wave_tok_max + 1;
+  const int wave_kv_lo = a.window > 0 ? max(0, start + min(row_begin, rows - 1) / G - a.window + 1) : 0;
+  // a tile needs no mask for this wave if it lies at or below its first row's position and at or
+  // above its last row's window edge
+  const int wave_pos_min = start + min(row_begin, rows - 1) / G;
+  const int wave_win_lo = a.window > 0 ? max(0, start + wave_tok_max - a.window + 1) : 0;
+  int my_pos[NT], my_tok[NT], my_head[NT];
+  bool row_ok[NT];
+  bf16x8 qreg[NT][DCH];
+#pragma unroll
+  for (int n = 0; n < NT; ++n) {
+    const int row = row_begin + 16 * n + li;
+    row_ok[n] = row < rows;
+    my_tok[n] = min(row / G, qlen - 1);
+    my_head[n] = kvh * G + row % G;
+    my_pos[n] = start + my_tok[n];
+    const uint16_t* qp = a.q + static_cast<int64_t>(row0 + my_tok[n]) * a.q_stride + my_head[n] * D;
+#pragma unroll
+    for (int c = 0; c < DCH; ++c) {
+      const int d = 32 * c + 8 * g;
+      qreg[n][c] = (EXACT || (c < n_dch && d < D)) ? load_bf16x8(qp + d) : zero_bf16x8();
+    }
+  }
+  f32x4 acc[NT][DTL];
+  float m[NT], l[NT];
+#pragma unroll
+  for (int n = 0; n < NT; ++n) {
+    m[n] = -INFINITY;
+    l[n] = 0.f;
+#pragma unroll
+    for (int t = 0; t < DTL; ++t) acc[n][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int64_t head_off = static_cast<int64_t>(kvh) * P * D;
+  const int64_t page_elems = static_cast<int64_t>(a.nkv) * P * D;
+  // What each thread moves per tile never changes: work the indices out once (they take divisions),
+  // leave only "which page" to the loop.
+  const int ps = a.p_shift, pm = P - 1;
+  const int k_chunks = D / 8;                    // 16-byte pieces of a key row
+  const int k_total = kPfKeys * k_chunks;
+  const int kp = min(P, kPfKeys);                // keys of one page inside a tile
+  const int v_per_row = kp / 4;                  // 8-byte pieces of one d row of a page, inside the tile
+  const int v_total = (kPfKeys / 4) * D;
+  int k_key[kKPieces], k_col[kKPieces], k_lds[kKPieces];
+  int v_d[kVPieces], v_off[kVPieces], v_lds[kVPieces];
+#pragma unroll
+  for (int j = 0; j < kKPieces; ++j) {
+    const int p = tid + j * (kPfWaves * kWave);
+    k_key[j] = p < k_total ? p / k_chunks : -1;  // -1: this thread has no such piece
+    k_col[j] = (p % k_chunks) * 8;
+    k_lds[j] = (p / k_chunks) * k_pitch + k_col[j];
+  }
+#pragma unroll
+  for (int j = 0; j < kVPieces; ++j) {
+    const int p = tid + j * (kPfWaves * kWave);
+    const int qi = p % v_per_row, d = (p / v_per_row) % D, pg = p / (v_per_row * D);
+    v_d[j] = p < v_total ? d : -1;
+    v_off[j] = pg * kp + 4 * qi;  // first of 4 keys, inside the tile
+    v_lds[j] = d * v_pitch + v_off[j];
+  }
+
+  // Page ids of 64 consecutive logical pages sit in one register across the wave (lane i: page
+  // pg_base + i), so a piece's address needs a cross-lane read, not a block-table load of its own.
+  const int pg_last = (kv_hi - 1) >> ps;
+  int pg_base = 0, pg_reg = 0;
+  auto cover = [&](int tile) {  // make the register hold the pages of this tile
+    const int first = min(max(tile * kPfKeys, kv_lo), kv_hi - 1) >> ps;
+    const int last = min(max(tile * kPfKeys + kPfKeys - 1, kv_lo), kv_hi - 1) >> ps;
+    if (tile == t0 || first < pg_base || last >= pg_base + kWave) {
+      pg_base = first;
+      pg_reg = table[min(first + lane, pg_last)];
+    }
+  };
+
+  uint4 kstage[kKPieces];
+  uint2 vstage[kVPieces];
+  auto fetch = [&](int tile) {
+    const int base = tile * kPfKeys;
+    cover(tile);
+#pragma unroll
+    for (int j = 0; j < kKPieces; ++j) {
+      const int key = min(max(base + max(k_key[j], 0), kv_lo), kv_hi - 1);
+      const int page = __shfl(pg_reg, (key >> ps) - pg_base, kWave);  // every lane takes part
+      if (EXACT || k_key[j] >= 0)
+        kstage[j] = *reinterpret_cast<const uint4*>(a.k_pages + page * page_elems + head_off +
+                                                    static_cast<int64_t>(key & pm) * D + k_col[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < kVPieces; ++j) {
+      const int off = base + v_off[j];
+      const int key4 = min(max(off, kv_lo & ~3), (kv_hi - 1) & ~3);
+      const int page = __shfl(pg_reg, (key4 >> ps) - pg_base, kWave);
+      if (EXACT || v_d[j] >= 0) {
+        uint2 v = *reinterpret_cast<const uint2*>(a.v_pages + page * page_elems + head_off +
+                                                  static_cast<int64_t>(v_d[j]) * P + (key4 & pm));
+        if (off + 4 > kv_total) {  // never written in this request: may hold anything
+          if (off + 0 >= kv_total) v.x &= 0xffff0000u;
+          if (off + 1 >= kv_total) v.x &= 0x0000ffffu;
+          if (off + 2 >= kv_total) v.y &= 0xffff0000u;
+          if (off + 3 >= kv_total) v.y &= 0x0000ffffu;
+        }
+        vstage[j] = v;
+      }
+    }
+  };
+  auto park = [&](int stage) {
+    uint16_t* ks = lds + stage * stage_elems;
+    uint16_t* vs = ks + kPfKeys * k_pitch;
+#pragma unroll
+    for (int j = 0; j < kKPieces; ++j)
+      if (EXACT || k_key[j] >= 0) *reinterpret_cast<uint4*>(ks + k_lds[j]) = kstage[j];
+#pragma unroll
+    for (int j = 0; j < kVPieces; ++j)
+      if (EXACT || v_d[j] >= 0) *reinterpret_cast<uint2*>(vs + v_lds[j]) = vstage[j];
+  };
+
+  fetch(t0);
+  park(0);
+  __syncthreads();
+
+  for (int tile = t0; tile < t1; ++tile) {
+    const int stage = (tile - t0) & 1;
+    const bool more = tile + 1 < t1;
+    if (more) fetch(tile + 1);
+
+    const int key_base = tile * kPfKeys;
+    // a wave whose rows see none of this tile's keys only helps with the loads
+    if (wave_has_rows && key_base < wave_kv_hi && key_base + kPfKeys > wave_kv_lo) {
+      const uint16_t* ks = lds + stage * stage_elems;
+      const uint16_t* vs = ks + kPfKeys * k_pitch;
+      f32x4 s[NT][4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        f32x4 z[NT];
+#pragma unroll
+        for (int n = 0; n < NT; ++n) z[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < DCH; ++c) {
+          if (EXACT || c < n_dch) {
+            const int d = 32 * c + 8 * g;
+            const bf16x8 kop = (EXACT || d < D) ? __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(ks + (16 * t + li) * k_pitch + d))
+                                     : zero_bf16x8();
+#pragma unroll
+            for (int n = 0; n < NT; ++n) z[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qreg[n][c], z[n], 0, 0, 0);
+          }
+        }
+#pragma unroll
+        for (int n = 0; n < NT; ++n) s[n][t] = z[n];
+      }
+
+      // Only tiles that touch a row's causal edge or window edge need the mask; the others take
+      // the short path.  m is kept in the exponent's domain (score * scale * log2 e).
+      const bool masked = key_base + kPfKeys - 1 > wave_pos_min || key_base < wave_win_lo;
+      bf16x8 pb[NT][2];
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        if (masked) {
+          const int lo = a.window > 0 ? my_pos[n] - a.window + 1 : 0;
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int key = key_base + 16 * t + 4 * g + r;
+              if (!(key >= lo && key <= my_pos[n])) s[n][t][r] = -INFINITY;
+            }
+        }
+        float bmax = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) bmax = fmaxf(bmax, s[n][t][r]);
+        bmax = group_max4(bmax) * a.scale_log2;  // scale > 0: the maximum commutes with it
+        const float m_new = fmaxf(m[n], bmax);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
+        const float alpha = __builtin_amdgcn_exp2f(m[n] - m_use);
+        float psum = 0.f;
+        uint32_t packed[8];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int r = 0; r < 4; r += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(s[n][t][r], a.scale_log2, -m_use));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(s[n][t][r + 1], a.scale_log2, -m_use));
+            psum += p0 + p1;
+            packed[2 * t + r / 2] = pack_bf16x2(p0, p1);
+          }
+        psum = group_sum4(psum);
+        l[n] = l[n] * alpha + psum;
+        // the accumulators need the factor only if some row's maximum moved
+        if (__builtin_amdgcn_ballot_w64(m_new > m[n]) != 0) {
+#pragma unroll
+          for (int dt = 0; dt < DTL; ++dt) {
+            acc[n][dt][0] *= alpha;
+            acc[n][dt][1] *= alpha;
+            acc[n][dt][2] *= alpha;
+            acc[n][dt][3] *= alpha;
+          }
+        }
+        m[n] = m_new;
+        uint4 p01 = {packed[0], packed[1], packed[2], packed[3]};  // keys 4g.. of tiles 0 and 1
+        uint4 p23 = {packed[4], packed[5], packed[6], packed[7]};  // ... of tiles 2 and 3
+        pb[n][0] = __builtin_bit_cast(bf16x8, p01);
+        pb[n][1] = __builtin_bit_cast(bf16x8, p23);
+      }
+
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int dt = 0; dt < DTL; ++dt) {
+          if (EXACT || dt < n_dt) {
+            const uint16_t* vrow = vs + (16 * dt + li) * v_pitch + 32 * u + 4 * g;
+            const uint2 va = *reinterpret_cast<const uint2*>(vrow);
+            const uint2 vb = *reinterpret_cast<const uint2*>(vrow + 16);
+            uint4 vv = {va.x, va.y, vb.x, vb.y};
+            const bf16x8 vop = __builtin_bit_cast(bf16x8, vv);
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+              acc[n][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pb[n][u], acc[n][dt], 0, 0, 0);
+          }
+        }
+    }
+
+    if (more) park(stage ^ 1);  // the other stage was last read before the barrier that ended the previous round
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int n = 0; n < NT; ++n) {
+    if (!row_ok[n]) continue;
+    const float inv_l = l[n] > 0.f ? 1.0f / l[n] : 0.f;
+    uint16_t* op = a.out + static_cast<int64_t>(row0 + my_tok[n]) * a.o_stride + my_head[n] * D;
+#pragma unroll
+    for (int dt = 0; dt < DTL; ++dt) {
+      if (EXACT || dt < n_dt) {
+        uint2 w;
+        w.x = static_cast<uint32_t>(f32_to_bf16_bits(acc[n][dt][0] * inv_l)) |
+              (static_cast<uint32_t>(f32_to_bf16_bits(acc[n][dt][1] * inv_l)) << 16);
+        w.y = static_cast<uint32_t>(f32_to_bf16_bits(acc[n][dt][2] * inv_l)) |
+              (static_cast<uint32_t>(f32_to_bf16_bits(acc[n][dt][3] * inv_l)) << 16);
+        *reinterpret_cast<uint2*>(op + 16 * dt + 4 * g) = w;
+      }
+    }
   }
 }
 
 template <int NT>
 int launch_attn(const AttnArgs& a, dim3 grid, hipStream_t s) {
+  // This kernel is bound by memory, not by instruction issue: it always runs with head_dim as a
+  // run-time value (the compile-time variant is kept for the LDS kernel, where it pays).
   if (a.D <= 64)
-    attn_mfma_kernel<NT, 64><<<grid, kWave, 0, s>>>(a);
+    attn_mfma_kernel<NT, 64, false><<<grid, kWave, 0, s>>>(a);
   else if (a.D <= 128)
-    attn_mfma_kernel<NT, 128><<<grid, kWave, 0, s>>>(a);
+    attn_mfma_kernel<NT, 128, false><<<grid, kWave, 0, s>>>(a);
   else
-    attn_mfma_kernel<NT, 256><<<grid, kWave, 0, s>>>(a);
+    attn_mfma_kernel<NT, 256, false><<<grid, kWave, 0, s>>>(a);
+  return launch_status();
+}
+
+inline size_t prefill_lds_bytes(int D) {
+  return 2 * (static_cast<size_t>(kPfKeys) * (D + 8) + static_cast<size_t>(D) * (kPfKeys + 8)) * sizeof(uint16_t);
+}
+
+template <int DMAX, bool EXACT>
+int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s) {
+  const size_t lds = prefill_lds_bytes(a.D);
+  static size_t allowed = 64 * 1024;  // dynamic LDS above 64 KiB has to be asked for, once per kernel
+  if (lds > allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_lds_kernel<DMAX, EXACT>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) return static_cast<int>(e);
+    allowed = lds;
+  }
+  attn_prefill_lds_kernel<DMAX, EXACT><<<grid, kPfWaves * kWave, lds, s>>>(a, min_rows);
   return launch_status();
 }
 
@@ -365,17 +713,19 @@ using namespace arle;
 // q, out: bfloat16 [token rows, nq*D] (row strides in elements).  Segments describe the packed
 // step: seg_row0[s]..seg_row0[s+1] are the token rows of segment s, whose first token sits at
 // position seg_start[s] of the request in block-table row seg_slot[s]; the cache already holds
-// the keys and values of these tokens.  max_qlen is the longest segment.  With splits > 1,
+// the keys and values of these tokens.  max_qlen / min_qlen are the longest and shortest segment.  With splits > 1,
 // ws_o/ws_ml must hold [token rows][nq][splits][D] and [..][2] floats and the merge runs after.
-// Requires D % 16 == 0, D <= 256, page_size % 4 == 0.
+// Requires D % 16 == 0, D <= 256, page_size a power of two >= 4.
 extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out, long long o_stride,
                                     const void* k_pages, const void* v_pages, const int* block_table,
                                     int table_stride, const int* seg_row0, const int* seg_slot,
-                                    const int* seg_start, int segments, int max_qlen, int token_rows,
+                                    const int* seg_start, int segments, int max_qlen, int min_qlen,
+                                    int token_rows,
                                     int nq, int nkv, int D, int page_size, float scale, int window,
                                     int splits, float* ws_o, float* ws_ml, void* stream) {
   if (segments == 0 || token_rows == 0) return 0;
-  if (D % 16 != 0 || D > 256 || D <= 0 || page_size % 4 != 0 || nq % nkv != 0 || splits < 1 || splits > 64)
+  if (D % 16 != 0 || D > 256 || D <= 0 || page_size < 4 || (page_size & (page_size - 1)) != 0 || nq % nkv != 0 ||
+      splits < 1 || splits > 64)
     return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   AttnArgs a;
@@ -396,19 +746,41 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
   a.nkv = nkv;
   a.D = D;
   a.P = page_size;
+  a.p_shift = __builtin_ctz(static_cast<unsigned>(page_size));
   a.scale_log2 = scale * 1.4426950408889634f;
   a.window = window;
   a.splits = splits;
+  a.rows_max = 0;
   const int G = nq / nkv;
-  const int max_rows = max_qlen * G;
-  // one row tile of 16 when a segment's rows fit it (decoded tokens), else two
-  const int nt = max_rows <= 16 ? 1 : 2;
+  const int max_rows = max_qlen * G, min_rows = min_qlen * G;
   const long long z = static_cast<long long>(segments) * splits;
   if (nkv > 65535 || z > 65535) return static_cast<int>(hipErrorInvalidValue);
+  int rc = 0;
+  const bool lds_ok = prefill_lds_bytes(D) <= 160 * 1024;
+  if (max_rows > 16 && lds_ok) {
+    // prompt portions through the LDS kernel; segments of at most 16 rows (decoded tokens of a mixed
+    // step) through the streaming kernel
+    dim3 grid((max_rows + kPfRows - 1) / kPfRows, nkv, segments);
+    if (D == 64)
+      rc = launch_prefill_lds<64, true>(a, grid, 17, s);
+    else if (D == 128)
+      rc = launch_prefill_lds<128, true>(a, grid, 17, s);
+    else if (D <= 64)
+      rc = launch_prefill_lds<64, false>(a, grid, 17, s);
+    else if (D <= 128)
+      rc = launch_prefill_lds<128, false>(a, grid, 17, s);
+    else
+      rc = launch_prefill_lds<256, false>(a, grid, 17, s);
+    if (rc != 0 || min_rows > 16) return rc;
+    a.rows_max = 16;
+    return launch_attn<1>(a, dim3(1, nkv, segments), s);
+  }
+  // one row tile of 16 when a segment's rows fit it (decoded tokens), else two
+  const int nt = max_rows <= 16 ? 1 : 2;
   dim3 grid((max_rows + 16 * nt - 1) / (16 * nt), nkv, static_cast<unsigned>(z));
-  int rc = nt == 1 ? launch_attn<1>(a, grid, s) : launch_attn<2>(a, grid, s);
+  rc = nt == 1 ? launch_attn<1>(a, grid, s) : launch_attn<2>(a, grid, s);
   if (rc != 0 || splits == 1) return rc;
   dim3 mgrid(token_rows, nq);
-  attn_merge_kernel<<<mgrid, kWave, 0, s>>>(ws_o, ws_ml, a.out, o_stride, nq, D, splits);
+  attn_merge_kernel<<<mgrid, kMergeWaves * kWave, 0, s>>>(ws_o, ws_ml, a.out, o_stride, nq, D, splits);
   return launch_status();
 }

@@ -22,12 +22,17 @@ __device__ __forceinline__ float to_float(bf16 v) {
   return __uint_as_float(static_cast<uint32_t>(v.bits) << 16);
 }
 
-// Round to nearest, ties to even; NaN stays NaN.
+// Round to nearest, ties to even (the hardware conversion of gfx950, v_cvt_pk_bf16_f32).
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+}
+
+// Two floats to two bfloat16 in one register: a in the low half, b in the high half.
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 template <typename T>

@@ -36,6 +36,7 @@ class StepBatch:
     segments: list
     max_position: int
     max_qlen: int                # longest segment
+    min_qlen: int                # shortest segment
     token_ids: torch.Tensor      # int32 [T]
     positions: torch.Tensor      # int32 [T]  absolute position of each row in its request
     slot_of_token: torch.Tensor  # int32 [T]  row of the block tables / state buffers
@@ -110,4 +111,5 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device, into=
         dev[k] = packed[off:off + n]
         off += n
     return StepBatch(num_tokens=row, segments=segments, max_position=max(pos),
-                     max_qlen=max(s.length for s in segments), host=host, **dev)
+                     max_qlen=max(s.length for s in segments), min_qlen=min(s.length for s in segments),
+                     host=host, **dev)

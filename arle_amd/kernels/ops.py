@@ -286,7 +286,7 @@ _MFMA_TARGET_WAVES = 4096   # waves wanted in flight for a decode launch (256 CU
 
 def attn_mfma_supported(dtype, head_dim: int, page_size: int) -> bool:
     return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 0 < head_dim <= MFMA_MAX_HEAD_DIM
-            and page_size % 4 == 0)
+            and page_size >= 4 and page_size & (page_size - 1) == 0)
 
 
 def decode_split_cap(max_kv_len: int) -> int:
@@ -301,7 +301,8 @@ def decode_splits(segments: int, num_kv_heads: int, max_kv_len: int) -> int:
 
 def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *,
                     max_qlen: int, max_kv_len: int, num_q_heads: int, num_kv_heads: int, head_dim: int,
-                    page_size: int, scale: float, window: int = 0, splits: int | None = None):
+                    page_size: int, scale: float, window: int = 0, splits: int | None = None,
+                    min_qlen: int = 1):
     """Causal attention of a packed step on the matrix cores (bfloat16).
 
     Segments: rows seg_row0[s]..seg_row0[s+1] belong to block-table row seg_slot[s] and start at
@@ -314,7 +315,7 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
     _need(q.shape == (tokens, num_q_heads * head_dim) and out.shape == q.shape and out.is_contiguous(),
           "q must be [T, nq*D] and out contiguous [T, nq*D]")
     _need(attn_mfma_supported(q.dtype, head_dim, page_size),
-          f"the MFMA attention needs head_dim % 16 == 0, head_dim <= {MFMA_MAX_HEAD_DIM} and page_size % 4 == 0 "
+          f"the MFMA attention needs head_dim % 16 == 0, head_dim <= {MFMA_MAX_HEAD_DIM} and a power-of-two page_size >= 4 "
           f"(got head_dim {head_dim}, page_size {page_size})")
     _need(q.data_ptr() % 16 == 0 and (q.stride(0) * 2) % 16 == 0, "q rows must be 16-byte aligned")
     _need(num_kv_heads > 0 and num_q_heads % num_kv_heads == 0, "q heads must be a multiple of kv heads")
@@ -325,7 +326,7 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
     _i32(seg_row0, "seg_row0", segments + 1)
     _i32(seg_slot, "seg_slot")
     _i32(seg_start, "seg_start", segments)
-    _need(1 <= max_qlen <= tokens, "max_qlen must lie in 1..tokens")
+    _need(1 <= min_qlen <= max_qlen <= tokens, "need 1 <= min_qlen <= max_qlen <= tokens")
     if splits is None:
         splits = decode_splits(segments, num_kv_heads, max_kv_len) if max_qlen == 1 else 1
     _need(splits == 1 or max_qlen == 1, "split-KV is for steps of single decoded tokens")
@@ -336,7 +337,8 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
         ws_ml = torch.empty((tokens, num_q_heads, splits, 2), dtype=torch.float32, device=q.device)
     lib.call("arle_attn_paged_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
              k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
-             seg_row0.data_ptr(), seg_slot.data_ptr(), seg_start.data_ptr(), segments, int(max_qlen), tokens,
+             seg_row0.data_ptr(), seg_slot.data_ptr(), seg_start.data_ptr(), segments, int(max_qlen),
+             int(min_qlen), tokens,
              num_q_heads, num_kv_heads, head_dim, page_size, float(scale), int(window), int(splits),
              _ptr(ws_o), _ptr(ws_ml), _stream())
     return out

@@ -121,7 +121,7 @@ def paged_attention(q, out, cache, batch, *, num_q_heads, num_kv_heads, head_dim
     """
     if ops.attn_mfma_supported(q.dtype, head_dim, cache.page_size):
         ops.attn_paged_mfma(q, out, cache.k_pages, cache.v_pages, cache.block_table, batch.seg_row0,
-                            batch.seg_slot, batch.seg_start, max_qlen=batch.max_qlen,
+                            batch.seg_slot, batch.seg_start, max_qlen=batch.max_qlen, min_qlen=batch.min_qlen,
                             max_kv_len=batch.max_position + 1, num_q_heads=num_q_heads,
                             num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=cache.page_size,
                             scale=scale, window=window, splits=getattr(batch, "kv_splits", None))

@@ -314,7 +314,7 @@ def _mfma_case(nq, nkv, D, P, segs, window, splits, seed):
     out = torch.full_like(q_all, float("nan"))
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
     ops.attn_paged_mfma(q_all, out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0),
-                        i32(list(range(len(segs)))), i32(seg_start), max_qlen=max(n for _, n in segs),
+                        i32(list(range(len(segs)))), i32(seg_start), max_qlen=max(n for _, n in segs), min_qlen=min(n for _, n in segs),
                         max_kv_len=max(lengths), num_q_heads=nq, num_kv_heads=nkv, head_dim=D, page_size=P,
                         scale=1.0 / math.sqrt(D), window=window, splits=splits)
     return out.cpu(), torch.cat(wants)
@@ -362,7 +362,7 @@ def test_attention_mfma_mixed_step_and_stale_pages():
     out = torch.empty_like(q_all)
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
     ops.attn_paged_mfma(q_all, out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0), i32([0, 1, 2, 3]),
-                        i32(starts), max_qlen=30, max_kv_len=max(lengths), num_q_heads=nq, num_kv_heads=nkv,
+                        i32(starts), max_qlen=30, min_qlen=1, max_kv_len=max(lengths), num_q_heads=nq, num_kv_heads=nkv,
                         head_dim=D, page_size=P, scale=1.0 / math.sqrt(D))
     assert torch.isfinite(out).all()
     assert _rel(out.cpu(), torch.cat(wants)) < 8e-3
@@ -385,7 +385,7 @@ def test_attention_mfma_finds_a_far_key():
         qq = q[n - rows:].reshape(rows, -1).to(DEV).contiguous()
         out = torch.empty_like(qq)
         ops.attn_paged_mfma(qq, out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32([0, rows]), i32([0]),
-                            i32([n - rows]), max_qlen=rows, max_kv_len=n, num_q_heads=nq, num_kv_heads=nkv,
+                            i32([n - rows]), max_qlen=rows, min_qlen=rows, max_kv_len=n, num_q_heads=nq, num_kv_heads=nkv,
                             head_dim=D, page_size=P, scale=1.0 / math.sqrt(D), splits=splits)
         got = out.cpu().reshape(rows, nq, D)
         assert torch.allclose(got[-1, 1].float(), v[far, 0].float(), atol=2e-2)
@@ -394,6 +394,7 @@ def test_attention_mfma_finds_a_far_key():
 def test_attention_mfma_refuses_shapes_it_was_not_written_for():
     assert not ops.attn_mfma_supported(torch.bfloat16, 24, 16)
     assert not ops.attn_mfma_supported(torch.bfloat16, 128, 6)
+    assert not ops.attn_mfma_supported(torch.bfloat16, 128, 12)   # such pages go to the fixed-order kernel
     assert not ops.attn_mfma_supported(torch.float32, 128, 16)
     assert not ops.attn_mfma_supported(torch.bfloat16, 272, 16)
     q = torch.zeros(2, 2 * 24, dtype=torch.bfloat16, device=DEV)
