@@ -392,8 +392,10 @@ constexpr int kPfWaves = 4;
 constexpr int kPfRows = 32 * kPfWaves;  // rows of a workgroup
 constexpr int kPfKeys = 64;             // keys of a tile
 
+// Up to head_dim 128 two workgroups share a CU (LDS: 2 x 72 KB), so that one computes while the
+// other waits for LDS or memory; the register budget is set accordingly.
 template <int DMAX, bool EXACT>
-__global__ __launch_bounds__(kPfWaves* kWave) void attn_prefill_lds_kernel(const AttnArgs a, int min_rows) {
+__global__ __launch_bounds__(kPfWaves* kWave, DMAX <= 128 ? 2 : 1) void attn_prefill_lds_kernel(const AttnArgs a, int min_rows) {
   constexpr int NT = 2;
   constexpr int DCH = DMAX / 32, DTL = DMAX / 16;
   constexpr int kKPieces = (kPfKeys * (DMAX / 8) + kPfWaves * kWave - 1) / (kPfWaves * kWave);  // 16-byte pieces per thread
@@ -406,7 +408,9 @@ __global__ __launch_bounds__(kPfWaves* kWave) void attn_prefill_lds_kernel(const
   const int qlen = a.seg_row0[seg + 1] - row0;
   const int rows = qlen * G;
   if (rows < min_rows) return;  // short segments (decoded tokens) belong to the other kernel
-  const int wg_row = blockIdx.x * kPfRows;
+  // the last rows of a segment see the most keys: hand them out first, so that the longest
+  // workgroups do not start last and leave the chip waiting for them
+  const int wg_row = (gridDim.x - 1 - blockIdx.x) * kPfRows;
   if (wg_row >= rows) return;
   const int start = a.seg_start[seg];
   const int* table = a.block_table + static_cast<int64_t>(a.seg_slot[seg]) * a.table_stride;
@@ -560,24 +564,34 @@ __global__ __launch_bounds__(kPfWaves* kWave) void attn_prefill_lds_kernel(const
     if (wave_has_rows && key_base < wave_kv_hi && key_base + kPfKeys > wave_kv_lo) {
       const uint16_t* ks = lds + stage * stage_elems;
       const uint16_t* vs = ks + kPfKeys * k_pitch;
+      // all key operands of the tile are asked for before the first product needs one, so that the
+      // LDS latency is paid once, not once per product
       f32x4 s[NT][4];
+      {
+        bf16x8 kop[4][DCH];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        f32x4 z[NT];
+        for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int n = 0; n < NT; ++n) z[n] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int c = 0; c < DCH; ++c) {
-          if (EXACT || c < n_dch) {
+          for (int c = 0; c < DCH; ++c) {
             const int d = 32 * c + 8 * g;
-            const bf16x8 kop = (EXACT || d < D) ? __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(ks + (16 * t + li) * k_pitch + d))
-                                     : zero_bf16x8();
-#pragma unroll
-            for (int n = 0; n < NT; ++n) z[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qreg[n][c], z[n], 0, 0, 0);
+            kop[t][c] = (EXACT || (c < n_dch && d < D))
+                            ? __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(ks + (16 * t + li) * k_pitch + d))
+                            : zero_bf16x8();
           }
-        }
 #pragma unroll
-        for (int n = 0; n < NT; ++n) s[n][t] = z[n];
+        for (int t = 0; t < 4; ++t) {
+          f32x4 z[NT];
+#pragma unroll
+          for (int n = 0; n < NT; ++n) z[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int c = 0; c < DCH; ++c)
+            if (EXACT || c < n_dch) {
+#pragma unroll
+              for (int n = 0; n < NT; ++n) z[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[t][c], qreg[n][c], z[n], 0, 0, 0);
+            }
+#pragma unroll
+          for (int n = 0; n < NT; ++n) s[n][t] = z[n];
+        }
       }
 
       // Only tiles that touch a row's causal edge or window edge need the mask; the others take
@@ -636,20 +650,25 @@ __global__ __launch_bounds__(kPfWaves* kWave) void attn_prefill_lds_kernel(const
       }
 
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < 2; ++u) {
+        uint2 va[DTL], vb[DTL];  // the value operands of 32 keys, all asked for first
 #pragma unroll
-        for (int dt = 0; dt < DTL; ++dt) {
+        for (int dt = 0; dt < DTL; ++dt)
           if (EXACT || dt < n_dt) {
             const uint16_t* vrow = vs + (16 * dt + li) * v_pitch + 32 * u + 4 * g;
-            const uint2 va = *reinterpret_cast<const uint2*>(vrow);
-            const uint2 vb = *reinterpret_cast<const uint2*>(vrow + 16);
-            uint4 vv = {va.x, va.y, vb.x, vb.y};
+            va[dt] = *reinterpret_cast<const uint2*>(vrow);
+            vb[dt] = *reinterpret_cast<const uint2*>(vrow + 16);
+          }
+#pragma unroll
+        for (int dt = 0; dt < DTL; ++dt)
+          if (EXACT || dt < n_dt) {
+            uint4 vv = {va[dt].x, va[dt].y, vb[dt].x, vb[dt].y};
             const bf16x8 vop = __builtin_bit_cast(bf16x8, vv);
 #pragma unroll
             for (int n = 0; n < NT; ++n)
               acc[n][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pb[n][u], acc[n][dt], 0, 0, 0);
           }
-        }
+      }
     }
 
     if (more) park(stage ^ 1);  // the other stage was last read before the barrier that ended the previous round
