@@ -42,32 +42,88 @@ def test_first_tokens_of_a_sequence(model_b, dtype):
     replay.compare(got, cfg, weights, {"y": toks}, TOL[dtype], f"first tokens in portions/{dtype}")
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_far_key_and_a_page_edge_show_in_the_logits(model_b, dtype, tmp_path):
-    """Scale one layer's q and k weights so that attention is sharp: a wrong key (off by one at a
-    page's edge, a stale page, a missing far key) then changes the logits far beyond rounding."""
-    from arle_amd.weights import write_safetensors
+def _write_folder(folder, cfg, weights):
     import json, os
+    from arle_amd.weights import write_safetensors
 
+    os.makedirs(folder)
+    json.dump(cfg, open(os.path.join(folder, "config.json"), "w"))
+    write_safetensors(os.path.join(folder, "model.safetensors"), {k: v.bfloat16() for k, v in weights.items()})
+    return read_folder(folder)
+
+
+def test_sharp_attention_shows_a_wrong_key_in_float32(model_b, tmp_path):
+    """Scale one layer's q and k norm weights so that attention is sharp: a wrong key (off by one at a
+    page's edge, a stale page, a missing far key) then changes the logits far beyond the float32
+    tolerance.  (In bfloat16 sharp but unsaturated scores amplify the rounding of the stored keys just as
+    much as they amplify a fault, so that mode is tested with saturated scores below.)"""
     d, cfg, weights = model_b
     sharp = {k: v.clone() for k, v in weights.items()}
     for name in ("q_norm", "k_norm"):
         sharp[f"model.layers.0.self_attn.{name}.weight"] *= 4.0   # scores x16
-    sharp_dir = str(tmp_path / "sharp")
-    os.makedirs(sharp_dir)
-    json.dump(cfg, open(os.path.join(sharp_dir, "config.json"), "w"))
-    write_safetensors(os.path.join(sharp_dir, "model.safetensors"), {k: v.bfloat16() for k, v in sharp.items()})
-    cfg2, weights2 = read_folder(sharp_dir)
+    cfg2, weights2 = _write_folder(str(tmp_path / "sharp"), cfg, sharp)
     toks = random_tokens(200, cfg["vocab_size"], 12)
-    eng = Engine.from_folder(sharp_dir, dtype=dtype, page_size=TINY["B"][1], max_tokens=256, max_slots=2)
+    eng = Engine.from_folder(str(tmp_path / "sharp"), dtype="float32", page_size=TINY["B"][1], max_tokens=256, max_slots=2)
     got = replay.run_steps(eng, replay.portions("x", toks, sizes=(8, 9, 7, 16, 1, 24, 3)))
-    replay.compare(got, cfg2, weights2, {"x": toks}, TOL[dtype] * (1 if dtype == "float32" else 2), f"sharp/{dtype}")
+    replay.compare(got, cfg2, weights2, {"x": toks}, TOL["float32"], "sharp/float32")
     # the test has teeth: reading one wrong key at a page's edge moves the last logits far beyond the tolerance
     other = list(toks)
     other[TINY["B"][1] - 1] = (other[TINY["B"][1] - 1] + 1) % cfg["vocab_size"]
     ref = plain.forward_logits(weights2, cfg2, toks, dtype=torch.float64)[-1]
     moved = plain.forward_logits(weights2, cfg2, other, dtype=torch.float64)[-1]
     assert float((ref - moved).abs().max() / ref.abs().max()) > 100 * TOL["float32"]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_planted_keys_at_page_edges_and_far_away_decide_the_logits(model_b, dtype, tmp_path):
+    """Layer 0 is made to look at one key only, with a margin that rounding cannot close.
+
+    Hidden column 0 is a positive constant in every embedding row and feeds, through q_proj, the
+    slowest-rotating dimension of every query head; hidden column 1 is zero except for three planted
+    tokens and feeds the same dimension of every key head; the q/k norm weights of that dimension are
+    large.  Every query therefore gives all its weight to the strongest planted key so far.  The three
+    are placed at position 0 (soon hundreds of keys away), in the last slot of a page and in the first
+    slot of a page, so a kernel that drops a far page, a page's last slot, the newest key or a page's
+    first slot returns another token's value.  Saturated scores do not amplify rounding, so bfloat16
+    keeps its ordinary tolerance."""
+    d, cfg, weights = model_b
+    P, D, nq, nkv = TINY["B"][1], cfg["head_dim"], cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    w = {k: v.clone() for k, v in weights.items()}
+    emb, slow = w["model.embed_tokens.weight"], D // 2 - 1      # NeoX pair (D/2-1, D-1) turns slowest
+    planted = {cfg["vocab_size"] - 3: 0.05, cfg["vocab_size"] - 2: 0.10, cfg["vocab_size"] - 1: 0.15}
+    emb[:, 0], emb[:, 1] = 0.15, 0.0
+    for tok, level in planted.items():
+        emb[tok, 1] = level
+    pre = "model.layers.0.self_attn."
+    for h in range(nq):
+        w[pre + "q_proj.weight"][h * D + slow] = 0.0
+        w[pre + "q_proj.weight"][h * D + slow, 0] = 2.0
+    for h in range(nkv):
+        w[pre + "k_proj.weight"][h * D + slow] = 0.0
+        w[pre + "k_proj.weight"][h * D + slow, 1] = 2.0
+    w[pre + "q_norm.weight"][slow] = 6.0
+    w[pre + "k_norm.weight"][slow] = 6.0
+    cfg2, weights2 = _write_folder(str(tmp_path / "planted"), cfg, w)
+
+    weak, mid, strong = planted
+    toks = [t % (cfg["vocab_size"] - 3) for t in random_tokens(200, cfg["vocab_size"], 14)]
+    places = {0: weak, 3 * P - 1: mid, 11 * P: strong}
+    for pos, tok in places.items():
+        toks[pos] = tok
+    eng = Engine.from_folder(str(tmp_path / "planted"), dtype=dtype, page_size=P, max_tokens=256, max_slots=2)
+    got = replay.run_steps(eng, replay.portions("x", toks, sizes=(8, 9, 7, 16, 1, 24, 3, 1, 1, 30)))
+    replay.compare(got, cfg2, weights2, {"x": toks}, TOL[dtype], f"planted/{dtype}")
+
+    # teeth: were the planted key at a page's edge not seen, the next position's logits would be those of
+    # the sequence without it (only attention carries one position's token to another's logits)
+    ref = plain.forward_logits(weights2, cfg2, toks, dtype=torch.float64)
+    for pos in (3 * P - 1, 11 * P):
+        without = list(toks)
+        without[pos] = 5
+        moved = plain.forward_logits(weights2, cfg2, without, dtype=torch.float64)
+        for at in (pos + 1, len(toks) - 1):
+            change = float((ref[at] - moved[at]).abs().max() / ref.abs().max())
+            assert change > 10 * TOL["bfloat16"], (pos, at, change)
 
 
 def test_step_refuses_bad_input(model_b):
