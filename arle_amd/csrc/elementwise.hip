@@ -33,6 +33,18 @@ __global__ void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict_
   out[static_cast<int64_t>(t) * width + j] = from_float<T>(act * u);
 }
 
+// out[i] = parts[0][i] + parts[1][i] + ..., added in that order: the sum of the float32 partial
+// products that a matrix product with K split over workgroups leaves behind.
+template <typename TOut>
+__global__ void sum_partials_kernel(const float* __restrict__ parts, int n_parts, int64_t stride,
+                                    TOut* __restrict__ out, int64_t count) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float v = parts[i];
+  for (int sp = 1; sp < n_parts; ++sp) v += parts[sp * stride + i];
+  out[i] = from_float<TOut>(v);
+}
+
 }  // namespace arle
 
 using namespace arle;
@@ -65,5 +77,19 @@ extern "C" int arle_silu_mul(const void* gate, const void* up, long long in_stri
                                                static_cast<const bf16*>(up), in_stride,
                                                static_cast<bf16*>(out), width, block);
   }
+  return launch_status();
+}
+
+// parts [n_parts][count] float32 (stride elements apart) -> out [count] float32 or bfloat16.
+extern "C" int arle_sum_partials(const float* parts, int n_parts, long long stride, void* out, int out_dtype,
+                                 long long count, void* stream) {
+  if (count == 0) return 0;
+  if (n_parts < 1) return static_cast<int>(hipErrorInvalidValue);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const unsigned blocks = static_cast<unsigned>((count + 255) / 256);
+  if (out_dtype == kF32)
+    sum_partials_kernel<float><<<blocks, 256, 0, s>>>(parts, n_parts, stride, static_cast<float*>(out), count);
+  else
+    sum_partials_kernel<bf16><<<blocks, 256, 0, s>>>(parts, n_parts, stride, static_cast<bf16*>(out), count);
   return launch_status();
 }

@@ -36,21 +36,28 @@ __global__ void rmsnorm_kernel(const TIn* __restrict__ x, int64_t x_stride,
   }
 }
 
-// residual[src(r), :] += delta[src(r), :]; out[r, :] = norm(residual[src(r), :]).
+// residual[src(r), :] += delta[0][src(r), :] + delta[1][src(r), :] + ...; out[r, :] = norm(residual[src(r), :]).
+// `delta` is a stack of n_delta tensors delta_stride elements apart (the partial products of a matrix
+// product whose K was split over workgroups), added in the order of the stack.
 // With `rows` given the sum is not written back: the rows are read for the last
 // time (final norm before the output head).
 template <typename TD, typename TOut, typename TW>
-__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
-                                   const TW* __restrict__ w, TOut* __restrict__ out,
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta, int n_delta,
+                                   int64_t delta_stride, const TW* __restrict__ w, TOut* __restrict__ out,
                                    const int* __restrict__ rows, int width, float eps) {
   __shared__ float lds[kNormWaves];
   const int r = blockIdx.x;
   const int64_t src = rows ? rows[r] : r;
   float* res = residual + src * width;
   const TD* d = delta + src * width;
+  auto summed = [&](int i) {  // residual + (delta 0 + delta 1 + ...), as the register-resident kernel adds them
+    float dv = to_float(d[i]);
+    for (int sp = 1; sp < n_delta; ++sp) dv += to_float(d[sp * delta_stride + i]);
+    return res[i] + dv;
+  };
   float ss = 0.f;
   for (int i = threadIdx.x; i < width; i += kNormThreads) {
-    const float v = res[i] + to_float(d[i]);
+    const float v = summed(i);
     if (!rows) res[i] = v;
     ss += v * v;
   }
@@ -58,7 +65,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
   TOut* o = out + static_cast<int64_t>(r) * width;
   for (int i = threadIdx.x; i < width; i += kNormThreads) {
-    const float v = rows ? res[i] + to_float(d[i]) : res[i];
+    const float v = rows ? summed(i) : res[i];
     o[i] = from_float<TOut>(v * inv * to_float(w[i]));
   }
 }
@@ -96,10 +103,12 @@ __device__ __forceinline__ void store4<bf16>(bf16* p, float4 v) {
   *reinterpret_cast<uint2*>(p) = raw;
 }
 
-// HAS_DELTA: residual row += delta row first (written back unless `rows` picks rows for the last time).
+// HAS_DELTA: residual row += the rows of the delta stack first, in the order of the stack (written back unless
+// `rows` picks rows for the last time).
 template <typename TIn, typename TD, typename TOut, typename TW, bool HAS_DELTA>
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_vec_kernel(TIn* __restrict__ x, int64_t x_stride,
-                                                                   const TD* __restrict__ delta,
+                                                                   const TD* __restrict__ delta, int n_delta,
+                                                                   int64_t delta_stride,
                                                                    const TW* __restrict__ w,
                                                                    TOut* __restrict__ out,
                                                                    const int* __restrict__ rows, int width,
@@ -117,6 +126,27 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_vec_kernel(TIn* __restri
       v[j] = load4<TIn>(xr + i);
       if (HAS_DELTA) d[j] = load4<TD>(dr + i);
       wv[j] = load4<TW>(w + i);
+    }
+  }
+  if (HAS_DELTA) {  // the rest of the stack, a few rows of loads in flight at a time
+#pragma unroll 4
+    for (int sp = 1; sp < n_delta; ++sp) {
+      float4 e[kVecPerThread];
+#pragma unroll
+      for (int j = 0; j < kVecPerThread; ++j) {
+        const int i = 4 * (threadIdx.x + j * kNormThreads);
+        if (i < width) e[j] = load4<TD>(dr + sp * delta_stride + i);
+      }
+#pragma unroll
+      for (int j = 0; j < kVecPerThread; ++j) {
+        const int i = 4 * (threadIdx.x + j * kNormThreads);
+        if (i < width) {
+          d[j].x += e[j].x;
+          d[j].y += e[j].y;
+          d[j].z += e[j].z;
+          d[j].w += e[j].w;
+        }
+      }
     }
   }
   float ss = 0.f;
@@ -146,6 +176,56 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_vec_kernel(TIn* __restri
   }
 }
 
+// A stack of float32 deltas (the partial products of a matrix product whose K was split over
+// workgroups) added into the residual row, then the norm.  Few rows make few workgroups here, so the
+// time is the latency of the loads: a workgroup of 1024 threads owns a row, every thread one group of
+// four columns, and the loads of the whole stack (up to kStackUnroll at a time) are in flight together.
+// Order of addition: residual + (delta 0 + delta 1 + ...), as in the kernels above.
+constexpr int kStackThreads = 1024;
+constexpr int kStackUnroll = 16;
+
+template <typename TOut, typename TW>
+__global__ __launch_bounds__(kStackThreads) void add_stack_rmsnorm_kernel(
+    float* __restrict__ residual, const float* __restrict__ delta, int n_delta, int64_t delta_stride,
+    const TW* __restrict__ w, TOut* __restrict__ out, const int* __restrict__ rows, int width, float eps) {
+  __shared__ float lds[kStackThreads / kWave];
+  const int r = blockIdx.x;
+  const int64_t src = rows ? rows[r] : r;
+  const int i = 4 * threadIdx.x;
+  const bool mine = i < width;
+  float* res = residual + src * width;
+  const float* dr = delta + src * width;
+  float4 v = {0.f, 0.f, 0.f, 0.f}, wv = v, d = v;
+  if (mine) {
+    v = load4<float>(res + i);
+    wv = load4<TW>(w + i);
+  }
+  for (int base = 0; base < n_delta; base += kStackUnroll) {
+    float4 e[kStackUnroll];
+#pragma unroll
+    for (int u = 0; u < kStackUnroll; ++u)
+      if (mine && base + u < n_delta) e[u] = load4<float>(dr + (base + u) * delta_stride + i);
+#pragma unroll
+    for (int u = 0; u < kStackUnroll; ++u)
+      if (mine && base + u < n_delta) {
+        d.x += e[u].x;
+        d.y += e[u].y;
+        d.z += e[u].z;
+        d.w += e[u].w;
+      }
+  }
+  v.x += d.x;
+  v.y += d.y;
+  v.z += d.z;
+  v.w += d.w;
+  if (mine && !rows) store4<float>(res + i, v);
+  const float total = block_sum<kStackThreads / kWave>(v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w, lds);
+  const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
+  if (mine)
+    store4<TOut>(out + static_cast<int64_t>(r) * width + i,
+                 float4{v.x * inv * wv.x, v.y * inv * wv.y, v.z * inv * wv.z, v.w * inv * wv.w});
+}
+
 inline bool vec_ok(int width, long long x_stride, const void* a, const void* b, const void* c, const void* d) {
   auto al = [](const void* p) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0; };
   return width % 4 == 0 && width <= kVecMax && x_stride % 4 == 0 && al(a) && al(b) && al(c) && al(d);
@@ -158,10 +238,10 @@ int launch_rmsnorm(const void* x, long long x_stride, const void* w, int w_dtype
     TIn* xp = const_cast<TIn*>(static_cast<const TIn*>(x));
     if (w_dtype == kF32)
       rmsnorm_vec_kernel<TIn, TIn, TOut, float, false><<<n_rows, kNormThreads, 0, s>>>(
-          xp, x_stride, nullptr, static_cast<const float*>(w), static_cast<TOut*>(out), rows, width, eps);
+          xp, x_stride, nullptr, 0, 0, static_cast<const float*>(w), static_cast<TOut*>(out), rows, width, eps);
     else
       rmsnorm_vec_kernel<TIn, TIn, TOut, bf16, false><<<n_rows, kNormThreads, 0, s>>>(
-          xp, x_stride, nullptr, static_cast<const bf16*>(w), static_cast<TOut*>(out), rows, width, eps);
+          xp, x_stride, nullptr, 0, 0, static_cast<const bf16*>(w), static_cast<TOut*>(out), rows, width, eps);
     return launch_status();
   }
   if (w_dtype == kF32) {
@@ -177,26 +257,40 @@ int launch_rmsnorm(const void* x, long long x_stride, const void* w, int w_dtype
 }
 
 template <typename TD, typename TOut>
-int launch_add_rmsnorm(float* residual, const void* delta, const void* w, int w_dtype, void* out,
-                       const int* rows, int n_rows, int width, float eps, hipStream_t s) {
-  if (vec_ok(width, width, residual, delta, w, out)) {
+int launch_add_rmsnorm(float* residual, const void* delta, int n_delta, long long delta_stride, const void* w,
+                       int w_dtype, void* out, const int* rows, int n_rows, int width, float eps, hipStream_t s) {
+  if constexpr (sizeof(TD) == 4) {
+    if (n_delta > 1 && vec_ok(width, width, residual, delta, w, out) && delta_stride % 4 == 0 &&
+        width <= 4 * kStackThreads) {
+      if (w_dtype == kF32)
+        add_stack_rmsnorm_kernel<TOut, float><<<n_rows, kStackThreads, 0, s>>>(
+            residual, static_cast<const float*>(delta), n_delta, delta_stride, static_cast<const float*>(w),
+            static_cast<TOut*>(out), rows, width, eps);
+      else
+        add_stack_rmsnorm_kernel<TOut, bf16><<<n_rows, kStackThreads, 0, s>>>(
+            residual, static_cast<const float*>(delta), n_delta, delta_stride, static_cast<const bf16*>(w),
+            static_cast<TOut*>(out), rows, width, eps);
+      return launch_status();
+    }
+  }
+  if (vec_ok(width, width, residual, delta, w, out) && delta_stride % 4 == 0) {
     if (w_dtype == kF32)
       rmsnorm_vec_kernel<float, TD, TOut, float, true><<<n_rows, kNormThreads, 0, s>>>(
-          residual, width, static_cast<const TD*>(delta), static_cast<const float*>(w),
+          residual, width, static_cast<const TD*>(delta), n_delta, delta_stride, static_cast<const float*>(w),
           static_cast<TOut*>(out), rows, width, eps);
     else
       rmsnorm_vec_kernel<float, TD, TOut, bf16, true><<<n_rows, kNormThreads, 0, s>>>(
-          residual, width, static_cast<const TD*>(delta), static_cast<const bf16*>(w),
+          residual, width, static_cast<const TD*>(delta), n_delta, delta_stride, static_cast<const bf16*>(w),
           static_cast<TOut*>(out), rows, width, eps);
     return launch_status();
   }
   if (w_dtype == kF32) {
     add_rmsnorm_kernel<TD, TOut, float><<<n_rows, kNormThreads, 0, s>>>(
-        residual, static_cast<const TD*>(delta), static_cast<const float*>(w),
+        residual, static_cast<const TD*>(delta), n_delta, delta_stride, static_cast<const float*>(w),
         static_cast<TOut*>(out), rows, width, eps);
   } else {
     add_rmsnorm_kernel<TD, TOut, bf16><<<n_rows, kNormThreads, 0, s>>>(
-        residual, static_cast<const TD*>(delta), static_cast<const bf16*>(w),
+        residual, static_cast<const TD*>(delta), n_delta, delta_stride, static_cast<const bf16*>(w),
         static_cast<TOut*>(out), rows, width, eps);
   }
   return launch_status();
@@ -221,16 +315,18 @@ extern "C" int arle_rmsnorm(const void* x, int in_dtype, long long x_stride, con
   return launch_rmsnorm<bf16, bf16>(x, x_stride, w, w_dtype, out, rows, n_rows, width, eps, s);
 }
 
-extern "C" int arle_add_rmsnorm(float* residual, const void* delta, int delta_dtype, const void* w,
-                                int w_dtype, void* out, int out_dtype, const int* rows, int n_rows,
-                                int width, float eps, void* stream) {
+// delta: n_delta >= 1 tensors [*, width] of `delta_dtype`, delta_stride elements apart, added in order.
+extern "C" int arle_add_rmsnorm(float* residual, const void* delta, int n_delta, long long delta_stride,
+                                int delta_dtype, const void* w, int w_dtype, void* out, int out_dtype,
+                                const int* rows, int n_rows, int width, float eps, void* stream) {
   if (n_rows == 0) return 0;
+  if (n_delta < 1) return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (delta_dtype == kF32 && out_dtype == kF32)
-    return launch_add_rmsnorm<float, float>(residual, delta, w, w_dtype, out, rows, n_rows, width, eps, s);
+    return launch_add_rmsnorm<float, float>(residual, delta, n_delta, delta_stride, w, w_dtype, out, rows, n_rows, width, eps, s);
   if (delta_dtype == kF32 && out_dtype == kBF16)
-    return launch_add_rmsnorm<float, bf16>(residual, delta, w, w_dtype, out, rows, n_rows, width, eps, s);
+    return launch_add_rmsnorm<float, bf16>(residual, delta, n_delta, delta_stride, w, w_dtype, out, rows, n_rows, width, eps, s);
   if (delta_dtype == kBF16 && out_dtype == kF32)
-    return launch_add_rmsnorm<bf16, float>(residual, delta, w, w_dtype, out, rows, n_rows, width, eps, s);
-  return launch_add_rmsnorm<bf16, bf16>(residual, delta, w, w_dtype, out, rows, n_rows, width, eps, s);
+    return launch_add_rmsnorm<bf16, float>(residual, delta, n_delta, delta_stride, w, w_dtype, out, rows, n_rows, width, eps, s);
+  return launch_add_rmsnorm<bf16, bf16>(residual, delta, n_delta, delta_stride, w, w_dtype, out, rows, n_rows, width, eps, s);
 }

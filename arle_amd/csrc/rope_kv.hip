@@ -10,6 +10,9 @@
 //   when no cache is given.
 // cos/sin are 32-bit tables [positions, rot/2]; all arithmetic is 32-bit and the
 // result is rounded once at the store.
+// The projections may also come as a stack of float32 partial products [n_parts][T, (nq + 2 nkv) D]
+// (a matrix product whose K was split over workgroups): then every value is the sum of the stack in
+// order, q is written to its own buffer and k, v only to the cache.
 // reference counterparts: crates/cuda-kernels/csrc/attention/prefill_attention_paged_prep.cu:8-106,
 // crates/cuda-kernels/csrc/attention/decode_prep_paged.cu:73-160 (head_dim fixed to 128 there).
 //
@@ -29,7 +32,8 @@ __global__ __launch_bounds__(kPrepWaves* kWave) void qk_prep_kernel(
     const TW* __restrict__ k_w, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     int rot, const int* __restrict__ positions, const int* __restrict__ slot_of_token,
     const int* __restrict__ block_table, int table_stride, T* __restrict__ k_pages,
-    T* __restrict__ v_pages, int nq, int nkv, int D, int page_size, float eps) {
+    T* __restrict__ v_pages, int nq, int nkv, int D, int page_size, float eps,
+    const float* __restrict__ parts, int n_parts, int64_t part_stride, int64_t part_row_stride) {
   extern __shared__ float lds[];  // [kPrepWaves][D]
   const int t = blockIdx.x;
   const int wave = threadIdx.x / kWave;
@@ -50,11 +54,28 @@ __global__ __launch_bounds__(kPrepWaves* kWave) void qk_prep_kernel(
     page_base = static_cast<int64_t>(page) * nkv * page_size * D;
   }
 
+  // column `col` of token t's fused [q | k | v] row, summed over the stack of partial products
+  const float* part_row = parts ? parts + static_cast<int64_t>(t) * part_row_stride : nullptr;
+  auto summed = [&](int col) {  // the loads of up to 16 parts are in flight together, the adds are in order
+    float acc = 0.f;
+    for (int base = 0; base < n_parts; base += 16) {
+      float e[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+        if (base + u < n_parts) e[u] = part_row[(base + u) * part_stride + col];
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+        if (base + u < n_parts) acc += e[u];
+    }
+    return acc;
+  };
+
   if (is_v && v_pages) {  // v head: copy into the cache, d-major inside the page
     const int kvh = head - nq - nkv;
     const T* vsrc = v + static_cast<int64_t>(t) * v_stride + kvh * D;
     T* vdst = v_pages + page_base + static_cast<int64_t>(kvh) * page_size * D + in_page;
-    for (int d = lane; d < D; d += kWave) vdst[static_cast<int64_t>(d) * page_size] = vsrc[d];
+    for (int d = lane; d < D; d += kWave)
+      vdst[static_cast<int64_t>(d) * page_size] = parts ? from_float<T>(summed(head * D + d)) : vsrc[d];
   }
 
   const int local = is_q ? head : head - nq;
@@ -64,7 +85,7 @@ __global__ __launch_bounds__(kPrepWaves* kWave) void qk_prep_kernel(
     const TW* w = is_q ? q_w : k_w;
     float ss = 0.f;
     for (int d = lane; d < D; d += kWave) {
-      const float val = to_float(src[d]);
+      const float val = parts ? summed(head * D + d) : to_float(src[d]);
       x[d] = val;
       ss += val * val;
     }
@@ -103,6 +124,7 @@ int launch_prep(void* q, long long q_stride, void* k, long long k_stride, const 
                 const float* cos_t, const float* sin_t, int rot, const int* positions,
                 const int* slot_of_token, const int* block_table, int table_stride, void* k_pages,
                 void* v_pages, int tokens, int nq, int nkv, int D, int page_size, float eps,
+                const float* parts, int n_parts, long long part_stride, long long part_row_stride,
                 hipStream_t s) {
   dim3 grid(tokens, (nq + 2 * nkv + kPrepWaves - 1) / kPrepWaves);
   const size_t lds = static_cast<size_t>(kPrepWaves) * D * sizeof(float);
@@ -111,13 +133,13 @@ int launch_prep(void* q, long long q_stride, void* k, long long k_stride, const 
         static_cast<T*>(q), q_stride, static_cast<T*>(k), k_stride, static_cast<const T*>(v),
         v_stride, static_cast<const float*>(q_w), static_cast<const float*>(k_w), cos_t, sin_t, rot,
         positions, slot_of_token, block_table, table_stride, static_cast<T*>(k_pages),
-        static_cast<T*>(v_pages), nq, nkv, D, page_size, eps);
+        static_cast<T*>(v_pages), nq, nkv, D, page_size, eps, parts, n_parts, part_stride, part_row_stride);
   } else {
     qk_prep_kernel<T, bf16><<<grid, kPrepWaves * kWave, lds, s>>>(
         static_cast<T*>(q), q_stride, static_cast<T*>(k), k_stride, static_cast<const T*>(v),
         v_stride, static_cast<const bf16*>(q_w), static_cast<const bf16*>(k_w), cos_t, sin_t, rot,
         positions, slot_of_token, block_table, table_stride, static_cast<T*>(k_pages),
-        static_cast<T*>(v_pages), nq, nkv, D, page_size, eps);
+        static_cast<T*>(v_pages), nq, nkv, D, page_size, eps, parts, n_parts, part_stride, part_row_stride);
   }
   return launch_status();
 }
@@ -130,20 +152,28 @@ using namespace arle;
 // buffers or three column blocks of one fused buffer both fit).  q_w/k_w may be
 // null (no per-head norm); rot may be 0 (no rotation; cos/sin unused); k_pages /
 // v_pages may be null (no cache write; k is then rewritten in place).
+// parts != null: the inputs are n_parts float32 tensors [tokens, (nq + 2 nkv) D] (row stride
+// part_row_stride, part_stride elements apart), summed in order; q is only written (a buffer of its
+// own), k and v go to the cache only (k_pages and v_pages must be given unless nkv == 0).
 extern "C" int arle_qk_prep(void* q, long long q_stride, void* k, long long k_stride, const void* v,
                             long long v_stride, int dtype, const void* q_w, const void* k_w,
                             int w_dtype, const float* cos_t, const float* sin_t, int rot,
                             const int* positions, const int* slot_of_token, const int* block_table,
                             int table_stride, void* k_pages, void* v_pages, int tokens, int nq,
-                            int nkv, int D, int page_size, float eps, void* stream) {
+                            int nkv, int D, int page_size, float eps, const float* parts, int n_parts,
+                            long long part_stride, long long part_row_stride, void* stream) {
   if (tokens == 0) return 0;
   if (D > kMaxHeadDim || rot > D || (rot & 1)) return static_cast<int>(hipErrorInvalidValue);
+  if (parts != nullptr && (n_parts < 1 || (nkv > 0 && (k_pages == nullptr || v_pages == nullptr))))
+    return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == kF32)
     return launch_prep<float>(q, q_stride, k, k_stride, v, v_stride, q_w, k_w, w_dtype, cos_t, sin_t,
                               rot, positions, slot_of_token, block_table, table_stride, k_pages,
-                              v_pages, tokens, nq, nkv, D, page_size, eps, s);
+                              v_pages, tokens, nq, nkv, D, page_size, eps, parts, n_parts, part_stride,
+                              part_row_stride, s);
   return launch_prep<bf16>(q, q_stride, k, k_stride, v, v_stride, q_w, k_w, w_dtype, cos_t, sin_t,
                            rot, positions, slot_of_token, block_table, table_stride, k_pages,
-                           v_pages, tokens, nq, nkv, D, page_size, eps, s);
+                           v_pages, tokens, nq, nkv, D, page_size, eps, parts, n_parts, part_stride,
+                           part_row_stride, s);
 }

@@ -26,7 +26,7 @@ SOURCES = {
     "elementwise": "elementwise.hip",
     "norm": "norm.hip",
     "gemm_f32": "gemm_f32.hip",
-    "gemm_bf16": "gemm_bf16.hip",
+    "gemm_rows": "gemm_rows.hip",
     "rope_kv": "rope_kv.hip",
     "attention_simt": "attention_simt.hip",
     "attention_mfma": "attention_mfma.hip",

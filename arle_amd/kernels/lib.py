@@ -22,11 +22,13 @@ SIGNATURES = {
     "arle_embed_gather": ("elementwise", [_p, _i, _p, _p, _i, _i, _p]),
     "arle_silu_mul": ("elementwise", [_p, _p, _ll, _p, _i, _i, _i, _i, _p]),
     "arle_rmsnorm": ("norm", [_p, _i, _ll, _p, _i, _p, _i, _p, _i, _i, _f, _p]),
-    "arle_add_rmsnorm": ("norm", [_p, _p, _i, _p, _i, _p, _i, _p, _i, _i, _f, _p]),
-    "arle_gemm_bf16_skinny": ("gemm_bf16", [_p, _ll, _p, _ll, _p, _ll, _i, _i, _i, _i, _i, _i, _p]),
+    "arle_add_rmsnorm": ("norm", [_p, _p, _i, _ll, _i, _p, _i, _p, _i, _p, _i, _i, _f, _p]),
+    "arle_sum_partials": ("elementwise", [_p, _i, _ll, _p, _i, _ll, _p]),
+    "arle_gemm_rows": ("gemm_rows", [_p, _ll, _p, _ll, _p, _ll, _ll, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "arle_gemm_rows_geometry": ("gemm_rows", [_i]),
     "arle_gemm_f32": ("gemm_f32", [_p, _ll, _p, _ll, _p, _ll, _i, _i, _i, _p]),
     "arle_qk_prep": ("rope_kv", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _p, _i, _p, _p, _i, _p, _p, _p,
-                                 _i, _p, _p, _i, _i, _i, _i, _i, _f, _p]),
+                                 _i, _p, _p, _i, _i, _i, _i, _i, _f, _p, _i, _ll, _ll, _p]),
     "arle_attn_paged_simt": ("attention_simt", [_p, _ll, _p, _ll, _p, _p, _i, _p, _i, _p, _p, _p, _i,
                                                 _i, _i, _i, _i, _f, _i, _p]),
     "arle_attn_paged_mfma": ("attention_mfma", [_p, _ll, _p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i,

@@ -136,11 +136,17 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
 def add_rmsnorm(residual: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: torch.Tensor | None = None,
                 out: torch.Tensor | None = None):
-    """residual += delta (float32, in place unless `rows` is given); out = rmsnorm(residual)."""
+    """residual += delta (float32, in place unless `rows` is given); out = rmsnorm(residual).
+
+    delta is [T, H], or a stack [S, T, H] of partial sums that are added in the order of the stack
+    (what a matrix product with K split over workgroups leaves behind)."""
     _gpu(residual, delta, weight, rows, out)
     _need(residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous(),
           "residual must be contiguous float32 [T, H]")
-    _need(delta.shape == residual.shape and delta.is_contiguous(), "delta must match the residual")
+    _need(delta.dim() in (2, 3) and tuple(delta.shape[-2:]) == tuple(residual.shape) and delta.is_contiguous()
+          and delta.dtype in _CODES and (delta.dim() == 2 or delta.shape[0] >= 1),
+          "delta must match the residual ([T, H] or a stack [S, T, H])")
+    n_delta = delta.shape[0] if delta.dim() == 3 else 1
     width = residual.shape[1]
     _need(weight.shape == (width,) and weight.is_contiguous(), "norm weight must be [width]")
     n_rows = residual.shape[0]
@@ -151,7 +157,7 @@ def add_rmsnorm(residual: torch.Tensor, delta: torch.Tensor, weight: torch.Tenso
         out = torch.empty((n_rows, width), dtype=out_dtype, device=residual.device)
     _need(out.shape == (n_rows, width) and out.dtype == out_dtype and out.is_contiguous(),
           "add_rmsnorm output must be contiguous [rows, width]")
-    lib.call("arle_add_rmsnorm", residual.data_ptr(), delta.data_ptr(), _code(delta),
+    lib.call("arle_add_rmsnorm", residual.data_ptr(), delta.data_ptr(), n_delta, residual.numel(), _code(delta),
              weight.data_ptr(), _code(weight), out.data_ptr(), _code(out), _ptr(rows), n_rows, width,
              float(eps), _stream())
     return out
@@ -185,20 +191,37 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None):
 def qk_prep(q, k, v, *, num_q_heads: int, num_kv_heads: int, head_dim: int, eps: float,
             q_weight=None, k_weight=None, cos=None, sin=None, rotary_dim: int = 0,
             positions=None, slot_of_token=None, block_table=None, k_pages=None, v_pages=None,
-            page_size: int = 0):
+            page_size: int = 0, parts=None):
     """Per-head norm + rotation of q and k in place; k and v written to the paged cache.
 
     q [T, nq*D], k, v [T, nkv*D] (row views of one fused buffer are fine).  With no
     cache given k is rewritten in place and v is left alone.
+
+    parts: float32 [S, T, (nq + 2 nkv) * D], a stack of partial products of the fused q|k|v projection.
+    Then the values are the sums over the stack (in order), q is an output only, and k, v are None:
+    they go to the cache, which must be given unless num_kv_heads is 0 (a layer that only needs q).
     """
-    _gpu(q, k, v, q_weight, k_weight, cos, sin, positions, slot_of_token, block_table, k_pages, v_pages)
+    _gpu(q, k, v, q_weight, k_weight, cos, sin, positions, slot_of_token, block_table, k_pages, v_pages, parts)
     tokens = q.shape[0]
     D = head_dim
     _need(0 < D <= MAX_HEAD_DIM, f"head_dim {D} is outside the supported range 1..{MAX_HEAD_DIM}")
-    for name, t, heads in (("q", q, num_q_heads), ("k", k, num_kv_heads), ("v", v, num_kv_heads)):
-        _rows(t, name)
-        _need(t.shape == (tokens, heads * D), f"{name} must be [T, heads*D]")
-        _need(t.dtype == q.dtype, "q, k and v must share one element type")
+    part_args = (0, 0, 0, 0)
+    if parts is not None:
+        width = (num_q_heads + 2 * num_kv_heads) * D
+        _need(parts.dtype == torch.float32 and parts.dim() == 3 and parts.shape[0] >= 1
+              and tuple(parts.shape[1:]) == (tokens, width) and parts.is_contiguous(),
+              f"parts must be contiguous float32 [S, {tokens}, {width}]")
+        _need(k is None and v is None, "with parts, k and v are not given: they go to the cache")
+        _need(num_kv_heads == 0 or k_pages is not None, "with parts, k and v need the cache to go to")
+        _rows(q, "q")
+        _need(q.shape == (tokens, num_q_heads * D), "q must be [T, heads*D]")
+        part_args = (parts.data_ptr(), parts.shape[0], tokens * width, width)
+        k = v = q   # never read or written in this mode
+    else:
+        for name, t, heads in (("q", q, num_q_heads), ("k", k, num_kv_heads), ("v", v, num_kv_heads)):
+            _rows(t, name)
+            _need(t.shape == (tokens, heads * D), f"{name} must be [T, heads*D]")
+            _need(t.dtype == q.dtype, "q, k and v must share one element type")
     _need((q_weight is None) == (k_weight is None), "give both q and k norm weights or neither")
     w_code = F32
     if q_weight is not None:
@@ -228,7 +251,7 @@ def qk_prep(q, k, v, *, num_q_heads: int, num_kv_heads: int, head_dim: int, eps:
              v.stride(0), _code(q), _ptr(q_weight), _ptr(k_weight), w_code, _ptr(cos), _ptr(sin),
              int(rotary_dim), positions.data_ptr(), _ptr(slot_of_token), _ptr(block_table),
              table_stride, _ptr(k_pages), _ptr(v_pages), tokens, num_q_heads, num_kv_heads, D,
-             int(page_size), float(eps), _stream())
+             int(page_size), float(eps), *part_args, _stream())
 
 
 # ------------------------------------------------------------------ attention
@@ -395,62 +418,126 @@ def apply_penalties(logits, indptr, tokens, counts, repetition, frequency, prese
 # ------------------------------------------------------------ bfloat16 products
 
 
-SKINNY_MAX_ROWS = 64
-SKINNY_PREFERRED_ROWS = 16   # up to here the kernel beats the library on MI355X; beyond, the library is used
+ROWS_KERNEL_MAX = 64          # most rows the hand-written few-rows kernel takes
 EPI_NONE, EPI_SILU_MUL = 0, 1
-_SKINNY_TARGET_WAVES = 2048
+# How the few-rows kernel is shaped for a product (measured on MI355X together with the kernel that adds
+# the stack of partial products; see the kernel for the variants):
+_ROWS_TARGET_WORKGROUPS = 640    # K is split until about this many workgroups stream W
+_ROWS_MAX_SPLITS = 8             # ... the consumer pays for every part of the stack
+_ROWS_PARTIAL_BYTES = 3 << 20    # ... and the float32 partial products stay below this
+_ROWS_WIDE_N = 32768             # from here on (an output head) N alone gives enough workgroups
+_ROWS_NARROW_N = 4096            # with more than 16 rows the kernel beats the library only up to here
+_V_GENERAL, _V_FUSED, _V_NARROW_LONG, _V_WIDE, _V_NARROW_SHORT = 0, 1, 2, 3, 4
+ROWS_VARIANTS = 5
 
 
-def gemm_skinny_supported(rows: int, k: int, x_stride: int) -> bool:
-    return 0 < rows <= SKINNY_MAX_ROWS and k % 8 == 0 and x_stride % 8 == 0
+def gemm_rows_supported(rows: int, k: int, x_stride: int) -> bool:
+    return 0 < rows <= ROWS_KERNEL_MAX and k % 8 == 0 and x_stride % 8 == 0
 
 
-def gemm_skinny_preferred(rows: int, k: int, x_stride: int) -> bool:
-    return rows <= SKINNY_PREFERRED_ROWS and gemm_skinny_supported(rows, k, x_stride)
+def gemm_rows_preferred(rows: int, n: int, k: int, x_stride: int, fused: bool = False) -> bool:
+    """Whether the hand-written kernel, not the library, should run this product."""
+    if not gemm_rows_supported(rows, k, x_stride):
+        return False
+    if rows <= 16:
+        return True
+    if fused:
+        return False
+    return n <= _ROWS_NARROW_N or (n >= _ROWS_WIDE_N and rows <= 32)
 
 
-def _skinny_waves(M: int, N: int, K: int, fused: bool) -> int:
-    """Waves of a workgroup that split K: enough waves in flight to fill the chip, each with at least
-    four 32-wide steps of its own, within what the reduction's LDS allows."""
-    nt = 1 if (M <= 16 and not fused) else 2
-    tiles = -(-N // (16 * nt))
-    steps = -(-K // 32)
-    cap = 8 if M > 16 else 16
-    want = max(1, -(-_SKINNY_TARGET_WAVES // tiles))
-    return max(1, min(want, cap, max(1, steps // 4)))
+def _rows_geometry(variant: int):
+    """(k steps of 32 per round, output columns per workgroup, column tiles a wave) of a variant."""
+    packed = lib.function("arle_gemm_rows_geometry")(variant)
+    _need(packed > 0, f"gemm_rows has no variant {variant}")
+    return packed >> 20, (packed >> 4) & 0xFFFF, packed & 15
 
 
-def gemm_bf16_skinny(x, w, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE):
-    """out = x . w^T for 1..64 rows of x on the matrix cores, streaming w once from HBM.
+def gemm_rows_plan(M: int, N: int, K: int, fused: bool = False):
+    """(variant, splits) for a product: small workgroups, K split across workgroups until enough of them
+    stream W, within a budget for the stack of partial products that the consumer has to add."""
+    if fused:
+        return _V_FUSED, 1
+    if N >= _ROWS_WIDE_N:
+        return _V_WIDE, 1
+    if M <= 16 and N <= _ROWS_NARROW_N:
+        variant = _V_NARROW_SHORT if K <= 4096 else _V_NARROW_LONG
+    else:
+        variant = _V_GENERAL
+    round_steps, columns, _ = _rows_geometry(variant)
+    groups = -(-N // columns)
+    rounds = -(-(-(-K // 32)) // round_steps)
+    splits = min(-(-_ROWS_TARGET_WORKGROUPS // groups), _ROWS_MAX_SPLITS, rounds,
+                 max(1, _ROWS_PARTIAL_BYTES // (M * N * 4)))
+    return variant, max(1, splits)
 
+
+def gemm_rows(x, w, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, variant: int | None = None,
+              splits: int | None = None):
+    """x . w^T for 1..64 rows of x, with x shared through LDS inside a workgroup.
+
+    splits == 1: returns [M, N] (or [M, N/2] with EPI_SILU_MUL) in `out_dtype`.
+    splits > 1: K is also split across workgroups; returns float32 [S, M, N] partial products (S <= splits,
+    no split is empty) for the consumer to add in the order of S.  With `variant` and `splits` left out
+    the shape decides (gemm_rows_plan), so callers must be ready for either form.
     EPI_SILU_MUL: w holds gate and up rows interleaved in blocks of 16; out[m, j] = silu(gate_j) * up_j.
     """
     _gpu(x, w)
     _rows(x, "x")
     _need(w.dim() == 2 and w.is_contiguous(), "w must be contiguous [N, K]")
-    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_bf16_skinny takes bfloat16 operands")
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_rows takes bfloat16 operands")
     M, K = x.shape
     N = w.shape[0]
-    _need(w.shape[1] == K, f"gemm_bf16_skinny: inner sizes differ ({K} vs {w.shape[1]})")
-    _need(gemm_skinny_supported(M, K, x.stride(0)),
-          f"gemm_bf16_skinny takes 1..{SKINNY_MAX_ROWS} rows and K % 8 == 0 (got {M} rows, K = {K})")
+    _need(w.shape[1] == K, f"gemm_rows: inner sizes differ ({K} vs {w.shape[1]})")
+    _need(gemm_rows_supported(M, K, x.stride(0)),
+          f"gemm_rows takes 1..{ROWS_KERNEL_MAX} rows and K % 8 == 0 (got {M} rows, K = {K})")
     _need(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
-    _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_bf16_skinny writes bfloat16 or float32")
+    _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_rows writes bfloat16 or float32")
     fused = epilogue == EPI_SILU_MUL
+    if variant is None or splits is None:
+        plan = gemm_rows_plan(M, N, K, fused)
+        variant = plan[0] if variant is None else variant
+        splits = plan[1] if splits is None else splits
     if fused:
         _need(N % 32 == 0, "the fused activation needs gate/up interleaved in blocks of 16")
-    out = torch.empty((M, N // 2 if fused else N), dtype=out_dtype, device=x.device)
-    lib.call("arle_gemm_bf16_skinny", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(),
-             out.stride(0), _CODES[out_dtype], M, N, K, int(epilogue), _skinny_waves(M, N, K, fused), _stream())
+    round_steps, _, tiles = _rows_geometry(variant)
+    if fused:
+        _need(tiles == 2 and splits == 1,
+              "the fused activation needs a variant with two column tiles a wave, and whole sums")
+    rounds_total = -(-(-(-K // 32)) // round_steps)
+    per_split = -(-rounds_total // max(1, min(splits, rounds_total)))
+    splits = -(-rounds_total // per_split)
+    if splits > 1:
+        out = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
+        ldo, stride, code = N, M * N, F32
+    else:
+        out = torch.empty((M, N // 2 if fused else N), dtype=out_dtype, device=x.device)
+        ldo, stride, code = out.stride(0), 0, _CODES[out_dtype]
+    lib.call("arle_gemm_rows", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), ldo, stride,
+             code, M, N, K, int(epilogue), variant, splits, per_split, _stream())
     return out
 
 
-def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16):
+def sum_partials(parts: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """[S, ...] float32 -> [...]: the stack added in order."""
+    _gpu(parts)
+    _need(parts.dtype == torch.float32 and parts.dim() >= 2 and parts.is_contiguous() and parts.shape[0] >= 1,
+          "sum_partials takes a contiguous float32 stack")
+    _need(out_dtype in _CODES, "sum_partials writes bfloat16 or float32")
+    out = torch.empty(parts.shape[1:], dtype=out_dtype, device=parts.device)
+    lib.call("arle_sum_partials", parts.data_ptr(), parts.shape[0], out.numel(), out.data_ptr(), _CODES[out_dtype],
+             out.numel(), _stream())
+    return out
+
+
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, partials_ok: bool = False):
     """out[M, N] = x[M, K] . w[N, K]^T, bfloat16 operands, float32 accumulation.
 
-    Up to 64 rows (decode steps) run the hand-written weight-streaming kernel.  More rows go to the
-    vendor library (hipBLASLt through torch.matmul), the matrix product the reference also leaves to
-    a library (crates/cuda-kernels/csrc/gemm/gemv.cu:240-330).
+    Few rows (decode steps, short portions) run the hand-written weight-streaming kernel.  More rows go
+    to the vendor library (hipBLASLt through torch.matmul), the matrix product the reference also leaves
+    to a library (crates/cuda-kernels/csrc/gemm/gemv.cu:240-330).
+    partials_ok: the caller adds a float32 stack [S, M, N] itself (in the order of S) if that is what the
+    kernel leaves behind; otherwise the stack is added here by one more small kernel.
     """
     _gpu(x, w)
     _rows(x, "x")
@@ -458,14 +545,17 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_bf16 takes bfloat16 operands")
     _need(x.shape[1] == w.shape[1], f"gemm_bf16: inner sizes differ ({x.shape[1]} vs {w.shape[1]})")
     _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_bf16 writes bfloat16 or float32")
-    if gemm_skinny_preferred(x.shape[0], x.shape[1], x.stride(0)) and x.data_ptr() % 16 == 0:
-        return gemm_bf16_skinny(x, w, out_dtype)
+    if gemm_rows_preferred(x.shape[0], w.shape[0], x.shape[1], x.stride(0)) and x.data_ptr() % 16 == 0:
+        out = gemm_rows(x, w, out_dtype)
+        if out.dim() == 3 and not partials_ok:
+            out = sum_partials(out, out_dtype)
+        return out
     if out_dtype == torch.float32:
         return _library_mm_f32out(x, w)
     return torch.matmul(x, w.t())
 
 
-_MM_OUT_DTYPE_OK: bool | None = None
+_MM_OUT_DTYPE_OK = None
 
 
 def _library_mm_f32out(x, w):

@@ -79,37 +79,44 @@ class PagedAttention(Part):
         return PagedNeed(num_kv_heads=self.nkv, head_dim=self.D, window=self.window)
 
     def forward(self, x, batch, cache):
+        """x [T, H] -> [T, H], or a float32 stack [S, T, H] to be added in order (see Linear)."""
         Q, KV = self.q_width, self.kv_width
         self.position.ensure_positions(batch.max_position + 1)
         cos, sin, rot = self.position.fused_rotary()
         fused = getattr(self.position, "fusable", False)
-        common = dict(num_q_heads=self.nq, num_kv_heads=self.nkv, head_dim=self.D, eps=self.eps,
+        nkv = self.nkv if cache.writes else 0   # a layer that reads another layer's cache only needs q
+        common = dict(num_q_heads=self.nq, num_kv_heads=nkv, head_dim=self.D, eps=self.eps,
                       positions=batch.positions)
+        to_cache = {}
         if cache.writes:
-            qkv = self.qkv(x)
-            q, k, v = qkv[:, :Q], qkv[:, Q:Q + KV], qkv[:, Q + KV:]
             to_cache = dict(slot_of_token=batch.slot_of_token, block_table=cache.block_table,
                             k_pages=cache.k_pages, v_pages=cache.v_pages, page_size=cache.page_size)
+        # the fused preparation kernel can add a stack of partial products itself
+        projected = (self.qkv if cache.writes else self.q_only)(x, partials_ok=fused)
+        if projected.dim() == 3:
+            q = torch.empty((x.shape[0], Q), dtype=x.dtype, device=x.device)
+            ops.qk_prep(q, None, None, q_weight=self.q_norm, k_weight=self.k_norm, cos=cos, sin=sin,
+                        rotary_dim=rot, parts=projected, **to_cache, **common)
         else:
-            # this layer reads a cache that an earlier layer wrote: only q is needed; the k
-            # operand of the preparation kernel is a scratch row that is thrown away
-            q = self.q_only(x)
-            k = v = torch.zeros((x.shape[0], KV), dtype=q.dtype, device=q.device)
-            to_cache = {}
-        if fused:
-            ops.qk_prep(q, k, v, q_weight=self.q_norm, k_weight=self.k_norm, cos=cos, sin=sin,
-                        rotary_dim=rot, **to_cache, **common)
-        else:
-            # a position encoding the fused kernel does not know: norm, encode, then write
-            if self.q_norm is not None:
-                ops.qk_prep(q, k, v, q_weight=self.q_norm, k_weight=self.k_norm, **common)
-            self.position.apply(q, k, batch.positions, self.nq, self.nkv)
-            if to_cache:
-                ops.qk_prep(q, k, v, **to_cache, **common)
+            if cache.writes:
+                q, k, v = projected[:, :Q], projected[:, Q:Q + KV], projected[:, Q + KV:]
+            else:
+                q = projected
+                k = v = projected[:, :0]
+            if fused:
+                ops.qk_prep(q, k, v, q_weight=self.q_norm, k_weight=self.k_norm, cos=cos, sin=sin,
+                            rotary_dim=rot, **to_cache, **common)
+            else:
+                # a position encoding the fused kernel does not know: norm, encode, then write
+                if self.q_norm is not None:
+                    ops.qk_prep(q, k, v, q_weight=self.q_norm, k_weight=self.k_norm, **common)
+                self.position.apply(q, k, batch.positions, self.nq, nkv)
+                if to_cache:
+                    ops.qk_prep(q, k, v, **to_cache, **common)
         out = torch.empty((x.shape[0], Q), dtype=q.dtype, device=q.device)
         paged_attention(q, out, cache, batch, num_q_heads=self.nq, num_kv_heads=self.nkv,
                         head_dim=self.D, scale=self.scale, window=self.window or 0)
-        return self.o(out)
+        return self.o(out, partials_ok=True)
 
 
 def paged_attention(q, out, cache, batch, *, num_q_heads, num_kv_heads, head_dim, scale, window):

@@ -7,13 +7,15 @@ learns which model it is in.
 
 Interfaces (T = tokens of the packed step, H = hidden size, A = activation dtype):
 
-* norm          `forward(x[T,W]) -> A[T,W]`;  `add_norm(residual f32[T,H], delta A[T,H] | None,
+* norm          `forward(x[T,W]) -> A[T,W]`;  `add_norm(residual f32[T,H], delta | None,
                 rows=None) -> A[rows or T, H]` adds the delta into the residual (in place) first.
+                A delta is A[T,H], or a float32 stack [S,T,H] of partial sums to be added in the order
+                of S (what a matrix product with K split over workgroups leaves behind).
 * position      `fused_rotary() -> (cos, sin, rotary_dim) | None`;  `apply(q, k, positions)` in place.
 * mixer         `cache_need() -> PagedNeed | StateNeed | None`;
-                `forward(x A[T,H], batch: StepBatch, cache_view) -> A[T,H]`.
-* feed_forward  `forward(x A[T,H]) -> A[T,H]`.
-* block         `forward(residual f32[T,H], delta A[T,H] | None, batch, cache_view) -> (residual, delta)`;
+                `forward(x A[T,H], batch: StepBatch, cache_view) -> delta`.
+* feed_forward  `forward(x A[T,H]) -> delta`.
+* block         `forward(residual f32[T,H], delta | None, batch, cache_view) -> (residual, delta)`;
                 the returned delta is what the next block (or the final norm) still has to add.
 * embedding     `forward(token_ids i32[T]) -> f32[T,H]`.
 * head          `forward(x A[R,H]) -> f32[R,V]`.

@@ -43,12 +43,14 @@ class SwiGLU(Part):
         self.down = Linear(tensors["down"])
 
     def forward(self, x):
+        """x [T, H] -> [T, H], or a float32 stack [S, T, H] to be added in order (see Linear)."""
         if self.block:
-            if ops.gemm_skinny_preferred(x.shape[0], x.shape[1], x.stride(0)):
-                act = ops.gemm_bf16_skinny(x, self.gate_up.weight, x.dtype, ops.EPI_SILU_MUL)
+            w = self.gate_up.weight
+            if x.shape[0] and ops.gemm_rows_preferred(x.shape[0], w.shape[0], x.shape[1], x.stride(0), fused=True):
+                act = ops.gemm_rows(x, w, x.dtype, ops.EPI_SILU_MUL)
             else:
                 act = ops.silu_mul_interleaved(self.gate_up(x), self.block)
         else:
             gu = self.gate_up(x)
             act = ops.silu_mul(gu[:, : self.inter], gu[:, self.inter:])
-        return self.down(act)
+        return self.down(act, partials_ok=True)

@@ -8,6 +8,11 @@ Which kernel runs depends only on the types of the operands:
   cuBLAS for its projections (infer/src/ops/linear.rs:921-959);
 * bfloat16 x, float32 W (a tensor that the checkpoint stores in 32 bits stays so):
   x is widened and the float32 kernel runs.
+
+The few-rows kernel may split K over workgroups and leave a stack of float32 partial products
+[S, T, out] behind.  A caller whose consumer can add such a stack in order (the residual add fused
+into RMSNorm, the q/k/v preparation) says `partials_ok=True` and passes it on; otherwise the stack
+is added here.
 """
 from __future__ import annotations
 
@@ -23,8 +28,9 @@ class Linear:
         self.weight = weight
         self.out_features, self.in_features = weight.shape
 
-    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-        """x [T, in] -> [T, out] in `out_dtype` (default: the type of x)."""
+    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None, partials_ok: bool = False) -> torch.Tensor:
+        """x [T, in] -> [T, out] in `out_dtype` (default: the type of x); with `partials_ok` possibly a
+        float32 stack [S, T, out] whose sum over S, in order, is the product."""
         out_dtype = out_dtype or x.dtype
         w = self.weight
         if x.shape[0] == 0:
@@ -34,4 +40,4 @@ class Linear:
             return y if out_dtype == torch.float32 else y.to(out_dtype)
         if x.dtype != torch.bfloat16:
             raise ops.ShapeError(f"a bfloat16 weight needs bfloat16 activations, got {x.dtype}")
-        return ops.gemm_bf16(x, w, out_dtype)
+        return ops.gemm_bf16(x, w, out_dtype, partials_ok=partials_ok)

@@ -172,6 +172,35 @@ def test_qk_prep_norm_rope_and_cache_write(nq, nkv, D, rot, dt):
         written[int(table[slots[t], positions[t] // P]), positions[t] % P] = True
     assert torch.count_nonzero(dk.transpose(1, 2)[~written]) == 0
 
+    # the same projections as a stack of three float32 partial products: same q, same cache
+    stack = torch.randn(3, T, (nq + 2 * nkv) * D, generator=_g(24))
+    stack[2] = qkv.float() - stack[0] - stack[1]
+    x = stack.double().sum(0)
+    q = plain.qk_norm(x[:, :Q].reshape(T, nq, D), qw.double(), eps)
+    k = plain.qk_norm(x[:, Q:Q + KV].reshape(T, nkv, D), kw.double(), eps)
+    v = x[:, Q + KV:].reshape(T, nkv, D)
+    if rot:
+        q = torch.cat([plain.apply_rope(q[..., :rot], c, s), q[..., rot:]], -1)
+        k = torch.cat([plain.apply_rope(k[..., :rot], c, s), k[..., rot:]], -1)
+    dq = torch.zeros(T, Q, dtype=dt, device=DEV)
+    dk, dv = k_pages.to(DEV), v_pages.to(DEV)
+    ops.qk_prep(dq, None, None, num_q_heads=nq, num_kv_heads=nkv, head_dim=D, eps=eps, q_weight=qw.to(DEV),
+                k_weight=kw.to(DEV), cos=None if cos is None else cos.to(DEV), sin=None if sin is None else sin.to(DEV),
+                rotary_dim=rot, positions=positions.to(DEV), slot_of_token=slots.to(DEV),
+                block_table=table.to(DEV), k_pages=dk, v_pages=dv, page_size=P, parts=stack.to(DEV))
+    assert _rel(dq.cpu().reshape(T, nq, D), q) < tol
+    dk, dv = dk.cpu(), dv.cpu()
+    for t in range(T):
+        page = int(table[slots[t], positions[t] // P])
+        assert _rel(dk[page, :, positions[t] % P], k[t]) < tol
+        assert _rel(dv[page, :, :, positions[t] % P], v[t]) < tol
+    # only q (a layer that reads another layer's cache)
+    dq2 = torch.zeros(T, Q, dtype=dt, device=DEV)
+    ops.qk_prep(dq2, None, None, num_q_heads=nq, num_kv_heads=0, head_dim=D, eps=eps, q_weight=qw.to(DEV),
+                k_weight=kw.to(DEV), cos=None if cos is None else cos.to(DEV), sin=None if sin is None else sin.to(DEV),
+                rotary_dim=rot, positions=positions.to(DEV), parts=stack[:, :, :Q].contiguous().to(DEV))
+    assert torch.equal(dq2, dq)
+
 
 def _fill_cache(table, k_pages, v_pages, slot, k, v, P):
     for pos in range(k.shape[0]):
@@ -407,46 +436,95 @@ def test_attention_mfma_refuses_shapes_it_was_not_written_for():
                             max_qlen=2, max_kv_len=2, num_q_heads=2, num_kv_heads=1, head_dim=24, page_size=16, scale=1.0)
 
 
+def _whole(out):
+    """A product, or the stack of partial products a split K leaves behind, as one float64 matrix."""
+    return out.double().sum(0).cpu() if out.dim() == 3 else out.double().cpu()
+
+
 @pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 64])
 @pytest.mark.parametrize("N,K", [(96, 64), (333, 88), (2560, 4096), (6144, 2560), (40, 8), (2560, 9728)])
-def test_gemm_bf16_skinny(M, N, K):
+def test_gemm_rows_as_planned(M, N, K):
     a = torch.randn(M, K, generator=_g(100)).bfloat16()
     w = (torch.randn(N, K, generator=_g(101)) * 0.1).bfloat16()
     want = a.double() @ w.double().T
-    got = ops.gemm_bf16_skinny(a.to(DEV), w.to(DEV), torch.float32).cpu()
-    assert _rel(got, want) < 1e-5          # float32 accumulation of exact bfloat16 products
-    got = ops.gemm_bf16_skinny(a.to(DEV), w.to(DEV), torch.bfloat16).cpu()
-    assert got.dtype == torch.bfloat16 and _rel(got, want) < 5e-3
+    got = ops.gemm_rows(a.to(DEV), w.to(DEV), torch.float32)
+    assert _rel(_whole(got), want) < 1e-5          # float32 accumulation of exact bfloat16 products
+    # the general entry point always hands back whole sums, in the type asked for
+    got = ops.gemm_bf16(a.to(DEV), w.to(DEV), torch.bfloat16).cpu()
+    assert got.dtype == torch.bfloat16 and got.shape == (M, N) and _rel(got, want) < 5e-3
     # a view with a row stride (rows of a wider buffer)
     wide = torch.randn(M, K + 24, generator=_g(102)).bfloat16().to(DEV)
-    got = ops.gemm_bf16_skinny(wide[:, 8:8 + K], w.to(DEV), torch.float32).cpu()
-    assert _rel(got, wide[:, 8:8 + K].double().cpu() @ w.double().T) < 1e-5
+    got = ops.gemm_rows(wide[:, 8:8 + K], w.to(DEV), torch.float32)
+    assert _rel(_whole(got), wide[:, 8:8 + K].double().cpu() @ w.double().T) < 1e-5
+
+
+@pytest.mark.parametrize("variant", range(ops.ROWS_VARIANTS))
+@pytest.mark.parametrize("M,N,K,splits", [(5, 333, 88, 1), (16, 96, 1096, 3), (20, 200, 520, 2), (64, 72, 2056, 5),
+                                          (33, 2560, 4096, 16)])
+def test_gemm_rows_every_variant_and_split(variant, M, N, K, splits):
+    a = torch.randn(M, K, generator=_g(103)).bfloat16()
+    w = (torch.randn(N, K, generator=_g(104)) * 0.1).bfloat16()
+    got = ops.gemm_rows(a.to(DEV), w.to(DEV), torch.float32, variant=variant, splits=splits)
+    # a stack of at most `splits` partial products, or whole sums when K holds a single round of this variant
+    assert (got.dim() == 2 or 1 < got.shape[0] <= splits) and (splits > 1 or got.dim() == 2)
+    assert _rel(_whole(got), a.double() @ w.double().T) < 1e-5
+    again = ops.gemm_rows(a.to(DEV), w.to(DEV), torch.float32, variant=variant, splits=splits)
+    assert torch.equal(got, again)                 # nothing in the kernel depends on timing
 
 
 @pytest.mark.parametrize("M", [1, 8, 20, 64])
 @pytest.mark.parametrize("inter,K", [(48, 64), (224, 96), (9728, 2560)])
-def test_gemm_bf16_skinny_with_fused_activation(M, inter, K):
+def test_gemm_rows_with_fused_activation(M, inter, K):
     x = torch.randn(M, K, generator=_g(110)).bfloat16()
     gate = (torch.randn(inter, K, generator=_g(111)) * 0.1).bfloat16()
     up = (torch.randn(inter, K, generator=_g(112)) * 0.1).bfloat16()
     fused = torch.stack([gate.view(-1, 16, K), up.view(-1, 16, K)], dim=1).reshape(2 * inter, K).contiguous()
     want = plain.silu(x.double() @ gate.double().T) * (x.double() @ up.double().T)
-    got = ops.gemm_bf16_skinny(x.to(DEV), fused.to(DEV), torch.float32, ops.EPI_SILU_MUL).cpu()
-    assert got.shape == (M, inter) and _rel(got, want) < 1e-5
+    for variant in (None, 1, 3):
+        got = ops.gemm_rows(x.to(DEV), fused.to(DEV), torch.float32, ops.EPI_SILU_MUL, variant=variant, splits=1).cpu()
+        assert got.shape == (M, inter) and _rel(got, want) < 1e-5
     # the same weights through the library product and the interleaved activation kernel
     gu = (x.double() @ fused.double().T).bfloat16().to(DEV)
     got = ops.silu_mul_interleaved(gu, 16).cpu()
     assert _rel(got, want) < 1e-2
 
 
-def test_gemm_bf16_skinny_refuses_what_it_cannot_take():
+def test_sum_partials_and_stacked_residual_add():
+    parts = torch.randn(5, 7, 88, generator=_g(113))
+    want = parts.double().sum(0)
+    assert _rel(ops.sum_partials(parts.to(DEV), torch.float32).cpu(), want) < 1e-6
+    assert ops.sum_partials(parts.to(DEV), torch.bfloat16).dtype == torch.bfloat16
+    for width in (88, 2560, 4100):                  # register-resident kernel, and the general one
+        parts = torch.randn(6, 3, width, generator=_g(114))
+        res = torch.randn(3, width, generator=_g(115)) * 2.0
+        nw = 1.0 + 0.2 * torch.randn(width, generator=_g(116))
+        on_gpu = res.clone().to(DEV)
+        got = ops.add_rmsnorm(on_gpu, parts.to(DEV), nw.to(DEV), 1e-5, torch.float32).cpu()
+        summed = res.double() + parts.double().sum(0)
+        assert _rel(on_gpu.cpu(), summed) < 1e-6
+        assert _rel(got, plain.rms_norm(summed, nw.double(), 1e-5)) < 1e-5
+        # picked rows (the final norm): nothing is written back
+        rows = torch.tensor([2, 0], dtype=torch.int32, device=DEV)
+        on_gpu = res.clone().to(DEV)
+        got = ops.add_rmsnorm(on_gpu, parts.to(DEV), nw.to(DEV), 1e-5, torch.float32, rows=rows).cpu()
+        assert torch.equal(on_gpu.cpu(), res)
+        assert _rel(got, plain.rms_norm(summed[[2, 0]], nw.double(), 1e-5)) < 1e-5
+
+
+def test_gemm_rows_refuses_what_it_cannot_take():
     x = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
     w = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ops.ShapeError, match="1..64 rows"):
-        ops.gemm_bf16_skinny(x, w)
+        ops.gemm_rows(x, w)
     with pytest.raises(ops.ShapeError, match="K % 8"):
-        ops.gemm_bf16_skinny(torch.zeros(2, 20, dtype=torch.bfloat16, device=DEV),
-                             torch.zeros(4, 20, dtype=torch.bfloat16, device=DEV))
+        ops.gemm_rows(torch.zeros(2, 20, dtype=torch.bfloat16, device=DEV),
+                      torch.zeros(4, 20, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(ops.ShapeError, match="no variant"):
+        ops.gemm_rows(x[:4], w, variant=99, splits=1)
+    with pytest.raises(ops.ShapeError, match="two column tiles"):
+        ops.gemm_rows(x[:4], w, epilogue=ops.EPI_SILU_MUL, variant=0, splits=1)
+    with pytest.raises(ops.ShapeError, match="whole sums"):
+        ops.gemm_rows(x[:4], w, epilogue=ops.EPI_SILU_MUL, variant=1, splits=2)
     # the general entry point still serves such shapes, through the library
     out = ops.gemm_bf16(torch.ones(2, 20, dtype=torch.bfloat16, device=DEV), torch.ones(4, 20, dtype=torch.bfloat16, device=DEV))
     assert out.shape == (2, 4) and float(out[0, 0]) == 20.0

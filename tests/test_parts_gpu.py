@@ -22,6 +22,11 @@ def _rel(a, b):
     return float((a.double().cpu() - b.double()).abs().max() / b.double().abs().max())
 
 
+def _delta(d):
+    """What a mixer or feed-forward hands to the residual add: [T, H], or a float32 stack to be summed."""
+    return d.double().sum(0) if d.dim() == 3 else d
+
+
 def _tensors(shapes, dtype, seed=0, scale=0.2):
     g = torch.Generator().manual_seed(seed)
     return {k: (torch.randn(*s, generator=g) * scale + (1.0 if len(s) == 1 else 0.0)).to(dtype) for k, s in shapes.items()}
@@ -48,7 +53,7 @@ def test_feed_forward_part(dtype, tol):
                                                {"gate": "g", "up": "u", "down": "d"}), lambda n: w[n].to(DEV), _rt(dtype))
     x = torch.randn(7, 88).to(dtype)
     want = plain.swiglu_mlp(x.double(), w["g"].double(), w["u"].double(), w["d"].double())
-    assert _rel(part.forward(x.to(DEV)), want) < tol
+    assert _rel(_delta(part.forward(x.to(DEV))), want) < tol
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -101,7 +106,7 @@ def test_attention_part_over_its_cache(dtype, tol, window):
         batch = build_step_batch([StepEntry("r", [0] * (hi - lo), [])], cache.slot_of.__getitem__, cache.length, 10, DEV)
         cache.append([("r", hi - lo)])
         cache.sync_tables()
-        outs.append(part.forward(x[lo:hi].to(DEV), batch, cache.view(0)))
+        outs.append(_delta(part.forward(x[lo:hi].to(DEV), batch, cache.view(0))).double())
         cache.trim_windows("r")
     got = torch.cat(outs)
     wd = {k: v.double() for k, v in w.items()}
