@@ -118,6 +118,114 @@ __global__ __launch_bounds__(kPrepWaves* kWave) void qk_prep_kernel(
   }
 }
 
+// bfloat16, head_dim a power of two (64..512), rotary_dim a multiple of 16: eight contiguous dims a lane,
+// one 16-byte load and one 16-byte store (q in place, k into its cache row), LPH = head_dim / 8 lanes a head.
+// The per-head sum of squares and the rotation partner (the lane rot/16 away) go through lane shuffles.
+template <int LPH, typename TW>
+__global__ __launch_bounds__(256) void qk_prep_bf16x8_kernel(
+    uint16_t* __restrict__ q, int64_t q_stride, uint16_t* __restrict__ k, int64_t k_stride,
+    const uint16_t* __restrict__ v, int64_t v_stride, const TW* __restrict__ q_w, const TW* __restrict__ k_w,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, const int* __restrict__ positions,
+    const int* __restrict__ slot_of_token, const int* __restrict__ block_table, int table_stride,
+    uint16_t* __restrict__ k_pages, uint16_t* __restrict__ v_pages, int nq, int nkv, int page_size, float eps) {
+  constexpr int D = LPH * 8;
+  const int t = blockIdx.x;
+  const int unit = blockIdx.y * blockDim.x + threadIdx.x;
+  const int head = unit / LPH, d0 = (unit % LPH) * 8;
+  const bool valid = head < nq + 2 * nkv;
+  const bool is_q = head < nq, is_v = valid && head >= nq + nkv;
+  const int local = is_q ? head : (is_v ? head - nq - nkv : head - nq);
+  const int pos = positions[t];
+  const int in_page = pos % page_size;
+  int64_t page_base = 0;
+  if (valid && !is_q && k_pages) {
+    const int page = block_table[static_cast<int64_t>(slot_of_token[t]) * table_stride + pos / page_size];
+    page_base = static_cast<int64_t>(page) * nkv * page_size * D;
+  }
+  uint16_t* src = is_q ? q + static_cast<int64_t>(t) * q_stride + local * D + d0
+                       : (is_v ? const_cast<uint16_t*>(v) + static_cast<int64_t>(t) * v_stride + local * D + d0
+                               : k + static_cast<int64_t>(t) * k_stride + local * D + d0);
+  uint4 raw = {0u, 0u, 0u, 0u};
+  if (valid) raw = *reinterpret_cast<const uint4*>(src);
+  if (is_v) {
+    if (v_pages) {
+      uint16_t* dst = v_pages + page_base + (static_cast<int64_t>(local) * D + d0) * page_size + in_page;
+      const uint32_t wds[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        dst[static_cast<int64_t>(e) * page_size] = static_cast<uint16_t>(wds[e / 2] >> (16 * (e & 1)));
+    }
+  }
+  // every lane takes part in the shuffles below (v lanes and lanes past the last head with zeros)
+  float x[8];
+  {
+    const uint32_t wds[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      x[2 * e] = __uint_as_float(wds[e] << 16);
+      x[2 * e + 1] = __uint_as_float(wds[e] & 0xffff0000u);
+    }
+  }
+  const TW* w = is_q ? q_w : k_w;
+  if (w != nullptr) {
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, kWave);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(D) + eps);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = x[e] * inv * to_float(w[d0 + e]);
+  }
+  const int half = rot / 2;
+  float y[8];
+  {
+    const bool low = d0 < half, rotated = d0 < rot;
+    const int lane = threadIdx.x % kWave;
+    const int from = rotated ? (low ? lane + half / 8 : lane - half / 8) : lane;
+    const int cd = low ? d0 : d0 - half;  // column of the cos/sin row
+    const float* cs = cos_t + static_cast<int64_t>(pos) * half + cd;
+    const float* sn = sin_t + static_cast<int64_t>(pos) * half + cd;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float other = __shfl(x[e], from, kWave);
+      if (rotated && valid && !is_v) {
+        const float c = cs[e], sv = sn[e];
+        y[e] = low ? x[e] * c - other * sv : other * sv + x[e] * c;
+      } else {
+        y[e] = x[e];
+      }
+    }
+  }
+  if (!valid || is_v) return;
+  uint16_t* dst = src;
+  if (!is_q && k_pages) dst = k_pages + page_base + (static_cast<int64_t>(local) * page_size + in_page) * D + d0;
+  *reinterpret_cast<uint4*>(dst) = uint4{pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3]), pack_bf16x2(y[4], y[5]),
+                                         pack_bf16x2(y[6], y[7])};
+}
+
+template <int LPH>
+int launch_prep_bf16x8(void* q, long long q_stride, void* k, long long k_stride, const void* v, long long v_stride,
+                       const void* q_w, const void* k_w, int w_dtype, const float* cos_t, const float* sin_t, int rot,
+                       const int* positions, const int* slot_of_token, const int* block_table, int table_stride,
+                       void* k_pages, void* v_pages, int tokens, int nq, int nkv, int page_size, float eps,
+                       hipStream_t s) {
+  const int units = (nq + 2 * nkv) * LPH;
+  dim3 grid(tokens, (units + 255) / 256);
+  auto u16 = [](const void* p) { return static_cast<uint16_t*>(const_cast<void*>(p)); };
+  if (w_dtype == kF32)
+    qk_prep_bf16x8_kernel<LPH, float><<<grid, 256, 0, s>>>(
+        u16(q), q_stride, u16(k), k_stride, u16(v), v_stride, static_cast<const float*>(q_w),
+        static_cast<const float*>(k_w), cos_t, sin_t, rot, positions, slot_of_token, block_table, table_stride,
+        u16(k_pages), u16(v_pages), nq, nkv, page_size, eps);
+  else
+    qk_prep_bf16x8_kernel<LPH, bf16><<<grid, 256, 0, s>>>(
+        u16(q), q_stride, u16(k), k_stride, u16(v), v_stride, static_cast<const bf16*>(q_w),
+        static_cast<const bf16*>(k_w), cos_t, sin_t, rot, positions, slot_of_token, block_table, table_stride,
+        u16(k_pages), u16(v_pages), nq, nkv, page_size, eps);
+  return launch_status();
+}
+
 template <typename T>
 int launch_prep(void* q, long long q_stride, void* k, long long k_stride, const void* v,
                 long long v_stride, const void* q_w, const void* k_w, int w_dtype,
@@ -167,6 +275,21 @@ extern "C" int arle_qk_prep(void* q, long long q_stride, void* k, long long k_st
   if (parts != nullptr && (n_parts < 1 || (nkv > 0 && (k_pages == nullptr || v_pages == nullptr))))
     return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool pow2 = D >= 64 && (D & (D - 1)) == 0;
+  if (dtype == kBF16 && parts == nullptr && pow2 && rot % 16 == 0 && q_stride % 8 == 0 && k_stride % 8 == 0 &&
+      v_stride % 8 == 0 && aligned(q) && aligned(k) && aligned(v) && aligned(k_pages) &&
+      (cos_t == nullptr || (reinterpret_cast<uintptr_t>(cos_t) % 4 == 0))) {
+#define ARLE_PREP(LPH)                                                                                          \
+  return launch_prep_bf16x8<LPH>(q, q_stride, k, k_stride, v, v_stride, q_w, k_w, w_dtype, cos_t, sin_t, rot,    \
+                                 positions, slot_of_token, block_table, table_stride, k_pages, v_pages, tokens, \
+                                 nq, nkv, page_size, eps, s)
+    if (D == 64) ARLE_PREP(8);
+    if (D == 128) ARLE_PREP(16);
+    if (D == 256) ARLE_PREP(32);
+    if (D == 512) ARLE_PREP(64);
+#undef ARLE_PREP
+  }
   if (dtype == kF32)
     return launch_prep<float>(q, q_stride, k, k_stride, v, v_stride, q_w, k_w, w_dtype, cos_t, sin_t,
                               rot, positions, slot_of_token, block_table, table_stride, k_pages,

@@ -98,13 +98,18 @@ def test_gemm_bf16(M, N, K):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
-def test_silu_mul(dt):
-    gu = torch.randn(5, 2 * 136, generator=_g(10)).to(dt)
-    g, u = gu[:, :136].double(), gu[:, 136:].double()
+@pytest.mark.parametrize("width", [136, 132, 9728])      # eight columns a thread in bfloat16, or one by one
+def test_silu_mul(dt, width):
+    gu = (torch.randn(5, 2 * width, generator=_g(10)) * 3.0).to(dt)
+    g, u = gu[:, :width].double(), gu[:, width:].double()
     want = plain.silu(g) * u
     d = gu.to(DEV)
-    got = ops.silu_mul(d[:, :136], d[:, 136:]).cpu()
+    got = ops.silu_mul(d[:, :width], d[:, width:]).cpu()
     assert _rel(got, want) < (1e-6 if dt == torch.float32 else 5e-3)
+    if width % 16 == 0:
+        inter = torch.stack([gu[:, :width].view(5, -1, 16), gu[:, width:].view(5, -1, 16)], dim=2).reshape(5, 2 * width)
+        got = ops.silu_mul_interleaved(inter.contiguous().to(DEV), 16).cpu()
+        assert _rel(got, want) < (1e-6 if dt == torch.float32 else 5e-3)
     z = torch.zeros(2, 8, dtype=dt, device=DEV)
     assert torch.count_nonzero(ops.silu_mul(z, torch.ones_like(z))) == 0
 
@@ -127,7 +132,7 @@ def _paged_setup(lengths, nkv, D, P, dtype, seed, shuffle=True):
 
 
 @pytest.mark.parametrize("nq,nkv,D,rot", [(3, 1, 48, 48), (4, 2, 16, 16), (8, 2, 128, 128), (2, 2, 64, 32),
-                                           (5, 5, 32, 0)])
+                                           (5, 5, 32, 0), (2, 1, 256, 64), (3, 3, 64, 0), (32, 8, 128, 128)])
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
 def test_qk_prep_norm_rope_and_cache_write(nq, nkv, D, rot, dt):
     P, eps, theta = 8, 1e-5, 1e4
