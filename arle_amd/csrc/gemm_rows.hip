@@ -1,33 +1,35 @@
 // bfloat16 matrix product for few rows (decode steps and short prompt portions):
 //   C[M,N] = X[M,K] . W[N,K]^T,  1 <= M <= 64.
 //
-// With few rows the product is one pass over W, and HBM bandwidth is the bound.  Reads of X are
-// not free either: every workgroup needs the rows of X for the k range it works on, and on
-// MI355X bytes that come from the L2 cost about as much as bytes that come from HBM.  So the
-// kernel shares X inside a workgroup and makes a workgroup's tile of W wide:
+// With few rows the product is one pass over W, and HBM bandwidth is the bound.  What decides the
+// speed on MI355X is how many independent loads of W are in flight on every CU at every moment, so
+// the kernel is built around that:
 //
-//   * a workgroup has WN x WK waves.  Wave (wn, wk) owns 16*NT output columns (rows of W) and
-//     every wk-th block of kBlockSteps 32-wide k steps of the workgroup's k slice;
-//   * X for one round (WK blocks of k) is staged once through LDS (coalesced 16-byte loads,
-//     rows padded by 16 bytes against bank conflicts) and read from there as the B operand of
-//     v_mfma_f32_16x16x32_bf16 by all WN waves: X traffic drops by the factor WN;
-//   * W goes straight from global memory into the A operand, 16 bytes a lane, one round ahead
-//     of its use, so that every wave keeps kBlockSteps * NT kilobyte-sized loads in flight;
-//   * the WK partial sums of a column tile are added through LDS in the fixed order wk = 0..WK-1;
-//   * gridDim.y splits K further across workgroups when N alone gives too few of them (small
-//     workgroups in great number stream best on MI355X).  Each split writes its own float32
-//     partial product out[s][M][N]; the kernel that consumes the product (the residual add fused
-//     into RMSNorm, the q/k/v preparation) adds the splits in the order s = 0, 1, ..., so results
+//   * many small workgroups of WN x WK waves.  Wave (wn, wk) owns 16 output columns (rows of W: one
+//     tile a wave streams better than two) and the wk-th part of the workgroup's k slice;
+//   * gridDim.y splits K across workgroups when N alone gives too few of them.  Each split writes its
+//     own float32 partial product out[s][M][N]; the kernel that consumes the product (the residual add
+//     fused into RMSNorm, the q/k/v preparation) adds the splits in the order s = 0, 1, ..., so results
 //     do not depend on timing.  (Adding them here, by the workgroup that arrives last, needs
 //     device-scope fences or write-through accesses, and both cost more than they save.)
+//   * the rows of X for the workgroup's whole k slice are staged once into LDS (reads of X come from
+//     the L2 but cost about as much as reads from HBM, so the WN waves share them).  After that one
+//     barrier the waves run free: there is no barrier inside the loop over k;
+//   * W goes straight from global memory into the A operand of v_mfma_f32_16x16x32_bf16, 16 bytes a
+//     lane, through a ring of PD registers: the load of step s + PD is issued as soon as step s has
+//     been multiplied, so every wave keeps PD kilobyte-sized loads in flight.  The X operand comes
+//     from LDS through a shorter ring of its own, so that no step waits for an LDS read;
+//   * the WK partial sums of a column tile are added through LDS in the fixed order wk = 0..WK-1.
 //
 // Operand layout (lane = 16 g + i):  A lane (i, g) = W[n0 + i][32 s + 8 g .. +7],
 // B lane (j, g) = X[m0 + j][32 s + 8 g .. +7], C lane (j, g) register r = C[m0 + j][n0 + 4 g + r].
-// Rows past M or N are clamped for the loads and skipped at the store; K % 8 == 0.
+// Rows past M or N are clamped for the loads and skipped at the store.  K % 8 == 0; where a step of 32
+// reaches past K, W is read from a clamped address and meets zeros that the staging put into X.
 //
-// Epilogue kEpiSiluMul: W holds gate and up rows interleaved in blocks of 16 and the kernel
-// writes silu(gate) * up, [M, N/2] (the reference runs an elementwise kernel for this,
-// crates/cuda-kernels/csrc/misc/split_qkv.cu:35-52).  Plain product: the reference's
+// Epilogue kEpiSiluMul: W holds gate and up rows interleaved in blocks of 16, so even column tiles are
+// gate and odd ones the matching up columns.  Neighbouring waves (WN is even) own such a pair; the odd
+// wave hands its sums over through LDS and the even one writes silu(gate) * up, [M, N/2] (the reference
+// runs an elementwise kernel for this, crates/cuda-kernels/csrc/misc/split_qkv.cu:35-52).  Plain product: the reference's
 // crates/cuda-kernels/csrc/gemm/gemv.cu:45-,240-330 and cuBLAS for more rows.
 #include "common.h"
 
@@ -37,7 +39,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kEpiNone = 0, kEpiSiluMul = 1;
-constexpr int kPad = 8;  // elements of padding per LDS row of X
+constexpr int kPad = 8;  // elements of padding per LDS row of X (16 bytes: rows start in different banks)
 
 struct RowsArgs {
   const uint16_t* x;
@@ -47,261 +49,225 @@ struct RowsArgs {
   void* out;
   int64_t ldo;
   int M, N, K;
-  int rounds_per_split;  // rounds (WK * KBS steps of 32) that one k split covers
+  int steps_per_split;   // k steps of 32 that one k split covers
   int64_t split_stride;  // elements between the partial products of two k splits
 };
 
-template <int MT, int NT, int WN, int WK, int KBS, int EPI, typename TOut>
+template <int MT, int WN, int WK, int PD, int XD, int EPI, typename TOut>
 __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a) {
   constexpr int kThreads = WN * WK * 64;
-  constexpr int kRows = MT * 16;
-  constexpr int kRoundK = WK * KBS * 32;          // elements of k per round
-  constexpr int kPitch = kRoundK + kPad;          // LDS row pitch in elements
-  constexpr int kChunksPerRow = kRoundK / 8;      // 16-byte chunks of one row of a round
-  constexpr int kChunks = kRows * kChunksPerRow;
-  constexpr int kCPT = (kChunks + kThreads - 1) / kThreads;  // chunks each thread stages per round
-  static_assert(EPI != kEpiSiluMul || NT == 2, "the fused activation needs the gate and the up tile side by side");
-  extern __shared__ __align__(16) uint16_t lds[];  // [2][kRows][kPitch] X, later the partial sums
+  static_assert(PD % XD == 0, "the X ring must divide the W ring");
+  static_assert(EPI != kEpiSiluMul || WN % 2 == 0, "the fused activation pairs neighbouring waves");
+  // [M][pitch] X, then [WK-1][WN][MT][64][4] partial sums, then [WN/2][MT][64][4] for the gate/up exchange
+  extern __shared__ __align__(16) uint16_t lds[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wn = wave % WN, wk = wave / WN;
   const int li = lane & 15, g = lane >> 4;
-  const int n0 = (blockIdx.x * WN + wn) * (16 * NT);
+  const int n0 = (blockIdx.x * WN + wn) * 16;
   const int M = a.M, N = a.N, K = a.K;
 
   const int steps_total = (K + 31) / 32;
-  const int round0 = blockIdx.y * a.rounds_per_split;
-  const int rounds = min(a.rounds_per_split, (steps_total + WK * KBS - 1) / (WK * KBS) - round0);
+  const int s_begin = blockIdx.y * a.steps_per_split;
+  const int s_end = min(s_begin + a.steps_per_split, steps_total);
+  const int pitch = a.steps_per_split * 32 + kPad;
 
-  const uint16_t* wp[NT];
-#pragma unroll
-  for (int t = 0; t < NT; ++t) wp[t] = a.w + static_cast<int64_t>(min(n0 + 16 * t + li, N - 1)) * a.ldw + 8 * g;
+  // this wave's steps: the wk-th part of the slice
+  const int per = (s_end - s_begin + WK - 1) / WK;
+  const int w_begin = s_begin + wk * per;
+  const int n_steps = max(0, min(w_begin + per, s_end) - w_begin);
 
-  // staging: chunk c = tid + i * kThreads -> row c / kChunksPerRow, 16-byte column c % kChunksPerRow
-  // (threads past the last chunk, when there are more threads than chunks, stage nothing)
-  const uint16_t* xsrc[kCPT];
-  int xcol[kCPT], xdst[kCPT];
-#pragma unroll
-  for (int i = 0; i < kCPT; ++i) {
-    const int c = tid + i * kThreads;
-    const int row = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
-    xsrc[i] = a.x + static_cast<int64_t>(min(row, M - 1)) * a.ldx + col;
-    xcol[i] = col;
-    xdst[i] = c < kChunks ? row * kPitch + col : -1;
-  }
+  const uint16_t* wrow = a.w + static_cast<int64_t>(min(n0 + li, N - 1)) * a.ldw;
+  auto load_w = [&](int s) {
+    const int e = min(32 * s + 8 * g, K - 8);  // clamped: always inside the row
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(wrow + e));
+  };
 
-  f32x4 acc[NT][MT];
+  // the first PD steps of W are on their way before anything else happens
+  bf16x8 ring[PD];
 #pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int b = 0; b < MT; ++b) acc[t][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int u = 0; u < PD; ++u)
+    if (u < n_steps) ring[u] = load_w(w_begin + u);
 
-  uint4 xs[kCPT];
-  bf16x8 wcur[KBS][NT], wnext[KBS][NT];
-
-  // Loads past K (the last round of a matrix whose K is no multiple of the round) read a clamped,
-  // valid address and are zeroed afterwards: the select is on the value, never on the address, so
-  // every load stays a plain global load.  K % 8 == 0: a chunk of 8 is inside or outside as a whole.
-  auto load_x = [&](int r) {  // global -> registers, round r of this split
-    const int k0 = (round0 + r) * kRoundK;
-    const bool whole = k0 + kRoundK <= K;
+  // X rows of the slice -> LDS, zeros past K; four 16-byte chunks a thread in flight
+  {
+    const int cpr = a.steps_per_split * 4;  // chunks of 8 elements per row
+    const int chunks = M * cpr;
+    const int k0 = s_begin * 32, k1 = min(s_end * 32, K);
+    for (int c0 = tid; c0 < chunks; c0 += 4 * kThreads) {
+      uint4 v[4];
+      int dst[4];
 #pragma unroll
-    for (int i = 0; i < kCPT; ++i) {
-      if (kChunks % kThreads != 0 && xdst[i] < 0) continue;
-      if (whole) {
-        xs[i] = *reinterpret_cast<const uint4*>(xsrc[i] + k0);
-      } else {
-        const bool in = k0 + xcol[i] < K;
-        const uint4 v = *reinterpret_cast<const uint4*>(xsrc[i] + (in ? k0 : 0) - (in ? 0 : xcol[i]));
-        xs[i] = uint4{in ? v.x : 0u, in ? v.y : 0u, in ? v.z : 0u, in ? v.w : 0u};
+      for (int i = 0; i < 4; ++i) {
+        const int c = c0 + i * kThreads;
+        const int row = min(c, chunks - 1) / cpr, col = (min(c, chunks - 1) % cpr) * 8;
+        const bool in = k0 + col < k1;
+        const uint4 raw = *reinterpret_cast<const uint4*>(a.x + static_cast<int64_t>(row) * a.ldx + (in ? k0 + col : 0));
+        v[i] = uint4{in ? raw.x : 0u, in ? raw.y : 0u, in ? raw.z : 0u, in ? raw.w : 0u};
+        dst[i] = c < chunks ? row * pitch + col : -1;
       }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (dst[i] >= 0) *reinterpret_cast<uint4*>(lds + dst[i]) = v[i];
     }
-  };
-  auto store_x = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < kCPT; ++i)
-      if (kChunks % kThreads == 0 || xdst[i] >= 0) *reinterpret_cast<uint4*>(lds + buf * (kRows * kPitch) + xdst[i]) = xs[i];
-  };
-  auto load_w = [&](int r, bf16x8 (&dst)[KBS][NT]) {
-    const int k0 = (round0 + r) * kRoundK + wk * (KBS * 32);
-    if (k0 + KBS * 32 <= K) {
-#pragma unroll
-      for (int u = 0; u < KBS; ++u)
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
-          dst[u][t] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(wp[t] + k0 + 32 * u));
-    } else {
-#pragma unroll
-      for (int u = 0; u < KBS; ++u) {
-        const int k = k0 + 32 * u;
-        const bool in = k + 8 * g < K;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          const uint4 v = *reinterpret_cast<const uint4*>(wp[t] + (in ? k : -8 * g));  // row start when outside
-          dst[u][t] = __builtin_bit_cast(bf16x8, uint4{in ? v.x : 0u, in ? v.y : 0u, in ? v.z : 0u, in ? v.w : 0u});
-        }
-      }
-    }
-  };
-
-  // One round: start the loads of the next round, multiply this round's W registers with X from LDS,
-  // park the next round's X in the other LDS buffer.  The two W register sets swap roles from round
-  // to round (the loop is unrolled by two), so the loads of round r + 1 stay in flight while round r
-  // is computed and nothing is copied.
-  auto round_body = [&](int r, bf16x8 (&cur)[KBS][NT], bf16x8 (&nxt)[KBS][NT]) {
-    const bool more = r + 1 < rounds;
-    if (more) {
-      load_x(r + 1);
-      load_w(r + 1, nxt);
-    }
-    const uint16_t* xb = lds + (r & 1) * (kRows * kPitch) + li * kPitch + wk * (KBS * 32) + 8 * g;
-#pragma unroll
-    for (int u = 0; u < KBS; ++u) {
-      bf16x8 xv[MT];
-#pragma unroll
-      for (int b = 0; b < MT; ++b)
-        xv[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(xb + b * 16 * kPitch + 32 * u));
-#pragma unroll
-      for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int b = 0; b < MT; ++b)
-          acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u][t], xv[b], acc[t][b], 0, 0, 0);
-    }
-    if (more) store_x((r + 1) & 1);
-    __syncthreads();
-  };
-
-  if (rounds > 0) {
-    load_x(0);
-    load_w(0, wcur);
-    store_x(0);
   }
   __syncthreads();
-  for (int r = 0; r < rounds; r += 2) {
-    round_body(r, wcur, wnext);
-    if (r + 1 < rounds) round_body(r + 1, wnext, wcur);
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int b = 0; b < MT; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const uint16_t* xrow[MT];  // lanes past the last row read the last row; their results are not stored
+#pragma unroll
+  for (int b = 0; b < MT; ++b) xrow[b] = lds + min(16 * b + li, M - 1) * pitch + (w_begin - s_begin) * 32 + 8 * g;
+  auto load_x = [&](int s, bf16x8 (&dst)[MT]) {
+#pragma unroll
+    for (int b = 0; b < MT; ++b) dst[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(xrow[b] + 32 * s));
+  };
+  bf16x8 xring[XD][MT];
+#pragma unroll
+  for (int u = 0; u < XD; ++u)
+    if (u < n_steps) load_x(u, xring[u]);
+
+  for (int base = 0; base < n_steps; base += PD) {
+#pragma unroll
+    for (int u = 0; u < PD; ++u) {
+      const int s = base + u;  // relative to w_begin
+      if (s < n_steps) {
+#pragma unroll
+        for (int b = 0; b < MT; ++b)
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
+        if (s + XD < n_steps) load_x(s + XD, xring[u % XD]);
+        if (s + PD < n_steps) ring[u] = load_w(w_begin + s + PD);
+      }
+    }
   }
 
   // add the WK partial sums of every column tile in the order wk = 0, 1, ...: waves wk > 0 park
-  // their registers in LDS (the X buffers are free after the last barrier), waves wk == 0 add
+  // their registers in LDS behind X, waves wk == 0 add
+  float* red = reinterpret_cast<float*>(lds + ((M * pitch + 7) / 8) * 8);  // [WK-1][WN][MT][64][4]
   if constexpr (WK > 1) {
-    float* red = reinterpret_cast<float*>(lds);  // [WK-1][WN][NT*MT][64][4]
     if (wk > 0) {
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int b = 0; b < MT; ++b)
-          *reinterpret_cast<f32x4*>(red + ((((wk - 1) * WN + wn) * (NT * MT) + t * MT + b) * 64 + lane) * 4) = acc[t][b];
+      for (int b = 0; b < MT; ++b)
+        *reinterpret_cast<f32x4*>(red + ((((wk - 1) * WN + wn) * MT + b) * 64 + lane) * 4) = acc[b];
     }
     __syncthreads();
     if (wk > 0) return;
 #pragma unroll
     for (int v = 1; v < WK; ++v)
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int b = 0; b < MT; ++b) {
-          const f32x4 p = *reinterpret_cast<const f32x4*>(red + ((((v - 1) * WN + wn) * (NT * MT) + t * MT + b) * 64 + lane) * 4);
-          acc[t][b][0] += p[0];
-          acc[t][b][1] += p[1];
-          acc[t][b][2] += p[2];
-          acc[t][b][3] += p[3];
-        }
+      for (int b = 0; b < MT; ++b) {
+        const f32x4 p = *reinterpret_cast<const f32x4*>(red + ((((v - 1) * WN + wn) * MT + b) * 64 + lane) * 4);
+        acc[b][0] += p[0];
+        acc[b][1] += p[1];
+        acc[b][2] += p[2];
+        acc[b][3] += p[3];
+      }
   }
 
-  // acc[t][b][r] = C[m = 16 b + li][n = n0 + 16 t + 4 g + r]
+  // acc[b][r] = C[m = 16 b + li][n = n0 + 4 g + r]
   TOut* out = static_cast<TOut*>(a.out) + static_cast<int64_t>(blockIdx.y) * a.split_stride;
   if constexpr (EPI == kEpiSiluMul) {
+    float* swap = red + (WK - 1) * WN * MT * 256;  // [WN/2][MT][64][4]: the up sums on their way to the gate wave
+    if (wn & 1) {
+#pragma unroll
+      for (int b = 0; b < MT; ++b) *reinterpret_cast<f32x4*>(swap + (((wn >> 1) * MT + b) * 64 + lane) * 4) = acc[b];
+    }
+    __syncthreads();  // the waves wk == 0, all that are left
+    if (wn & 1) return;
     const int c0 = (n0 / 2) + 4 * g;  // output column of register 0
 #pragma unroll
     for (int b = 0; b < MT; ++b) {
       const int mrow = 16 * b + li;
       if (mrow >= M) continue;
+      const f32x4 up = *reinterpret_cast<const f32x4*>(swap + (((wn >> 1) * MT + b) * 64 + lane) * 4);
       TOut* o = out + static_cast<int64_t>(mrow) * a.ldo + c0;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         if (n0 + 16 + 4 * g + r >= N) continue;
-        const float gate = acc[0][b][r], up = acc[1][b][r];
-        o[r] = from_float<TOut>(gate / (1.0f + expf(-gate)) * up);
+        const float gate = acc[b][r];
+        o[r] = from_float<TOut>(gate / (1.0f + expf(-gate)) * up[r]);
       }
     }
   } else {
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
+    for (int b = 0; b < MT; ++b) {
+      const int mrow = 16 * b + li;
+      if (mrow >= M) continue;
+      const int ncol = n0 + 4 * g;
+      TOut* o = out + static_cast<int64_t>(mrow) * a.ldo + ncol;
 #pragma unroll
-      for (int b = 0; b < MT; ++b) {
-        const int mrow = 16 * b + li;
-        if (mrow >= M) continue;
-        const int ncol = n0 + 16 * t + 4 * g;
-        TOut* o = out + static_cast<int64_t>(mrow) * a.ldo + ncol;
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (ncol + r < N) o[r] = from_float<TOut>(acc[t][b][r]);
-      }
-  }
-}
-
-template <int MT, int NT, int WN, int WK, int KBS>
-constexpr size_t rows_lds_bytes() {
-  const size_t x = 2ull * (MT * 16) * (WK * KBS * 32 + kPad) * sizeof(uint16_t);
-  const size_t red = WK > 1 ? static_cast<size_t>(WK - 1) * WN * NT * MT * 64 * 4 * sizeof(float) : 0;
-  return x > red ? x : red;
-}
-
-template <int MT, int NT, int WN, int WK, int KBS, int EPI, typename TOut>
-int launch_rows(const RowsArgs& a, int splits, hipStream_t s) {
-  constexpr size_t lds = rows_lds_bytes<MT, NT, WN, WK, KBS>();
-  auto kernel = gemm_rows_kernel<MT, NT, WN, WK, KBS, EPI, TOut>;
-  if (lds > 64 * 1024) {
-    static bool raised = false;  // per instantiation; the attribute belongs to the function, set once
-    if (!raised) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         static_cast<int>(lds));
-      if (e != hipSuccess) {
-        (void)hipGetLastError();  // do not leave the error behind for the next call to find
-        return static_cast<int>(e);
-      }
-      raised = true;
+      for (int r = 0; r < 4; ++r)
+        if (ncol + r < N) o[r] = from_float<TOut>(acc[b][r]);
     }
   }
-  const int col_groups = (a.N + WN * NT * 16 - 1) / (WN * NT * 16);
+}
+
+// LDS of a launch: the X rows of one k slice and, behind them, the partial sums of the waves wk > 0 and the
+// gate/up exchange.
+inline size_t rows_lds_bytes(int M, int steps_per_split, int mt, int wn, int wk) {
+  const size_t x = (static_cast<size_t>(M) * (steps_per_split * 32 + kPad) + 7) / 8 * 8 * sizeof(uint16_t);
+  const size_t red = static_cast<size_t>(wk - 1) * wn * mt * 64 * 4 * sizeof(float);
+  const size_t swap = static_cast<size_t>((wn + 1) / 2) * mt * 64 * 4 * sizeof(float);
+  return x + red + swap;
+}
+constexpr size_t kRowsLdsMax = 144 * 1024;  // of the 160 KB of a CU
+
+template <int MT, int WN, int WK, int PD, int XD, int EPI, typename TOut>
+int launch_rows(const RowsArgs& a, int splits, hipStream_t s) {
+  const size_t lds = rows_lds_bytes(a.M, a.steps_per_split, MT, WN, WK);
+  if (lds > kRowsLdsMax) return static_cast<int>(hipErrorInvalidValue);
+  auto kernel = gemm_rows_kernel<MT, WN, WK, PD, XD, EPI, TOut>;
+  static size_t allowed = 64 * 1024;  // per instantiation: what the function may use so far
+  if (lds > allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       static_cast<int>(kRowsLdsMax));
+    if (e != hipSuccess) {
+      (void)hipGetLastError();  // do not leave the error behind for the next call to find
+      return static_cast<int>(e);
+    }
+    allowed = kRowsLdsMax;
+  }
+  const int col_groups = (a.N + WN * 16 - 1) / (WN * 16);
   kernel<<<dim3(col_groups, splits), WN * WK * 64, lds, s>>>(a);
   return launch_status();
 }
 
-template <int MT, int NT, int WN, int WK, int KBS, int EPI>
+template <int MT, int WN, int WK, int PD, int XD, int EPI>
 int launch_rows_out(const RowsArgs& a, int splits, int out_dtype, hipStream_t s) {
-  if (out_dtype == kF32) return launch_rows<MT, NT, WN, WK, KBS, EPI, float>(a, splits, s);
-  return launch_rows<MT, NT, WN, WK, KBS, EPI, bf16>(a, splits, s);
+  if (out_dtype == kF32) return launch_rows<MT, WN, WK, PD, XD, EPI, float>(a, splits, s);
+  return launch_rows<MT, WN, WK, PD, XD, EPI, bf16>(a, splits, s);
 }
 
-template <int MT, int NT, int WN, int WK, int KBS>
+template <int MT, int WN, int WK, int PD>
 int dispatch_rows(const RowsArgs& a, int splits, int out_dtype, int epilogue, hipStream_t s) {
-  if constexpr (NT == 2) {
-    if (epilogue == kEpiSiluMul) return launch_rows_out<MT, NT, WN, WK, KBS, kEpiSiluMul>(a, splits, out_dtype, s);
+  constexpr int XD = MT == 1 ? 4 : 2;  // X steps read ahead from LDS (registers: XD * MT * 4)
+  if constexpr (WN % 2 == 0) {
+    if (epilogue == kEpiSiluMul) return launch_rows_out<MT, WN, WK, PD, XD, kEpiSiluMul>(a, splits, out_dtype, s);
   }
-  return launch_rows_out<MT, NT, WN, WK, KBS, kEpiNone>(a, splits, out_dtype, s);
+  return launch_rows_out<MT, WN, WK, PD, XD, kEpiNone>(a, splits, out_dtype, s);
 }
 
 }  // namespace arle
 
 using namespace arle;
 
-// Shapes of a workgroup, by `variant`: (NT, WN, WK, KBS), picked by the caller per matrix shape and row count
-// from measurements on MI355X:
-//   0  general product                      1  gate/up with the fused activation (two column tiles a wave)
-//   2  few output columns, long K           3  very many output columns (an output head)
-//   4  few output columns, short K
-#define ARLE_ROWS_VARIANTS(X) X(0, 1, 4, 2, 4) X(1, 2, 4, 2, 8) X(2, 1, 2, 4, 4) X(3, 2, 4, 2, 4) X(4, 1, 1, 2, 8)
+// Shapes of a workgroup, by `variant`: (WN, WK, PD), picked by the caller per matrix shape and row count
+// from measurements on MI355X.  The fused activation needs an even WN.
+//   0  general product               1  gate/up with the fused activation, up to 8 rows
+//   2  few output columns            3  more than 8 rows with the fused activation, or very many columns
+//   4  general, more columns a workgroup
+#define ARLE_ROWS_VARIANTS(X) X(0, 2, 2, 4) X(1, 2, 4, 4) X(2, 1, 4, 4) X(3, 8, 1, 4) X(4, 4, 1, 8)
 constexpr int kVariants = 5;
 
-// (k steps of 32 that one round covers) << 20 | (output columns of one workgroup) << 4 | (column tiles a wave);
-// -1 for an unknown variant
+// (waves that share the k slice) << 20 | (output columns of one workgroup) << 4 | (1 if the variant can apply
+// the fused activation); -1 for an unknown variant
 extern "C" int arle_gemm_rows_geometry(int variant) {
   switch (variant) {
-#define X(ID, NT, WN, WK, KBS) \
-  case ID:                     \
-    return ((WK * KBS) << 20) | ((WN * NT * 16) << 4) | NT;
+#define X(ID, WN, WK, PD) \
+  case ID:                \
+    return (WK << 20) | ((WN * 16) << 4) | (WN % 2 == 0 ? 1 : 0);
     ARLE_ROWS_VARIANTS(X)
 #undef X
     default:
@@ -309,33 +275,50 @@ extern "C" int arle_gemm_rows_geometry(int variant) {
   }
 }
 
+// Bytes of LDS that a launch of `variant` needs for M rows and k slices of steps_per_split steps; the launch
+// is refused above arle_gemm_rows_lds_max().
+extern "C" long long arle_gemm_rows_lds(int variant, int M, int steps_per_split) {
+  const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  switch (variant) {
+#define X(ID, WN, WK, PD) \
+  case ID:                \
+    return static_cast<long long>(rows_lds_bytes(M, steps_per_split, mt, WN, WK));
+    ARLE_ROWS_VARIANTS(X)
+#undef X
+    default:
+      return -1;
+  }
+}
+extern "C" long long arle_gemm_rows_lds_max() { return static_cast<long long>(kRowsLdsMax); }
+
 // x [M, K] and w [N, K] bfloat16 with row strides in elements (multiples of 8), 1 <= M <= 64, K % 8 == 0.
 // splits == 1: out [M, N] (or [M, N/2] with the fused activation) bfloat16 or float32.
 // splits  > 1: out [splits, M, N] float32 partial products, split_stride elements apart, no activation;
-//              split s covers rounds [s * rounds_per_split, (s + 1) * rounds_per_split) and none may be empty.
+//              split s covers steps [s * steps_per_split, (s + 1) * steps_per_split) and none may be empty.
 extern "C" int arle_gemm_rows(const void* x, long long ldx, const void* w, long long ldw, void* out, long long ldo,
                               long long split_stride, int out_dtype, int M, int N, int K, int epilogue, int variant,
-                              int splits, int rounds_per_split, void* stream) {
+                              int splits, int steps_per_split, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K % 8 != 0 || K <= 0 || ldx % 8 != 0 || ldw % 8 != 0 || splits < 1 || splits > 65535 ||
-      rounds_per_split < 1 || variant < 0 || variant >= kVariants)
+      steps_per_split < 1 || variant < 0 || variant >= kVariants)
     return static_cast<int>(hipErrorInvalidValue);
-  const int round_steps = arle_gemm_rows_geometry(variant) >> 20;
-  const int rounds_total = ((K + 31) / 32 + round_steps - 1) / round_steps;
-  if (static_cast<long long>(splits - 1) * rounds_per_split >= rounds_total) return static_cast<int>(hipErrorInvalidValue);
+  const int steps_total = (K + 31) / 32;
+  if (static_cast<long long>(splits - 1) * steps_per_split >= steps_total ||
+      static_cast<long long>(splits) * steps_per_split < steps_total)
+    return static_cast<int>(hipErrorInvalidValue);
   if (splits > 1 && (out_dtype != kF32 || epilogue != kEpiNone)) return static_cast<int>(hipErrorInvalidValue);
-  if (epilogue == kEpiSiluMul && (N % 32 != 0 || (arle_gemm_rows_geometry(variant) & 15) != 2))
+  if (epilogue == kEpiSiluMul && (N % 32 != 0 || (arle_gemm_rows_geometry(variant) & 15) != 1))
     return static_cast<int>(hipErrorInvalidValue);
   if (epilogue != kEpiNone && epilogue != kEpiSiluMul) return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const RowsArgs a{static_cast<const uint16_t*>(x), ldx, static_cast<const uint16_t*>(w), ldw, out, ldo, M, N, K,
-                   rounds_per_split, split_stride};
+                   steps_per_split, split_stride};
   switch (variant) {
-#define X(ID, NT, WN, WK, KBS)                                                                      \
-  case ID:                                                                                          \
-    if (M <= 16) return dispatch_rows<1, NT, WN, WK, KBS>(a, splits, out_dtype, epilogue, s);       \
-    if (M <= 32) return dispatch_rows<2, NT, WN, WK, KBS>(a, splits, out_dtype, epilogue, s);       \
-    return dispatch_rows<4, NT, WN, WK, KBS>(a, splits, out_dtype, epilogue, s);
+#define X(ID, WN, WK, PD)                                                                       \
+  case ID:                                                                                      \
+    if (M <= 16) return dispatch_rows<1, WN, WK, PD>(a, splits, out_dtype, epilogue, s);        \
+    if (M <= 32) return dispatch_rows<2, WN, WK, PD>(a, splits, out_dtype, epilogue, s);        \
+    return dispatch_rows<4, WN, WK, PD>(a, splits, out_dtype, epilogue, s);
     ARLE_ROWS_VARIANTS(X)
 #undef X
   }

@@ -7,6 +7,8 @@ live on the GPU.
 """
 from __future__ import annotations
 
+import ctypes
+import functools
 import math
 
 import torch
@@ -426,8 +428,9 @@ _ROWS_TARGET_WORKGROUPS = 640    # K is split until about this many workgroups s
 _ROWS_MAX_SPLITS = 8             # ... the consumer pays for every part of the stack
 _ROWS_PARTIAL_BYTES = 3 << 20    # ... and the float32 partial products stay below this
 _ROWS_WIDE_N = 32768             # from here on (an output head) N alone gives enough workgroups
-_ROWS_NARROW_N = 4096            # with more than 16 rows the kernel beats the library only up to here
-_V_GENERAL, _V_FUSED, _V_NARROW_LONG, _V_WIDE, _V_NARROW_SHORT = 0, 1, 2, 3, 4
+_ROWS_NARROW_N = 4096            # up to here N gives so few that one column tile a workgroup is best
+_ROWS_PREFERRED = 16             # with more rows the library is at least as fast on MI355X
+_V_GENERAL, _V_FUSED_FEW, _V_NARROW, _V_SHARED = 0, 1, 2, 3
 ROWS_VARIANTS = 5
 
 
@@ -435,41 +438,56 @@ def gemm_rows_supported(rows: int, k: int, x_stride: int) -> bool:
     return 0 < rows <= ROWS_KERNEL_MAX and k % 8 == 0 and x_stride % 8 == 0
 
 
+def _fused_variant(rows: int) -> int:
+    return _V_FUSED_FEW if rows <= 8 else _V_SHARED
+
+
 def gemm_rows_preferred(rows: int, n: int, k: int, x_stride: int, fused: bool = False) -> bool:
     """Whether the hand-written kernel, not the library, should run this product."""
-    if not gemm_rows_supported(rows, k, x_stride):
+    if not gemm_rows_supported(rows, k, x_stride) or rows > _ROWS_PREFERRED:
         return False
-    if rows <= 16:
-        return True
-    if fused:
-        return False
-    return n <= _ROWS_NARROW_N or (n >= _ROWS_WIDE_N and rows <= 32)
+    if fused:   # the activation needs whole sums: the rows of all of K in LDS at once
+        return _rows_min_splits(_fused_variant(rows), rows, k) == 1
+    return True
 
 
+@functools.lru_cache(maxsize=None)
 def _rows_geometry(variant: int):
-    """(k steps of 32 per round, output columns per workgroup, column tiles a wave) of a variant."""
+    """(waves that share a k slice, output columns per workgroup, can apply the fused activation) of a variant."""
     packed = lib.function("arle_gemm_rows_geometry")(variant)
     _need(packed > 0, f"gemm_rows has no variant {variant}")
     return packed >> 20, (packed >> 4) & 0xFFFF, packed & 15
 
 
+@functools.lru_cache(maxsize=4096)
+def _rows_min_splits(variant: int, M: int, K: int) -> int:
+    """Fewest k splits with which the X rows of one slice fit into LDS."""
+    fn = lib.function("arle_gemm_rows_lds")
+    fn.restype = ctypes.c_longlong
+    cap_fn = lib.function("arle_gemm_rows_lds_max")
+    cap_fn.restype = ctypes.c_longlong
+    cap, steps = cap_fn(), -(-K // 32)
+    splits = 1
+    while fn(variant, M, -(-steps // splits)) > cap:
+        splits += 1
+        _need(splits <= steps, f"gemm_rows: {M} rows of one k step do not fit into LDS")
+    return splits
+
+
+@functools.lru_cache(maxsize=4096)
 def gemm_rows_plan(M: int, N: int, K: int, fused: bool = False):
     """(variant, splits) for a product: small workgroups, K split across workgroups until enough of them
     stream W, within a budget for the stack of partial products that the consumer has to add."""
     if fused:
-        return _V_FUSED, 1
+        return _fused_variant(M), 1
     if N >= _ROWS_WIDE_N:
-        return _V_WIDE, 1
-    if M <= 16 and N <= _ROWS_NARROW_N:
-        variant = _V_NARROW_SHORT if K <= 4096 else _V_NARROW_LONG
+        variant, want = (_V_NARROW if M <= 4 else _V_SHARED), 1
     else:
-        variant = _V_GENERAL
-    round_steps, columns, _ = _rows_geometry(variant)
-    groups = -(-N // columns)
-    rounds = -(-(-(-K // 32)) // round_steps)
-    splits = min(-(-_ROWS_TARGET_WORKGROUPS // groups), _ROWS_MAX_SPLITS, rounds,
-                 max(1, _ROWS_PARTIAL_BYTES // (M * N * 4)))
-    return variant, max(1, splits)
+        variant = _V_NARROW if N <= _ROWS_NARROW_N else _V_GENERAL
+        _, columns, _ = _rows_geometry(variant)
+        groups = -(-N // columns)
+        want = min(-(-_ROWS_TARGET_WORKGROUPS // groups), _ROWS_MAX_SPLITS, max(1, _ROWS_PARTIAL_BYTES // (M * N * 4)))
+    return variant, max(want, _rows_min_splits(variant, M, K))
 
 
 def gemm_rows(x, w, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, variant: int | None = None,
@@ -498,15 +516,16 @@ def gemm_rows(x, w, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, varia
         plan = gemm_rows_plan(M, N, K, fused)
         variant = plan[0] if variant is None else variant
         splits = plan[1] if splits is None else splits
+    _, _, can_fuse = _rows_geometry(variant)
+    steps = -(-K // 32)
+    per_split = -(-steps // max(1, min(splits, steps)))
+    splits = -(-steps // per_split)
     if fused:
         _need(N % 32 == 0, "the fused activation needs gate/up interleaved in blocks of 16")
-    round_steps, _, tiles = _rows_geometry(variant)
-    if fused:
-        _need(tiles == 2 and splits == 1,
-              "the fused activation needs a variant with two column tiles a wave, and whole sums")
-    rounds_total = -(-(-(-K // 32)) // round_steps)
-    per_split = -(-rounds_total // max(1, min(splits, rounds_total)))
-    splits = -(-rounds_total // per_split)
+        _need(can_fuse == 1 and splits == 1,
+              "the fused activation needs a variant with an even number of column tiles, and whole sums")
+    _need(splits >= _rows_min_splits(variant, M, K),
+          f"gemm_rows: {M} rows of {per_split * 32} columns do not fit into LDS; split K further")
     if splits > 1:
         out = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
         ldo, stride, code = N, M * N, F32

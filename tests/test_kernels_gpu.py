@@ -485,7 +485,10 @@ def test_gemm_rows_with_fused_activation(M, inter, K):
     up = (torch.randn(inter, K, generator=_g(112)) * 0.1).bfloat16()
     fused = torch.stack([gate.view(-1, 16, K), up.view(-1, 16, K)], dim=1).reshape(2 * inter, K).contiguous()
     want = plain.silu(x.double() @ gate.double().T) * (x.double() @ up.double().T)
-    for variant in (None, 1, 3):
+    for variant in (None, 0, 1, 3, 4):
+        planned = ops.gemm_rows_plan(M, 2 * inter, K, True)[0] if variant is None else variant
+        if ops._rows_min_splits(planned, M, K) > 1:
+            continue      # these rows of all of K do not fit into LDS: no whole sums, no fused activation
         got = ops.gemm_rows(x.to(DEV), fused.to(DEV), torch.float32, ops.EPI_SILU_MUL, variant=variant, splits=1).cpu()
         assert got.shape == (M, inter) and _rel(got, want) < 1e-5
     # the same weights through the library product and the interleaved activation kernel
@@ -526,10 +529,13 @@ def test_gemm_rows_refuses_what_it_cannot_take():
                       torch.zeros(4, 20, dtype=torch.bfloat16, device=DEV))
     with pytest.raises(ops.ShapeError, match="no variant"):
         ops.gemm_rows(x[:4], w, variant=99, splits=1)
-    with pytest.raises(ops.ShapeError, match="two column tiles"):
-        ops.gemm_rows(x[:4], w, epilogue=ops.EPI_SILU_MUL, variant=0, splits=1)
+    with pytest.raises(ops.ShapeError, match="even number of column tiles"):
+        ops.gemm_rows(x[:4], w, epilogue=ops.EPI_SILU_MUL, variant=2, splits=1)
     with pytest.raises(ops.ShapeError, match="whole sums"):
         ops.gemm_rows(x[:4], w, epilogue=ops.EPI_SILU_MUL, variant=1, splits=2)
+    with pytest.raises(ops.ShapeError, match="do not fit into LDS"):
+        ops.gemm_rows(torch.zeros(64, 9728, dtype=torch.bfloat16, device=DEV),
+                      torch.zeros(32, 9728, dtype=torch.bfloat16, device=DEV), variant=0, splits=2)
     # the general entry point still serves such shapes, through the library
     out = ops.gemm_bf16(torch.ones(2, 20, dtype=torch.bfloat16, device=DEV), torch.ones(4, 20, dtype=torch.bfloat16, device=DEV))
     assert out.shape == (2, 4) and float(out[0, 0]) == 20.0
