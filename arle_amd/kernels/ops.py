@@ -306,7 +306,7 @@ def attn_paged_simt(q, out, k_pages, v_pages, block_table, positions, slot_of_to
 
 
 MFMA_MAX_HEAD_DIM = 256
-_MFMA_TARGET_WAVES = 4096   # waves wanted in flight for a decode launch (256 CUs x 16)
+_MFMA_TARGET_WAVES = 2048   # workgroups wanted for a decode launch (measured: 8 per CU of an MI355X)
 
 
 def attn_mfma_supported(dtype, head_dim: int, page_size: int) -> bool:

@@ -119,6 +119,54 @@ def test_attention_part_over_its_cache(dtype, tol, window):
     assert _rel(got, plain.linear(att.reshape(T, -1), wd["o"])) < tol
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 5e-6), (torch.bfloat16, 2e-2)])
+def test_block_part_alone_equals_a_plain_decoder_layer(dtype, tol):
+    """One pre-norm block built from the recipe of a tiny configuration: residual and pending delta in,
+    residual and pending delta out, over a portion of 20 rows, a single row and a portion of 6."""
+    from arle_amd.config import Qwen3Config
+    from arle_amd.models.qwen3 import qwen3_spec
+    from arle_amd.parts import lookup as lookup_part
+    from tiny import TINY_C
+
+    cfg = dict(TINY_C, num_hidden_layers=1)
+    layer = qwen3_spec(Qwen3Config.from_dict(cfg)).layers[0]
+    names = {**layer.mixer.weights, **layer.feed_forward.weights, "n1": layer.norms["mixer_in"].weights["weight"],
+             "n2": layer.norms["ffn_in"].weights["weight"]}
+    H, nq, nkv, D, I = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["intermediate_size"]
+    shapes = {names["q"]: (nq * D, H), names["k"]: (nkv * D, H), names["v"]: (nkv * D, H), names["o"]: (H, nq * D),
+              names["q_norm"]: (D,), names["k_norm"]: (D,), names["gate"]: (I, H), names["up"]: (I, H),
+              names["down"]: (H, I), names["n1"]: (H,), names["n2"]: (H,)}
+    w = _tensors(shapes, dtype, seed=9, scale=0.1)
+    fetch = lambda n: w[n].to(DEV)
+    rt = _rt(dtype)
+    mixer = build_part("mixer", layer.mixer, fetch, rt)
+    ffn = build_part("feed_forward", layer.feed_forward, fetch, rt)
+    norms = {role: build_part("norm", spec, fetch, rt) for role, spec in layer.norms.items()}
+    block = lookup_part("block", layer.block)(mixer, ffn, norms)
+    cache = CacheManager([mixer.cache_need()], page_size=16, num_pages=8, max_slots=2, max_request_tokens=64,
+                         device=DEV, dtype=dtype)
+    T = 27
+    h0 = torch.randn(T, H)
+    pending = (torch.randn(T, H) * 0.3).to(dtype)     # what the block before this one has not added yet
+    cache.admit("r")
+    out_rows = []
+    for lo, hi in ((0, 20), (20, 21), (21, 27)):
+        batch = build_step_batch([StepEntry("r", [0] * (hi - lo), [])], cache.slot_of.__getitem__, cache.length, 10, DEV)
+        cache.append([("r", hi - lo)])
+        cache.sync_tables()
+        residual, delta = block.forward(h0[lo:hi].clone().to(DEV), pending[lo:hi].to(DEV), batch, cache.view(0))
+        out_rows.append(residual.double().cpu() + _delta(delta).double().cpu())
+    got = torch.cat(out_rows)
+    wd = {k: v.double() for k, v in w.items()}
+    qw = {"model.layers.0." + k: wd[v] for k, v in (("self_attn.q_proj.weight", names["q"]), ("self_attn.k_proj.weight", names["k"]),
+          ("self_attn.v_proj.weight", names["v"]), ("self_attn.o_proj.weight", names["o"]), ("self_attn.q_norm.weight", names["q_norm"]),
+          ("self_attn.k_norm.weight", names["k_norm"]), ("mlp.gate_proj.weight", names["gate"]), ("mlp.up_proj.weight", names["up"]),
+          ("mlp.down_proj.weight", names["down"]), ("input_layernorm.weight", names["n1"]),
+          ("post_attention_layernorm.weight", names["n2"]))}
+    want = plain.decoder_layer(h0.double() + pending.double(), qw, 0, cfg, list(range(T)))
+    assert _rel(got, want) < tol
+
+
 def test_unknown_part_and_bad_head_dim_are_refused():
     with pytest.raises(KeyError, match="no mixer part named 'nope'"):
         lookup("mixer", "nope")

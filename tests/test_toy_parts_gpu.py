@@ -1,0 +1,261 @@
+"""Toy parts of every other role, defined here and registered without touching the framework:
+a feed-forward with routing (top-1 of a few experts), a position encoding the fused kernels do not
+know (adjacent-pair rotation with a learned angle table), a norm with a bias, and a block that runs
+mixer and feed-forward side by side.  Built from torch operations: they show the interfaces, they
+are nobody's model.  The attention layers around them are the stock part, so this also drives its
+path for position encodings that are applied between the norm and the cache write."""
+from dataclasses import asdict, dataclass
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import replay
+from arle_amd.config import register_architecture
+from arle_amd.engine import Engine
+from arle_amd.parts import LayerSpec, ModelSpec, Part, PartSpec, ScheduleEntry, WeightDecl, register
+from arle_amd.weights import write_random_model
+from tiny import random_tokens, read_folder
+
+pytestmark = pytest.mark.gpu
+
+
+def _whole(delta):
+    """A delta as one tensor: stock parts may hand over a stack of partial sums."""
+    return delta.float().sum(0) if delta.dim() == 3 else delta.float()
+
+
+@register("norm", "toy_biased")
+class BiasedNorm(Part):
+    """(x - mean) / sqrt(var + eps) * w + b."""
+
+    @classmethod
+    def declare_weights(cls, params):
+        return {"weight": WeightDecl((params["width"],), init="ones"), "bias": WeightDecl((params["width"],))}
+
+    def __init__(self, params, tensors, rt, children=None):
+        super().__init__(params, tensors, rt, children)
+        self.w, self.b, self.eps = tensors["weight"].float(), tensors["bias"].float(), float(params["eps"])
+
+    def forward(self, x, rows=None):
+        x = x.float() if rows is None else x.float()[rows.long()]
+        mu = x.mean(-1, keepdim=True)
+        var = (x - mu).pow(2).mean(-1, keepdim=True)
+        return ((x - mu) / torch.sqrt(var + self.eps) * self.w + self.b).to(self.rt.act_dtype)
+
+    def add_norm(self, residual, delta, rows=None):
+        if delta is not None:
+            if rows is None:
+                residual += _whole(delta)
+            else:
+                return self.forward(residual + _whole(delta), rows)
+        return self.forward(residual, rows)
+
+
+@register("position", "toy_pairs")
+class PairRotation(Part):
+    """Rotates the adjacent pairs (2i, 2i+1) of every head by angle[position, i], a learned table."""
+
+    fusable = False
+
+    @classmethod
+    def declare_weights(cls, params):
+        return {"angle": WeightDecl((params["max_positions"], params["head_dim"] // 2))}
+
+    def __init__(self, params, tensors, rt, children=None):
+        super().__init__(params, tensors, rt, children)
+        self.angle, self.D = tensors["angle"].float(), int(params["head_dim"])
+
+    def ensure_positions(self, n):
+        assert n <= self.angle.shape[0], "the learned table is as long as it is"
+
+    def fused_rotary(self):
+        return None, None, 0
+
+    def apply(self, q, k, positions, num_q_heads, num_kv_heads):
+        a = self.angle[positions.long()]                     # [T, D/2]
+        cos, sin = a.cos()[:, None, :], a.sin()[:, None, :]
+        for x, heads in ((q, num_q_heads), (k, num_kv_heads)):
+            if heads == 0:
+                continue
+            v = x.float().reshape(x.shape[0], heads, self.D // 2, 2)
+            even, odd = v[..., 0], v[..., 1]
+            out = torch.stack([even * cos - odd * sin, even * sin + odd * cos], dim=-1)
+            x.copy_(out.reshape(x.shape[0], heads * self.D).to(x.dtype))
+
+
+@register("feed_forward", "toy_routed")
+class RoutedFFN(Part):
+    """Every row goes to the one expert with the largest router logit: relu(x W1_e^T) W2_e^T, scaled by the
+    softmax weight of that expert.  Router logits and softmax in float32."""
+
+    @classmethod
+    def declare_weights(cls, params):
+        e, h, i = params["experts"], params["hidden_size"], params["intermediate_size"]
+        return {"router": WeightDecl((e, h)), "w1": WeightDecl((e * i, h)), "w2": WeightDecl((e * h, i))}
+
+    def __init__(self, params, tensors, rt, children=None):
+        super().__init__(params, tensors, rt, children)
+        e, h, i = params["experts"], params["hidden_size"], params["intermediate_size"]
+        self.router = tensors["router"].float()
+        self.w1, self.w2 = tensors["w1"].float().reshape(e, i, h), tensors["w2"].float().reshape(e, h, i)
+
+    def forward(self, x):
+        xf = x.float()
+        probs = torch.softmax(xf @ self.router.T, dim=-1)
+        weight, expert = probs.max(dim=-1)
+        hidden = torch.relu(torch.einsum("th,tih->ti", xf, self.w1[expert]))
+        return (torch.einsum("ti,thi->th", hidden, self.w2[expert]) * weight[:, None]).to(x.dtype)
+
+
+@register("block", "toy_parallel")
+class ParallelBlock:
+    """h += mixer(norm(h)) + feed_forward(norm(h)): one norm, both branches read it."""
+
+    norm_roles = ("in",)
+
+    def __init__(self, mixer, feed_forward, norms):
+        self.mixer, self.feed_forward, self.norm = mixer, feed_forward, norms["in"]
+
+    def forward(self, residual, delta, batch, cache_view):
+        a = self.norm.add_norm(residual, delta)
+        m = _whole(self.mixer.forward(a, batch, cache_view))
+        f = _whole(self.feed_forward.forward(a))
+        return residual, m + f
+
+
+@dataclass(frozen=True)
+class ToyPartsConfig:
+    hidden_size: int
+    intermediate_size: int
+    experts: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    vocab_size: int
+    eps: float
+    layers: int
+    max_position_embeddings: int = 128
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(**{k: raw[k] for k in cls.__dataclass_fields__})
+
+    def to_dict(self):
+        return dict(asdict(self), architectures=["ToyPartsLM"])
+
+
+def toy_parts_spec(c: ToyPartsConfig, stop_token_ids=()):
+    def norm(name):
+        return PartSpec("toy_biased", {"width": c.hidden_size, "eps": c.eps}, {"weight": name + ".w", "bias": name + ".b"})
+
+    layers = []
+    for i in range(c.layers):
+        p = f"l{i}."
+        pos = PartSpec("toy_pairs", {"head_dim": c.head_dim, "max_positions": c.max_position_embeddings},
+                       {"angle": p + "angle"})
+        mixer = PartSpec("paged_attention",
+                         {"hidden_size": c.hidden_size, "num_q_heads": c.heads, "num_kv_heads": c.kv_heads,
+                          "head_dim": c.head_dim, "qk_norm": i % 2 == 0, "eps": c.eps, "position": pos, "window": None},
+                         dict({"q": p + "q", "k": p + "k", "v": p + "v", "o": p + "o"},
+                              **({"q_norm": p + "qn", "k_norm": p + "kn"} if i % 2 == 0 else {})))
+        ffn = PartSpec("toy_routed", {"hidden_size": c.hidden_size, "intermediate_size": c.intermediate_size,
+                                      "experts": c.experts}, {"router": p + "router", "w1": p + "w1", "w2": p + "w2"})
+        layers.append(LayerSpec("toy_parallel", mixer, ffn, {"in": norm(p + "n")}))
+    sizes = {"vocab_size": c.vocab_size, "hidden_size": c.hidden_size}
+    # the last entry runs layer 0 again on the cache that its first run wrote (only q is projected there)
+    schedule = [ScheduleEntry(i) for i in range(c.layers)] + [ScheduleEntry(0, cache_from=0)]
+    return ModelSpec(hidden_size=c.hidden_size, vocab_size=c.vocab_size, max_positions=c.max_position_embeddings,
+                     embedding=PartSpec("token_table", sizes, {"table": "embed"}), layers=layers, schedule=schedule,
+                     final_norm=norm("final"), head=PartSpec("linear", sizes, {"weight": "head"}),
+                     stop_token_ids=tuple(stop_token_ids))
+
+
+register_architecture("ToyPartsLM", ToyPartsConfig, toy_parts_spec)
+
+TOY = ToyPartsConfig(hidden_size=40, intermediate_size=24, experts=3, heads=3, kv_heads=1, head_dim=16,
+                     vocab_size=90, eps=1e-5, layers=2)
+
+
+def _biased_norm(x, w, b, eps):
+    mu = x.mean(-1, keepdim=True)
+    return (x - mu) / torch.sqrt((x - mu).pow(2).mean(-1, keepdim=True) + eps) * w + b
+
+
+def _pair_rotate(x, angle):
+    """x [T, heads, D], angle [T, D/2]."""
+    T, H, D = x.shape
+    v = x.reshape(T, H, D // 2, 2)
+    c, s = angle.cos()[:, None, :], angle.sin()[:, None, :]
+    return torch.stack([v[..., 0] * c - v[..., 1] * s, v[..., 0] * s + v[..., 1] * c], dim=-1).reshape(T, H, D)
+
+
+def toy_parts_plain_logits(c: ToyPartsConfig, w, tokens):
+    w = {k: v.double() for k, v in w.items()}
+    T = len(tokens)
+    h = plain.embedding(w["embed"], tokens)
+    kv0 = None
+    for entry, layer in enumerate(list(range(c.layers)) + [0]):
+        p = f"l{layer}."
+        a = _biased_norm(h, w[p + "n.w"], w[p + "n.b"], c.eps)
+        angle = w[p + "angle"][:T]
+        q = plain.linear(a, w[p + "q"]).reshape(T, c.heads, c.head_dim)
+        if layer % 2 == 0:
+            q = plain.qk_norm(q, w[p + "qn"], c.eps)
+        q = _pair_rotate(q, angle)
+        if entry < c.layers:
+            k = plain.linear(a, w[p + "k"]).reshape(T, c.kv_heads, c.head_dim)
+            if layer % 2 == 0:
+                k = plain.qk_norm(k, w[p + "kn"], c.eps)
+            k = _pair_rotate(k, angle)
+            v = plain.linear(a, w[p + "v"]).reshape(T, c.kv_heads, c.head_dim)
+            if layer == 0:
+                kv0 = (k, v)
+        else:
+            k, v = kv0
+        m = plain.linear(plain.causal_attention(q, k, v, c.kv_heads).reshape(T, -1), w[p + "o"])
+        probs = torch.softmax(a @ w[p + "router"].T, dim=-1)
+        weight, expert = probs.max(dim=-1)
+        w1 = w[p + "w1"].reshape(c.experts, c.intermediate_size, c.hidden_size)
+        w2 = w[p + "w2"].reshape(c.experts, c.hidden_size, c.intermediate_size)
+        f = torch.stack([w2[e] @ torch.relu(w1[e] @ a[t]) * weight[t] for t, e in enumerate(expert.tolist())])
+        h = h + m + f
+    return plain.linear(_biased_norm(h, w["final.w"], w["final.b"], c.eps), w["head"])
+
+
+@pytest.fixture(scope="module")
+def folder(tmp_path_factory):
+    d = str(tmp_path_factory.mktemp("toyparts") / "toy")
+    write_random_model(d, "ToyPartsLM", TOY, seed=5, std=0.15, norm_std=0.05)
+    return d
+
+
+def test_toy_parts_are_built_and_stepped(folder):
+    """float32: the routed feed-forward switches experts on tiny differences, so only the 32-bit path is
+    compared row by row."""
+    _, weights = read_folder(folder)
+    eng = Engine.from_folder(folder, dtype="float32", page_size=4, max_tokens=4 * 64, max_slots=4)
+    reqs = {f"t{i}": random_tokens(n, TOY.vocab_size, 70 + i) for i, n in enumerate([23, 40, 9, 31])}
+    got = replay.run_steps(eng, replay.mixed(reqs, max_live=3, seed=4))
+    for rid, toks in reqs.items():
+        ref = toy_parts_plain_logits(TOY, weights, toks)
+        for pos in range(len(toks)):
+            err = float((got[(rid, pos)].double() - ref[pos]).abs().max() / ref.abs().max())
+            assert err <= 2e-5, f"request {rid} position {pos}: {err:.3e}"
+    assert all(f == g.pool.num_pages for f, g in zip(eng.cache.free_pages(), eng.cache.groups))
+
+
+def test_toy_parts_run_in_bfloat16_too(folder):
+    """The stock attention, cache and kernels under the toy parts in bfloat16: finite logits of the right shape,
+    equal however the prompt is cut wherever the routing is the same (rounding may flip an expert, so rows are
+    compared by their best token against the float32 engine, with most of them required to agree)."""
+    toks = random_tokens(36, TOY.vocab_size, 91)
+    outs = {}
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine.from_folder(folder, dtype=dtype, page_size=4, max_tokens=64, max_slots=2)
+        got = replay.run_steps(eng, replay.portions("x", toks, sizes=(5, 1, 9, 2)))
+        rows = torch.stack([got[("x", p)] for p in range(len(toks))])
+        assert torch.isfinite(rows).all() and rows.shape == (len(toks), TOY.vocab_size)
+        outs[dtype] = rows
+    agree = (outs["float32"].argmax(-1) == outs["bfloat16"].argmax(-1)).float().mean()
+    assert float(agree) >= 0.8
