@@ -13,6 +13,8 @@ from dataclasses import dataclass, field
 import numpy as np
 import torch
 
+from ..cache import native
+
 
 @dataclass
 class StepEntry:
@@ -63,42 +65,55 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device, into=
     if not entries:
         raise ValueError("a step needs at least one entry")
     seen = set()
-    segments, ids, pos, slots, want_rows = [], [], [], [], []
-    row = 0
+    segments, row = [], 0
     for e in entries:
         if e.request in seen:
             raise ValueError(f"request {e.request!r} appears twice in one step")
         seen.add(e.request)
-        n = len(e.tokens)
-        if n == 0:
+        if len(e.tokens) == 0:
             raise ValueError(f"request {e.request!r} brings no tokens")
-        slot, start = slot_of(e.request), length_of(e.request)
-        for t in e.tokens:
-            if not 0 <= int(t) < vocab_size:
-                raise ValueError(f"token id {t} of request {e.request!r} is outside the vocabulary "
-                                 f"(size {vocab_size})")
-        for w in e.want:
-            if not 0 <= int(w) < n:
-                raise ValueError(f"wanted place {w} of request {e.request!r} is outside its {n} tokens")
-            want_rows.append(row + int(w))
-        segments.append(Segment(e.request, slot, start, n, row))
-        ids.extend(int(t) for t in e.tokens)
-        pos.extend(range(start, start + n))
-        slots.extend([slot] * n)
-        row += n
-    host = {
-        "token_ids": np.asarray(ids, dtype=np.int32),
-        "positions": np.asarray(pos, dtype=np.int32),
-        "slot_of_token": np.asarray(slots, dtype=np.int32),
-        "want_rows": np.asarray(want_rows, dtype=np.int32),
-        "seg_row0": np.asarray([s.row0 for s in segments] + [row], dtype=np.int32),
-        "seg_slot": np.asarray([s.slot for s in segments], dtype=np.int32),
-        "seg_start": np.asarray([s.start for s in segments], dtype=np.int32),
-    }
+        segments.append(Segment(e.request, slot_of(e.request), length_of(e.request), len(e.tokens), row))
+        row += len(e.tokens)
+    # the arrays themselves are laid out by the native runtime core, which also checks ids and places;
+    # its inputs go over in one int32 array: slots, starts, token counts, want counts, tokens, wants
+    S = len(segments)
+    staged = [s.slot for s in segments]
+    staged += [s.start for s in segments]
+    staged += [s.length for s in segments]
+    staged += [len(e.want) for e in entries]
+    for e in entries:
+        staged += e.tokens
+    for e in entries:
+        staged += e.want
+    wide = np.array(staged, dtype=np.int64)
+    np.clip(wide, -1, 2**31 - 1, out=wide)     # what is out of range stays out of range
+    inputs = wide.astype(np.int32)
+    num_wanted = inputs.size - 4 * S - row
+    base = inputs.ctypes.data
+    at = lambda elements: base + 4 * elements
+    slot_p, start_p, ntok_p, nwant_p, tokens_p, wants_p = at(0), at(S), at(2 * S), at(3 * S), at(4 * S), at(4 * S + row)
+    flat_np = np.empty(packed_size(row, S, num_wanted), dtype=np.int32)
+    meta, where = native.int_array(5), native.int_array(2)
+    code = native.lib().arle_pack_step(S, slot_p, start_p, ntok_p, tokens_p, nwant_p, wants_p, int(vocab_size),
+                                       flat_np.ctypes.data, flat_np.size, meta, where)
+    if code == 1:
+        e = entries[where[0]]
+        bad = next(t for t in e.tokens if not 0 <= int(t) < vocab_size)
+        raise ValueError(f"token id {bad} of request {e.request!r} is outside the vocabulary (size {vocab_size})")
+    if code == 2:
+        e = entries[where[0]]
+        bad = next(w for w in e.want if not 0 <= int(w) < len(e.tokens))
+        raise ValueError(f"wanted place {bad} of request {e.request!r} is outside its {len(e.tokens)} tokens")
+    if code != 0:
+        raise ValueError(f"the step could not be packed (code {code})")
+    sizes = [row, row, row, num_wanted, S + 1, S, S]
+    order = ["token_ids", "positions", "slot_of_token", "want_rows", "seg_row0", "seg_slot", "seg_start"]
+    host, off = {}, 0
+    for k, n in zip(order, sizes):
+        host[k] = flat_np[off:off + n]
+        off += n
     # one host->device copy for all arrays
-    order = list(host)
-    sizes = [host[k].size for k in order]
-    flat = torch.from_numpy(np.concatenate([host[k] for k in order]))
+    flat = torch.from_numpy(flat_np)
     if into is None:
         packed = flat.to(device, non_blocking=False)
     else:
@@ -110,6 +125,5 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device, into=
     for k, n in zip(order, sizes):
         dev[k] = packed[off:off + n]
         off += n
-    return StepBatch(num_tokens=row, segments=segments, max_position=max(pos),
-                     max_qlen=max(s.length for s in segments), min_qlen=min(s.length for s in segments),
+    return StepBatch(num_tokens=row, segments=segments, max_position=meta[2], max_qlen=meta[3], min_qlen=meta[4],
                      host=host, **dev)

@@ -134,9 +134,15 @@ class Engine:
         if not decode_only:
             batch = build_step_batch(entries, self.cache.slot_of.__getitem__, self.cache.length,
                                      self.spec.vocab_size, self.device)
-        else:   # check the entries before anything is changed
-            build_step_batch(entries, self.cache.slot_of.__getitem__, self.cache.length,
-                             self.spec.vocab_size, "cpu")
+        else:   # the packing inside the captured path checks the token ids; on an error the lengths are rolled back
+            if len({e.request for e in entries}) != len(entries):
+                raise ValueError("a request appears twice in one step")
+            for e in entries:
+                if any(int(w) != 0 for w in e.want):
+                    raise ValueError(f"wanted place outside the one token of request {e.request!r}")
+                if not 0 <= int(e.tokens[0]) < self.spec.vocab_size:
+                    raise ValueError(f"token id {e.tokens[0]} of request {e.request!r} is outside the vocabulary "
+                                     f"(size {self.spec.vocab_size})")
         self.cache.append([(e.request, len(e.tokens)) for e in entries])
         try:
             self.cache.sync_tables()

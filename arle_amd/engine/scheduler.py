@@ -31,10 +31,13 @@ runs two forwards, `Split`).
 """
 from __future__ import annotations
 
+import ctypes
+
 import time
 from collections import deque
 from dataclasses import dataclass, field
 
+from ..cache import native
 from ..cache.pages import OutOfPages
 from ..sampling.params import SamplingParams
 from .batch import StepEntry
@@ -107,8 +110,12 @@ class StepPlan:
 
 
 def retract_victim(decoding: list):
-    """Fewest generated tokens first; ties: the longest prompt (decode.rs:16-21)."""
-    return min(decoding, key=lambda r: (len(r.generated), -len(r.prompt)))
+    """Fewest generated tokens first; ties: the longest prompt (decode.rs:16-21).  Decided by the native
+    runtime core."""
+    n = len(decoding)
+    generated = (ctypes.c_int * n)(*[len(r.generated) for r in decoding])
+    prompts = (ctypes.c_int * n)(*[len(r.prompt) for r in decoding])
+    return decoding[native.lib().arle_retract_victim(n, generated, prompts)]
 
 
 def plan_prefill(queue, decode_rows: int, cfg: SchedulerConfig, fits) -> list:

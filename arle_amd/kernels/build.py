@@ -1,4 +1,5 @@
-"""Compile the HIP sources under `arle_amd/csrc` into shared libraries for gfx950.
+"""Compile the HIP sources under `arle_amd/csrc` into shared libraries for gfx950, and the
+host-side C++ runtime core (`csrc/host/`, no GPU code) with the host compiler.
 
 One library per source file, built with plain `hipcc` (no torch headers, so a
 file compiles in seconds).  Libraries live in `arle_amd/_lib/`, or in a per-user
@@ -31,8 +32,11 @@ SOURCES = {
     "attention_simt": "attention_simt.hip",
     "attention_mfma": "attention_mfma.hip",
     "sampling": "sampling.hip",
+    "host": "host/runtime.cpp",
 }
 HEADERS = ("common.h",)
+HOST_LIBS = ("host",)   # plain C++: page pool, block tables, step packing
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared"]
 
 HIPCC_FLAGS = [
     f"--offload-arch={OFFLOAD_ARCH}",
@@ -104,12 +108,20 @@ def existing_lib(name: str) -> str | None:
     return None
 
 
+def find_host_compiler() -> str:
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++")):
+        if cand and (os.path.exists(cand) or shutil.which(cand)):
+            return cand
+    return find_hipcc()   # hipcc compiles plain C++ too
+
+
 def source_hash(name: str) -> str:
     h = hashlib.sha256()
-    for fname in (SOURCES[name], *HEADERS):
+    host = name in HOST_LIBS
+    for fname in ((SOURCES[name],) if host else (SOURCES[name], *HEADERS)):
         with open(os.path.join(CSRC_DIR, fname), "rb") as fh:
             h.update(fh.read())
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(HOST_FLAGS if host else HIPCC_FLAGS).encode())
     return h.hexdigest()
 
 
@@ -129,8 +141,12 @@ def build(name: str) -> str:
     out_dir = lib_dir()
     out = os.path.join(out_dir, f"libarle_{name}.so")
     tmp = f"{out}.tmp{os.getpid()}"
-    cmd = [find_hipcc(), *HIPCC_FLAGS, f"-I{CSRC_DIR}", src, "-o", tmp]
-    _say(f"compiling {SOURCES[name]} for {OFFLOAD_ARCH} ...")
+    if name in HOST_LIBS:
+        cmd = [find_host_compiler(), *HOST_FLAGS, src, "-o", tmp]
+        _say(f"compiling {SOURCES[name]} for the host ...")
+    else:
+        cmd = [find_hipcc(), *HIPCC_FLAGS, f"-I{CSRC_DIR}", src, "-o", tmp]
+        _say(f"compiling {SOURCES[name]} for {OFFLOAD_ARCH} ...")
     t0 = time.time()
     env = dict(os.environ)
     env.setdefault("TMPDIR", tempfile.gettempdir())
@@ -152,7 +168,7 @@ def build(name: str) -> str:
     if proc.returncode != 0:
         if os.path.exists(tmp):
             os.remove(tmp)
-        raise BuildError(f"hipcc failed on {SOURCES[name]} (exit {proc.returncode}):\n{output}")
+        raise BuildError(f"{os.path.basename(cmd[0])} failed on {SOURCES[name]} (exit {proc.returncode}):\n{output}")
     os.replace(tmp, out)
     with open(out + ".srchash", "w") as fh:
         fh.write(source_hash(name))
