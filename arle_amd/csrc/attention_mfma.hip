@@ -34,6 +34,8 @@ namespace arle {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 struct AttnArgs {
   const uint16_t* q;
@@ -383,42 +385,66 @@ __global__ __launch_bounds__(kMergeWaves* kWave) void attn_merge_kernel(
 // ---------------------------------------------------------------------------------------------
 // Prompt portions: the same products, with keys and values staged through LDS.
 //
-// A workgroup of four waves owns 128 rows (32 per wave, two row tiles) of one segment and kv head
+// A workgroup of eight waves owns 128 rows (16 per wave) of one segment and kv head
 // and walks the keys in tiles of 64.  All 256 threads fetch a tile with coalesced loads (a key page
 // [slot][d] and a value page [d][slot] are contiguous in memory), park it in LDS, and every wave
 // reads its MFMA operands from there, so a key or value is read from L2 once per 128 rows instead
-// of once per 32.  Two LDS stages: tile i+1 is on its way from memory while tile i is computed.
-constexpr int kPfWaves = 4;
-constexpr int kPfRows = 32 * kPfWaves;  // rows of a workgroup
+// of once per 16.  Two LDS stages: tile i+1 is on its way from memory while tile i is computed.
+constexpr int kPfWaves = 8;
+constexpr int kPfNT = 1;                          // row tiles of 16 a wave
+constexpr int kPfRows = 16 * kPfNT * kPfWaves;    // rows of a workgroup
 constexpr int kPfKeys = 64;             // keys of a tile
+constexpr int kPfVPad = 4;              // padding of a value row in LDS: 34 dwords a row, so that the 16 rows which
+                                        // 16 lanes read or write together (8 bytes each) fall into 16 different bank pairs
 
-// Up to head_dim 128 two workgroups share a CU (LDS: 2 x 72 KB), so that one computes while the
-// other waits for LDS or memory; the register budget is set accordingly.
+// Work is handed out at run time.  A causal prompt is a triangle: the last 128 rows of a segment see 32 times
+// the keys of the first 128, and a fixed assignment of row blocks to workgroups leaves most of the chip idle
+// while the heaviest ones finish.  So the launch has two workgroups per CU and every workgroup takes the next
+// item (row block, kv head, segment), heaviest row blocks first, from a counter until none is left.  The counter
+// is a device variable of this module, put to zero by a one-thread kernel before every launch: launches of this
+// kernel on one device must not overlap (they never do on one stream).
+__device__ unsigned int g_prefill_next_item;
+
+__global__ void attn_prefill_reset_kernel() { g_prefill_next_item = 0u; }
+
+// One workgroup a CU: two waves on every SIMD, each with the registers it wants (16 rows a wave keep the
+// pieces of the next tile in registers beside the accumulators; with 32 rows they are spilled, and a spilled
+// load is waited for at once).  The staging registers are plain vector types on purpose: arrays of HIP's
+// uint4/uint2 structs went through scratch memory here.
 template <int DMAX, bool EXACT>
-__global__ __launch_bounds__(kPfWaves* kWave, DMAX <= 128 ? 2 : 1) void attn_prefill_lds_kernel(const AttnArgs a, int min_rows) {
-  constexpr int NT = 2;
+__global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_prefill_lds_kernel(const AttnArgs a, int min_rows,
+                                                                                         int blocks_x, int segments) {
+  constexpr int NT = kPfNT;
   constexpr int DCH = DMAX / 32, DTL = DMAX / 16;
   constexpr int kKPieces = (kPfKeys * (DMAX / 8) + kPfWaves * kWave - 1) / (kPfWaves * kWave);  // 16-byte pieces per thread
   constexpr int kVPieces = (kPfKeys / 4 * DMAX + kPfWaves * kWave - 1) / (kPfWaves * kWave);    // 8-byte pieces per thread
   extern __shared__ __align__(16) unsigned char lds_raw[];
+  __shared__ unsigned int item_of_workgroup;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, g = lane >> 4;
-  const int seg = blockIdx.z, kvh = blockIdx.y;
   const int G = a.nq / a.nkv;
+  const unsigned int per_block = static_cast<unsigned int>(a.nkv) * segments;
+  const unsigned int items = per_block * blocks_x;
+ for (;;) {  // one item per round; every wave of the workgroup leaves at the same round
+  if (tid == 0) item_of_workgroup = atomicAdd(&g_prefill_next_item, 1u);
+  __syncthreads();
+  const unsigned int item = item_of_workgroup;
+  __syncthreads();  // everyone has read it before thread 0 asks for the next
+  if (item >= items) return;
+  const int seg = (item % per_block) / a.nkv, kvh = (item % per_block) % a.nkv;
   const int row0 = a.seg_row0[seg];
   const int qlen = a.seg_row0[seg + 1] - row0;
   const int rows = qlen * G;
-  if (rows < min_rows) return;  // short segments (decoded tokens) belong to the other kernel
-  // the last rows of a segment see the most keys: hand them out first, so that the longest
-  // workgroups do not start last and leave the chip waiting for them
-  const int wg_row = (gridDim.x - 1 - blockIdx.x) * kPfRows;
-  if (wg_row >= rows) return;
+  if (rows < min_rows) continue;  // short segments (decoded tokens) belong to the other kernel
+  // the last rows of a segment see the most keys: they are handed out first
+  const int wg_row = (blocks_x - 1 - static_cast<int>(item / per_block)) * kPfRows;
+  if (wg_row >= rows) continue;
   const int start = a.seg_start[seg];
   const int* table = a.block_table + static_cast<int64_t>(a.seg_slot[seg]) * a.table_stride;
   const int D = EXACT ? DMAX : a.D, P = a.P;
   const int n_dch = EXACT ? DCH : (D + 31) / 32, n_dt = EXACT ? DTL : D / 16;
 
-  // LDS: two stages of [64 keys][D + 8] keys and [D][64 + 8] values (bfloat16; rows padded by 16 bytes)
-  const int k_pitch = D + 8, v_pitch = kPfKeys + 8;
+  // LDS: two stages of [64 keys][D + 8] keys and [D][64 + 4] values (bfloat16; rows padded against bank conflicts)
+  const int k_pitch = D + 8, v_pitch = kPfKeys + kPfVPad;
   const int stage_elems = kPfKeys * k_pitch + D * v_pitch;
   uint16_t* lds = reinterpret_cast<uint16_t*>(lds_raw);
 
@@ -431,9 +457,9 @@ __global__ __launch_bounds__(kPfWaves* kWave, DMAX <= 128 ? 2 : 1) void attn_pre
   const int t0 = kv_lo / kPfKeys, t1 = (kv_hi + kPfKeys - 1) / kPfKeys;
 
   // this wave's rows
-  const int row_begin = wg_row + 32 * wave;
+  const int row_begin = wg_row + 16 * NT * wave;
   const bool wave_has_rows = row_begin < rows;
-  const int wave_tok_max = wave_has_rows ? (min(row_begin + 32, rows) - 1) / G : 0;
+  const int wave_tok_max = wave_has_rows ? (min(row_begin + 16 * NT, rows) - 1) / G : 0;
   const int wave_kv_hi = start + wave_tok_max + 1;
   const int wave_kv_lo = a.window > 0 ? max(0, start + min(row_begin, rows - 1) / G - a.window + 1) : 0;
   // a tile needs no mask for this wave if it lies at or below its first row's position and at or
@@ -488,8 +514,10 @@ __global__ __launch_bounds__(kPfWaves* kWave, DMAX <= 128 ? 2 : 1) void attn_pre
   }
 #pragma unroll
   for (int j = 0; j < kVPieces; ++j) {
+    // 16 lanes next to each other take 16 consecutive d rows at the same keys (LDS: 16 bank pairs; memory: a
+    // wave still covers whole 128-byte lines, because its other lanes take the neighbouring keys)
     const int p = tid + j * (kPfWaves * kWave);
-    const int qi = p % v_per_row, d = (p / v_per_row) % D, pg = p / (v_per_row * D);
+    const int qi = (p / 16) % v_per_row, d = p % 16 + 16 * ((p / (16 * v_per_row)) % (D / 16)), pg = p / (v_per_row * D);
     v_d[j] = p < v_total ? d : -1;
     v_off[j] = pg * kp + 4 * qi;  // first of 4 keys, inside the tile
     v_lds[j] = d * v_pitch + v_off[j];
@@ -508,8 +536,8 @@ __global__ __launch_bounds__(kPfWaves* kWave, DMAX <= 128 ? 2 : 1) void attn_pre
     }
   };
 
-  uint4 kstage[kKPieces];
-  uint2 vstage[kVPieces];
+  u32x4 kstage[kKPieces];  // plain vector types: they stay in registers
+  u32x2 vstage[kVPieces];
   auto fetch = [&](int tile) {
     const int base = tile * kPfKeys;
     cover(tile);
@@ -518,7 +546,7 @@ __global__ __launch_bounds__(kPfWaves* kWave, DMAX <= 128 ? 2 : 1) void attn_pre
       const int key = min(max(base + max(k_key[j], 0), kv_lo), kv_hi - 1);
       const int page = __shfl(pg_reg, (key >> ps) - pg_base, kWave);  // every lane takes part
       if (EXACT || k_key[j] >= 0)
-        kstage[j] = *reinterpret_cast<const uint4*>(a.k_pages + page * page_elems + head_off +
+        kstage[j] = *reinterpret_cast<const u32x4*>(a.k_pages + page * page_elems + head_off +
                                                     static_cast<int64_t>(key & pm) * D + k_col[j]);
     }
 #pragma unroll
@@ -527,46 +555,53 @@ __global__ __launch_bounds__(kPfWaves* kWave, DMAX <= 128 ? 2 : 1) void attn_pre
       const int key4 = min(max(off, kv_lo & ~3), (kv_hi - 1) & ~3);
       const int page = __shfl(pg_reg, (key4 >> ps) - pg_base, kWave);
       if (EXACT || v_d[j] >= 0) {
-        uint2 v = *reinterpret_cast<const uint2*>(a.v_pages + page * page_elems + head_off +
-                                                  static_cast<int64_t>(v_d[j]) * P + (key4 & pm));
-        if (off + 4 > kv_total) {  // never written in this request: may hold anything
+        // nothing here looks at the loaded value, so no load has to be waited for before the next is issued
+        vstage[j] = *reinterpret_cast<const u32x2*>(a.v_pages + page * page_elems + head_off +
+                                                    static_cast<int64_t>(v_d[j]) * P + (key4 & pm));
+      }
+    }
+  };
+  auto park = [&](int stage, int tile) {  // the pieces of `tile` go from registers to LDS
+    uint16_t* ks = lds + stage * stage_elems;
+    uint16_t* vs = ks + kPfKeys * k_pitch;
+#pragma unroll
+    for (int j = 0; j < kKPieces; ++j)
+      if (EXACT || k_key[j] >= 0) *reinterpret_cast<u32x4*>(ks + k_lds[j]) = kstage[j];
+    const bool unwritten = tile * kPfKeys + kPfKeys > kv_total;  // the request's last tile only
+#pragma unroll
+    for (int j = 0; j < kVPieces; ++j)
+      if (EXACT || v_d[j] >= 0) {
+        u32x2 v = vstage[j];
+        if (unwritten) {  // slots past the last token may hold anything, also NaN: zero them for the products
+          const int off = tile * kPfKeys + v_off[j];
           if (off + 0 >= kv_total) v.x &= 0xffff0000u;
           if (off + 1 >= kv_total) v.x &= 0x0000ffffu;
           if (off + 2 >= kv_total) v.y &= 0xffff0000u;
           if (off + 3 >= kv_total) v.y &= 0x0000ffffu;
         }
-        vstage[j] = v;
+        *reinterpret_cast<u32x2*>(vs + v_lds[j]) = v;
       }
-    }
-  };
-  auto park = [&](int stage) {
-    uint16_t* ks = lds + stage * stage_elems;
-    uint16_t* vs = ks + kPfKeys * k_pitch;
-#pragma unroll
-    for (int j = 0; j < kKPieces; ++j)
-      if (EXACT || k_key[j] >= 0) *reinterpret_cast<uint4*>(ks + k_lds[j]) = kstage[j];
-#pragma unroll
-    for (int j = 0; j < kVPieces; ++j)
-      if (EXACT || v_d[j] >= 0) *reinterpret_cast<uint2*>(vs + v_lds[j]) = vstage[j];
   };
 
   fetch(t0);
-  park(0);
+  park(0, t0);
   __syncthreads();
 
   for (int tile = t0; tile < t1; ++tile) {
     const int stage = (tile - t0) & 1;
     const bool more = tile + 1 < t1;
+    // the next tile is on its way while this one is computed; its pieces wait in registers (they must not be
+    // spilled: a spill has to wait for the loads at once, which is why a wave has 16 rows, not 32)
     if (more) fetch(tile + 1);
-
     const int key_base = tile * kPfKeys;
     // a wave whose rows see none of this tile's keys only helps with the loads
-    if (wave_has_rows && key_base < wave_kv_hi && key_base + kPfKeys > wave_kv_lo) {
-      const uint16_t* ks = lds + stage * stage_elems;
-      const uint16_t* vs = ks + kPfKeys * k_pitch;
+    const bool computes = wave_has_rows && key_base < wave_kv_hi && key_base + kPfKeys > wave_kv_lo;
+    const uint16_t* ks = lds + stage * stage_elems;
+    const uint16_t* vs = ks + kPfKeys * k_pitch;
+    f32x4 s[NT][4];
+    if (computes) {
       // all key operands of the tile are asked for before the first product needs one, so that the
       // LDS latency is paid once, not once per product
-      f32x4 s[NT][4];
       {
         bf16x8 kop[4][DCH];
 #pragma unroll
@@ -578,6 +613,8 @@ __global__ __launch_bounds__(kPfWaves* kWave, DMAX <= 128 ? 2 : 1) void attn_pre
                             ? __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(ks + (16 * t + li) * k_pitch + d))
                             : zero_bf16x8();
           }
+        // keep the reads above the products: moved in between them, every read's latency shows
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           f32x4 z[NT];
@@ -593,7 +630,8 @@ __global__ __launch_bounds__(kPfWaves* kWave, DMAX <= 128 ? 2 : 1) void attn_pre
           for (int n = 0; n < NT; ++n) s[n][t] = z[n];
         }
       }
-
+    }
+    if (computes) {
       // Only tiles that touch a row's causal edge or window edge need the mask; the others take
       // the short path.  m is kept in the exponent's domain (score * scale * log2 e).
       const bool masked = key_base + kPfKeys - 1 > wave_pos_min || key_base < wave_win_lo;
@@ -659,6 +697,7 @@ __global__ __launch_bounds__(kPfWaves* kWave, DMAX <= 128 ? 2 : 1) void attn_pre
             va[dt] = *reinterpret_cast<const uint2*>(vrow);
             vb[dt] = *reinterpret_cast<const uint2*>(vrow + 16);
           }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int dt = 0; dt < DTL; ++dt)
           if (EXACT || dt < n_dt) {
@@ -671,7 +710,7 @@ __global__ __launch_bounds__(kPfWaves* kWave, DMAX <= 128 ? 2 : 1) void attn_pre
       }
     }
 
-    if (more) park(stage ^ 1);  // the other stage was last read before the barrier that ended the previous round
+    if (more) park(stage ^ 1, tile + 1);  // the other stage was last read before the barrier that ended the previous round
     __syncthreads();
   }
 
@@ -692,6 +731,7 @@ __global__ __launch_bounds__(kPfWaves* kWave, DMAX <= 128 ? 2 : 1) void attn_pre
       }
     }
   }
+ }  // next item
 }
 
 template <int NT>
@@ -708,7 +748,7 @@ int launch_attn(const AttnArgs& a, dim3 grid, hipStream_t s) {
 }
 
 inline size_t prefill_lds_bytes(int D) {
-  return 2 * (static_cast<size_t>(kPfKeys) * (D + 8) + static_cast<size_t>(D) * (kPfKeys + 8)) * sizeof(uint16_t);
+  return 2 * (static_cast<size_t>(kPfKeys) * (D + 8) + static_cast<size_t>(D) * (kPfKeys + kPfVPad)) * sizeof(uint16_t);
 }
 
 template <int DMAX, bool EXACT>
@@ -721,7 +761,19 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
     if (e != hipSuccess) return static_cast<int>(e);
     allowed = lds;
   }
-  attn_prefill_lds_kernel<DMAX, EXACT><<<grid, kPfWaves * kWave, lds, s>>>(a, min_rows);
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cus = n;
+  }
+  const long long items = static_cast<long long>(grid.x) * grid.y * grid.z;
+  const int per_cu = 1;  // eight waves: two on every SIMD, with all the registers they want
+  const unsigned workgroups = static_cast<unsigned>(items < static_cast<long long>(per_cu) * cus ? items : per_cu * cus);
+  attn_prefill_reset_kernel<<<1, 1, 0, s>>>();
+  attn_prefill_lds_kernel<DMAX, EXACT><<<workgroups, kPfWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
+                                                                                static_cast<int>(grid.z));
   return launch_status();
 }
 

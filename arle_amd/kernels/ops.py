@@ -425,7 +425,7 @@ EPI_NONE, EPI_SILU_MUL = 0, 1
 # How the few-rows kernel is shaped for a product (measured on MI355X together with the kernel that adds
 # the stack of partial products; see the kernel for the variants):
 _ROWS_TARGET_WORKGROUPS = 640    # K is split until about this many workgroups stream W
-_ROWS_MAX_SPLITS = 8             # ... the consumer pays for every part of the stack
+_ROWS_MAX_SPLITS = 4             # ... the consumer pays for every part of the stack (4, 8, 16 measure alike)
 _ROWS_PARTIAL_BYTES = 3 << 20    # ... and the float32 partial products stay below this
 _ROWS_WIDE_N = 32768             # from here on (an output head) N alone gives enough workgroups
 _ROWS_NARROW_N = 4096            # up to here N gives so few that one column tile a workgroup is best
