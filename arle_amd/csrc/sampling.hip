@@ -71,6 +71,73 @@ __global__ __launch_bounds__(kSampThreads) void argmax_rows_kernel(const float* 
   if (threadIdx.x == 0) out[blockIdx.x] = r.i;
 }
 
+// A row cut into gridDim.x chunks, so that a few rows still fill the chip: every workgroup leaves the best
+// (value, index) of its chunk in parts[row][chunk], and argmax_merge_kernel picks among them by the same rule.
+constexpr int kChunkThreads = 256;
+
+__global__ __launch_bounds__(kChunkThreads) void argmax_chunks_kernel(const float* __restrict__ logits, int vocab,
+                                                                     int chunk_len, ArgMax* __restrict__ parts) {
+  __shared__ ArgMax lds[kChunkThreads / kWave];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const float* x = logits + static_cast<int64_t>(row) * vocab;
+  const int begin = chunk * chunk_len, end = min(vocab, begin + chunk_len);
+  ArgMax a;
+  a.v = -INFINITY;
+  a.i = 0x7fffffff;
+  auto take = [&](float v, int i) {
+    ArgMax c;
+    c.v = v;
+    c.i = i;
+    a = better(a, c);
+  };
+  // chunk_len is a multiple of 4: with a 16-byte aligned row, four logits a load
+  if (reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+    const int whole = begin + (max(end - begin, 0) & ~3);
+    for (int i = begin + 4 * static_cast<int>(threadIdx.x); i < whole; i += 4 * kChunkThreads) {
+      const float4 v = *reinterpret_cast<const float4*>(x + i);
+      take(v.x, i);
+      take(v.y, i + 1);
+      take(v.z, i + 2);
+      take(v.w, i + 3);
+    }
+    for (int i = whole + static_cast<int>(threadIdx.x); i < end; i += kChunkThreads) take(x[i], i);
+  } else {
+    for (int i = begin + static_cast<int>(threadIdx.x); i < end; i += kChunkThreads) take(x[i], i);
+  }
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    ArgMax o;
+    o.v = __shfl_xor(a.v, off, kWave);
+    o.i = __shfl_xor(a.i, off, kWave);
+    a = better(a, o);
+  }
+  if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = a;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    ArgMax r = lds[0];
+    for (int i = 1; i < kChunkThreads / kWave; ++i) r = better(r, lds[i]);
+    parts[static_cast<int64_t>(row) * gridDim.x + chunk] = r;
+  }
+}
+
+__global__ __launch_bounds__(kWave) void argmax_merge_kernel(const ArgMax* __restrict__ parts, int chunks,
+                                                             int* __restrict__ out) {
+  const ArgMax* p = parts + static_cast<int64_t>(blockIdx.x) * chunks;
+  ArgMax a;
+  a.v = -INFINITY;
+  a.i = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += kWave) a = better(a, p[c]);
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    ArgMax o;
+    o.v = __shfl_xor(a.v, off, kWave);
+    o.i = __shfl_xor(a.i, off, kWave);
+    a = better(a, o);
+  }
+  // a row of NaNs (no value ever wins) yields index 0, as in the one-workgroup kernel
+  if (threadIdx.x == 0) out[blockIdx.x] = a.i == 0x7fffffff ? 0 : a.i;
+}
+
 __device__ __forceinline__ float block_sum_f(float v, float* lds) {
   return block_sum<kSampWaves>(v, lds);
 }
@@ -247,9 +314,27 @@ __global__ void apply_penalties_kernel(float* __restrict__ logits, int vocab,
 
 using namespace arle;
 
-extern "C" int arle_argmax_rows(const float* logits, int rows, int vocab, int* out, void* stream) {
+// parts: scratch of arle_argmax_chunks(rows, vocab) * rows pairs of 8 bytes, or null when that count is 1.
+extern "C" int arle_argmax_chunks(int rows, int vocab) {
+  if (rows <= 0 || vocab < 8192) return 1;
+  const int wanted = (512 + rows - 1) / rows;            // about 512 workgroups in all
+  const int most = vocab / 2048;                         // at least 2048 logits a chunk
+  return max(1, min(min(wanted, most), 256));
+}
+
+extern "C" int arle_argmax_rows(const float* logits, int rows, int vocab, int* out, void* parts, void* stream) {
   if (rows == 0) return 0;
-  argmax_rows_kernel<<<rows, kSampThreads, 0, static_cast<hipStream_t>(stream)>>>(logits, vocab, out);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int chunks = arle_argmax_chunks(rows, vocab);
+  if (chunks == 1) {
+    argmax_rows_kernel<<<rows, kSampThreads, 0, s>>>(logits, vocab, out);
+    return launch_status();
+  }
+  if (parts == nullptr) return static_cast<int>(hipErrorInvalidValue);
+  const int chunk_len = (((vocab + chunks - 1) / chunks) + 3) & ~3;
+  argmax_chunks_kernel<<<dim3(chunks, rows), kChunkThreads, 0, s>>>(logits, vocab, chunk_len,
+                                                                    static_cast<ArgMax*>(parts));
+  argmax_merge_kernel<<<rows, kWave, 0, s>>>(static_cast<const ArgMax*>(parts), chunks, out);
   return launch_status();
 }
 

@@ -379,10 +379,19 @@ def _logits(logits):
     return logits.shape
 
 
+@functools.lru_cache(maxsize=None)
+def _argmax_chunks(rows: int, vocab: int) -> int:
+    """Into how many chunks the argmax kernel cuts each row (it wants scratch for more than one)."""
+    return int(lib.function("arle_argmax_chunks")(rows, vocab))
+
+
 def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
     rows, vocab = _logits(logits)
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
-    lib.call("arle_argmax_rows", logits.data_ptr(), rows, vocab, out.data_ptr(), _stream())
+    chunks = _argmax_chunks(rows, vocab)
+    parts = torch.empty((rows, chunks, 2), dtype=torch.int32, device=logits.device) if chunks > 1 else None
+    lib.call("arle_argmax_rows", logits.data_ptr(), rows, vocab, out.data_ptr(),
+             parts.data_ptr() if parts is not None else 0, _stream())
     return out
 
 

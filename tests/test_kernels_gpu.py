@@ -131,6 +131,48 @@ def _paged_setup(lengths, nkv, D, P, dtype, seed, shuffle=True):
     return table, k_pages, v_pages
 
 
+@pytest.mark.parametrize("nq,nkv,D,P", [(4, 2, 128, 16), (2, 1, 64, 16), (3, 3, 128, 32), (2, 2, 64, 64),
+                                         (2, 1, 256, 16), (2, 2, 128, 8)])
+def test_qk_prep_runs_of_positions_fill_value_pages(nq, nkv, D, P):
+    """Portions of prompts: runs of consecutive positions that start on and off a multiple of 16, one after
+    the other in the packed rows, with single decoded tokens between them.  Every value lands in its slot
+    and no other slot of the cache changes."""
+    dt, eps, theta, rot = torch.bfloat16, 1e-6, 1e4, D
+    runs = [(0, 16, 48), (1, 5, 37), (2, 70, 1), (3, 32, 32), (1, 42, 1), (0, 64, 19)]   # (slot, start, count)
+    lengths = [83, 43, 71, 64]
+    table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, 40)
+    positions = torch.tensor([s + i for _, s, n in runs for i in range(n)], dtype=torch.int32)
+    slots = torch.tensor([r for r, _, n in runs for _ in range(n)], dtype=torch.int32)
+    T = positions.numel()
+    qkv = torch.randn(T, (nq + 2 * nkv) * D, generator=_g(41)).to(dt)
+    qw = (1.0 + 0.2 * torch.randn(D, generator=_g(42))).to(dt)
+    kw = (1.0 + 0.2 * torch.randn(D, generator=_g(43))).to(dt)
+    cos, sin = plain.rope_cos_sin(range(96), rot, theta)
+    d_qkv = qkv.to(DEV)
+    Q, KV = nq * D, nkv * D
+    dk, dv = k_pages.to(DEV), v_pages.to(DEV)
+    ops.qk_prep(d_qkv[:, :Q], d_qkv[:, Q:Q + KV], d_qkv[:, Q + KV:], num_q_heads=nq, num_kv_heads=nkv,
+                head_dim=D, eps=eps, q_weight=qw.to(DEV), k_weight=kw.to(DEV), cos=cos.to(DEV), sin=sin.to(DEV),
+                rotary_dim=rot, positions=positions.to(DEV), slot_of_token=slots.to(DEV),
+                block_table=table.to(DEV), k_pages=dk, v_pages=dv, page_size=P)
+    x = qkv.double()
+    c, s = plain.rope_cos_sin(positions.tolist(), rot, theta, dtype=torch.float64)
+    q = plain.apply_rope(plain.qk_norm(x[:, :Q].reshape(T, nq, D), qw.double(), eps), c, s)
+    k = plain.apply_rope(plain.qk_norm(x[:, Q:Q + KV].reshape(T, nkv, D), kw.double(), eps), c, s)
+    v = x[:, Q + KV:].reshape(T, nkv, D)
+    assert _rel(d_qkv[:, :Q].cpu().reshape(T, nq, D), q) < 6e-3
+    dk, dv = dk.cpu(), dv.cpu()
+    want_v = torch.zeros_like(dv)
+    written = torch.zeros(dk.shape[0], P, dtype=torch.bool)
+    for t in range(T):
+        page, at = int(table[slots[t], positions[t] // P]), int(positions[t]) % P
+        assert _rel(dk[page, :, at], k[t]) < 6e-3
+        want_v[page, :, :, at] = v[t].to(dt)
+        written[page, at] = True
+    assert torch.equal(dv, want_v)
+    assert torch.count_nonzero(dk.transpose(1, 2)[~written]) == 0
+
+
 @pytest.mark.parametrize("nq,nkv,D,rot", [(3, 1, 48, 48), (4, 2, 16, 16), (8, 2, 128, 128), (2, 2, 64, 32),
                                            (5, 5, 32, 0), (2, 1, 256, 64), (3, 3, 64, 0), (32, 8, 128, 128)])
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
@@ -273,6 +315,29 @@ def test_argmax_rows_first_maximum_wins():
     big[3, 7] = 60.0
     big[3, 100000] = 60.0
     assert ops.argmax_rows(big.to(DEV)).tolist() == big.argmax(-1).tolist()
+
+
+@pytest.mark.parametrize("rows,vocab", [(1, 151936), (3, 151937), (8, 32003), (64, 50257), (2, 8192), (7, 8191)])
+def test_argmax_rows_cut_into_chunks(rows, vocab):
+    """Rows long enough to be cut into chunks, with widths that leave the rows unaligned: the maximum at the
+    last place, at the first, twice (the first one wins, also from another chunk), and a row of NaNs."""
+    x = torch.randn(rows, vocab, generator=_g(51))
+    x[0, vocab - 1] = 40.0
+    want = x.argmax(-1).tolist()
+    if rows > 1:
+        x[1, 0] = 41.0
+        want[1] = 0
+    if rows > 2:
+        x[2, vocab // 2 + 1] = 42.0
+        x[2, vocab - 3] = 42.0
+        want[2] = vocab // 2 + 1
+    if rows > 3:
+        x[3] = float("nan")
+        want[3] = 0
+    if rows > 4:
+        x[4] = -5.0                                   # all equal: index 0
+        want[4] = 0
+    assert ops.argmax_rows(x.to(DEV)).tolist() == want
 
 
 def _sample(logits, temperature, u, top_k=-1, top_p=1.0, min_p=0.0):
