@@ -42,8 +42,8 @@ struct AttnArgs {
   int64_t q_stride;
   uint16_t* out;
   int64_t o_stride;
-  float* ws_o;   // [token row][q head][split][D]   (splits > 1)
-  float* ws_ml;  // [token row][q head][split][2]
+  float* ws_o;   // [segment * ws_rows + token of the segment][q head][split][D]   (splits > 1)
+  float* ws_ml;  // [segment * ws_rows + token of the segment][q head][split][2]
   const uint16_t* k_pages;  // [page][kv head][slot][D]
   const uint16_t* v_pages;  // [page][kv head][D][slot]
   const int* block_table;
@@ -56,6 +56,7 @@ struct AttnArgs {
   float scale_log2;
   int window;  // 0: all earlier keys
   int splits;
+  int ws_rows;   // token rows that the split-KV workspace holds for a segment
   int rows_max;  // the streaming kernel skips segments with more rows than this (0: takes all)
 };
 
@@ -310,7 +311,8 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
         }
       }
     } else {
-      const int64_t slot = (tok_row * a.nq + my_head[n]) * a.splits + split;
+      const int64_t ws_row = static_cast<int64_t>(seg) * a.ws_rows + my_tok[n];
+      const int64_t slot = (ws_row * a.nq + my_head[n]) * a.splits + split;
       float* wo = a.ws_o + slot * D;
 #pragma unroll
       for (int dt = 0; dt < DTL; ++dt) {
@@ -328,18 +330,24 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
 }
 
 // out[row][head][:] = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).   One workgroup of four waves
-// per (row, head).  Lane s of every wave holds the statistics of split s (splits <= 64) and the
+// per (workspace row, head); a workspace row is (segment, token of the segment), and rows past a segment's
+// length or of a segment that the streaming kernel left to the LDS kernel are skipped.  Lane s of every wave holds the statistics of split s (splits <= 64) and the
 // weights travel by cross-lane reads; wave w adds the splits s = w, w+4, ... with all its loads
 // independent of one another, and the four partial sums meet in LDS in wave order.
 constexpr int kMergeWaves = 4;
 constexpr int kMergeMaxD = 256;
 __global__ __launch_bounds__(kMergeWaves* kWave) void attn_merge_kernel(
     const float* __restrict__ ws_o, const float* __restrict__ ws_ml, uint16_t* __restrict__ out,
-    int64_t o_stride, int nq, int D, int splits) {
+    int64_t o_stride, const int* __restrict__ seg_row0, int ws_rows, int rows_max, int nq, int nkv, int D,
+    int splits) {
   __shared__ float part[kMergeWaves][kMergeMaxD];
-  const int row = blockIdx.x, head = blockIdx.y;
+  const int head = blockIdx.y;
+  const int seg = blockIdx.x / ws_rows, tok = blockIdx.x % ws_rows;
+  const int first = seg_row0[seg], qlen = seg_row0[seg + 1] - first;
+  if (tok >= qlen || (rows_max > 0 && qlen * (nq / nkv) > rows_max)) return;  // the whole workgroup leaves
+  const int row = first + tok;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int64_t base = (static_cast<int64_t>(row) * nq + head) * splits;
+  const int64_t base = (static_cast<int64_t>(blockIdx.x) * nq + head) * splits;
   float ms = -INFINITY, ls = 0.f;
   if (lane < splits) {
     const float2 ml = *reinterpret_cast<const float2*>(ws_ml + (base + lane) * 2);
@@ -399,13 +407,55 @@ constexpr int kPfVPad = 4;              // padding of a value row in LDS: 34 dwo
 
 // Work is handed out at run time.  A causal prompt is a triangle: the last 128 rows of a segment see 32 times
 // the keys of the first 128, and a fixed assignment of row blocks to workgroups leaves most of the chip idle
-// while the heaviest ones finish.  So the launch has two workgroups per CU and every workgroup takes the next
+// while the heaviest ones finish.  So the launch has one workgroup per CU and every workgroup takes the next
 // item (row block, kv head, segment), heaviest row blocks first, from a counter until none is left.  The counter
-// is a device variable of this module, put to zero by a one-thread kernel before every launch: launches of this
+// is a device variable of this module, put to zero by the planning kernel before every launch: launches of this
 // kernel on one device must not overlap (they never do on one stream).
+//
+// The planning kernel (one workgroup) also lists the live (row block, segment) pairs in that order: a step
+// that mixes a few portions with many decoded tokens has far more pairs that are dead (segments left to the
+// other kernel, row blocks past a short segment's end) than live ones, and asking for an item only to drop it
+// costs a round trip to the counter each time.  Steps with more pairs than the list holds go without it.
+constexpr int kPfPlanMax = 16384;
 __device__ unsigned int g_prefill_next_item;
+__device__ unsigned int g_prefill_pairs;              // entries of g_prefill_plan
+__device__ unsigned int g_prefill_plan[kPfPlanMax];   // (row block << 16) | segment
 
-__global__ void attn_prefill_reset_kernel() { g_prefill_next_item = 0u; }
+__global__ __launch_bounds__(256) void attn_prefill_plan_kernel(const int* __restrict__ seg_row0, int segments,
+                                                                 int blocks_x, int G, int min_rows, int listed) {
+  __shared__ unsigned int wave_count[4];
+  __shared__ unsigned int base;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) {
+    base = 0u;
+    g_prefill_next_item = 0u;
+  }
+  if (!listed) return;  // the whole workgroup
+  __syncthreads();
+  const int total = blocks_x * segments;
+  for (int i0 = 0; i0 < total; i0 += 256) {
+    const int i = i0 + tid;
+    bool live = false;
+    unsigned int entry = 0u;
+    if (i < total) {
+      const int seg = i % segments, rb = blocks_x - 1 - i / segments;  // the last rows see the most keys: first
+      const int rows = (seg_row0[seg + 1] - seg_row0[seg]) * G;
+      live = rows >= min_rows && rb * kPfRows < rows;
+      entry = (static_cast<unsigned int>(rb) << 16) | static_cast<unsigned int>(seg);
+    }
+    const unsigned long long votes = __ballot(live);
+    const unsigned int before = __popcll(votes & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_count[wave] = __popcll(votes);
+    __syncthreads();
+    unsigned int offset = base;
+    for (int w = 0; w < wave; ++w) offset += wave_count[w];
+    if (live) g_prefill_plan[offset + before] = entry;
+    __syncthreads();
+    if (tid == 0) base += wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
+    __syncthreads();
+  }
+  if (tid == 0) g_prefill_pairs = base;
+}
 
 // One workgroup a CU: two waves on every SIMD, each with the registers it wants (16 rows a wave keep the
 // pieces of the next tile in registers beside the accumulators; with 32 rows they are spilled, and a spilled
@@ -413,7 +463,7 @@ __global__ void attn_prefill_reset_kernel() { g_prefill_next_item = 0u; }
 // uint4/uint2 structs went through scratch memory here.
 template <int DMAX, bool EXACT>
 __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_prefill_lds_kernel(const AttnArgs a, int min_rows,
-                                                                                         int blocks_x, int segments) {
+                                                                                         int blocks_x, int segments, int listed) {
   constexpr int NT = kPfNT;
   constexpr int DCH = DMAX / 32, DTL = DMAX / 16;
   constexpr int kKPieces = (kPfKeys * (DMAX / 8) + kPfWaves * kWave - 1) / (kPfWaves * kWave);  // 16-byte pieces per thread
@@ -422,21 +472,28 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
   __shared__ unsigned int item_of_workgroup;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, g = lane >> 4;
   const int G = a.nq / a.nkv;
-  const unsigned int per_block = static_cast<unsigned int>(a.nkv) * segments;
-  const unsigned int items = per_block * blocks_x;
+  const unsigned int nkv = static_cast<unsigned int>(a.nkv);
+  const unsigned int pairs = listed ? g_prefill_pairs : static_cast<unsigned int>(blocks_x) * segments;
+  const unsigned int items = pairs * nkv;
  for (;;) {  // one item per round; every wave of the workgroup leaves at the same round
   if (tid == 0) item_of_workgroup = atomicAdd(&g_prefill_next_item, 1u);
   __syncthreads();
   const unsigned int item = item_of_workgroup;
   __syncthreads();  // everyone has read it before thread 0 asks for the next
   if (item >= items) return;
-  const int seg = (item % per_block) / a.nkv, kvh = (item % per_block) % a.nkv;
+  const unsigned int pair = item / nkv;
+  const int kvh = static_cast<int>(item % nkv);
+  // the last rows of a segment see the most keys: they are handed out first
+  int seg = static_cast<int>(pair % segments), wg_row = (blocks_x - 1 - static_cast<int>(pair / segments)) * kPfRows;
+  if (listed) {
+    const unsigned int entry = g_prefill_plan[pair];
+    seg = static_cast<int>(entry & 0xffffu);
+    wg_row = static_cast<int>(entry >> 16) * kPfRows;
+  }
   const int row0 = a.seg_row0[seg];
   const int qlen = a.seg_row0[seg + 1] - row0;
   const int rows = qlen * G;
   if (rows < min_rows) continue;  // short segments (decoded tokens) belong to the other kernel
-  // the last rows of a segment see the most keys: they are handed out first
-  const int wg_row = (blocks_x - 1 - static_cast<int>(item / per_block)) * kPfRows;
   if (wg_row >= rows) continue;
   const int start = a.seg_start[seg];
   const int* table = a.block_table + static_cast<int64_t>(a.seg_slot[seg]) * a.table_stride;
@@ -771,9 +828,11 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
   const long long items = static_cast<long long>(grid.x) * grid.y * grid.z;
   const int per_cu = 1;  // eight waves: two on every SIMD, with all the registers they want
   const unsigned workgroups = static_cast<unsigned>(items < static_cast<long long>(per_cu) * cus ? items : per_cu * cus);
-  attn_prefill_reset_kernel<<<1, 1, 0, s>>>();
+  const int listed = static_cast<long long>(grid.x) * grid.z <= kPfPlanMax && grid.x <= 65535 && grid.z <= 65535;
+  attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
+                                             a.nq / a.nkv, min_rows, listed);
   attn_prefill_lds_kernel<DMAX, EXACT><<<workgroups, kPfWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
-                                                                                static_cast<int>(grid.z));
+                                                                                static_cast<int>(grid.z), listed);
   return launch_status();
 }
 
@@ -781,11 +840,20 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
 
 using namespace arle;
 
+// Token rows that the split-KV workspace holds for every segment: the most tokens of a segment whose rows
+// (tokens x q heads of a kv head) fit one row tile of 16.
+extern "C" int arle_attn_ws_rows(int max_qlen, int nq, int nkv) {
+  const int G = nkv > 0 ? nq / nkv : 1;
+  return max(1, min(max_qlen, 16 / max(G, 1)));
+}
+
 // q, out: bfloat16 [token rows, nq*D] (row strides in elements).  Segments describe the packed
 // step: seg_row0[s]..seg_row0[s+1] are the token rows of segment s, whose first token sits at
 // position seg_start[s] of the request in block-table row seg_slot[s]; the cache already holds
 // the keys and values of these tokens.  max_qlen / min_qlen are the longest and shortest segment.  With splits > 1,
-// ws_o/ws_ml must hold [token rows][nq][splits][D] and [..][2] floats and the merge runs after.
+// ws_o/ws_ml must hold [segments * ws_rows][nq][splits][D] and [..][2] floats, ws_rows = arle_attn_ws_rows(...),
+// and the merge runs after; the split is over the keys of segments of at most 16 rows (decoded tokens and
+// portions of a few tokens); longer portions, which the LDS kernel takes, have rows enough to fill the chip.
 // Requires D % 16 == 0, D <= 256, page_size a power of two >= 4.
 extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out, long long o_stride,
                                     const void* k_pages, const void* v_pages, const int* block_table,
@@ -821,6 +889,7 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
   a.scale_log2 = scale * 1.4426950408889634f;
   a.window = window;
   a.splits = splits;
+  a.ws_rows = arle_attn_ws_rows(max_qlen, nq, nkv);
   a.rows_max = 0;
   const int G = nq / nkv;
   const int max_rows = max_qlen * G, min_rows = min_qlen * G;
@@ -844,14 +913,19 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
       rc = launch_prefill_lds<256, false>(a, grid, 17, s);
     if (rc != 0 || min_rows > 16) return rc;
     a.rows_max = 16;
-    return launch_attn<1>(a, dim3(1, nkv, segments), s);
+    rc = launch_attn<1>(a, dim3(1, nkv, static_cast<unsigned>(z)), s);
+    if (rc != 0 || splits == 1) return rc;
+    attn_merge_kernel<<<dim3(segments * a.ws_rows, nq), kMergeWaves * kWave, 0, s>>>(
+        ws_o, ws_ml, a.out, o_stride, seg_row0, a.ws_rows, a.rows_max, nq, nkv, D, splits);
+    return launch_status();
   }
+  if (max_rows > 16 && splits > 1) return static_cast<int>(hipErrorInvalidValue);  // two row tiles: no split
   // one row tile of 16 when a segment's rows fit it (decoded tokens), else two
   const int nt = max_rows <= 16 ? 1 : 2;
   dim3 grid((max_rows + 16 * nt - 1) / (16 * nt), nkv, static_cast<unsigned>(z));
   rc = nt == 1 ? launch_attn<1>(a, grid, s) : launch_attn<2>(a, grid, s);
   if (rc != 0 || splits == 1) return rc;
-  dim3 mgrid(token_rows, nq);
-  attn_merge_kernel<<<mgrid, kMergeWaves * kWave, 0, s>>>(ws_o, ws_ml, a.out, o_stride, nq, D, splits);
+  attn_merge_kernel<<<dim3(segments * a.ws_rows, nq), kMergeWaves * kWave, 0, s>>>(
+      ws_o, ws_ml, a.out, o_stride, seg_row0, a.ws_rows, 0, nq, nkv, D, splits);
   return launch_status();
 }

@@ -83,32 +83,36 @@ __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(wrow + e));
   };
 
-  // the first PD steps of W are on their way before anything else happens
+  // the first PD steps of W are on their way before anything else happens; without a condition (a step past
+  // the wave's last one is clamped into the row and never used), because a load under a condition is waited
+  // for at the end of its branch
   bf16x8 ring[PD];
 #pragma unroll
-  for (int u = 0; u < PD; ++u)
-    if (u < n_steps) ring[u] = load_w(w_begin + u);
+  for (int u = 0; u < PD; ++u) ring[u] = load_w(w_begin + u);
 
-  // X rows of the slice -> LDS, zeros past K; four 16-byte chunks a thread in flight
+  // X rows of the slice -> LDS, straight from memory (no registers in between, so every piece of the slice is
+  // on its way at once): a wave's 64 lanes fill 1 KB of LDS in lane order from 64 addresses of their own.  A
+  // row in LDS is its 16-byte pieces and one piece of padding; padding lanes and lanes past K fetch a piece
+  // that exists, and the pieces past K are put to zero afterwards (W is clamped there, X must not count).
   {
-    const int cpr = a.steps_per_split * 4;  // chunks of 8 elements per row
-    const int chunks = M * cpr;
+    const int cpr = a.steps_per_split * 4;  // pieces of 8 elements per row
+    const int cpp = cpr + kPad / 8;         // ... with the padding
+    const int total = M * cpp;
     const int k0 = s_begin * 32, k1 = min(s_end * 32, K);
-    for (int c0 = tid; c0 < chunks; c0 += 4 * kThreads) {
-      uint4 v[4];
-      int dst[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int c = c0 + i * kThreads;
-        const int row = min(c, chunks - 1) / cpr, col = (min(c, chunks - 1) % cpr) * 8;
-        const bool in = k0 + col < k1;
-        const uint4 raw = *reinterpret_cast<const uint4*>(a.x + static_cast<int64_t>(row) * a.ldx + (in ? k0 + col : 0));
-        v[i] = uint4{in ? raw.x : 0u, in ? raw.y : 0u, in ? raw.z : 0u, in ? raw.w : 0u};
-        dst[i] = c < chunks ? row * pitch + col : -1;
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (dst[i] >= 0) *reinterpret_cast<uint4*>(lds + dst[i]) = v[i];
+    for (int q0 = wave * 64; q0 < total; q0 += kThreads) {
+      const int q = min(q0 + lane, total - 1);
+      const int row = q / cpp, cc = q % cpp;
+      const int col = k0 + cc * 8;
+      const uint16_t* src = a.x + static_cast<int64_t>(row) * a.ldx + ((cc < cpr && col < k1) ? col : k0);
+      __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)(lds + q0 * 8),
+                                       16, 0, 0);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (k1 < s_end * 32) {
+      __syncthreads();  // the pieces put to zero were fetched by other waves: all of them have to be in first
+      const int z0 = (k1 - k0) / 8, nz = (s_end * 32 - k1) / 8;
+      for (int i = tid; i < M * nz; i += kThreads)
+        *reinterpret_cast<uint4*>(lds + (i / nz) * pitch + (z0 + i % nz) * 8) = uint4{0u, 0u, 0u, 0u};
     }
   }
   __syncthreads();
@@ -129,23 +133,49 @@ __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a
   for (int u = 0; u < XD; ++u)
     if (u < n_steps) load_x(u, xring[u]);
 
-  for (int base = 0; base < n_steps; base += PD) {
+  // While a whole round of PD steps and of PD loads ahead is left, the round runs without a condition: only
+  // then does each product wait for its own load alone (a load under a condition in a loop makes the next wait
+  // a wait for every load).  The last two rounds are written out, not looped over.
+  int base = 0;
+  for (; base + 2 * PD <= n_steps; base += PD) {
 #pragma unroll
     for (int u = 0; u < PD; ++u) {
       const int s = base + u;  // relative to w_begin
-      if (s < n_steps) {
 #pragma unroll
-        for (int b = 0; b < MT; ++b)
-          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
-        if (s + XD < n_steps) load_x(s + XD, xring[u % XD]);
-        if (s + PD < n_steps) ring[u] = load_w(w_begin + s + PD);
-      }
+      for (int b = 0; b < MT; ++b)
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
+      load_x(s + XD, xring[u % XD]);
+      ring[u] = load_w(w_begin + s + PD);
+      __builtin_amdgcn_sched_barrier(0);  // keep each load right behind its product: PD - 1 stay in flight
+    }
+  }
+  if (base + PD <= n_steps) {  // a whole round of products, fewer than PD loads ahead
+#pragma unroll
+    for (int u = 0; u < PD; ++u) {
+      const int s = base + u;
+#pragma unroll
+      for (int b = 0; b < MT; ++b)
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
+      if (s + XD < n_steps) load_x(s + XD, xring[u % XD]);
+      if (s + PD < n_steps) ring[u] = load_w(w_begin + s + PD);
+    }
+    base += PD;
+  }
+  // the last steps, fewer than PD: W is in the ring or on its way, only X is left to fetch
+#pragma unroll
+  for (int u = 0; u < PD; ++u) {
+    const int s = base + u;
+    if (s < n_steps) {
+#pragma unroll
+      for (int b = 0; b < MT; ++b)
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
+      if (s + XD < n_steps) load_x(s + XD, xring[u % XD]);
     }
   }
 
   // add the WK partial sums of every column tile in the order wk = 0, 1, ...: waves wk > 0 park
   // their registers in LDS behind X, waves wk == 0 add
-  float* red = reinterpret_cast<float*>(lds + ((M * pitch + 7) / 8) * 8);  // [WK-1][WN][MT][64][4]
+  float* red = reinterpret_cast<float*>(lds + ((M * pitch + 511) / 512) * 512);  // [WK-1][WN][MT][64][4]; X ends on a whole wave's fill
   if constexpr (WK > 1) {
     if (wk > 0) {
 #pragma unroll
@@ -207,7 +237,7 @@ __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a
 // LDS of a launch: the X rows of one k slice and, behind them, the partial sums of the waves wk > 0 and the
 // gate/up exchange.
 inline size_t rows_lds_bytes(int M, int steps_per_split, int mt, int wn, int wk) {
-  const size_t x = (static_cast<size_t>(M) * (steps_per_split * 32 + kPad) + 7) / 8 * 8 * sizeof(uint16_t);
+  const size_t x = (static_cast<size_t>(M) * (steps_per_split * 32 + kPad) + 511) / 512 * 512 * sizeof(uint16_t);
   const size_t red = static_cast<size_t>(wk - 1) * wn * mt * 64 * 4 * sizeof(float);
   const size_t swap = static_cast<size_t>((wn + 1) / 2) * mt * 64 * 4 * sizeof(float);
   return x + red + swap;

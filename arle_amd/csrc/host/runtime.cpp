@@ -242,7 +242,7 @@ int arle_group_check(void* h, char* msg, int cap) {
 //   token_ids[T] positions[T] slot_of_token[T] want_rows[R] seg_row0[S+1] seg_slot[S] seg_start[S]
 // Entry e brings n_tokens[e] tokens (concatenated in `tokens`) of the request in slot[e] that holds start[e]
 // tokens already, and wants n_want[e] places among them (concatenated in `wants`).
-// meta: T, R, max position, longest entry, shortest entry.  Returns 0, or
+// meta (six ints): T, R, max position, longest entry, shortest entry, entries of one token.  Returns 0, or
 //   1: a token id outside the vocabulary   2: a wanted place outside its entry   3: an entry without tokens
 //   4: `out` has not exactly the size of the step;   where[0..1] = entry and the offending value.
 int arle_pack_step(int n_entries, const int* slot, const int* start, const int* n_tokens, const int* tokens,
@@ -267,7 +267,7 @@ int arle_pack_step(int n_entries, const int* slot, const int* start, const int* 
   int* seg_row0 = want_rows + R;
   int* seg_slot = seg_row0 + S + 1;
   int* seg_start = seg_slot + S;
-  int row = 0, w = 0, t = 0, r = 0, max_pos = 0, longest = 0, shortest = INT32_MAX;
+  int row = 0, w = 0, t = 0, r = 0, max_pos = 0, longest = 0, shortest = INT32_MAX, singles = 0;
   for (int e = 0; e < n_entries; ++e) {
     const int n = n_tokens[e];
     for (int i = 0; i < n; ++i) {
@@ -296,6 +296,7 @@ int arle_pack_step(int n_entries, const int* slot, const int* start, const int* 
     max_pos = std::max(max_pos, start[e] + n - 1);
     longest = std::max(longest, n);
     shortest = std::min(shortest, n);
+    singles += n == 1;
     row += n;
     t += n;
     w += n_want[e];
@@ -306,6 +307,7 @@ int arle_pack_step(int n_entries, const int* slot, const int* start, const int* 
   meta[2] = max_pos;
   meta[3] = longest;
   meta[4] = shortest;
+  meta[5] = singles;
   return 0;
 }
 

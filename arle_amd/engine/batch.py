@@ -47,6 +47,7 @@ class StepBatch:
     seg_slot: torch.Tensor       # int32 [S]
     seg_start: torch.Tensor      # int32 [S]  position of a segment's first row
     host: dict                   # the same arrays as numpy, for parts that plan on the host
+    single_segments: int = 0     # segments of one token (decoded tokens)
     kv_splits: int | None = None  # split-KV factor fixed by the caller (a captured graph), else chosen per call
 
 
@@ -93,7 +94,7 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device, into=
     at = lambda elements: base + 4 * elements
     slot_p, start_p, ntok_p, nwant_p, tokens_p, wants_p = at(0), at(S), at(2 * S), at(3 * S), at(4 * S), at(4 * S + row)
     flat_np = np.empty(packed_size(row, S, num_wanted), dtype=np.int32)
-    meta, where = native.int_array(5), native.int_array(2)
+    meta, where = native.int_array(6), native.int_array(2)
     code = native.lib().arle_pack_step(S, slot_p, start_p, ntok_p, tokens_p, nwant_p, wants_p, int(vocab_size),
                                        flat_np.ctypes.data, flat_np.size, meta, where)
     if code == 1:
@@ -126,4 +127,5 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device, into=
         dev[k] = packed[off:off + n]
         off += n
     return StepBatch(num_tokens=row, segments=segments, max_position=meta[2], max_qlen=meta[3], min_qlen=meta[4],
+                     single_segments=meta[5],
                      host=host, **dev)

@@ -319,6 +319,9 @@ def decode_split_cap(max_kv_len: int) -> int:
     return max(1, min(-(-max_kv_len // 32) // 2, 32))
 
 
+_ATTN_ROW_TILE = 16   # rows of the matrix-core tile: a segment with more rows goes to the LDS kernel
+
+
 def decode_splits(segments: int, num_kv_heads: int, max_kv_len: int) -> int:
     """Split-KV factor of a step of single decoded tokens: enough waves to fill the chip."""
     return max(1, min(-(-_MFMA_TARGET_WAVES // (segments * num_kv_heads)), decode_split_cap(max_kv_len)))
@@ -327,11 +330,13 @@ def decode_splits(segments: int, num_kv_heads: int, max_kv_len: int) -> int:
 def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *,
                     max_qlen: int, max_kv_len: int, num_q_heads: int, num_kv_heads: int, head_dim: int,
                     page_size: int, scale: float, window: int = 0, splits: int | None = None,
-                    min_qlen: int = 1):
+                    min_qlen: int = 1, short_segments: int | None = None):
     """Causal attention of a packed step on the matrix cores (bfloat16).
 
     Segments: rows seg_row0[s]..seg_row0[s+1] belong to block-table row seg_slot[s] and start at
-    position seg_start[s].  A step of single decoded tokens is split over the keys (split-KV).
+    position seg_start[s].  Segments whose rows (tokens x q heads of a kv head) fit one row tile of 16,
+    decoded tokens above all, are split over the keys (split-KV), also beside longer portions in one
+    step; `short_segments` says how many there are (default: all), which sets the number of splits.
     """
     _gpu(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start)
     tokens = q.shape[0]
@@ -352,14 +357,18 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
     _i32(seg_slot, "seg_slot")
     _i32(seg_start, "seg_start", segments)
     _need(1 <= min_qlen <= max_qlen <= tokens, "need 1 <= min_qlen <= max_qlen <= tokens")
-    if splits is None:
-        splits = decode_splits(segments, num_kv_heads, max_kv_len) if max_qlen == 1 else 1
-    _need(splits == 1 or max_qlen == 1, "split-KV is for steps of single decoded tokens")
+    group = num_q_heads // num_kv_heads
+    if min_qlen * group > _ATTN_ROW_TILE:
+        splits = 1                      # no segment is short enough for the kernel that splits the keys
+    elif splits is None:
+        short = segments if short_segments is None else max(1, min(short_segments, segments))
+        splits = decode_splits(short, num_kv_heads, max_kv_len)
     _need(segments * splits <= _GRID_Y_MAX and num_kv_heads <= _GRID_Y_MAX, "too many segments for one launch")
     ws_o = ws_ml = None
     if splits > 1:
-        ws_o = torch.empty((tokens, num_q_heads, splits, head_dim), dtype=torch.float32, device=q.device)
-        ws_ml = torch.empty((tokens, num_q_heads, splits, 2), dtype=torch.float32, device=q.device)
+        ws_rows = segments * max(1, min(max_qlen, _ATTN_ROW_TILE // group))   # arle_attn_ws_rows a segment
+        ws_o = torch.empty((ws_rows, num_q_heads, splits, head_dim), dtype=torch.float32, device=q.device)
+        ws_ml = torch.empty((ws_rows, num_q_heads, splits, 2), dtype=torch.float32, device=q.device)
     lib.call("arle_attn_paged_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
              k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
              seg_row0.data_ptr(), seg_slot.data_ptr(), seg_start.data_ptr(), segments, int(max_qlen),

@@ -131,7 +131,8 @@ def paged_attention(q, out, cache, batch, *, num_q_heads, num_kv_heads, head_dim
                             batch.seg_slot, batch.seg_start, max_qlen=batch.max_qlen, min_qlen=batch.min_qlen,
                             max_kv_len=batch.max_position + 1, num_q_heads=num_q_heads,
                             num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=cache.page_size,
-                            scale=scale, window=window, splits=getattr(batch, "kv_splits", None))
+                            scale=scale, window=window, splits=getattr(batch, "kv_splits", None),
+                            short_segments=getattr(batch, "single_segments", 0) or None)
     else:
         ops.attn_paged_simt(q, out, cache.k_pages, cache.v_pages, cache.block_table, batch.positions,
                             batch.slot_of_token, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads,

@@ -439,11 +439,14 @@ def test_attention_mfma_decoded_tokens_split_over_the_keys(nq, nkv, D, P, splits
     assert _rel(got, want) < 8e-3
 
 
-def test_attention_mfma_mixed_step_and_stale_pages():
-    """Decoded tokens beside portions in one launch; pages hold NaN bits beyond each request's length."""
-    nq, nkv, D, P = 8, 2, 128, 16
+@pytest.mark.parametrize("nq,nkv,D", [(8, 2, 128), (3, 3, 64), (16, 1, 128)])
+@pytest.mark.parametrize("splits", [None, 1, 5])
+def test_attention_mfma_mixed_step_and_stale_pages(nq, nkv, D, splits):
+    """Decoded tokens and portions of a few tokens (split over the keys) beside longer portions in one
+    launch; pages hold NaN bits beyond each request's length, and so does the output before the call."""
+    P = 16
     dt = torch.bfloat16
-    segs = [(200, 1), (17, 30), (63, 1), (0, 5)]
+    segs = [(200, 1), (17, 30), (63, 1), (0, 5), (40, 3), (0, 2), (330, 1), (100, 16)]
     lengths = [a + b for a, b in segs]
     table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, 90)
     k_pages.fill_(float("nan"))
@@ -458,11 +461,12 @@ def test_attention_mfma_mixed_step_and_stale_pages():
         row0.append(row0[-1] + n)
         starts.append(cached)
     q_all = torch.cat(qs).to(DEV)
-    out = torch.empty_like(q_all)
+    out = torch.full_like(q_all, float("nan"))
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
-    ops.attn_paged_mfma(q_all, out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0), i32([0, 1, 2, 3]),
-                        i32(starts), max_qlen=30, min_qlen=1, max_kv_len=max(lengths), num_q_heads=nq, num_kv_heads=nkv,
-                        head_dim=D, page_size=P, scale=1.0 / math.sqrt(D))
+    ops.attn_paged_mfma(q_all, out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0),
+                        i32(list(range(len(segs)))), i32(starts), max_qlen=30, min_qlen=1, max_kv_len=max(lengths),
+                        num_q_heads=nq, num_kv_heads=nkv, head_dim=D, page_size=P, scale=1.0 / math.sqrt(D),
+                        splits=splits, short_segments=3)
     assert torch.isfinite(out).all()
     assert _rel(out.cpu(), torch.cat(wants)) < 8e-3
 
@@ -530,7 +534,7 @@ def test_gemm_rows_as_planned(M, N, K):
 
 @pytest.mark.parametrize("variant", range(ops.ROWS_VARIANTS))
 @pytest.mark.parametrize("M,N,K,splits", [(5, 333, 88, 1), (16, 96, 1096, 3), (20, 200, 520, 2), (64, 72, 2056, 5),
-                                          (33, 2560, 4096, 16)])
+                                          (33, 2560, 4096, 16), (64, 72, 2056, 3), (48, 100, 4104, 4)])
 def test_gemm_rows_every_variant_and_split(variant, M, N, K, splits):
     a = torch.randn(M, K, generator=_g(103)).bfloat16()
     w = (torch.randn(N, K, generator=_g(104)) * 0.1).bfloat16()
