@@ -176,7 +176,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
   };
 
   // values of a block: for each 16-key tile the 4 keys 4g..4g+3, at d = 16*dt + li
-  auto load_v = [&](int blk, uint2 (&vreg)[2][DTL]) {
+  auto load_v = [&](int blk, u32x4 (&vreg)[DTL]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       int key4 = blk * 32 + 16 * t + 4 * g;
@@ -185,13 +185,17 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
       const uint16_t* vp = a.v_pages + page * page_elems + k_head + (key4 & pm);
 #pragma unroll
       for (int dt = 0; dt < DTL; ++dt) {
-        if (EXACT || dt < n_dt) vreg[t][dt] = *reinterpret_cast<const uint2*>(vp + static_cast<int64_t>(16 * dt + li) * P);
+        if (EXACT || dt < n_dt) {
+          const u32x2 four = *reinterpret_cast<const u32x2*>(vp + static_cast<int64_t>(16 * dt + li) * P);
+          vreg[dt][2 * t] = four[0];
+          vreg[dt][2 * t + 1] = four[1];
+        }
       }
     }
   };
 
   bf16x8 kcur[2][DCH];
-  uint2 vraw[2][DTL];
+  u32x4 vraw[DTL];  // the second product's operand for each d tile: keys 4g..4g+3 of both 16-key tiles
   if (b0 < b1) {
     refill_pages(clamp_key(b0 * 32) >> ps);
     load_k(b0, kcur);
@@ -226,10 +230,10 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
 #pragma unroll
         for (int dt = 0; dt < DTL; ++dt) {
           if (!EXACT && dt >= n_dt) continue;
-          if (key4 + 0 >= kv_total) vraw[t][dt].x &= 0xffff0000u;
-          if (key4 + 1 >= kv_total) vraw[t][dt].x &= 0x0000ffffu;
-          if (key4 + 2 >= kv_total) vraw[t][dt].y &= 0xffff0000u;
-          if (key4 + 3 >= kv_total) vraw[t][dt].y &= 0x0000ffffu;
+          if (key4 + 0 >= kv_total) vraw[dt][2 * t] &= 0xffff0000u;
+          if (key4 + 1 >= kv_total) vraw[dt][2 * t] &= 0x0000ffffu;
+          if (key4 + 2 >= kv_total) vraw[dt][2 * t + 1] &= 0xffff0000u;
+          if (key4 + 3 >= kv_total) vraw[dt][2 * t + 1] &= 0x0000ffffu;
         }
       }
     }
@@ -280,8 +284,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
 #pragma unroll
     for (int dt = 0; dt < DTL; ++dt) {
       if (EXACT || dt < n_dt) {
-        uint4 vv = {vraw[0][dt].x, vraw[0][dt].y, vraw[1][dt].x, vraw[1][dt].y};
-        const bf16x8 vop = __builtin_bit_cast(bf16x8, vv);
+        const bf16x8 vop = __builtin_bit_cast(bf16x8, vraw[dt]);
 #pragma unroll
         for (int n = 0; n < NT; ++n)
           acc[n][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pb[n], acc[n][dt], 0, 0, 0);
@@ -746,20 +749,27 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
 
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        uint2 va[DTL], vb[DTL];  // the value operands of 32 keys, all asked for first
+        // the value operands of 32 keys, all asked for first.  Each is one four-dword vector filled half by
+        // half: an operand put together from the scalars of two two-dword vectors just before the product was
+        // compiled wrongly in the streaming kernel (the registers of the second pair were handed out again
+        // before the product had read them).
+        u32x4 vv[DTL];
 #pragma unroll
         for (int dt = 0; dt < DTL; ++dt)
           if (EXACT || dt < n_dt) {
             const uint16_t* vrow = vs + (16 * dt + li) * v_pitch + 32 * u + 4 * g;
-            va[dt] = *reinterpret_cast<const uint2*>(vrow);
-            vb[dt] = *reinterpret_cast<const uint2*>(vrow + 16);
+            const u32x2 va = *reinterpret_cast<const u32x2*>(vrow);
+            const u32x2 vb = *reinterpret_cast<const u32x2*>(vrow + 16);
+            vv[dt][0] = va[0];
+            vv[dt][1] = va[1];
+            vv[dt][2] = vb[0];
+            vv[dt][3] = vb[1];
           }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int dt = 0; dt < DTL; ++dt)
           if (EXACT || dt < n_dt) {
-            uint4 vv = {va[dt].x, va[dt].y, vb[dt].x, vb[dt].y};
-            const bf16x8 vop = __builtin_bit_cast(bf16x8, vv);
+            const bf16x8 vop = __builtin_bit_cast(bf16x8, vv[dt]);
 #pragma unroll
             for (int n = 0; n < NT; ++n)
               acc[n][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pb[n][u], acc[n][dt], 0, 0, 0);
@@ -793,9 +803,14 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
 
 template <int NT>
 int launch_attn(const AttnArgs& a, dim3 grid, hipStream_t s) {
-  // This kernel is bound by memory, not by instruction issue: it always runs with head_dim as a
-  // run-time value (the compile-time variant is kept for the LDS kernel, where it pays).
-  if (a.D <= 64)
+  // head_dim 64 and 128 as compile-time values: no test and no branch around a load, so that the keys and
+  // values of the next block stay in flight while this block is computed (a load inside a branch makes the
+  // next wait a wait for everything)
+  if (a.D == 128)
+    attn_mfma_kernel<NT, 128, true><<<grid, kWave, 0, s>>>(a);
+  else if (a.D == 64)
+    attn_mfma_kernel<NT, 64, true><<<grid, kWave, 0, s>>>(a);
+  else if (a.D <= 64)
     attn_mfma_kernel<NT, 64, false><<<grid, kWave, 0, s>>>(a);
   else if (a.D <= 128)
     attn_mfma_kernel<NT, 128, false><<<grid, kWave, 0, s>>>(a);

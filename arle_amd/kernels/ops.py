@@ -315,8 +315,11 @@ def attn_mfma_supported(dtype, head_dim: int, page_size: int) -> bool:
 
 
 def decode_split_cap(max_kv_len: int) -> int:
-    """Most splits worth making for keys up to max_kv_len: at least two 32-key blocks each, at most 32."""
-    return max(1, min(-(-max_kv_len // 32) // 2, 32))
+    """Most splits worth making for keys up to max_kv_len: at least two 32-key blocks each, at most 64
+    (the merge keeps the statistics of one split in each lane of a wave), and a power of two, so that a
+    context that grows passes through few different values (a captured decode step is made for one)."""
+    most = max(1, min(-(-max_kv_len // 32) // 2, 64))
+    return 1 << (most.bit_length() - 1)
 
 
 _ATTN_ROW_TILE = 16   # rows of the matrix-core tile: a segment with more rows goes to the LDS kernel
