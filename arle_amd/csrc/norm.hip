@@ -182,7 +182,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_vec_kernel(TIn* __restri
 // four columns, and the loads of the whole stack (up to kStackUnroll at a time) are in flight together.
 // Order of addition: residual + (delta 0 + delta 1 + ...), as in the kernels above.
 constexpr int kStackThreads = 1024;
-constexpr int kStackUnroll = 16;
+constexpr int kStackUnroll = 4;   // parts of the stack that a thread has in flight at a time
 
 template <typename TOut, typename TW>
 __global__ __launch_bounds__(kStackThreads) void add_stack_rmsnorm_kernel(
@@ -195,31 +195,47 @@ __global__ __launch_bounds__(kStackThreads) void add_stack_rmsnorm_kernel(
   const bool mine = i < width;
   float* res = residual + src * width;
   const float* dr = delta + src * width;
-  float4 v = {0.f, 0.f, 0.f, 0.f}, wv = v, d = v;
-  if (mine) {
-    v = load4<float>(res + i);
-    wv = load4<TW>(w + i);
-  }
-  for (int base = 0; base < n_delta; base += kStackUnroll) {
+  const int ic = mine ? i : 0;
+  float4 v = load4<float>(res + ic), d = {0.f, 0.f, 0.f, 0.f};
+  const float4 wv = load4<TW>(w + ic);
+  // The loads of a round carry no condition (a load under a condition is waited for before the next one is
+  // issued, and the parts would arrive one after the other): whole rounds of four parts first, then one round
+  // whose loads past the last part fetch the last part again and are not added.  Threads past the width read
+  // column 0.
+  const float* dc = dr + ic;
+  int base = 0;
+  for (; base + kStackUnroll <= n_delta; base += kStackUnroll) {
     float4 e[kStackUnroll];
 #pragma unroll
-    for (int u = 0; u < kStackUnroll; ++u)
-      if (mine && base + u < n_delta) e[u] = load4<float>(dr + (base + u) * delta_stride + i);
+    for (int u = 0; u < kStackUnroll; ++u) e[u] = load4<float>(dc + (base + u) * delta_stride);
 #pragma unroll
-    for (int u = 0; u < kStackUnroll; ++u)
-      if (mine && base + u < n_delta) {
-        d.x += e[u].x;
-        d.y += e[u].y;
-        d.z += e[u].z;
-        d.w += e[u].w;
-      }
+    for (int u = 0; u < kStackUnroll; ++u) {
+      d.x += e[u].x;
+      d.y += e[u].y;
+      d.z += e[u].z;
+      d.w += e[u].w;
+    }
+  }
+  if (base < n_delta) {
+    float4 e[kStackUnroll - 1];
+#pragma unroll
+    for (int u = 0; u < kStackUnroll - 1; ++u) e[u] = load4<float>(dc + min(base + u, n_delta - 1) * delta_stride);
+#pragma unroll
+    for (int u = 0; u < kStackUnroll - 1; ++u) {
+      const bool in = base + u < n_delta;
+      d.x += in ? e[u].x : 0.f;
+      d.y += in ? e[u].y : 0.f;
+      d.z += in ? e[u].z : 0.f;
+      d.w += in ? e[u].w : 0.f;
+    }
   }
   v.x += d.x;
   v.y += d.y;
   v.z += d.z;
   v.w += d.w;
   if (mine && !rows) store4<float>(res + i, v);
-  const float total = block_sum<kStackThreads / kWave>(v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w, lds);
+  const float total =
+      block_sum<kStackThreads / kWave>(mine ? v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w : 0.f, lds);
   const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
   if (mine)
     store4<TOut>(out + static_cast<int64_t>(r) * width + i,

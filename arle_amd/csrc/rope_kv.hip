@@ -56,16 +56,26 @@ __global__ __launch_bounds__(kPrepWaves* kWave) void qk_prep_kernel(
 
   // column `col` of token t's fused [q | k | v] row, summed over the stack of partial products
   const float* part_row = parts ? parts + static_cast<int64_t>(t) * part_row_stride : nullptr;
-  auto summed = [&](int col) {  // the loads of up to 16 parts are in flight together, the adds are in order
+  // The loads carry no condition (a load under a condition is waited for before the next one is issued):
+  // whole rounds of four parts, then one round that fetches the last part again where there is none and
+  // does not add it.  The adds are in the order of the parts.
+  auto summed = [&](int col) {
+    const float* p = part_row + col;
     float acc = 0.f;
-    for (int base = 0; base < n_parts; base += 16) {
-      float e[16];
+    int base = 0;
+    for (; base + 4 <= n_parts; base += 4) {
+      float e[4];
 #pragma unroll
-      for (int u = 0; u < 16; ++u)
-        if (base + u < n_parts) e[u] = part_row[(base + u) * part_stride + col];
+      for (int u = 0; u < 4; ++u) e[u] = p[(base + u) * part_stride];
 #pragma unroll
-      for (int u = 0; u < 16; ++u)
-        if (base + u < n_parts) acc += e[u];
+      for (int u = 0; u < 4; ++u) acc += e[u];
+    }
+    if (base < n_parts) {
+      float e[3];
+#pragma unroll
+      for (int u = 0; u < 3; ++u) e[u] = p[min(base + u, n_parts - 1) * part_stride];
+#pragma unroll
+      for (int u = 0; u < 3; ++u) acc += base + u < n_parts ? e[u] : 0.f;
     }
     return acc;
   };

@@ -138,140 +138,395 @@ __global__ __launch_bounds__(kWave) void argmax_merge_kernel(const ArgMax* __res
   if (threadIdx.x == 0) out[blockIdx.x] = a.i == 0x7fffffff ? 0 : a.i;
 }
 
-__device__ __forceinline__ float block_sum_f(float v, float* lds) {
-  return block_sum<kSampWaves>(v, lds);
-}
+// ---------------------------------------------------------------------------------------------
+// Temperature sampling with min-p, top-k and top-p, many workgroups a row.
+//
+// e[i] = exp(x[i] / T - max) is kept unnormalised: every filter is "keep e[i] >= some threshold", and since
+// e >= 0 the order of the values is the order of their bit patterns.
+//   min_p:  e >= min_p                       (the largest e is exp(0) = 1)
+//   top_k:  e >= the k-th largest e           (ties of the k-th stay)
+//   top_p:  e >= the largest t whose kept mass reaches top_p of the mass kept so far
+// The k-th largest value and the mass threshold are found digit by digit, eight bits at a time: a pass over
+// the row fills a histogram of 256 bins with the next digit of the elements that match the digits found so
+// far; scanning the bins from the top gives the digit in which the count (the mass) is reached.  Counts are
+// integers and masses are summed as 64-bit fixed-point numbers (e * 2^40), so the histograms do not depend
+// on the order in which workgroups add to them, and every workgroup that reads them finds the same digits.
+// The token is then drawn by the inverse CDF in token order: u * (kept mass) falls into a chunk, and inside
+// the chunk into a token.
+constexpr int kSelThreads = kChunkThreads;
+constexpr int kSelWaves = kSelThreads / kWave;
+constexpr float kMassScale = 1099511627776.0f;  // 2^40
 
-// Largest threshold bits t such that pred(t) holds, pred being monotone
-// (true for small t).  Probabilities are >= 0, so their order as floats is
-// their order as unsigned bit patterns.
-template <typename Pred>
-__device__ __forceinline__ uint32_t bisect_bits(Pred pred) {
-  uint32_t t = 0;
-  for (int bit = 30; bit >= 0; --bit) {
-    const uint32_t cand = t | (1u << bit);
-    if (pred(cand)) t = cand;
-  }
-  return t;
-}
+struct SampleArgs {
+  const float* logits;
+  float* e;  // [rows, vocab]
+  int vocab, chunk_len, chunks;
+  const float* temperature;
+  const int* top_k;
+  const float* top_p;
+  const float* min_p;
+  const float* u;
+  const ArgMax* part_max;          // [rows, chunks]
+  unsigned int* hist_k;            // [rows, 4, 256] counts
+  unsigned long long* hist_p;      // [rows, 4, 256] masses
+  float* chunk_mass;               // [rows, chunks]
+  unsigned int* threshold;         // [rows] bits of the final threshold
+  int use_top_k, use_top_p;        // 0: no row of this call uses the filter (its passes are not launched)
+  int* out;
+};
 
-__global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
-    const float* __restrict__ logits, int vocab, float* __restrict__ probs /* [rows, vocab] */,
-    const float* __restrict__ temperature, const int* __restrict__ top_k,
-    const float* __restrict__ top_p, const float* __restrict__ min_p, const float* __restrict__ u,
-    int* __restrict__ out) {
-  __shared__ ArgMax lds_arg[kSampWaves];
-  __shared__ float lds[kSampWaves];
-  __shared__ float chunk_sum[kSampThreads];
-  __shared__ int chosen;
-  const int row = blockIdx.x;
-  const float* x = logits + static_cast<int64_t>(row) * vocab;
-  float* p = probs + static_cast<int64_t>(row) * vocab;
-  const float temp = temperature[row];
-  const int k = top_k[row];
-  const float tp = top_p[row];
-  const float mp = min_p[row];
+struct RowParams {
+  float inv_t, min_p, top_p;
+  int k;
+  bool greedy, k_active, p_active;
+};
 
+__device__ __forceinline__ RowParams row_params(const SampleArgs& a, int row) {
+  RowParams r;
+  const float temp = a.temperature[row];
+  r.k = a.top_k[row];
+  r.top_p = a.top_p[row];
+  r.min_p = a.min_p[row];
   // Greedy rule of the reference: (T <= 0 or top_k == 1) and no stochastic filter.
-  const bool greedy = (temp <= 0.f || k == 1) && tp >= 1.f && mp <= 0.f;
-  if (greedy) {
-    ArgMax r = row_argmax(x, vocab, lds_arg);
-    if (threadIdx.x == 0) out[row] = r.i;
+  r.greedy = (temp <= 0.f || r.k == 1) && r.top_p >= 1.f && r.min_p <= 0.f;
+  r.inv_t = temp > 0.f ? 1.0f / temp : 1.0f;
+  r.k_active = a.use_top_k && r.k > 0 && r.k < a.vocab;
+  r.p_active = a.use_top_p && r.top_p < 1.f;
+  return r;
+}
+
+__device__ __forceinline__ unsigned long long shfl_u64(unsigned long long v, int src) {
+  const unsigned int lo = __shfl(static_cast<unsigned int>(v), src, kWave);
+  const unsigned int hi = __shfl(static_cast<unsigned int>(v >> 32), src, kWave);
+  return (static_cast<unsigned long long>(hi) << 32) | lo;
+}
+__device__ __forceinline__ unsigned int shfl_any(unsigned int v, int src) { return __shfl(v, src, kWave); }
+__device__ __forceinline__ unsigned long long shfl_any(unsigned long long v, int src) { return shfl_u64(v, src); }
+
+// Digits of the threshold, most significant first, from `levels` histograms [levels][256] (level l holds the
+// elements that match the digits of the levels before it).  need: the rank (the mass) to reach, counted from
+// the top, at least 1.  Every thread of the workgroup calls this; bins is LDS [levels * 256], result LDS [4].
+// Returns false when the whole row does not reach `need` (then everything is kept).  prefix: the digits found,
+// rest: what is left to reach inside the bin of the last digit.
+template <typename T>
+__device__ bool select_digits(const T* __restrict__ hist, int levels, T need, T* bins, unsigned long long* result,
+                              unsigned int& prefix, T& rest) {
+  for (int l = 0; l < levels; ++l) bins[l * 256 + threadIdx.x] = hist[l * 256 + threadIdx.x];
+  __syncthreads();
+  if (threadIdx.x < kWave) {
+    const int lane = threadIdx.x;
+    unsigned int digits = 0;
+    bool ok = true;
+    for (int l = 0; l < levels && ok; ++l) {
+      T m[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) m[j] = bins[l * 256 + 4 * lane + j];
+      const T own = m[0] + m[1] + m[2] + m[3];
+      T suffix = own;  // sum over the bins of this lane and of the lanes above it
+#pragma unroll
+      for (int off = 1; off < kWave; off <<= 1) {
+        const T other = shfl_any(suffix, min(lane + off, kWave - 1));
+        if (lane + off < kWave) suffix += other;
+      }
+      const T above_lane = suffix - own;
+      const bool here = above_lane < need && suffix >= need;
+      unsigned int digit = 0;
+      T left = 0;
+      if (here) {
+        T above = above_lane;
+#pragma unroll
+        for (int j = 3; j >= 0; --j) {
+          if (left == 0 && above + m[j] >= need) {
+            digit = 4 * lane + j;
+            left = need - above;  // >= 1
+          }
+          above += m[j];
+        }
+      }
+      const unsigned long long votes = __ballot(here);
+      if (votes == 0ull) {
+        ok = false;
+      } else {
+        const int src = __ffsll(static_cast<long long>(votes)) - 1;
+        digits = (digits << 8) | shfl_any(digit, src);
+        need = shfl_any(left, src);
+      }
+    }
+    if (lane == 0) {
+      result[0] = ok ? 1ull : 0ull;
+      result[1] = digits;
+      result[2] = static_cast<unsigned long long>(need);
+    }
+  }
+  __syncthreads();
+  prefix = static_cast<unsigned int>(result[1]);
+  rest = static_cast<T>(result[2]);
+  const bool ok = result[0] != 0ull;
+  __syncthreads();  // bins and result may be used again
+  return ok;
+}
+
+struct SelectLds {
+  unsigned long long bins[4 * 256];
+  unsigned long long result[4];
+};
+
+// Bits of the top-k threshold of a row (0: keep everything), from the four count histograms.
+__device__ unsigned int top_k_bits(const SampleArgs& a, int row, const RowParams& r, SelectLds& lds) {
+  if (!r.k_active) return 0u;  // the same for every thread
+  unsigned int prefix, rest;
+  const bool ok = select_digits<unsigned int>(a.hist_k + static_cast<int64_t>(row) * 1024, 4,
+                                              static_cast<unsigned int>(r.k),
+                                              reinterpret_cast<unsigned int*>(lds.bins), lds.result, prefix, rest);
+  return ok ? prefix : 0u;
+}
+
+// The threshold below which min_p and top_k drop a token.
+__device__ unsigned int floor_bits(const SampleArgs& a, int row, const RowParams& r, SelectLds& lds) {
+  const unsigned int mp = r.min_p > 0.f ? __float_as_uint(r.min_p) : 0u;
+  return max(mp, top_k_bits(a, row, r, lds));
+}
+
+// What top_p asks of the kept mass, as a fixed-point number (at least 1).
+__device__ __forceinline__ unsigned long long top_p_need(float top_p, unsigned long long total) {
+  const unsigned long long need = static_cast<unsigned long long>(static_cast<double>(top_p) * static_cast<double>(total));
+  return need < 1ull ? 1ull : need;
+}
+
+__device__ __forceinline__ float merged_max(const SampleArgs& a, int row, float* lds /* [kSelWaves] */) {
+  float v = -INFINITY;
+  for (int c = threadIdx.x; c < a.chunks; c += kSelThreads)
+    v = fmaxf(v, a.part_max[static_cast<int64_t>(row) * a.chunks + c].v);
+  return block_max<kSelWaves>(v, lds);
+}
+
+// e = exp(x / T - max) for the chunk, and the first digit's histogram of top_k.
+__global__ __launch_bounds__(kSelThreads) void sample_exp_kernel(const SampleArgs a) {
+  __shared__ float red[kSelWaves];
+  __shared__ unsigned int hist[256];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const RowParams r = row_params(a, row);
+  if (r.greedy) return;
+  hist[threadIdx.x] = 0u;
+  const float mx = merged_max(a, row, red) * r.inv_t;  // the block reduction also orders the LDS writes above
+  const float* x = a.logits + static_cast<int64_t>(row) * a.vocab;
+  float* e = a.e + static_cast<int64_t>(row) * a.vocab;
+  const int begin = chunk * a.chunk_len, end = min(a.vocab, begin + a.chunk_len);
+  const unsigned int mp = r.min_p > 0.f ? __float_as_uint(r.min_p) : 0u;
+  for (int i = begin + static_cast<int>(threadIdx.x); i < end; i += kSelThreads) {
+    const float v = expf(x[i] * r.inv_t - mx);
+    e[i] = v;
+    const unsigned int bits = __float_as_uint(v);
+    if (r.k_active && v >= 0.f && bits >= mp) atomicAdd(&hist[bits >> 24], 1u);
+  }
+  if (!r.k_active) return;
+  __syncthreads();
+  const unsigned int n = hist[threadIdx.x];
+  if (n) atomicAdd(a.hist_k + static_cast<int64_t>(row) * 1024 + threadIdx.x, n);
+}
+
+// Digit `level` (1..3) of the top_k threshold.
+__global__ __launch_bounds__(kSelThreads) void sample_top_k_kernel(const SampleArgs a, int level) {
+  __shared__ SelectLds sel;
+  __shared__ unsigned int hist[256];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const RowParams r = row_params(a, row);
+  if (r.greedy || !r.k_active) return;
+  unsigned int prefix, rest;
+  const bool ok = select_digits<unsigned int>(a.hist_k + static_cast<int64_t>(row) * 1024, level,
+                                              static_cast<unsigned int>(r.k),
+                                              reinterpret_cast<unsigned int*>(sel.bins), sel.result, prefix, rest);
+  if (!ok) return;  // fewer than k tokens are left: all of them stay
+  hist[threadIdx.x] = 0u;
+  __syncthreads();
+  const float* e = a.e + static_cast<int64_t>(row) * a.vocab;
+  const int begin = chunk * a.chunk_len, end = min(a.vocab, begin + a.chunk_len);
+  const unsigned int mp = r.min_p > 0.f ? __float_as_uint(r.min_p) : 0u;
+  const int high = 32 - 8 * level, low = 24 - 8 * level;
+  for (int i = begin + static_cast<int>(threadIdx.x); i < end; i += kSelThreads) {
+    const float v = e[i];
+    const unsigned int bits = __float_as_uint(v);
+    if (v >= 0.f && bits >= mp && (bits >> high) == prefix) atomicAdd(&hist[(bits >> low) & 255u], 1u);
+  }
+  __syncthreads();
+  const unsigned int n = hist[threadIdx.x];
+  if (n) atomicAdd(a.hist_k + static_cast<int64_t>(row) * 1024 + level * 256 + threadIdx.x, n);
+}
+
+// Digit `level` (0..3) of the top_p threshold, over what min_p and top_k have kept.
+__global__ __launch_bounds__(kSelThreads) void sample_top_p_kernel(const SampleArgs a, int level) {
+  __shared__ SelectLds sel;
+  __shared__ unsigned long long hist[256];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const RowParams r = row_params(a, row);
+  if (r.greedy || !r.p_active) return;
+  const unsigned int floor = floor_bits(a, row, r, sel);
+  const unsigned long long* hp = a.hist_p + static_cast<int64_t>(row) * 1024;
+  unsigned int prefix = 0u;
+  if (level > 0) {
+    // the whole kept mass is the sum of the first histogram
+    sel.bins[threadIdx.x] = hp[threadIdx.x];
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      unsigned long long total = 0ull;
+      for (int b = 0; b < 256; ++b) total += sel.bins[b];
+      sel.result[3] = total;
+    }
+    __syncthreads();
+    const unsigned long long need = top_p_need(r.top_p, sel.result[3]);
+    __syncthreads();
+    unsigned long long rest;
+    if (!select_digits<unsigned long long>(hp, level, need, sel.bins, sel.result, prefix, rest)) return;
+  }
+  hist[threadIdx.x] = 0ull;
+  __syncthreads();
+  const float* e = a.e + static_cast<int64_t>(row) * a.vocab;
+  const int begin = chunk * a.chunk_len, end = min(a.vocab, begin + a.chunk_len);
+  const int high = 32 - 8 * level, low = 24 - 8 * level;
+  for (int i = begin + static_cast<int>(threadIdx.x); i < end; i += kSelThreads) {
+    const float v = e[i];
+    const unsigned int bits = __float_as_uint(v);
+    if (v >= 0.f && bits >= floor && (level == 0 || (bits >> high) == prefix))
+      atomicAdd(&hist[(bits >> low) & 255u], static_cast<unsigned long long>(v * kMassScale));
+  }
+  __syncthreads();
+  const unsigned long long n = hist[threadIdx.x];
+  if (n) atomicAdd(const_cast<unsigned long long*>(hp) + level * 256 + threadIdx.x, n);
+}
+
+// The final threshold of the row and the kept mass of every chunk.
+__global__ __launch_bounds__(kSelThreads) void sample_mass_kernel(const SampleArgs a) {
+  __shared__ SelectLds sel;
+  __shared__ float red[kSelWaves];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const RowParams r = row_params(a, row);
+  if (r.greedy) return;
+  unsigned int thr = floor_bits(a, row, r, sel);
+  if (r.p_active) {
+    const unsigned long long* hp = a.hist_p + static_cast<int64_t>(row) * 1024;
+    sel.bins[threadIdx.x] = hp[threadIdx.x];
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      unsigned long long total = 0ull;
+      for (int b = 0; b < 256; ++b) total += sel.bins[b];
+      sel.result[3] = total;
+    }
+    __syncthreads();
+    const unsigned long long need = top_p_need(r.top_p, sel.result[3]);
+    __syncthreads();
+    unsigned int prefix;
+    unsigned long long rest;
+    if (select_digits<unsigned long long>(hp, 4, need, sel.bins, sel.result, prefix, rest)) thr = max(thr, prefix);
+  }
+  if (chunk == 0 && threadIdx.x == 0) a.threshold[row] = thr;
+  const float* e = a.e + static_cast<int64_t>(row) * a.vocab;
+  const int begin = chunk * a.chunk_len, end = min(a.vocab, begin + a.chunk_len);
+  float mass = 0.f;
+  for (int i = begin + static_cast<int>(threadIdx.x); i < end; i += kSelThreads) {
+    const float v = e[i];
+    if (v >= 0.f && __float_as_uint(v) >= thr) mass += v;
+  }
+  mass = block_sum<kSelWaves>(mass, red);
+  if (threadIdx.x == 0) a.chunk_mass[static_cast<int64_t>(row) * a.chunks + chunk] = mass;
+}
+
+// The token: greedy rows take the first maximum; the others the inverse CDF in token order.
+__global__ __launch_bounds__(kSelThreads) void sample_pick_kernel(const SampleArgs a) {
+  __shared__ ArgMax best[kSelWaves];
+  __shared__ float part[kSelThreads];
+  __shared__ float chunk_start;
+  __shared__ int chunk_of_target, chosen;
+  const int row = blockIdx.x;
+  const RowParams r = row_params(a, row);
+  if (r.greedy) {
+    ArgMax m;
+    m.v = -INFINITY;
+    m.i = 0x7fffffff;
+    for (int c = threadIdx.x; c < a.chunks; c += kSelThreads)
+      m = better(m, a.part_max[static_cast<int64_t>(row) * a.chunks + c]);
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+      ArgMax o;
+      o.v = __shfl_xor(m.v, off, kWave);
+      o.i = __shfl_xor(m.i, off, kWave);
+      m = better(m, o);
+    }
+    if (threadIdx.x % kWave == 0) best[threadIdx.x / kWave] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      ArgMax t = best[0];
+      for (int w = 1; w < kSelWaves; ++w) t = better(t, best[w]);
+      a.out[row] = t.i == 0x7fffffff ? 0 : t.i;
+    }
     return;
   }
-  const float inv_t = temp > 0.f ? 1.0f / temp : 1.0f;
-
-  // softmax(x / T)
-  float mx = -INFINITY;
-  for (int i = threadIdx.x; i < vocab; i += kSampThreads) mx = fmaxf(mx, x[i] * inv_t);
-  mx = block_max<kSampWaves>(mx, lds);
-  float sum = 0.f;
-  for (int i = threadIdx.x; i < vocab; i += kSampThreads) {
-    const float e = expf(x[i] * inv_t - mx);
-    p[i] = e;
-    sum += e;
-  }
-  sum = block_sum_f(sum, lds);
-  float norm = 1.0f / sum;  // pending factor: true probability = p[i] * norm
-  float pmax = norm;        // exp(0) * norm
-
-  auto renormalise = [&](float threshold_true) {
-    // zero what is below the threshold, fold `norm` in, and renormalise the rest
-    float kept = 0.f;
-    for (int i = threadIdx.x; i < vocab; i += kSampThreads) {
-      float v = p[i] * norm;
-      if (v < threshold_true) v = 0.f;
-      p[i] = v;
-      kept += v;
+  const unsigned int thr = a.threshold[row];
+  const float* masses = a.chunk_mass + static_cast<int64_t>(row) * a.chunks;
+  if (threadIdx.x == 0) {
+    float total = 0.f;
+    for (int c = 0; c < a.chunks; ++c) total += masses[c];
+    const float target = a.u[row] * total;
+    float run = 0.f;
+    int at = -1, last = 0;
+    float start = 0.f, last_start = 0.f;
+    for (int c = 0; c < a.chunks; ++c) {
+      const float m = masses[c];
+      if (m > 0.f) {
+        last = c;
+        last_start = run;
+      }
+      if (at < 0 && target < run + m) {
+        at = c;
+        start = run;
+      }
+      run += m;
     }
-    kept = block_sum_f(kept, lds);
-    norm = 1.0f / kept;
-    pmax = pmax * norm;
-  };
-
-  if (mp > 0.f) renormalise(mp * pmax);
-
-  if (k > 0 && k < vocab) {
-    // fold the pending factor in so that thresholds compare stored values
-    for (int i = threadIdx.x; i < vocab; i += kSampThreads) p[i] *= norm;
-    norm = 1.0f;
-    __syncthreads();
-    const uint32_t bits = bisect_bits([&](uint32_t cand) {
-      float cnt = 0.f;
-      for (int i = threadIdx.x; i < vocab; i += kSampThreads)
-        cnt += (__float_as_uint(p[i]) >= cand) ? 1.f : 0.f;
-      return block_sum_f(cnt, lds) >= static_cast<float>(k);
-    });
-    renormalise(__uint_as_float(bits));  // keeps the k largest (and ties of the k-th)
-  }
-
-  if (tp < 1.f) {
-    for (int i = threadIdx.x; i < vocab; i += kSampThreads) p[i] *= norm;
-    norm = 1.0f;
-    __syncthreads();
-    const uint32_t bits = bisect_bits([&](uint32_t cand) {
-      float mass = 0.f;
-      for (int i = threadIdx.x; i < vocab; i += kSampThreads)
-        mass += (__float_as_uint(p[i]) >= cand) ? p[i] : 0.f;
-      return block_sum_f(mass, lds) >= tp;
-    });
-    renormalise(__uint_as_float(bits));  // smallest top set whose mass reaches top_p
+    chunk_of_target = at >= 0 ? at : last;  // u at or past the whole mass (rounding): the last chunk that holds any
+    chunk_start = at >= 0 ? start : last_start;
+    part[0] = target;
+    chosen = -1;
   }
   __syncthreads();
-
-  // inverse CDF in token order: thread i owns tokens [i*chunk, (i+1)*chunk)
-  const int chunk = (vocab + kSampThreads - 1) / kSampThreads;
-  const int lo = min(static_cast<int>(threadIdx.x) * chunk, vocab);
-  const int hi = min(lo + chunk, vocab);
+  const int chunk = chunk_of_target;
+  const float target = part[0];
+  const float before = chunk_start;
+  __syncthreads();
+  const float* e = a.e + static_cast<int64_t>(row) * a.vocab;
+  const int begin = chunk * a.chunk_len, end = min(a.vocab, begin + a.chunk_len);
+  // thread t owns the tokens [lo, hi) of the chunk, in token order
+  const int per = (end - begin + kSelThreads - 1) / kSelThreads;
+  const int lo = min(begin + static_cast<int>(threadIdx.x) * per, end), hi = min(lo + per, end);
+  auto kept = [&](int i) {
+    const float v = e[i];
+    return (v >= 0.f && __float_as_uint(v) >= thr) ? v : 0.f;
+  };
   float mine = 0.f;
-  for (int i = lo; i < hi; ++i) mine += p[i] * norm;
-  chunk_sum[threadIdx.x] = mine;
-  if (threadIdx.x == 0) chosen = -1;
+  for (int i = lo; i < hi; ++i) mine += kept(i);
+  part[threadIdx.x] = mine;
   __syncthreads();
   if (threadIdx.x == 0) {
-    float run = 0.f;  // exclusive prefix, serial: 1024 adds
-    for (int i = 0; i < kSampThreads; ++i) {
-      const float c = chunk_sum[i];
-      chunk_sum[i] = run;
+    float run = before;  // exclusive prefix, serial
+    for (int t = 0; t < kSelThreads; ++t) {
+      const float c = part[t];
+      part[t] = run;
       run += c;
     }
   }
   __syncthreads();
-  const float target = u[row];
-  const float start = chunk_sum[threadIdx.x];
+  const float start = part[threadIdx.x];
   if (target >= start && target < start + mine && hi > lo) {
     float run = start;
     int pick = -1;
     for (int i = lo; i < hi; ++i) {
-      run += p[i] * norm;
+      run += kept(i);
       if (target < run) {
         pick = i;
         break;
       }
     }
-    if (pick < 0) {  // rounding left the target past the chunk's end: last kept token here
+    if (pick < 0) {  // rounding left the target past this thread's end: its last kept token
       for (int i = hi - 1; i >= lo; --i)
-        if (p[i] > 0.f) {
+        if (kept(i) > 0.f) {
           pick = i;
           break;
         }
@@ -280,14 +535,21 @@ __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
   }
   __syncthreads();
   if (chosen < 0) {
-    // u at or beyond the total mass (rounding): the last token with p > 0
+    // the target lies outside what the threads found (rounding between the two ways of adding): the last kept
+    // token of the chunk, or of the row when the chunk holds none
     int last = -1;
-    for (int i = threadIdx.x; i < vocab; i += kSampThreads)
-      if (p[i] > 0.f) last = max(last, i);
-    atomicMax(&chosen, last);
+    for (int i = begin + static_cast<int>(threadIdx.x); i < end; i += kSelThreads)
+      if (kept(i) > 0.f) last = max(last, i);
+    if (last >= 0) atomicMax(&chosen, last);
     __syncthreads();
+    if (chosen < 0) {
+      for (int i = threadIdx.x; i < a.vocab; i += kSelThreads)
+        if (kept(i) > 0.f) last = max(last, i);
+      if (last >= 0) atomicMax(&chosen, last);
+      __syncthreads();
+    }
   }
-  if (threadIdx.x == 0) out[row] = chosen;
+  if (threadIdx.x == 0) a.out[row] = max(chosen, 0);
 }
 
 // logits[row, tok] for each (tok, count) listed for the row:
@@ -317,7 +579,7 @@ using namespace arle;
 // parts: scratch of arle_argmax_chunks(rows, vocab) * rows pairs of 8 bytes, or null when that count is 1.
 extern "C" int arle_argmax_chunks(int rows, int vocab) {
   if (rows <= 0 || vocab < 8192) return 1;
-  const int wanted = (512 + rows - 1) / rows;            // about 512 workgroups in all
+  const int wanted = (2048 + rows - 1) / rows;           // about 2048 workgroups of 256 threads in all
   const int most = vocab / 2048;                         // at least 2048 logits a chunk
   return max(1, min(min(wanted, most), 256));
 }
@@ -338,14 +600,61 @@ extern "C" int arle_argmax_rows(const float* logits, int rows, int vocab, int* o
   return launch_status();
 }
 
-// probs is scratch [rows, vocab] 32-bit; each listed token id must appear once per row in
-// the penalty lists.
+// Scratch of a sampling call, in bytes: the histograms (which the caller hands over filled with zeros: the whole
+// scratch may simply be zeroed), the chunk maxima and masses, and the thresholds.
+static inline size_t sample_hist_p_bytes(int rows) { return static_cast<size_t>(rows) * 1024 * sizeof(unsigned long long); }
+static inline size_t sample_hist_k_bytes(int rows) { return static_cast<size_t>(rows) * 1024 * sizeof(unsigned int); }
+extern "C" long long arle_sample_scratch_bytes(int rows, int vocab) {
+  const size_t chunks = static_cast<size_t>(arle_argmax_chunks(rows, vocab));
+  return static_cast<long long>(sample_hist_p_bytes(rows) + sample_hist_k_bytes(rows) +
+                                rows * chunks * (sizeof(ArgMax) + sizeof(float)) + rows * sizeof(unsigned int));
+}
+
+// One token id per row of logits [rows, vocab] (float32).  probs is scratch [rows, vocab] float32; scratch holds
+// arle_sample_scratch_bytes(rows, vocab) zeroed bytes, 8-byte aligned.  use_top_k / use_top_p == 0 promise that
+// no row of the call has the filter switched on (top_k in 1..vocab-1, top_p < 1); its passes are then left out.
 extern "C" int arle_sample_rows(const float* logits, int rows, int vocab, float* probs,
                                 const float* temperature, const int* top_k, const float* top_p,
-                                const float* min_p, const float* u, int* out, void* stream) {
+                                const float* min_p, const float* u, int* out, void* scratch, int use_top_k,
+                                int use_top_p, void* stream) {
   if (rows == 0) return 0;
-  sample_rows_kernel<<<rows, kSampThreads, 0, static_cast<hipStream_t>(stream)>>>(
-      logits, vocab, probs, temperature, top_k, top_p, min_p, u, out);
+  if (scratch == nullptr || reinterpret_cast<uintptr_t>(scratch) % 8 != 0 || rows > 65535)
+    return static_cast<int>(hipErrorInvalidValue);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SampleArgs a;
+  a.logits = logits;
+  a.e = probs;
+  a.vocab = vocab;
+  a.chunks = arle_argmax_chunks(rows, vocab);
+  a.chunk_len = (((vocab + a.chunks - 1) / a.chunks) + 3) & ~3;
+  a.temperature = temperature;
+  a.top_k = top_k;
+  a.top_p = top_p;
+  a.min_p = min_p;
+  a.u = u;
+  unsigned char* at = static_cast<unsigned char*>(scratch);
+  a.hist_p = reinterpret_cast<unsigned long long*>(at);
+  at += sample_hist_p_bytes(rows);
+  a.hist_k = reinterpret_cast<unsigned int*>(at);
+  at += sample_hist_k_bytes(rows);
+  ArgMax* part_max = reinterpret_cast<ArgMax*>(at);
+  a.part_max = part_max;
+  at += static_cast<size_t>(rows) * a.chunks * sizeof(ArgMax);
+  a.chunk_mass = reinterpret_cast<float*>(at);
+  at += static_cast<size_t>(rows) * a.chunks * sizeof(float);
+  a.threshold = reinterpret_cast<unsigned int*>(at);
+  a.use_top_k = use_top_k;
+  a.use_top_p = use_top_p;
+  a.out = out;
+  const dim3 grid(a.chunks, rows);
+  argmax_chunks_kernel<<<grid, kChunkThreads, 0, s>>>(logits, vocab, a.chunk_len, part_max);
+  sample_exp_kernel<<<grid, kSelThreads, 0, s>>>(a);
+  if (use_top_k)
+    for (int level = 1; level < 4; ++level) sample_top_k_kernel<<<grid, kSelThreads, 0, s>>>(a, level);
+  if (use_top_p)
+    for (int level = 0; level < 4; ++level) sample_top_p_kernel<<<grid, kSelThreads, 0, s>>>(a, level);
+  sample_mass_kernel<<<grid, kSelThreads, 0, s>>>(a);
+  sample_pick_kernel<<<rows, kSelThreads, 0, s>>>(a);
   return launch_status();
 }
 

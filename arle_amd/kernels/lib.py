@@ -37,7 +37,8 @@ SIGNATURES = {
                                                 _i, _i, _i, _f, _i, _i, _p, _p, _p]),
     "arle_argmax_chunks": ("sampling", [_i, _i]),
     "arle_argmax_rows": ("sampling", [_p, _i, _i, _p, _p, _p]),
-    "arle_sample_rows": ("sampling", [_p, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p]),
+    "arle_sample_scratch_bytes": ("sampling", [_i, _i]),
+    "arle_sample_rows": ("sampling", [_p, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _p]),
     "arle_apply_penalties": ("sampling", [_p, _i, _i, _p, _p, _p, _p, _p, _p, _p]),
 }
 

@@ -407,8 +407,20 @@ def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def sample_rows(logits, temperature, top_k, top_p, min_p, u) -> torch.Tensor:
-    """One token id per row; per-row float32 temperature/top_p/min_p/u and int32 top_k."""
+@functools.lru_cache(maxsize=None)
+def _sample_scratch_bytes(rows: int, vocab: int) -> int:
+    fn = lib.function("arle_sample_scratch_bytes")
+    fn.restype = ctypes.c_longlong
+    return int(fn(rows, vocab))
+
+
+def sample_rows(logits, temperature, top_k, top_p, min_p, u, *, use_top_k: bool = True,
+                use_top_p: bool = True) -> torch.Tensor:
+    """One token id per row; per-row float32 temperature/top_p/min_p/u and int32 top_k.
+
+    use_top_k / use_top_p = False promise that no row has that filter switched on (top_k in 1..vocab-1,
+    top_p < 1): the passes over the row that look for its threshold are then not launched.
+    """
     rows, vocab = _logits(logits)
     for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
                         ("top_p", top_p, torch.float32), ("min_p", min_p, torch.float32),
@@ -417,9 +429,12 @@ def sample_rows(logits, temperature, top_k, top_p, min_p, u) -> torch.Tensor:
         _need(t.dtype == dt and t.shape == (rows,) and t.is_contiguous(), f"{name} must be {dt} [rows]")
     probs = torch.empty((rows, vocab), dtype=torch.float32, device=logits.device)
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    words = -(-_sample_scratch_bytes(rows, vocab) // 8)
+    scratch = torch.zeros((words,), dtype=torch.int64, device=logits.device)   # histograms start at zero
     lib.call("arle_sample_rows", logits.data_ptr(), rows, vocab, probs.data_ptr(),
              temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), min_p.data_ptr(),
-             u.data_ptr(), out.data_ptr(), _stream())
+             u.data_ptr(), out.data_ptr(), scratch.data_ptr(), int(bool(use_top_k)), int(bool(use_top_p)),
+             _stream())
     return out
 
 

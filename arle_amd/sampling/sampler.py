@@ -12,6 +12,7 @@ is not kept.
 """
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from ..kernels import ops
@@ -48,14 +49,18 @@ class Sampler:
             self._penalise(logits, rows)
         if all(p.is_greedy() for p, _, _, _ in rows):
             return ops.argmax_rows(logits).tolist()
-        f32 = lambda vals: torch.tensor(vals, dtype=torch.float32, device=self.device)
-        out = ops.sample_rows(
-            logits,
-            f32([p.temperature for p, _, _, _ in rows]),
-            torch.tensor([p.top_k for p, _, _, _ in rows], dtype=torch.int32, device=self.device),
-            f32([p.top_p for p, _, _, _ in rows]),
-            f32([p.min_p for p, _, _, _ in rows]),
-            f32([uniform(seed, idx) for _, seed, idx, _ in rows]))
+        # one host->device copy for the five per-row arrays (top_k travels as the bits of an int32)
+        n, vocab = len(rows), logits.shape[1]
+        packed = np.empty((5, n), dtype=np.float32)
+        packed[0] = [p.temperature for p, _, _, _ in rows]
+        packed[1] = [p.top_p for p, _, _, _ in rows]
+        packed[2] = [p.min_p for p, _, _, _ in rows]
+        packed[3] = [uniform(seed, idx) for _, seed, idx, _ in rows]
+        packed[4].view(np.int32)[:] = [p.top_k for p, _, _, _ in rows]
+        dev = torch.from_numpy(packed).to(self.device)
+        out = ops.sample_rows(logits, dev[0], dev[4].view(torch.int32), dev[1], dev[2], dev[3],
+                              use_top_k=any(0 < p.top_k < vocab for p, _, _, _ in rows),
+                              use_top_p=any(p.top_p < 1.0 for p, _, _, _ in rows))
         return out.tolist()
 
     def _penalise(self, logits, rows) -> None:

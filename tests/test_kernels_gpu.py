@@ -370,6 +370,42 @@ def test_sampling_against_plain_inverse_cdf(vocab):
             assert got == want, (case, u)
 
 
+@pytest.mark.parametrize("rows,vocab", [(3, 151936), (9, 50257), (70, 8200)])
+def test_sampling_of_long_rows_cut_into_chunks(rows, vocab):
+    """Vocabularies long enough for several workgroups a row, widths that leave rows unaligned, rows that differ
+    in every parameter (greedy ones among them), and filters switched off for the whole call."""
+    g = _g(61)
+    logits = torch.randn(rows, vocab, generator=g) * 2.5
+    logits[0, vocab - 1] = 14.0                 # a peaked row: top_p keeps one token
+    logits[1, :4] = 9.0                         # ties at the top
+    pars = [dict(temperature=0.9, top_k=40, top_p=0.9, min_p=0.02), dict(temperature=1.2, top_k=3),
+            dict(temperature=0.0), dict(temperature=0.7, top_p=0.35), dict(temperature=1.0, min_p=0.1),
+            dict(temperature=1.5), dict(temperature=0.8, top_k=1), dict(temperature=1.0, top_k=vocab + 5, top_p=0.999),
+            dict(temperature=0.6, top_k=500, top_p=0.5)]
+    pars = [pars[i % len(pars)] for i in range(rows)]
+    f32 = lambda key, default: torch.tensor([p.get(key, default) for p in pars], dtype=torch.float32, device=DEV)
+    top_k = torch.tensor([p.get("top_k", -1) for p in pars], dtype=torch.int32, device=DEV)
+    check = range(rows) if rows <= 9 else range(0, rows, 7)
+    for u in (0.0, 0.31, 0.62, 0.9995):
+        us = torch.full((rows,), u, dtype=torch.float32, device=DEV)
+        got = ops.sample_rows(logits.to(DEV), f32("temperature", 1.0), top_k, f32("top_p", 1.0), f32("min_p", 0.0),
+                              us).tolist()
+        for r in check:
+            p = pars[r]
+            want = plain.sample_token(logits[r], p["temperature"], u, p.get("top_k", -1), p.get("top_p", 1.0),
+                                      p.get("min_p", 0.0))
+            assert got[r] == want, (r, p, u)
+    # no row with top_k or top_p: the passes that look for their thresholds are left out
+    plain_rows = [dict(temperature=0.9), dict(temperature=1.1, min_p=0.05), dict(temperature=0.0)]
+    pars = [plain_rows[i % 3] for i in range(rows)]
+    us = torch.full((rows,), 0.44, dtype=torch.float32, device=DEV)
+    got = ops.sample_rows(logits.to(DEV), f32("temperature", 1.0), torch.full((rows,), -1, dtype=torch.int32, device=DEV),
+                          f32("top_p", 1.0), f32("min_p", 0.0), us, use_top_k=False, use_top_p=False).tolist()
+    for r in check:
+        p = pars[r]
+        assert got[r] == plain.sample_token(logits[r], p["temperature"], 0.44, -1, 1.0, p.get("min_p", 0.0)), (r, p)
+
+
 def test_penalties():
     logits = torch.tensor([[2.0, -2.0, 1.0, 0.5], [1.0, 1.0, 1.0, 1.0]])
     d = logits.to(DEV)
