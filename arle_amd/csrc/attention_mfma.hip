@@ -57,6 +57,9 @@ struct AttnArgs {
   int window;  // 0: all earlier keys
   int splits;
   int ws_rows;   // token rows that the split-KV workspace holds for a segment
+  int portion_splits;  // parts into which the LDS kernel cuts the keys of a row block (1: whole; it writes out)
+  float* pws_o;        // [token row][q head][part][D]   (portion_splits > 1)
+  float* pws_ml;       // [token row][q head][part][2]
   int rows_max;  // the streaming kernel skips segments with more rows than this (0: takes all)
 };
 
@@ -477,15 +480,17 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
   const int G = a.nq / a.nkv;
   const unsigned int nkv = static_cast<unsigned int>(a.nkv);
   const unsigned int pairs = listed ? g_prefill_pairs : static_cast<unsigned int>(blocks_x) * segments;
-  const unsigned int items = pairs * nkv;
+  const unsigned int parts = static_cast<unsigned int>(a.portion_splits);
+  const unsigned int items = pairs * nkv * parts;
  for (;;) {  // one item per round; every wave of the workgroup leaves at the same round
   if (tid == 0) item_of_workgroup = atomicAdd(&g_prefill_next_item, 1u);
   __syncthreads();
   const unsigned int item = item_of_workgroup;
   __syncthreads();  // everyone has read it before thread 0 asks for the next
   if (item >= items) return;
-  const unsigned int pair = item / nkv;
-  const int kvh = static_cast<int>(item % nkv);
+  const unsigned int pair = item / (nkv * parts);
+  const int kvh = static_cast<int>((item / parts) % nkv);
+  const int part = static_cast<int>(item % parts);
   // the last rows of a segment see the most keys: they are handed out first
   int seg = static_cast<int>(pair % segments), wg_row = (blocks_x - 1 - static_cast<int>(pair / segments)) * kPfRows;
   if (listed) {
@@ -514,7 +519,12 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
   const int kv_total = start + qlen;
   const int kv_hi = start + tok_max + 1;
   const int kv_lo = a.window > 0 ? max(0, start + tok_min - a.window + 1) : 0;
-  const int t0 = kv_lo / kPfKeys, t1 = (kv_hi + kPfKeys - 1) / kPfKeys;
+  int t0 = kv_lo / kPfKeys, t1 = (kv_hi + kPfKeys - 1) / kPfKeys;
+  if (parts > 1) {  // this workgroup takes one part of the tiles (it may be empty) and leaves partial results
+    const int per = (t1 - t0 + static_cast<int>(parts) - 1) / static_cast<int>(parts);
+    t0 = t0 + part * per;
+    t1 = min(t0 + per, t1);
+  }
 
   // this wave's rows
   const int row_begin = wg_row + 16 * NT * wave;
@@ -784,6 +794,19 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
 #pragma unroll
   for (int n = 0; n < NT; ++n) {
     if (!row_ok[n]) continue;
+    if (parts > 1) {  // unnormalised sums and the statistics of this part, for attn_merge_portions_kernel
+      const int64_t slot = ((static_cast<int64_t>(row0 + my_tok[n]) * a.nq + my_head[n]) * parts + part);
+      float* wo = a.pws_o + slot * D;
+#pragma unroll
+      for (int dt = 0; dt < DTL; ++dt)
+        if (EXACT || dt < n_dt)
+          *reinterpret_cast<float4*>(wo + 16 * dt + 4 * g) = float4{acc[n][dt][0], acc[n][dt][1], acc[n][dt][2], acc[n][dt][3]};
+      if (g == 0) {
+        a.pws_ml[slot * 2] = m[n];
+        a.pws_ml[slot * 2 + 1] = l[n];
+      }
+      continue;
+    }
     const float inv_l = l[n] > 0.f ? 1.0f / l[n] : 0.f;
     uint16_t* op = a.out + static_cast<int64_t>(row0 + my_tok[n]) * a.o_stride + my_head[n] * D;
 #pragma unroll
@@ -799,6 +822,55 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
     }
   }
  }  // next item
+}
+
+// The parts of a portion's rows put together: out = sum_p o_p 2^(m_p - m) / sum_p l_p 2^(m_p - m), in the order
+// of the parts.  One workgroup per listed (row block, segment) pair and kv head; a wave takes every eighth row,
+// a lane four columns of it (head_dim <= 256).
+constexpr int kPortionPartsMax = 8;
+__global__ __launch_bounds__(kPfWaves* kWave) void attn_merge_portions_kernel(const AttnArgs a) {
+  if (blockIdx.x >= g_prefill_pairs) return;
+  const unsigned int entry = g_prefill_plan[blockIdx.x];
+  const int seg = static_cast<int>(entry & 0xffffu), wg_row = static_cast<int>(entry >> 16) * kPfRows;
+  const int kvh = blockIdx.y, G = a.nq / a.nkv, D = a.D, parts = a.portion_splits;
+  const int row0 = a.seg_row0[seg];
+  const int rows = (a.seg_row0[seg + 1] - row0) * G;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int d0 = 4 * lane;
+  for (int row = wg_row + wave; row < min(wg_row + kPfRows, rows); row += kPfWaves) {
+    const int head = kvh * G + row % G;
+    const int64_t tok_row = row0 + row / G;
+    const int64_t base = (tok_row * a.nq + head) * parts;
+    float ms[kPortionPartsMax], ls[kPortionPartsMax];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int p = 0; p < kPortionPartsMax; ++p) {
+      const float2 ml = *reinterpret_cast<const float2*>(a.pws_ml + (base + min(p, parts - 1)) * 2);
+      ms[p] = p < parts ? ml.x : -INFINITY;
+      ls[p] = p < parts ? ml.y : 0.f;
+      mx = fmaxf(mx, ms[p]);
+    }
+    float denom = 0.f;
+    float4 o = {0.f, 0.f, 0.f, 0.f};
+    const float* src = a.pws_o + base * D + (d0 < D ? d0 : 0);
+#pragma unroll
+    for (int p = 0; p < kPortionPartsMax; ++p) {
+      const float w = ms[p] > -INFINITY ? exp2f(ms[p] - mx) : 0.f;  // an empty part weighs nothing
+      denom += ls[p] * w;
+      const float4 v = *reinterpret_cast<const float4*>(src + static_cast<int64_t>(min(p, parts - 1)) * D);
+      o.x += v.x * w;
+      o.y += v.y * w;
+      o.z += v.z * w;
+      o.w += v.w * w;
+    }
+    const float inv = denom > 0.f ? 1.0f / denom : 0.f;
+    if (d0 < D) {
+      uint2 w;
+      w.x = static_cast<uint32_t>(f32_to_bf16_bits(o.x * inv)) | (static_cast<uint32_t>(f32_to_bf16_bits(o.y * inv)) << 16);
+      w.y = static_cast<uint32_t>(f32_to_bf16_bits(o.z * inv)) | (static_cast<uint32_t>(f32_to_bf16_bits(o.w * inv)) << 16);
+      *reinterpret_cast<uint2*>(a.out + tok_row * a.o_stride + head * D + d0) = w;
+    }
+  }
 }
 
 template <int NT>
@@ -840,14 +912,17 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
       n = 256;
     cus = n;
   }
-  const long long items = static_cast<long long>(grid.x) * grid.y * grid.z;
+  const long long items = static_cast<long long>(grid.x) * grid.y * grid.z * a.portion_splits;
   const int per_cu = 1;  // eight waves: two on every SIMD, with all the registers they want
   const unsigned workgroups = static_cast<unsigned>(items < static_cast<long long>(per_cu) * cus ? items : per_cu * cus);
   const int listed = static_cast<long long>(grid.x) * grid.z <= kPfPlanMax && grid.x <= 65535 && grid.z <= 65535;
   attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
                                              a.nq / a.nkv, min_rows, listed);
+  if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);  // the merge walks the list
   attn_prefill_lds_kernel<DMAX, EXACT><<<workgroups, kPfWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
                                                                                 static_cast<int>(grid.z), listed);
+  if (a.portion_splits > 1)
+    attn_merge_portions_kernel<<<dim3(grid.x * grid.z, grid.y), kPfWaves * kWave, 0, s>>>(a);
   return launch_status();
 }
 
@@ -868,7 +943,9 @@ extern "C" int arle_attn_ws_rows(int max_qlen, int nq, int nkv) {
 // the keys and values of these tokens.  max_qlen / min_qlen are the longest and shortest segment.  With splits > 1,
 // ws_o/ws_ml must hold [segments * ws_rows][nq][splits][D] and [..][2] floats, ws_rows = arle_attn_ws_rows(...),
 // and the merge runs after; the split is over the keys of segments of at most 16 rows (decoded tokens and
-// portions of a few tokens); longer portions, which the LDS kernel takes, have rows enough to fill the chip.
+// portions of a few tokens).  Longer portions go to the LDS kernel; when they have too few row blocks to fill
+// the chip, portion_splits > 1 cuts the keys of every row block into that many parts (at most 8), pws_o/pws_ml
+// must hold [token rows][nq][portion_splits][D] and [..][2] floats, and a merge of their own runs after.
 // Requires D % 16 == 0, D <= 256, page_size a power of two >= 4.
 extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out, long long o_stride,
                                     const void* k_pages, const void* v_pages, const int* block_table,
@@ -876,10 +953,12 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
                                     const int* seg_start, int segments, int max_qlen, int min_qlen,
                                     int token_rows,
                                     int nq, int nkv, int D, int page_size, float scale, int window,
-                                    int splits, float* ws_o, float* ws_ml, void* stream) {
+                                    int splits, float* ws_o, float* ws_ml, int portion_splits, float* pws_o,
+                                    float* pws_ml, void* stream) {
   if (segments == 0 || token_rows == 0) return 0;
   if (D % 16 != 0 || D > 256 || D <= 0 || page_size < 4 || (page_size & (page_size - 1)) != 0 || nq % nkv != 0 ||
-      splits < 1 || splits > 64)
+      splits < 1 || splits > 64 || portion_splits < 1 || portion_splits > kPortionPartsMax ||
+      (portion_splits > 1 && (pws_o == nullptr || pws_ml == nullptr)))
     return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   AttnArgs a;
@@ -905,6 +984,9 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
   a.window = window;
   a.splits = splits;
   a.ws_rows = arle_attn_ws_rows(max_qlen, nq, nkv);
+  a.portion_splits = portion_splits;
+  a.pws_o = pws_o;
+  a.pws_ml = pws_ml;
   a.rows_max = 0;
   const int G = nq / nkv;
   const int max_rows = max_qlen * G, min_rows = min_qlen * G;

@@ -79,7 +79,9 @@ class Engine:
         self.max_request_tokens = max_request_tokens
         self.steps_run = 0
         self.use_graphs = bool(cuda_graph) and self.model.graph_safe
-        self._graphs: dict = {}       # (rows, split cap) -> _DecodeGraph
+        self._graphs: dict = {}       # (rows, split cap) or a step shape -> (graph, input buffer, logits)
+        self._shapes_seen: set = set()
+        self.max_graphs = 64          # captured steps kept (each holds its activations)
         self._graph_pool = None
         self.graph_replays = 0
 
@@ -130,8 +132,11 @@ class Engine:
                 raise EngineError(f"request {e.request!r} is not live; add_request it first")
         before = {e.request: self.cache.length(e.request) for e in entries}
         decode_only = self.use_graphs and all(len(e.tokens) == 1 for e in entries)
+        shape_key = None if decode_only or not self.use_graphs else self._repeated_shape(entries, before)
         batch = None
-        if not decode_only:
+        if shape_key is not None:
+            pass    # packed inside the captured path, like a decode step
+        elif not decode_only:
             batch = build_step_batch(entries, self.cache.slot_of.__getitem__, self.cache.length,
                                      self.spec.vocab_size, self.device)
         else:   # the packing inside the captured path checks the token ids; on an error the lengths are rolled back
@@ -148,6 +153,8 @@ class Engine:
             self.cache.sync_tables()
             if decode_only:
                 logits = self._decode_step_graphed(entries, before)
+            elif shape_key is not None:
+                logits = self._step_graphed(shape_key, entries, before)
             else:
                 logits = self.model.forward(batch, self.cache)
         except Exception:
@@ -200,6 +207,62 @@ class Engine:
         if wanted == list(range(rows)):
             return logits
         return logits[torch.tensor(wanted, dtype=torch.long, device=self.device)]
+
+    # -- captured steps of any shape ---------------------------------------------------------------
+    def _repeated_shape(self, entries, before):
+        """Key of this step's launch shape if a step of the same shape has been seen before, else None.
+
+        Every launch of a step is fixed by the lengths of its entries (in order), by how many logits are
+        wanted, and by the cap that the longest context puts on the split-KV factor of its short entries.
+        Serving repeats shapes (equal portions of a long prompt; the same decoded tokens beside them), and
+        for a small step the host needs longer to launch the kernels one by one than the GPU to run them:
+        from its second occurrence on a shape is run from a captured graph.
+        """
+        lens = tuple(len(e.tokens) for e in entries)
+        if not lens or min(lens) == 0:
+            return None
+        max_kv = max(before[e.request] + len(e.tokens) for e in entries)
+        key = (lens, sum(len(e.want) for e in entries), ops.decode_split_cap(max_kv))
+        if key in self._graphs:
+            return key
+        if len(self._shapes_seen) > 4096:
+            self._shapes_seen.clear()
+        seen = key in self._shapes_seen
+        self._shapes_seen.add(key)
+        return key if seen else None
+
+    def _step_graphed(self, key, entries, before) -> torch.Tensor:
+        """A step whose shape repeats, through a HIP graph captured for that shape (see _repeated_shape).
+
+        As for decode steps, what varies (token ids, positions, slots, wanted rows) travels in the graph's
+        fixed input buffer.  The least recently used graph goes when there are too many.
+        """
+        length_before = before.__getitem__
+        slot_of = self.cache.slot_of.__getitem__
+        rec = self._graphs.pop(key, None)
+        if rec is None:
+            tokens, wanted = sum(key[0]), key[1]
+            static = torch.empty(packed_size(tokens, len(entries), wanted), dtype=torch.int32, device=self.device)
+            batch = build_step_batch(entries, slot_of, length_before, self.spec.vocab_size, self.device, into=static)
+            self._prepare_for_positions(self.max_request_tokens)
+            logits = self.model.forward(batch, self.cache)   # this step's result, and the warm-up
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                static_logits = self.model.forward(batch, self.cache)
+            rec = (graph, static, static_logits)
+            while len(self._graphs) >= self.max_graphs:
+                self._graphs.pop(next(iter(self._graphs)))
+        else:
+            graph, static, static_logits = rec
+            build_step_batch(entries, slot_of, length_before, self.spec.vocab_size, self.device, into=static)
+            graph.replay()
+            self.graph_replays += 1
+            logits = static_logits.clone()
+        self._graphs[key] = rec    # most recently used last
+        return logits
 
     def _prepare_for_positions(self, n: int) -> None:
         """Grow every position table to n positions now, so that no captured step has to."""

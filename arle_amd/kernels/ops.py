@@ -32,7 +32,14 @@ def _code(t: torch.Tensor) -> int:
         raise ShapeError(f"unsupported element type {t.dtype}; kernels take float32 and bfloat16")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """Handle of the current stream of the current device (the raw call is many times cheaper than building a
+    Stream object, and this runs once per kernel launch)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -330,16 +337,52 @@ def decode_splits(segments: int, num_kv_heads: int, max_kv_len: int) -> int:
     return max(1, min(-(-_MFMA_TARGET_WAVES // (segments * num_kv_heads)), decode_split_cap(max_kv_len)))
 
 
+_PORTION_SPLITS_MAX = 8         # parts into which the keys of a portion's row block may be cut
+_PORTION_ROWS = 128             # rows of a row block of the portions kernel
+_PORTION_LIST_MAX = 16384       # (row block, segment) pairs that its work list holds
+_PORTION_WS_BYTES = 256 << 20   # most memory for the parts
+
+
+@functools.lru_cache(maxsize=None)
+def _compute_units(device_index: int) -> int:
+    return int(torch.cuda.get_device_properties(device_index).multi_processor_count)
+
+
+def portion_key_splits(tokens: int, max_qlen: int, long_segments: int, num_q_heads: int, num_kv_heads: int,
+                       head_dim: int, max_kv_len: int, device) -> int:
+    """Into how many parts the keys of every row block of a prompt portion are cut.
+
+    The portions kernel gives a row block of 128 rows (tokens x q heads of a kv head) to a workgroup.  A short
+    portion has fewer row blocks than the chip has compute units, however long its context: then the keys are
+    cut too, each part at least 256 keys long, and the parts are merged afterwards.  The number depends on the
+    shape of the step and on the power-of-two class of the longest context only, like the split of decoded
+    tokens, so that a captured step and an eager one choose alike.
+    """
+    group = num_q_heads // num_kv_heads
+    blocks = -(-max_qlen * group // _PORTION_ROWS)
+    items = blocks * num_kv_heads * max(1, long_segments)
+    units = _compute_units(device.index if device.index is not None else torch.cuda.current_device())
+    if items >= units or blocks * max(1, long_segments) > _PORTION_LIST_MAX:
+        return 1
+    most = max(1, decode_split_cap(max_kv_len) // 4)
+    parts = min(-(-units // items), _PORTION_SPLITS_MAX, most)
+    while parts > 1 and tokens * num_q_heads * parts * (head_dim + 2) * 4 > _PORTION_WS_BYTES:
+        parts -= 1
+    return parts
+
+
 def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *,
                     max_qlen: int, max_kv_len: int, num_q_heads: int, num_kv_heads: int, head_dim: int,
                     page_size: int, scale: float, window: int = 0, splits: int | None = None,
-                    min_qlen: int = 1, short_segments: int | None = None):
+                    min_qlen: int = 1, short_segments: int | None = None, portion_splits: int | None = None):
     """Causal attention of a packed step on the matrix cores (bfloat16).
 
     Segments: rows seg_row0[s]..seg_row0[s+1] belong to block-table row seg_slot[s] and start at
     position seg_start[s].  Segments whose rows (tokens x q heads of a kv head) fit one row tile of 16,
     decoded tokens above all, are split over the keys (split-KV), also beside longer portions in one
     step; `short_segments` says how many there are (default: all), which sets the number of splits.
+    Longer portions that are too few to fill the chip have their keys cut into `portion_splits` parts
+    (default: portion_key_splits).
     """
     _gpu(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start)
     tokens = q.shape[0]
@@ -372,12 +415,23 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
         ws_rows = segments * max(1, min(max_qlen, _ATTN_ROW_TILE // group))   # arle_attn_ws_rows a segment
         ws_o = torch.empty((ws_rows, num_q_heads, splits, head_dim), dtype=torch.float32, device=q.device)
         ws_ml = torch.empty((ws_rows, num_q_heads, splits, 2), dtype=torch.float32, device=q.device)
+    if portion_splits is None:
+        long_segments = segments if short_segments is None else max(1, segments - short_segments)
+        portion_splits = portion_key_splits(tokens, max_qlen, long_segments, num_q_heads, num_kv_heads, head_dim,
+                                            max_kv_len, q.device)
+    if max_qlen * group <= _ATTN_ROW_TILE:
+        portion_splits = 1              # no portion for the kernel that they are for
+    _need(1 <= portion_splits <= _PORTION_SPLITS_MAX, f"portion_splits must be 1..{_PORTION_SPLITS_MAX}")
+    pws_o = pws_ml = None
+    if portion_splits > 1:
+        pws_o = torch.empty((tokens, num_q_heads, portion_splits, head_dim), dtype=torch.float32, device=q.device)
+        pws_ml = torch.empty((tokens, num_q_heads, portion_splits, 2), dtype=torch.float32, device=q.device)
     lib.call("arle_attn_paged_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
              k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
              seg_row0.data_ptr(), seg_slot.data_ptr(), seg_start.data_ptr(), segments, int(max_qlen),
              int(min_qlen), tokens,
              num_q_heads, num_kv_heads, head_dim, page_size, float(scale), int(window), int(splits),
-             _ptr(ws_o), _ptr(ws_ml), _stream())
+             _ptr(ws_o), _ptr(ws_ml), int(portion_splits), _ptr(pws_o), _ptr(pws_ml), _stream())
     return out
 
 

@@ -116,3 +116,36 @@ def test_captured_decode_steps_equal_eager_ones_on_every_replay(model, dtype):
     assert graphed.graph_replays >= 10
     for key in a:
         assert torch.equal(a[key], b[key]), f"graph replay differs from the eager step at {key}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_steps_of_repeated_shapes_equal_eager_ones(model, dtype):
+    """A step shape that repeats (equal portions of prompts, the same decoded tokens beside a portion) runs from
+    a captured graph from its second occurrence on.  Every replay, with steps of other shapes, requests that
+    end (pages used again) and synchronisations in between, must give the bits of the eager engine."""
+    name, d, cfg, _ = model
+    reqs = _requests(cfg, [90, 61, 75, 48], 950)
+    make = lambda graphs: Engine.from_folder(d, dtype=dtype, page_size=TINY[name][1], max_tokens=256, max_slots=4,
+                                             cuda_graph=graphs)
+    eager, graphed = make(False), make(True)
+    r = {k: list(v) for k, v in reqs.items()}
+    steps = []
+    # r0 in portions of 12 (the same shape seven times), logits wanted at every portion's end
+    for a in range(0, 84, 12):
+        steps.append({"entries": [("r0", r["r0"][a:a + 12], [11])], "end": []})
+    # r1 whole, then r0 and r1 decode beside portions of 10 of r2: the shape (1, 1, 10) repeats
+    steps.append({"entries": [("r1", r["r1"][:55], [54])], "end": []})
+    for i in range(6):
+        steps.append({"entries": [("r0", [r["r0"][84 + i]], [0]), ("r1", [r["r1"][55 + i]], [0]),
+                                  ("r2", r["r2"][10 * i:10 * i + 10], [3, 9])], "end": []})
+    steps[-1]["end"] = ["r0", "r1"]
+    # pages of r0 and r1 are used again by r3, in portions of 12 (the first shape, replayed once more)
+    for a in range(0, 48, 12):
+        steps.append({"entries": [("r3", r["r3"][a:a + 12], [11])], "end": []})
+    steps.append({"entries": [("r2", r["r2"][60:75], [14])], "end": ["r2", "r3"]})
+    a = replay.run_steps(eager, steps)
+    b = replay.run_steps(graphed, steps)
+    assert graphed.graph_replays >= 12
+    assert set(a) == set(b)
+    for key in a:
+        assert torch.equal(a[key], b[key]), f"graph replay differs from the eager step at {key}"

@@ -427,7 +427,7 @@ def test_kernels_refuse_what_they_were_not_written_for():
         ops.embed_gather(torch.zeros(4, 4, device=DEV), torch.zeros(2, dtype=torch.int64, device=DEV))
 
 
-def _mfma_case(nq, nkv, D, P, segs, window, splits, seed):
+def _mfma_case(nq, nkv, D, P, segs, window, splits, seed, portion_splits=None):
     """segs: [(cached length before the step, rows in the step)].  Returns (got, want) [T, nq*D]."""
     dt = torch.bfloat16
     lengths = [a + b for a, b in segs]
@@ -451,7 +451,7 @@ def _mfma_case(nq, nkv, D, P, segs, window, splits, seed):
     ops.attn_paged_mfma(q_all, out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0),
                         i32(list(range(len(segs)))), i32(seg_start), max_qlen=max(n for _, n in segs), min_qlen=min(n for _, n in segs),
                         max_kv_len=max(lengths), num_q_heads=nq, num_kv_heads=nkv, head_dim=D, page_size=P,
-                        scale=1.0 / math.sqrt(D), window=window, splits=splits)
+                        scale=1.0 / math.sqrt(D), window=window, splits=splits, portion_splits=portion_splits)
     return out.cpu(), torch.cat(wants)
 
 
@@ -461,6 +461,18 @@ def _mfma_case(nq, nkv, D, P, segs, window, splits, seed):
 def test_attention_mfma_prompt_portions(nq, nkv, D, P, window):
     # portions that start mid-page after a cached prefix, a whole prompt, and a single first token
     got, want = _mfma_case(nq, nkv, D, P, [(0, 70), (45, 39), (0, 1), (130, 2)], window, 1, 70)
+    assert torch.isfinite(got).all()
+    assert _rel(got, want) < 8e-3
+
+
+@pytest.mark.parametrize("nq,nkv,D,P", [(4, 2, 16, 4), (32, 8, 128, 16), (5, 1, 64, 16), (2, 2, 256, 16), (16, 1, 80, 64)])
+@pytest.mark.parametrize("parts", [None, 2, 5, 8])
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_mfma_portions_with_their_keys_cut_into_parts(nq, nkv, D, P, parts, window):
+    """Portions too few to fill the chip: every row block's keys are cut into parts (some of them empty: more
+    parts than tiles; parts that lie before a window or after a row's own position) and merged afterwards."""
+    got, want = _mfma_case(nq, nkv, D, P, [(300, 70), (45, 39), (0, 1), (130, 2), (0, 200)], window, 1, 75,
+                           portion_splits=parts)
     assert torch.isfinite(got).all()
     assert _rel(got, want) < 8e-3
 
@@ -505,6 +517,41 @@ def test_attention_mfma_mixed_step_and_stale_pages(nq, nkv, D, splits):
                         splits=splits, short_segments=3)
     assert torch.isfinite(out).all()
     assert _rel(out.cpu(), torch.cat(wants)) < 8e-3
+
+
+def test_attention_mfma_step_too_large_for_the_work_list():
+    """More (row block, segment) pairs than the planning kernel lists: the portions kernel then walks all
+    pairs itself.  One long portion beside many decoded tokens, against the same segments launched alone
+    (listed), which must agree bit for bit, and the decoded tokens against the plain implementation."""
+    nq, nkv, D, P = 16, 1, 64, 16
+    dt = torch.bfloat16
+    long_n, singles = 3400, 40                      # 3400 * 16 rows / 128 = 425 row blocks, * 41 segments > 16384
+    segs = [(0, long_n)] + [(20 + 3 * i, 1) for i in range(singles)]
+    lengths = [a + b for a, b in segs]
+    table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, 97)
+    qs, row0, starts, wants = [], [0], [], []
+    for s, (cached, n) in enumerate(segs):
+        g = _g(98 + s)
+        q, k, v = (torch.randn(cached + n, h, D, generator=g).to(dt) for h in (nq, nkv, nkv))
+        _fill_cache(table, k_pages, v_pages, s, k, v, P)
+        qs.append(q[cached:].reshape(n, -1))
+        if s > 0:
+            wants.append(plain.causal_attention(q.double(), k.double(), v.double(), nkv)[cached:].reshape(n, -1))
+        row0.append(row0[-1] + n)
+        starts.append(cached)
+    q_all = torch.cat(qs).to(DEV)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    dk, dv, dtab = k_pages.to(DEV), v_pages.to(DEV), table.to(DEV)
+    common = dict(num_q_heads=nq, num_kv_heads=nkv, head_dim=D, page_size=P, scale=1.0 / math.sqrt(D))
+    out = torch.full_like(q_all, float("nan"))
+    ops.attn_paged_mfma(q_all, out, dk, dv, dtab, i32(row0), i32(list(range(len(segs)))), i32(starts),
+                        max_qlen=long_n, min_qlen=1, max_kv_len=max(lengths), short_segments=singles, **common)
+    assert torch.isfinite(out).all()
+    alone = torch.full_like(q_all[:long_n], float("nan"))
+    ops.attn_paged_mfma(q_all[:long_n], alone, dk, dv, dtab, i32([0, long_n]), i32([0]), i32([0]),
+                        max_qlen=long_n, min_qlen=long_n, max_kv_len=long_n, **common)
+    assert torch.equal(out[:long_n], alone)
+    assert _rel(out[long_n:].cpu(), torch.cat(wants)) < 8e-3
 
 
 def test_attention_mfma_finds_a_far_key():
