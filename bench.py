@@ -58,6 +58,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=FULL_LAYERS)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 decode points")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="measure the 2,048-token prefill alone (for profiles of its kernels) and print that")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
@@ -105,6 +107,11 @@ def main() -> int:
     prefill = {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
                "frac": round(prefill_flops(raw, PROMPT) / prefill_s / PEAK_FLOPS[dkey], 4)}
     print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
+    if args.prefill_only:
+        print(json.dumps({"metric": "prefill tok/s at 2,048 tokens (Qwen3-4B shape, random weights)",
+                          "value": prefill["value"], "unit": "tok/s", "n_gpus": 1, "dtype": dkey,
+                          "higher_is_better": True, "prefill": prefill}))
+        return 0
 
     # ---- decode ---------------------------------------------------------------------------------
     def decode_run(batch, steps, warmup):
