@@ -234,6 +234,134 @@ __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same product for workgroups that stay: gridDim.x workgroups a k split, each of which stages its X slice
+// once and then walks the column groups blockIdx.x, blockIdx.x + gridDim.x, ... with the W ring running on from
+// one group into the next.  With more than 16 rows the X slice is large (64 rows of 640 columns are 80 KB), and
+// staging it again for every 128 columns, as the kernel above does, costs as much as reading W; here it is
+// read once per workgroup, so that W alone is streamed.  Waves: WN, one 16-column tile each; no split of the
+// slice inside the workgroup.  The slice is walked in rounds of PD steps; a last round that reaches past the
+// slice meets zeros in LDS (the staging puts zeros behind the slice up to a whole round).
+template <int MT, int WN, int PD, typename TOut>
+__global__ __launch_bounds__(WN * 64) void gemm_stream_kernel(const RowsArgs a) {
+  constexpr int kThreads = WN * 64;
+  constexpr int XD = 2;
+  static_assert(PD % XD == 0, "the X ring must divide the W ring");
+  extern __shared__ __align__(16) uint16_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int li = lane & 15, g = lane >> 4;
+  const int M = a.M, N = a.N, K = a.K;
+  const int steps_total = (K + 31) / 32;
+  const int s_begin = blockIdx.y * a.steps_per_split;
+  const int s_end = min(s_begin + a.steps_per_split, steps_total);
+  const int n_steps = s_end - s_begin;
+  const int rounds = (n_steps + PD - 1) / PD;
+  const int steps_padded = rounds * PD;
+  const int pitch = steps_padded * 32 + kPad;
+  const int groups_total = (N + WN * 16 - 1) / (WN * 16);
+  const int n_mine = (groups_total - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
+  if (n_mine <= 0) return;  // the whole workgroup
+
+  auto w_row = [&](int group) {
+    const int n0 = (group * WN + wave) * 16;
+    return a.w + static_cast<int64_t>(min(n0 + li, N - 1)) * a.ldw;
+  };
+  auto load_w = [&](const uint16_t* row, int s) {  // s: step inside the slice (may reach past it, not past K)
+    const int e = min(32 * (s_begin + s) + 8 * g, K - 8);
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(row + e));
+  };
+  const uint16_t* wcur = w_row(blockIdx.x);
+  bf16x8 ring[PD];
+#pragma unroll
+  for (int u = 0; u < PD; ++u) ring[u] = load_w(wcur, u);
+
+  {  // X slice -> LDS, as in the kernel above, zeros from the end of the slice to the end of the last round
+    const int cpr = steps_padded * 4;
+    const int cpp = cpr + kPad / 8;
+    const int total = M * cpp;
+    const int k0 = s_begin * 32, k1 = min(s_end * 32, K);
+    for (int q0 = wave * 64; q0 < total; q0 += kThreads) {
+      const int q = min(q0 + lane, total - 1);
+      const int row = q / cpp, cc = q % cpp;
+      const int col = k0 + cc * 8;
+      const uint16_t* src = a.x + static_cast<int64_t>(row) * a.ldx + ((cc < cpr && col < k1) ? col : k0);
+      __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)(lds + q0 * 8), 16, 0, 0);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const int z0 = (k1 - k0) / 8, nz = cpr - z0;
+    if (nz > 0) {
+      __syncthreads();  // the pieces put to zero were fetched by other waves
+      for (int i = tid; i < M * nz; i += kThreads)
+        *reinterpret_cast<uint4*>(lds + (i / nz) * pitch + (z0 + i % nz) * 8) = uint4{0u, 0u, 0u, 0u};
+    }
+  }
+  __syncthreads();
+
+  const uint16_t* xrow[MT];
+#pragma unroll
+  for (int b = 0; b < MT; ++b) xrow[b] = lds + min(16 * b + li, M - 1) * pitch + 8 * g;
+  auto load_x = [&](int s, bf16x8 (&dst)[MT]) {
+#pragma unroll
+    for (int b = 0; b < MT; ++b) dst[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(xrow[b] + 32 * s));
+  };
+  bf16x8 xring[XD][MT];
+#pragma unroll
+  for (int u = 0; u < XD; ++u) load_x(u, xring[u]);  // steps_padded >= PD >= XD
+
+  for (int gi = 0; gi < n_mine; ++gi) {
+    const int group = blockIdx.x + gi * gridDim.x;
+    // the ring runs on into the workgroup's next group (after the last one: into this one again, unused)
+    const uint16_t* wnext_group = w_row(gi + 1 < n_mine ? group + static_cast<int>(gridDim.x) : group);
+    f32x4 acc[MT];
+#pragma unroll
+    for (int b = 0; b < MT; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int rr = 0; rr < rounds; ++rr) {
+      const bool last = rr + 1 == rounds;
+      const uint16_t* wnext = last ? wnext_group : wcur;
+      const int snext = last ? 0 : (rr + 1) * PD;
+#pragma unroll
+      for (int u = 0; u < PD; ++u) {
+        const int s = rr * PD + u;
+#pragma unroll
+        for (int b = 0; b < MT; ++b)
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
+        int sx = s + XD;
+        if (sx >= steps_padded) sx -= steps_padded;  // the next group starts at the slice's first step again
+        load_x(sx, xring[u % XD]);
+        ring[u] = load_w(wnext, snext + u);
+        __builtin_amdgcn_sched_barrier(0);  // each load right behind its product
+      }
+    }
+    wcur = wnext_group;
+    // acc[b][r] = C[m = 16 b + li][n = n0 + 4 g + r]
+    TOut* out = static_cast<TOut*>(a.out) + static_cast<int64_t>(blockIdx.y) * a.split_stride;
+    const int ncol = (group * WN + wave) * 16 + 4 * g;
+#pragma unroll
+    for (int b = 0; b < MT; ++b) {
+      const int mrow = 16 * b + li;
+      if (mrow >= M) continue;
+      TOut* o = out + static_cast<int64_t>(mrow) * a.ldo + ncol;
+      if (ncol + 3 < N && (a.ldo & 3) == 0) {
+        if constexpr (sizeof(TOut) == 4) {
+          *reinterpret_cast<float4*>(o) = float4{acc[b][0], acc[b][1], acc[b][2], acc[b][3]};
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[r] = from_float<TOut>(acc[b][r]);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (ncol + r < N) o[r] = from_float<TOut>(acc[b][r]);
+      }
+    }
+  }
+}
+
+inline size_t stream_lds_bytes(int M, int steps_per_split, int pd) {
+  const int padded = (steps_per_split + pd - 1) / pd * pd;
+  return (static_cast<size_t>(M) * (padded * 32 + kPad) + 511) / 512 * 512 * sizeof(uint16_t);
+}
+
 // LDS of a launch: the X rows of one k slice and, behind them, the partial sums of the waves wk > 0 and the
 // gate/up exchange.
 inline size_t rows_lds_bytes(int M, int steps_per_split, int mt, int wn, int wk) {
@@ -350,6 +478,88 @@ extern "C" int arle_gemm_rows(const void* x, long long ldx, const void* w, long 
     if (M <= 32) return dispatch_rows<2, WN, WK, PD>(a, splits, out_dtype, epilogue, s);        \
     return dispatch_rows<4, WN, WK, PD>(a, splits, out_dtype, epilogue, s);
     ARLE_ROWS_VARIANTS(X)
+#undef X
+  }
+  return static_cast<int>(hipErrorInvalidValue);
+}
+
+// Shapes of a staying workgroup, by `variant`: (WN, PD).
+#define ARLE_STREAM_VARIANTS(X) X(0, 4, 8) X(1, 8, 4) X(2, 8, 8) X(3, 4, 4) X(4, 2, 8)
+constexpr int kStreamVariants = 5;
+
+// (output columns of one column group) << 8 | PD; -1 for an unknown variant
+extern "C" int arle_gemm_stream_geometry(int variant) {
+  switch (variant) {
+#define X(ID, WN, PD) \
+  case ID:            \
+    return ((WN * 16) << 8) | PD;
+    ARLE_STREAM_VARIANTS(X)
+#undef X
+    default:
+      return -1;
+  }
+}
+
+extern "C" long long arle_gemm_stream_lds(int variant, int M, int steps_per_split) {
+  const int geometry = arle_gemm_stream_geometry(variant);
+  if (geometry < 0) return -1;
+  return static_cast<long long>(stream_lds_bytes(M, steps_per_split, geometry & 255));
+}
+
+namespace arle {
+template <int MT, int WN, int PD, typename TOut>
+int launch_stream(const RowsArgs& a, int splits, int workgroups, hipStream_t s) {
+  const size_t lds = stream_lds_bytes(a.M, a.steps_per_split, PD);
+  if (lds > kRowsLdsMax) return static_cast<int>(hipErrorInvalidValue);
+  auto kernel = gemm_stream_kernel<MT, WN, PD, TOut>;
+  static size_t allowed = 64 * 1024;
+  if (lds > allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       static_cast<int>(kRowsLdsMax));
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return static_cast<int>(e);
+    }
+    allowed = kRowsLdsMax;
+  }
+  const int groups = (a.N + WN * 16 - 1) / (WN * 16);
+  kernel<<<dim3(min(workgroups, groups), splits), WN * 64, lds, s>>>(a);
+  return launch_status();
+}
+
+template <int WN, int PD>
+int dispatch_stream(const RowsArgs& a, int splits, int workgroups, int out_dtype, hipStream_t s) {
+  const bool f32 = out_dtype == kF32;
+  if (a.M <= 16)
+    return f32 ? launch_stream<1, WN, PD, float>(a, splits, workgroups, s) : launch_stream<1, WN, PD, bf16>(a, splits, workgroups, s);
+  if (a.M <= 32)
+    return f32 ? launch_stream<2, WN, PD, float>(a, splits, workgroups, s) : launch_stream<2, WN, PD, bf16>(a, splits, workgroups, s);
+  return f32 ? launch_stream<4, WN, PD, float>(a, splits, workgroups, s) : launch_stream<4, WN, PD, bf16>(a, splits, workgroups, s);
+}
+}  // namespace arle
+
+// The product with workgroups that stay (see gemm_stream_kernel): `workgroups` of them for every k split walk
+// the column groups.  Operands, splits and the stack of partial products as in arle_gemm_rows; no activation.
+extern "C" int arle_gemm_stream(const void* x, long long ldx, const void* w, long long ldw, void* out, long long ldo,
+                                long long split_stride, int out_dtype, int M, int N, int K, int variant, int splits,
+                                int steps_per_split, int workgroups, void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K % 8 != 0 || K <= 0 || ldx % 8 != 0 || ldw % 8 != 0 || splits < 1 || splits > 65535 ||
+      steps_per_split < 1 || workgroups < 1 || variant < 0 || variant >= kStreamVariants)
+    return static_cast<int>(hipErrorInvalidValue);
+  const int steps_total = (K + 31) / 32;
+  if (static_cast<long long>(splits - 1) * steps_per_split >= steps_total ||
+      static_cast<long long>(splits) * steps_per_split < steps_total)
+    return static_cast<int>(hipErrorInvalidValue);
+  if (splits > 1 && out_dtype != kF32) return static_cast<int>(hipErrorInvalidValue);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const RowsArgs a{static_cast<const uint16_t*>(x), ldx, static_cast<const uint16_t*>(w), ldw, out, ldo, M, N, K,
+                   steps_per_split, split_stride};
+  switch (variant) {
+#define X(ID, WN, PD) \
+  case ID:            \
+    return dispatch_stream<WN, PD>(a, splits, workgroups, out_dtype, s);
+    ARLE_STREAM_VARIANTS(X)
 #undef X
   }
   return static_cast<int>(hipErrorInvalidValue);

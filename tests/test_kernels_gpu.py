@@ -615,6 +615,35 @@ def test_gemm_rows_as_planned(M, N, K):
     assert _rel(_whole(got), wide[:, 8:8 + K].double().cpu() @ w.double().T) < 1e-5
 
 
+@pytest.mark.parametrize("variant", range(ops.STREAM_VARIANTS))
+@pytest.mark.parametrize("M,N,K,splits,workgroups", [(5, 333, 88, 1, 2), (16, 96, 1096, 3, 1), (20, 200, 520, 2, 64),
+                                                     (64, 72, 2056, 5, 1), (33, 2560, 4096, 6, 11), (64, 1000, 2056, 3, 3),
+                                                     (48, 100, 4104, 4, None), (1, 40, 8, 1, 7)])
+def test_gemm_stream_workgroups_that_walk_several_column_groups(variant, M, N, K, splits, workgroups):
+    """The kernel whose workgroups stay: widths that end inside a column group and inside a k step, slices that
+    end inside a round, one workgroup for all groups and more workgroups than groups, LDS beyond 64 KB."""
+    a = torch.randn(M, K, generator=_g(105)).bfloat16()
+    w = (torch.randn(N, K, generator=_g(106)) * 0.1).bfloat16()
+    got = ops.gemm_stream(a.to(DEV), w.to(DEV), torch.float32, variant=variant, splits=splits, workgroups=workgroups)
+    assert got.dim() == 2 or got.shape[0] >= splits
+    assert _rel(_whole(got), a.double() @ w.double().T) < 1e-5
+
+
+def test_gemm_bf16_takes_the_staying_kernel_for_narrow_outputs_of_17_to_64_rows():
+    for M in (17, 40, 64):
+        a = torch.randn(M, 4096, generator=_g(107)).bfloat16()
+        w = (torch.randn(2560, 4096, generator=_g(108)) * 0.05).bfloat16()
+        assert ops.gemm_stream_preferred(M, 2560, 4096, 4096)
+        stack = ops.gemm_bf16(a.to(DEV), w.to(DEV), torch.bfloat16, partials_ok=True)
+        assert stack.dim() == 3 and stack.dtype == torch.float32
+        whole = ops.gemm_bf16(a.to(DEV), w.to(DEV), torch.bfloat16)
+        assert whole.shape == (M, 2560) and whole.dtype == torch.bfloat16
+        want = a.double() @ w.double().T
+        assert _rel(stack.double().sum(0).cpu(), want) < 1e-5
+        assert _rel(whole.cpu(), want) < 6e-3
+    assert not ops.gemm_stream_preferred(64, 19456, 2560, 2560) and not ops.gemm_stream_preferred(16, 2560, 4096, 4096)
+
+
 @pytest.mark.parametrize("variant", range(ops.ROWS_VARIANTS))
 @pytest.mark.parametrize("M,N,K,splits", [(5, 333, 88, 1), (16, 96, 1096, 3), (20, 200, 520, 2), (64, 72, 2056, 5),
                                           (33, 2560, 4096, 16), (64, 72, 2056, 3), (48, 100, 4104, 4)])
