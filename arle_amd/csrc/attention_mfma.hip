@@ -28,6 +28,8 @@
 // batch_decode_paged_hd128.py:239-463).  Scores are scaled by scale*log2(e) and exponentiated
 // with exp2; probabilities are narrowed to bfloat16 before the second product, as the
 // reference does (batch_prefill_paged_hd128.py:219-225); the sum l uses the 32-bit values.
+#include <type_traits>
+
 #include "common.h"
 
 namespace arle {
@@ -205,9 +207,12 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
     load_v(b0, vraw);
   }
 
-  for (int blk = b0; blk < b1; ++blk) {
+  // One block of 32 keys.  `more` (is there a next block, whose keys and values are fetched meanwhile) is a
+  // compile-time value: all blocks but the last run without a condition around their loads, so that each
+  // product waits for its own operand only and the values of the next block stay in flight behind its keys.
+  auto block = [&](int blk, auto more_tag) {
+    constexpr bool more = decltype(more_tag)::value;
     const int key_base = blk * 32;
-    const bool more = blk + 1 < b1;
     if (more) cover(blk + 1);
 
     // scores S^T: s[n][t][r] belongs to key key_base + 16t + 4g + r and row (n, li)
@@ -295,7 +300,9 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
     }
     // and the value registers after the second product
     if (more) load_v(blk + 1, vraw);
-  }
+  };
+  for (int blk = b0; blk + 1 < b1; ++blk) block(blk, std::true_type{});
+  if (b0 < b1) block(b1 - 1, std::false_type{});
 
   // acc[n][dt][r] is O^T[d = 16dt + 4g + r][row (n, li)]
 #pragma unroll

@@ -82,6 +82,7 @@ class Engine:
         self._graphs: dict = {}       # (rows, split cap) or a step shape -> (graph, input buffer, logits)
         self._shapes_seen: set = set()
         self.max_graphs = 64          # captured steps kept (each holds its activations)
+        self.max_graph_logits_bytes = 64 << 20
         self._graph_pool = None
         self.graph_replays = 0
 
@@ -221,8 +222,11 @@ class Engine:
         lens = tuple(len(e.tokens) for e in entries)
         if not lens or min(lens) == 0:
             return None
+        wanted = sum(len(e.want) for e in entries)
+        if wanted * self.spec.vocab_size * 4 > self.max_graph_logits_bytes:
+            return None     # a captured step keeps its logits buffer for good
         max_kv = max(before[e.request] + len(e.tokens) for e in entries)
-        key = (lens, sum(len(e.want) for e in entries), ops.decode_split_cap(max_kv))
+        key = (lens, wanted, ops.decode_split_cap(max_kv))
         if key in self._graphs:
             return key
         if len(self._shapes_seen) > 4096:
