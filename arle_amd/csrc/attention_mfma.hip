@@ -28,8 +28,6 @@
 // batch_decode_paged_hd128.py:239-463).  Scores are scaled by scale*log2(e) and exponentiated
 // with exp2; probabilities are narrowed to bfloat16 before the second product, as the
 // reference does (batch_prefill_paged_hd128.py:219-225); the sum l uses the 32-bit values.
-#include <type_traits>
-
 #include "common.h"
 
 namespace arle {
@@ -130,8 +128,11 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
     const uint16_t* qp = a.q + static_cast<int64_t>(row0 + my_tok[n]) * a.q_stride + my_head[n] * D;
 #pragma unroll
     for (int c = 0; c < DCH; ++c) {
+      // always a load (from a clamped place) and a choice of the value afterwards: a load under a condition
+      // would be waited for on the spot, and would leave registers that are sometimes never written
       const int d = 32 * c + 8 * g;
-      qreg[n][c] = (EXACT || (c < n_dch && d < D)) ? load_bf16x8(qp + d) : zero_bf16x8();
+      const bf16x8 got = load_bf16x8(qp + (EXACT ? d : min(d, D - 8)));
+      qreg[n][c] = (EXACT || d < D) ? got : zero_bf16x8();
     }
   }
 
@@ -175,7 +176,8 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
 #pragma unroll
       for (int c = 0; c < DCH; ++c) {
         const int d = 32 * c + 8 * g;
-        kreg[t][c] = (EXACT || (c < n_dch && d < D)) ? load_bf16x8(kp + d) : zero_bf16x8();
+        const bf16x8 got = load_bf16x8(kp + (EXACT ? d : min(d, D - 8)));
+        kreg[t][c] = (EXACT || d < D) ? got : zero_bf16x8();
       }
     }
   };
@@ -190,11 +192,10 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
       const uint16_t* vp = a.v_pages + page * page_elems + k_head + (key4 & pm);
 #pragma unroll
       for (int dt = 0; dt < DTL; ++dt) {
-        if (EXACT || dt < n_dt) {
-          const u32x2 four = *reinterpret_cast<const u32x2*>(vp + static_cast<int64_t>(16 * dt + li) * P);
-          vreg[dt][2 * t] = four[0];
-          vreg[dt][2 * t + 1] = four[1];
-        }
+        const int drow = EXACT ? 16 * dt + li : min(16 * dt + li, D - 1);  // a tile past head_dim reads its last row
+        const u32x2 four = *reinterpret_cast<const u32x2*>(vp + static_cast<int64_t>(drow) * P);
+        vreg[dt][2 * t] = four[0];
+        vreg[dt][2 * t + 1] = four[1];
       }
     }
   };
@@ -207,12 +208,9 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
     load_v(b0, vraw);
   }
 
-  // One block of 32 keys.  `more` (is there a next block, whose keys and values are fetched meanwhile) is a
-  // compile-time value: all blocks but the last run without a condition around their loads, so that each
-  // product waits for its own operand only and the values of the next block stay in flight behind its keys.
-  auto block = [&](int blk, auto more_tag) {
-    constexpr bool more = decltype(more_tag)::value;
+  for (int blk = b0; blk < b1; ++blk) {
     const int key_base = blk * 32;
+    const bool more = blk + 1 < b1;
     if (more) cover(blk + 1);
 
     // scores S^T: s[n][t][r] belongs to key key_base + 16t + 4g + r and row (n, li)
@@ -300,9 +298,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
     }
     // and the value registers after the second product
     if (more) load_v(blk + 1, vraw);
-  };
-  for (int blk = b0; blk + 1 < b1; ++blk) block(blk, std::true_type{});
-  if (b0 < b1) block(b1 - 1, std::false_type{});
+  }
 
   // acc[n][dt][r] is O^T[d = 16dt + 4g + r][row (n, li)]
 #pragma unroll
@@ -556,8 +552,11 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
     const uint16_t* qp = a.q + static_cast<int64_t>(row0 + my_tok[n]) * a.q_stride + my_head[n] * D;
 #pragma unroll
     for (int c = 0; c < DCH; ++c) {
+      // always a load (from a clamped place) and a choice of the value afterwards: a load under a condition
+      // would be waited for on the spot, and would leave registers that are sometimes never written
       const int d = 32 * c + 8 * g;
-      qreg[n][c] = (EXACT || (c < n_dch && d < D)) ? load_bf16x8(qp + d) : zero_bf16x8();
+      const bf16x8 got = load_bf16x8(qp + (EXACT ? d : min(d, D - 8)));
+      qreg[n][c] = (EXACT || d < D) ? got : zero_bf16x8();
     }
   }
   f32x4 acc[NT][DTL];
