@@ -831,43 +831,53 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
 }
 
 // The parts of a portion's rows put together: out = sum_p o_p 2^(m_p - m) / sum_p l_p 2^(m_p - m), in the order
-// of the parts.  One workgroup per listed (row block, segment) pair and kv head; a wave takes every eighth row,
-// a lane four columns of it (head_dim <= 256).
+// of the parts.  Work items are (listed pair, kv head, eight rows of the row block): a workgroup of eight waves
+// takes items blockIdx.x, blockIdx.x + gridDim.x, ... and each wave one row of the item, a lane four columns
+// (head_dim <= 256).  No workgroup is launched for nothing, and no wave walks rows one after the other (a row
+// is two dependent loads: walking sixteen of them took longer than the attention itself).
 constexpr int kPortionPartsMax = 8;
 __global__ __launch_bounds__(kPfWaves* kWave) void attn_merge_portions_kernel(const AttnArgs a) {
-  if (blockIdx.x >= g_prefill_pairs) return;
-  const unsigned int entry = g_prefill_plan[blockIdx.x];
-  const int seg = static_cast<int>(entry & 0xffffu), wg_row = static_cast<int>(entry >> 16) * kPfRows;
-  const int kvh = blockIdx.y, G = a.nq / a.nkv, D = a.D, parts = a.portion_splits;
-  const int row0 = a.seg_row0[seg];
-  const int rows = (a.seg_row0[seg + 1] - row0) * G;
+  const int G = a.nq / a.nkv, D = a.D, parts = a.portion_splits;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int d0 = 4 * lane;
-  for (int row = wg_row + wave; row < min(wg_row + kPfRows, rows); row += kPfWaves) {
+  constexpr int kSubBlocks = kPfRows / kPfWaves;  // items of eight rows in a row block
+  const unsigned int items = g_prefill_pairs * a.nkv * kSubBlocks;
+  for (unsigned int item = blockIdx.x; item < items; item += gridDim.x) {
+    const unsigned int pair = item / (a.nkv * kSubBlocks);
+    const int kvh = static_cast<int>((item / kSubBlocks) % a.nkv), sub = static_cast<int>(item % kSubBlocks);
+    const unsigned int entry = g_prefill_plan[pair];
+    const int seg = static_cast<int>(entry & 0xffffu);
+    const int row = static_cast<int>(entry >> 16) * kPfRows + sub * kPfWaves + wave;
+    const int row0 = a.seg_row0[seg];
+    const int rows = (a.seg_row0[seg + 1] - row0) * G;
+    if (row >= rows) continue;  // this wave only
     const int head = kvh * G + row % G;
     const int64_t tok_row = row0 + row / G;
     const int64_t base = (tok_row * a.nq + head) * parts;
     float ms[kPortionPartsMax], ls[kPortionPartsMax];
-    float mx = -INFINITY;
+    float4 os[kPortionPartsMax];
+    const float* src = a.pws_o + base * D + (d0 < D ? d0 : 0);
 #pragma unroll
-    for (int p = 0; p < kPortionPartsMax; ++p) {
-      const float2 ml = *reinterpret_cast<const float2*>(a.pws_ml + (base + min(p, parts - 1)) * 2);
+    for (int p = 0; p < kPortionPartsMax; ++p) {  // every load first, none under a condition
+      const int q = min(p, parts - 1);
+      const float2 ml = *reinterpret_cast<const float2*>(a.pws_ml + (base + q) * 2);
+      os[p] = *reinterpret_cast<const float4*>(src + static_cast<int64_t>(q) * D);
       ms[p] = p < parts ? ml.x : -INFINITY;
       ls[p] = p < parts ? ml.y : 0.f;
-      mx = fmaxf(mx, ms[p]);
     }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int p = 0; p < kPortionPartsMax; ++p) mx = fmaxf(mx, ms[p]);
     float denom = 0.f;
     float4 o = {0.f, 0.f, 0.f, 0.f};
-    const float* src = a.pws_o + base * D + (d0 < D ? d0 : 0);
 #pragma unroll
     for (int p = 0; p < kPortionPartsMax; ++p) {
       const float w = ms[p] > -INFINITY ? exp2f(ms[p] - mx) : 0.f;  // an empty part weighs nothing
       denom += ls[p] * w;
-      const float4 v = *reinterpret_cast<const float4*>(src + static_cast<int64_t>(min(p, parts - 1)) * D);
-      o.x += v.x * w;
-      o.y += v.y * w;
-      o.z += v.z * w;
-      o.w += v.w * w;
+      o.x += os[p].x * w;
+      o.y += os[p].y * w;
+      o.z += os[p].z * w;
+      o.w += os[p].w * w;
     }
     const float inv = denom > 0.f ? 1.0f / denom : 0.f;
     if (d0 < D) {
@@ -927,8 +937,10 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
   if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);  // the merge walks the list
   attn_prefill_lds_kernel<DMAX, EXACT><<<workgroups, kPfWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
                                                                                 static_cast<int>(grid.z), listed);
-  if (a.portion_splits > 1)
-    attn_merge_portions_kernel<<<dim3(grid.x * grid.z, grid.y), kPfWaves * kWave, 0, s>>>(a);
+  if (a.portion_splits > 1) {
+    const long long most = static_cast<long long>(grid.x) * grid.y * grid.z * (kPfRows / kPfWaves);
+    attn_merge_portions_kernel<<<static_cast<unsigned>(most < 4LL * cus ? most : 4LL * cus), kPfWaves * kWave, 0, s>>>(a);
+  }
   return launch_status();
 }
 

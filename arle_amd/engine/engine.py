@@ -182,7 +182,7 @@ class Engine:
         key = (rows, ops.decode_split_cap(max_kv))
         all_rows = [StepEntry(e.request, e.tokens, [0]) for e in entries]
         length_before = before.__getitem__
-        rec = self._graphs.get(key)
+        rec = self._graphs.pop(key, None)
         if rec is None:
             static = torch.empty(packed_size(rows, rows, rows), dtype=torch.int32, device=self.device)
             batch = build_step_batch(all_rows, self.cache.slot_of.__getitem__, length_before,
@@ -196,7 +196,9 @@ class Engine:
                 self._graph_pool = torch.cuda.graph_pool_handle()
             with torch.cuda.graph(graph, pool=self._graph_pool):
                 static_logits = self.model.forward(batch, self.cache)
-            self._graphs[key] = (graph, static, static_logits)
+            rec = (graph, static, static_logits)
+            while len(self._graphs) >= self.max_graphs:      # the least recently used goes
+                self._graphs.pop(next(iter(self._graphs)))
         else:
             graph, static, static_logits = rec
             build_step_batch(all_rows, self.cache.slot_of.__getitem__, length_before,
@@ -204,6 +206,7 @@ class Engine:
             graph.replay()
             self.graph_replays += 1
             logits = static_logits.clone()
+        self._graphs[key] = rec    # most recently used last
         wanted = [i for i, e in enumerate(entries) for _ in e.want]
         if wanted == list(range(rows)):
             return logits

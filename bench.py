@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the Qwen3-4B shape with random weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
+    python bench.py --workload qwen3-8b-mixed | qwen3-32b-decode     (the baseline's two further workloads)
 
 A step is one decode step of `batch` requests, each holding a `prompt`-token random prompt
 (prefilled by the engine itself before the clock starts) and growing by one token per step.
@@ -21,6 +22,13 @@ PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 QWEN3_4B = dict(num_hidden_layers=36, hidden_size=2560, num_attention_heads=32, num_key_value_heads=8,
                 head_dim=128, intermediate_size=9728, vocab_size=151936, rope_theta=1000000.0,
                 rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=40960)
+# BASELINE.json configs[3] and [4]: the two other workloads (`--workload`)
+QWEN3_8B = dict(num_hidden_layers=36, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+                head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1000000.0,
+                rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960)
+QWEN3_32B = dict(num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8,
+                 head_dim=128, intermediate_size=25600, vocab_size=151936, rope_theta=1000000.0,
+                 rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960)
 FULL_LAYERS = QWEN3_4B["num_hidden_layers"]
 CONTEXT = 4096
 PROMPT = 2048
@@ -49,6 +57,136 @@ def prefill_flops(c, tokens: int) -> float:
     return gemm + attn + head
 
 
+def _timed(torch, fn):
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    fn()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t
+
+
+def mixed_8b(args) -> int:
+    """BASELINE.json configs[3]: 32 requests decoding at 1,024 tokens of context beside one 2,048-token prompt
+    that arrives in portions of 512: four steps of 32 + 512 rows.  Reports the mean step and the tokens a second
+    of both kinds."""
+    import torch
+
+    from arle_amd.config import Qwen3Config
+    from arle_amd.engine import Engine, StepEntry
+    from arle_amd.kernels import ops
+
+    raw = dict(QWEN3_8B, num_hidden_layers=args.layers or QWEN3_8B["num_hidden_layers"])
+    config = Qwen3Config.from_dict(raw)
+    decoders, context, prompt, portion = 32, 1024, 2048, 512
+    engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype="bfloat16", page_size=PAGE,
+                                max_tokens=decoders * (context + 64) + 2 * prompt, max_slots=decoders + 1,
+                                max_request_tokens=4096)
+    gen = torch.Generator().manual_seed(1234)
+    rand = lambda n: torch.randint(0, config.vocab_size, (n,), generator=gen).tolist()
+    keys = [("d", i) for i in range(decoders)]
+    last = []
+    for k in keys:
+        engine.add_request(k)
+    for i in range(0, decoders, 8):
+        out = engine.step([StepEntry(k, rand(context - 1), [context - 2]) for k in keys[i:i + 8]])
+        last.extend(ops.argmax_rows(out).tolist())
+    state = {"last": last}
+
+    def one_prompt(tag):
+        engine.add_request(tag)
+        toks = rand(prompt)
+        for a in range(0, prompt, portion):
+            entries = [StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])]
+            entries.append(StepEntry(tag, toks[a:a + portion], [portion - 1] if a + portion == prompt else []))
+            out = engine.step(entries)
+            state["last"] = ops.argmax_rows(out).tolist()[:decoders]
+        engine.end_request(tag)
+
+    for i in range(2):          # the second pass captures the four step shapes, later ones replay them
+        one_prompt(("warm", i))
+    # the decoders have grown by 8 tokens; the timed prompts run at 1,032..1,048 tokens of context
+    reps = max(1, args.steps // 4)
+    dt = _timed(torch, lambda: [one_prompt(("p", i)) for i in range(reps)])
+    steps = 4 * reps
+    ms = dt / steps * 1e3
+    flops = sum(prefill_flops_portion(raw, a, portion) for a in range(0, prompt, portion)) / 4.0
+    line = {"metric": "mixed step: 32 decoding requests at 1,024 tokens + a 512-token prompt portion (Qwen3-8B shape)",
+            "value": round(steps * (decoders + portion) / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps,
+            "warmup": 8, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic: seeded random weights N(0,0.02), uniform random token ids",
+            "config": {"model": "Qwen3-8B shape", "decoding_requests": decoders, "decode_context": context,
+                       "prompt_len": prompt, "portion": portion, "layers": raw["num_hidden_layers"],
+                       "hidden": raw["hidden_size"], "q_heads": 32, "kv_heads": 8, "head_dim": 128,
+                       "intermediate": raw["intermediate_size"], "vocab": raw["vocab_size"], "tied": False,
+                       "page_size": PAGE},
+            "points": {"decode_tok_s": round(decoders * steps / dt, 1), "prefill_tok_s": round(portion * steps / dt, 1)},
+            "roofline": {"bound": "mfma+hbm", "flops_per_step": round(flops / 1e12, 2), "unit": "TFLOP",
+                         "frac": round(flops / (dt / steps) / PEAK_FLOPS["bf16"], 4)}}
+    print(json.dumps(line))
+    return 0
+
+
+def prefill_flops_portion(c, start: int, n: int) -> float:
+    """Flops of a portion of n prompt tokens that starts at position `start` (products and causal attention)."""
+    L = c["num_hidden_layers"]
+    gemm = 2.0 * n * L * layer_params(c)
+    attn = 4.0 * c["num_attention_heads"] * c["head_dim"] * (n * start + n * (n + 1) / 2) * L
+    return gemm + attn
+
+
+def decode_32b(args) -> int:
+    """BASELINE.json configs[4]: 64 requests decoding at 8,192 tokens of context, Qwen3-32B shape (65 GB of
+    weights, 137 GB of cache)."""
+    import torch
+
+    from arle_amd.config import Qwen3Config
+    from arle_amd.engine import Engine, StepEntry
+    from arle_amd.kernels import ops
+
+    raw = dict(QWEN3_32B, num_hidden_layers=args.layers or QWEN3_32B["num_hidden_layers"])
+    config = Qwen3Config.from_dict(raw)
+    batch, context = args.batch if args.batch != 8 else 64, 8192
+    steps, warmup = min(args.steps, 16), min(args.warmup, 4)
+    t0 = time.time()
+    engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype="bfloat16", page_size=PAGE,
+                                max_tokens=batch * (context + 64), max_slots=batch, max_request_tokens=context + 64)
+    print(f"[bench] engine ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    gen = torch.Generator().manual_seed(1234)
+    rand = lambda n: torch.randint(0, config.vocab_size, (n,), generator=gen).tolist()
+    keys = [("d", i) for i in range(batch)]
+    last = []
+    for i, k in enumerate(keys):          # real prefill, one 8,191-token prompt a step
+        engine.add_request(k)
+        out = engine.step([StepEntry(k, rand(context - 1), [context - 2])])
+        last.extend(ops.argmax_rows(out).tolist())
+        if i % 8 == 7:
+            print(f"[bench] prefilled {i + 1} of {batch} requests ({time.time() - t0:.0f} s)", file=sys.stderr, flush=True)
+    state = {"last": last}
+
+    def one_step():
+        out = engine.step([StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])])
+        state["last"] = ops.argmax_rows(out).tolist()
+
+    for _ in range(warmup):
+        one_step()
+    ctx0 = engine.length(keys[0])
+    dt = _timed(torch, lambda: [one_step() for _ in range(steps)])
+    ctx_mean = ctx0 + (steps - 1) / 2.0 + 1
+    achieved = decode_bytes(raw, batch, ctx_mean) / (dt / steps) / 1e9
+    line = {"metric": f"decode tok/s at batch {batch}, 8,192 tokens of context (Qwen3-32B shape, random weights)",
+            "value": round(batch * steps / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": round(dt / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic: seeded random weights N(0,0.02), uniform random token ids",
+            "config": {"model": "Qwen3-32B shape", "global_batch": batch, "seq_len": context, "layers": raw["num_hidden_layers"],
+                       "layers_full": QWEN3_32B["num_hidden_layers"], "hidden": raw["hidden_size"], "q_heads": 64,
+                       "kv_heads": 8, "head_dim": 128, "intermediate": raw["intermediate_size"],
+                       "vocab": raw["vocab_size"], "tied": False, "page_size": PAGE},
+            "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(achieved / PEAK_HBM_GBS, 4)}}
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -60,10 +198,16 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 decode points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiles of its kernels) and print that")
+    ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode"],
+                    help="qwen3-4b is the contract's run; the other two are the further workloads of the baseline")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
         return 2
+    if args.workload != "qwen3-4b":
+        if args.layers == FULL_LAYERS:
+            args.layers = 0   # the workload's own depth
+        return mixed_8b(args) if args.workload == "qwen3-8b-mixed" else decode_32b(args)
 
     import torch
 
