@@ -728,7 +728,7 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
             out = sum_partials(out, out_dtype)
         return out
     if gemm_stream_preferred(x.shape[0], w.shape[0], x.shape[1], x.stride(0)) and x.data_ptr() % 16 == 0:
-        out = gemm_stream(x, w, out_dtype, variant=_STREAM_VARIANT, splits=_STREAM_SPLITS)
+        out = gemm_stream(x, w, out_dtype, variant=_STREAM_VARIANT, splits=_stream_splits(x.shape[0], x.shape[1]))
         if out.dim() == 3 and not partials_ok:
             out = sum_partials(out, out_dtype)
         return out
@@ -741,14 +741,27 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
 # o and down projections: 11 against 15 us and 19 against 29 us at 64 rows of the Qwen3-4B shapes); for wide
 # outputs (q|k|v, gate|up) the two are level and the library stays.
 _STREAM_VARIANT = 0
-_STREAM_SPLITS = 6
-_STREAM_MAX_N = 4096
+_STREAM_SPLITS = 6              # at least so many k splits ...
+_STREAM_STEPS_A_SPLIT = 50      # ... and at most so many steps of 32 in one (the 32B shape's down, K = 25600: 16 splits)
+_STREAM_MAX_N = 5120            # 60 against the library's 146 us there at 32 rows, 97 against 157 us at 64
 _STREAM_MIN_K = 2048
 
 
+_STREAM_PARTIAL_BYTES = 6 << 20  # most bytes of partial products: the consumer (one workgroup a row) pays for them
+
+
+def _stream_splits(rows: int, k: int) -> int:
+    return max(_STREAM_SPLITS, -(-k // (32 * _STREAM_STEPS_A_SPLIT)), _stream_min_splits(_STREAM_VARIANT, rows, k))
+
+
 def gemm_stream_preferred(rows: int, n: int, k: int, x_stride: int) -> bool:
-    return (_ROWS_PREFERRED < rows <= ROWS_KERNEL_MAX and n <= _STREAM_MAX_N and k >= _STREAM_MIN_K
-            and gemm_rows_supported(rows, k, x_stride))
+    """Whether the kernel whose workgroups stay, not the library, should run this product: 17..64 rows, a narrow
+    output and a long K, and a stack of partial products small enough (at the 32B shape's down projection the
+    kernel alone is a third faster than the library, but 23 partial products of 64 x 5120 cost more than that)."""
+    if not (_ROWS_PREFERRED < rows <= ROWS_KERNEL_MAX and n <= _STREAM_MAX_N and k >= _STREAM_MIN_K
+            and gemm_rows_supported(rows, k, x_stride)):
+        return False
+    return _stream_splits(rows, k) * rows * n * 4 <= _STREAM_PARTIAL_BYTES
 
 
 _MM_OUT_DTYPE_OK = None
