@@ -729,7 +729,8 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
         return out
     if gemm_stream_preferred(x.shape[0], w.shape[0], x.shape[1], x.stride(0)) and x.data_ptr() % 16 == 0:
         out = gemm_stream(x, w, out_dtype, variant=_STREAM_VARIANT, splits=_stream_splits(x.shape[0], x.shape[1]))
-        if out.dim() == 3 and not partials_ok:
+        # a large stack is added here by many workgroups; the consumer would add it with one workgroup a row
+        if out.dim() == 3 and (not partials_ok or out.numel() * 4 > _STREAM_PARTIAL_BYTES):
             out = sum_partials(out, out_dtype)
         return out
     if out_dtype == torch.float32:
@@ -747,7 +748,7 @@ _STREAM_MAX_N = 5120            # 60 against the library's 146 us there at 32 ro
 _STREAM_MIN_K = 2048
 
 
-_STREAM_PARTIAL_BYTES = 6 << 20  # most bytes of partial products: the consumer (one workgroup a row) pays for them
+_STREAM_PARTIAL_BYTES = 6 << 20  # a larger stack of partial products is added before it is handed on
 
 
 def _stream_splits(rows: int, k: int) -> int:
@@ -756,12 +757,9 @@ def _stream_splits(rows: int, k: int) -> int:
 
 def gemm_stream_preferred(rows: int, n: int, k: int, x_stride: int) -> bool:
     """Whether the kernel whose workgroups stay, not the library, should run this product: 17..64 rows, a narrow
-    output and a long K, and a stack of partial products small enough (at the 32B shape's down projection the
-    kernel alone is a third faster than the library, but 23 partial products of 64 x 5120 cost more than that)."""
-    if not (_ROWS_PREFERRED < rows <= ROWS_KERNEL_MAX and n <= _STREAM_MAX_N and k >= _STREAM_MIN_K
-            and gemm_rows_supported(rows, k, x_stride)):
-        return False
-    return _stream_splits(rows, k) * rows * n * 4 <= _STREAM_PARTIAL_BYTES
+    output and a long K."""
+    return (_ROWS_PREFERRED < rows <= ROWS_KERNEL_MAX and n <= _STREAM_MAX_N and k >= _STREAM_MIN_K
+            and gemm_rows_supported(rows, k, x_stride))
 
 
 _MM_OUT_DTYPE_OK = None
