@@ -149,3 +149,23 @@ def test_captured_steps_of_repeated_shapes_equal_eager_ones(model, dtype):
     assert set(a) == set(b)
     for key in a:
         assert torch.equal(a[key], b[key]), f"graph replay differs from the eager step at {key}"
+
+
+def test_captured_steps_are_kept_least_recently_used(model):
+    """More step shapes than the engine may keep as graphs: the least recently used goes, and a shape that comes
+    back is captured again; the logits stay those of the eager engine."""
+    name, d, cfg, _ = model
+    make = lambda graphs: Engine.from_folder(d, dtype="float32", page_size=TINY[name][1], max_tokens=256, max_slots=4,
+                                             cuda_graph=graphs)
+    eager, graphed = make(False), make(True)
+    graphed.max_graphs = 2
+    toks = random_tokens(120, cfg["vocab_size"], 77)
+    steps, at = [], 0
+    for n in (5, 5, 7, 7, 9, 9, 5, 5, 7, 1, 1, 1, 9, 9):     # portions of three sizes, and decoded tokens
+        steps.append({"entries": [("r", toks[at:at + n], [n - 1])], "end": []})
+        at += n
+    a = replay.run_steps(eager, steps)
+    b = replay.run_steps(graphed, steps)
+    assert len(graphed._graphs) <= 2 and graphed.graph_replays >= 4
+    for key in a:
+        assert torch.equal(a[key], b[key]), key

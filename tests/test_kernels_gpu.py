@@ -720,3 +720,19 @@ def test_gemm_rows_refuses_what_it_cannot_take():
     # the general entry point still serves such shapes, through the library
     out = ops.gemm_bf16(torch.ones(2, 20, dtype=torch.bfloat16, device=DEV), torch.ones(4, 20, dtype=torch.bfloat16, device=DEV))
     assert out.shape == (2, 4) and float(out[0, 0]) == 20.0
+
+
+def test_split_choices_depend_on_shape_and_context_class_only():
+    """The split-KV factor of decoded tokens and the key parts of a short portion are functions of the step's shape
+    and of the power-of-two class of the longest context, so that a captured step and an eager one choose alike."""
+    lengths = (1, 63, 64, 127, 128, 1000, 2048, 4095, 4096, 100000)
+    caps = [ops.decode_split_cap(n) for n in lengths]
+    assert caps == [1, 1, 1, 2, 2, 16, 32, 64, 64, 64]          # largest power of two <= (blocks of 32 keys) / 2, <= 64
+    assert all(c & (c - 1) == 0 for c in caps) and caps == sorted(caps)
+    dev = torch.device(DEV)
+    args = dict(num_q_heads=32, num_kv_heads=8, head_dim=128, device=dev)
+    assert ops.portion_key_splits(2048, 2048, 1, max_kv_len=2048, **args) == 1          # enough row blocks
+    few = ops.portion_key_splits(512, 512, 1, max_kv_len=2048, **args)
+    assert 2 <= few <= 8 and few == ops.portion_key_splits(512, 512, 1, max_kv_len=3000, **args)
+    assert ops.portion_key_splits(128, 128, 1, max_kv_len=200, **args) == 1              # too few keys to cut
+    assert ops.portion_key_splits(64, 64, 1, max_kv_len=65536, **args) == 8
