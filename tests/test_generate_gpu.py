@@ -166,3 +166,34 @@ def test_trace_run_program(folders, tmp_path, dtype, tol):
     finally:
         tr.close()
     replay.compare(got, cfg, weights, reqs, tol, f"trace_run/{dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_many_requests_through_the_scheduler_with_and_without_captured_steps(folders, dtype):
+    """Thirty requests of random lengths and budgets through few slots, small portions and a pool that runs out now
+    and then: prompt portions beside decoded tokens in ever changing shapes, some of which repeat and are captured.
+    With captured steps and without, every request must get the same tokens (and in float32 the plain ones)."""
+    from arle_amd.engine import Engine
+
+    cfg, weights = read_folder(folders["B"])
+    rng = np.random.default_rng(5)
+    prompts = [random_tokens(int(n), cfg["vocab_size"], 500 + i) for i, n in enumerate(rng.integers(1, 60, size=30))]
+    budgets = [int(b) for b in rng.integers(1, 14, size=30)]
+    results = {}
+    for graphs in (False, True):
+        eng = Engine.from_folder(folders["B"], dtype=dtype, page_size=TINY["B"][1], max_tokens=208, max_slots=5,
+                                 max_request_tokens=96, cuda_graph=graphs)
+        llm = LLM(eng, num_slots=5, chunked_prefill_size=16, max_num_batched_tokens=48, max_seq_len=96)
+        outs = []
+        for lo in range(0, 30, 10):     # three waves of ten requests, each wave through one scheduler
+            wave = llm.generate(prompts[lo:lo + 10], max_tokens=max(budgets[lo:lo + 10]),
+                                sampling=SamplingParams(temperature=0.0, ignore_eos=True))
+            outs.extend(o.response_token_ids[:b] for o, b in zip(wave, budgets[lo:lo + 10]))
+        results[graphs] = outs
+        if graphs:
+            assert eng.graph_replays > 20
+        assert not eng.cache.slot_of
+    assert results[False] == results[True]
+    if dtype == "float32":
+        for p, b, got in list(zip(prompts, budgets, results[True]))[::5]:
+            assert got == _plain_greedy(cfg, weights, p, b)
