@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 TOL = {"float32": 1e-5, "bfloat16": 2e-2}
 
 
-@pytest.fixture(scope="module", params=["A", "B", "C"])
+@pytest.fixture(scope="module", params=["A", "B", "C", "D", "E"])
 def model(request, tmp_path_factory):
     name = request.param
     d = make_model_dir(tmp_path_factory.mktemp("models"), name)

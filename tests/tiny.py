@@ -27,11 +27,22 @@ TINY_C = dict(num_hidden_layers=2, hidden_size=88, num_attention_heads=3, num_ke
               head_dim=48, intermediate_size=136, vocab_size=333, rope_theta=50000.0,
               rms_norm_eps=3e-6, tie_word_embeddings=False, max_position_embeddings=1024)
 
+# D: head_dim 64 (the matrix-core kernels with a compile-time head_dim), a group of four, a page of 32 slots;
+# E: head_dim 96 (their run-time head_dim variants, three quarters of a 128 tile), two kv heads of three q heads.
+TINY_D = dict(num_hidden_layers=2, hidden_size=120, num_attention_heads=8, num_key_value_heads=2,
+              head_dim=64, intermediate_size=200, vocab_size=1003, rope_theta=300000.0,
+              rms_norm_eps=2e-6, tie_word_embeddings=True, max_position_embeddings=2048)
+TINY_E = dict(num_hidden_layers=2, hidden_size=104, num_attention_heads=6, num_key_value_heads=2,
+              head_dim=96, intermediate_size=168, vocab_size=517, rope_theta=20000.0,
+              rms_norm_eps=1e-5, tie_word_embeddings=False, max_position_embeddings=1024)
+
 # name -> (config, page size, weight std, norm std, seed)
 TINY = {
     "A": (TINY_A, 4, 0.02, 0.02, 11),
     "B": (TINY_B, 8, 0.05, 0.05, 22),
     "C": (TINY_C, 16, 0.08, 0.1, 33),
+    "D": (TINY_D, 32, 0.06, 0.05, 44),
+    "E": (TINY_E, 16, 0.07, 0.08, 55),
 }
 
 
