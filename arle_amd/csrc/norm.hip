@@ -74,8 +74,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
 // Rows of up to kVecMax elements (a multiple of 4) are read once with 16-byte loads, kept in
 // registers across the reduction and written once.  All loads of a row are issued before anything
 // is stored, so that the in-place update of the residual does not serialise them.
-constexpr int kVecPerThread = 4;                                   // float4 groups per thread
-constexpr int kVecMax = kNormThreads * kVecPerThread * 4;          // 4096 elements
+constexpr int kVecPerThreadMax = 8;                                // float4 groups per thread: 2, 4 or 8 by width
+constexpr int kVecMax = kNormThreads * kVecPerThreadMax * 4;       // 8192 elements
 
 template <typename T>
 __device__ __forceinline__ float4 load4(const T* p);
@@ -104,8 +104,10 @@ __device__ __forceinline__ void store4<bf16>(bf16* p, float4 v) {
 }
 
 // HAS_DELTA: residual row += the rows of the delta stack first, in the order of the stack (written back unless
-// `rows` picks rows for the last time).
-template <typename TIn, typename TD, typename TOut, typename TW, bool HAS_DELTA>
+// `rows` picks rows for the last time).  VPT float4 groups a thread (width <= 256 * VPT * 4).  No load stands
+// under a condition (a group past the width reads the row's last group again and is left out of the sums and
+// stores), so that all of them are in flight together.
+template <typename TIn, typename TD, typename TOut, typename TW, bool HAS_DELTA, int VPT>
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_vec_kernel(TIn* __restrict__ x, int64_t x_stride,
                                                                    const TD* __restrict__ delta, int n_delta,
                                                                    int64_t delta_stride,
@@ -118,63 +120,66 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_vec_kernel(TIn* __restri
   const int64_t src = rows ? rows[r] : r;
   TIn* xr = x + src * x_stride;
   const TD* dr = HAS_DELTA ? delta + src * static_cast<int64_t>(width) : nullptr;
-  float4 v[kVecPerThread], d[kVecPerThread], wv[kVecPerThread];
+  float4 v[VPT], d[VPT], wv[VPT];
+  int at[VPT];
+  bool in[VPT];
 #pragma unroll
-  for (int j = 0; j < kVecPerThread; ++j) {
+  for (int j = 0; j < VPT; ++j) {
     const int i = 4 * (threadIdx.x + j * kNormThreads);
-    if (i < width) {
-      v[j] = load4<TIn>(xr + i);
-      if (HAS_DELTA) d[j] = load4<TD>(dr + i);
-      wv[j] = load4<TW>(w + i);
-    }
+    in[j] = i < width;
+    at[j] = in[j] ? i : width - 4;
+    v[j] = load4<TIn>(xr + at[j]);
+    if (HAS_DELTA) d[j] = load4<TD>(dr + at[j]);
+    wv[j] = load4<TW>(w + at[j]);
   }
   if (HAS_DELTA) {  // the rest of the stack, a few rows of loads in flight at a time
-#pragma unroll 4
+#pragma unroll 2
     for (int sp = 1; sp < n_delta; ++sp) {
-      float4 e[kVecPerThread];
+      float4 e[VPT];
 #pragma unroll
-      for (int j = 0; j < kVecPerThread; ++j) {
-        const int i = 4 * (threadIdx.x + j * kNormThreads);
-        if (i < width) e[j] = load4<TD>(dr + sp * delta_stride + i);
-      }
+      for (int j = 0; j < VPT; ++j) e[j] = load4<TD>(dr + sp * delta_stride + at[j]);
 #pragma unroll
-      for (int j = 0; j < kVecPerThread; ++j) {
-        const int i = 4 * (threadIdx.x + j * kNormThreads);
-        if (i < width) {
-          d[j].x += e[j].x;
-          d[j].y += e[j].y;
-          d[j].z += e[j].z;
-          d[j].w += e[j].w;
-        }
+      for (int j = 0; j < VPT; ++j) {
+        d[j].x += e[j].x;
+        d[j].y += e[j].y;
+        d[j].z += e[j].z;
+        d[j].w += e[j].w;
       }
     }
   }
   float ss = 0.f;
 #pragma unroll
-  for (int j = 0; j < kVecPerThread; ++j) {
-    const int i = 4 * (threadIdx.x + j * kNormThreads);
-    if (i < width) {
-      if (HAS_DELTA) {
-        v[j].x += d[j].x;
-        v[j].y += d[j].y;
-        v[j].z += d[j].z;
-        v[j].w += d[j].w;
-        if (!rows) store4<TIn>(xr + i, v[j]);
-      }
-      ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+  for (int j = 0; j < VPT; ++j) {
+    if (HAS_DELTA) {
+      v[j].x += d[j].x;
+      v[j].y += d[j].y;
+      v[j].z += d[j].z;
+      v[j].w += d[j].w;
+      if (!rows && in[j]) store4<TIn>(xr + at[j], v[j]);
     }
+    if (in[j]) ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
   }
   const float total = block_sum<kNormWaves>(ss, lds);
   const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
   TOut* o = out + static_cast<int64_t>(r) * width;
 #pragma unroll
-  for (int j = 0; j < kVecPerThread; ++j) {
-    const int i = 4 * (threadIdx.x + j * kNormThreads);
-    if (i < width)
-      store4<TOut>(o + i, float4{v[j].x * inv * wv[j].x, v[j].y * inv * wv[j].y, v[j].z * inv * wv[j].z,
-                                 v[j].w * inv * wv[j].w});
+  for (int j = 0; j < VPT; ++j) {
+    if (in[j])
+      store4<TOut>(o + at[j], float4{v[j].x * inv * wv[j].x, v[j].y * inv * wv[j].y, v[j].z * inv * wv[j].z,
+                                     v[j].w * inv * wv[j].w});
   }
 }
+
+// the variant with the fewest groups a thread that covers the width
+#define ARLE_NORM_VEC(TIN, TD, TOUT, TW, HAS_DELTA, ...)                                             \
+  do {                                                                                               \
+    if (width <= kNormThreads * 8)                                                                   \
+      rmsnorm_vec_kernel<TIN, TD, TOUT, TW, HAS_DELTA, 2><<<n_rows, kNormThreads, 0, s>>>(__VA_ARGS__); \
+    else if (width <= kNormThreads * 16)                                                             \
+      rmsnorm_vec_kernel<TIN, TD, TOUT, TW, HAS_DELTA, 4><<<n_rows, kNormThreads, 0, s>>>(__VA_ARGS__); \
+    else                                                                                             \
+      rmsnorm_vec_kernel<TIN, TD, TOUT, TW, HAS_DELTA, 8><<<n_rows, kNormThreads, 0, s>>>(__VA_ARGS__); \
+  } while (0)
 
 // A stack of float32 deltas (the partial products of a matrix product whose K was split over
 // workgroups) added into the residual row, then the norm.  Few rows make few workgroups here, so the
@@ -244,7 +249,7 @@ __global__ __launch_bounds__(kStackThreads) void add_stack_rmsnorm_kernel(
 
 inline bool vec_ok(int width, long long x_stride, const void* a, const void* b, const void* c, const void* d) {
   auto al = [](const void* p) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-  return width % 4 == 0 && width <= kVecMax && x_stride % 4 == 0 && al(a) && al(b) && al(c) && al(d);
+  return width % 4 == 0 && width >= 4 && width <= kVecMax && x_stride % 4 == 0 && al(a) && al(b) && al(c) && al(d);
 }
 
 template <typename TIn, typename TOut>
@@ -253,11 +258,11 @@ int launch_rmsnorm(const void* x, long long x_stride, const void* w, int w_dtype
   if (vec_ok(width, x_stride, x, w, out, nullptr)) {
     TIn* xp = const_cast<TIn*>(static_cast<const TIn*>(x));
     if (w_dtype == kF32)
-      rmsnorm_vec_kernel<TIn, TIn, TOut, float, false><<<n_rows, kNormThreads, 0, s>>>(
-          xp, x_stride, nullptr, 0, 0, static_cast<const float*>(w), static_cast<TOut*>(out), rows, width, eps);
+      ARLE_NORM_VEC(TIn, TIn, TOut, float, false, xp, x_stride, nullptr, 0, 0, static_cast<const float*>(w),
+                    static_cast<TOut*>(out), rows, width, eps);
     else
-      rmsnorm_vec_kernel<TIn, TIn, TOut, bf16, false><<<n_rows, kNormThreads, 0, s>>>(
-          xp, x_stride, nullptr, 0, 0, static_cast<const bf16*>(w), static_cast<TOut*>(out), rows, width, eps);
+      ARLE_NORM_VEC(TIn, TIn, TOut, bf16, false, xp, x_stride, nullptr, 0, 0, static_cast<const bf16*>(w),
+                    static_cast<TOut*>(out), rows, width, eps);
     return launch_status();
   }
   if (w_dtype == kF32) {
@@ -291,13 +296,11 @@ int launch_add_rmsnorm(float* residual, const void* delta, int n_delta, long lon
   }
   if (vec_ok(width, width, residual, delta, w, out) && delta_stride % 4 == 0) {
     if (w_dtype == kF32)
-      rmsnorm_vec_kernel<float, TD, TOut, float, true><<<n_rows, kNormThreads, 0, s>>>(
-          residual, width, static_cast<const TD*>(delta), n_delta, delta_stride, static_cast<const float*>(w),
-          static_cast<TOut*>(out), rows, width, eps);
+      ARLE_NORM_VEC(float, TD, TOut, float, true, residual, width, static_cast<const TD*>(delta), n_delta,
+                    delta_stride, static_cast<const float*>(w), static_cast<TOut*>(out), rows, width, eps);
     else
-      rmsnorm_vec_kernel<float, TD, TOut, bf16, true><<<n_rows, kNormThreads, 0, s>>>(
-          residual, width, static_cast<const TD*>(delta), n_delta, delta_stride, static_cast<const bf16*>(w),
-          static_cast<TOut*>(out), rows, width, eps);
+      ARLE_NORM_VEC(float, TD, TOut, bf16, true, residual, width, static_cast<const TD*>(delta), n_delta,
+                    delta_stride, static_cast<const bf16*>(w), static_cast<TOut*>(out), rows, width, eps);
     return launch_status();
   }
   if (w_dtype == kF32) {

@@ -28,7 +28,7 @@ def test_embed_gather():
         assert torch.equal(out.cpu(), table.to(dt).float()[ids.long()])
 
 
-@pytest.mark.parametrize("width", [4, 96, 260, 2560])
+@pytest.mark.parametrize("width", [4, 96, 260, 2044, 2560, 4096, 5120, 6004, 8192, 8196, 9001])
 @pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("wdt", [torch.float32, torch.bfloat16])
 def test_rmsnorm_and_fused_add(width, act, wdt):
