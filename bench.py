@@ -145,7 +145,7 @@ def decode_32b(args) -> int:
 
     raw = dict(QWEN3_32B, num_hidden_layers=args.layers or QWEN3_32B["num_hidden_layers"])
     config = Qwen3Config.from_dict(raw)
-    batch, context = args.batch if args.batch != 8 else 64, 8192
+    batch, context = args.batch or 64, args.context
     steps, warmup = min(args.steps, 16), min(args.warmup, 4)
     t0 = time.time()
     engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype="bfloat16", page_size=PAGE,
@@ -173,7 +173,7 @@ def decode_32b(args) -> int:
     dt = _timed(torch, lambda: [one_step() for _ in range(steps)])
     ctx_mean = ctx0 + (steps - 1) / 2.0 + 1
     achieved = decode_bytes(raw, batch, ctx_mean) / (dt / steps) / 1e9
-    line = {"metric": f"decode tok/s at batch {batch}, 8,192 tokens of context (Qwen3-32B shape, random weights)",
+    line = {"metric": f"decode tok/s at batch {batch}, {context:,} tokens of context (Qwen3-32B shape, random weights)",
             "value": round(batch * steps / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
             "ms_per_step": round(dt / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16", "data": "synthetic: seeded random weights N(0,0.02), uniform random token ids",
@@ -192,7 +192,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=None, help="decoding requests (default: 8; 64 for qwen3-32b-decode)")
+    ap.add_argument("--context", type=int, default=8192, help="tokens of context of the qwen3-32b-decode workload")
     ap.add_argument("--layers", type=int, default=FULL_LAYERS)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 decode points")
@@ -204,6 +205,8 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
         return 2
+    if args.workload == "qwen3-4b" and args.batch is None:
+        args.batch = 8
     if args.workload != "qwen3-4b":
         if args.layers == FULL_LAYERS:
             args.layers = 0   # the workload's own depth
