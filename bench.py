@@ -1,7 +1,7 @@
 """Decode and prefill throughput of the Qwen3-4B shape with random weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
-    python bench.py --workload qwen3-8b-mixed | qwen3-32b-decode     (the baseline's two further workloads)
+    python bench.py --workload qwen3-8b-mixed | qwen3-32b-decode     (two further workloads)
 
 A step is one decode step of `batch` requests, each holding a `prompt`-token random prompt
 (prefilled by the engine itself before the clock starts) and growing by one token per step.
@@ -18,11 +18,11 @@ import time
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-# BASELINE.json configs[2]: Qwen3-4B shape
+# the benchmark configuration: Qwen3-4B shape
 QWEN3_4B = dict(num_hidden_layers=36, hidden_size=2560, num_attention_heads=32, num_key_value_heads=8,
                 head_dim=128, intermediate_size=9728, vocab_size=151936, rope_theta=1000000.0,
                 rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=40960)
-# BASELINE.json configs[3] and [4]: the two other workloads (`--workload`)
+# the two further workloads (`--workload`): Qwen3-8B and Qwen3-32B shapes
 QWEN3_8B = dict(num_hidden_layers=36, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
                 head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1000000.0,
                 rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960)
@@ -66,7 +66,7 @@ def _timed(torch, fn):
 
 
 def mixed_8b(args) -> int:
-    """BASELINE.json configs[3]: 32 requests decoding at 1,024 tokens of context beside one 2,048-token prompt
+    """Qwen3-8B shape: 32 requests decoding at 1,024 tokens of context beside one 2,048-token prompt
     that arrives in portions of 512: four steps of 32 + 512 rows.  Reports the mean step and the tokens a second
     of both kinds."""
     import torch
@@ -135,7 +135,7 @@ def prefill_flops_portion(c, start: int, n: int) -> float:
 
 
 def decode_32b(args) -> int:
-    """BASELINE.json configs[4]: 64 requests decoding at 8,192 tokens of context, Qwen3-32B shape (65 GB of
+    """Qwen3-32B shape: 64 requests decoding at 8,192 tokens of context by default (65 GB of
     weights, 137 GB of cache)."""
     import torch
 
@@ -200,7 +200,7 @@ def main() -> int:
     ap.add_argument("--prefill-only", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiles of its kernels) and print that")
     ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode"],
-                    help="qwen3-4b is the contract's run; the other two are the further workloads of the baseline")
+                    help="qwen3-4b is the default run; the other two are further workloads at larger shapes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
