@@ -830,6 +830,309 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
  }  // next item
 }
 
+// ---------------------------------------------------------------------------------------------
+// Prompt portions, head_dim 128: the same work as attn_prefill_lds_kernel, built around three facts that its
+// counters showed (no unit busy half the time; a third of the vector instructions spent on moving tiles; every
+// wave reading the whole tile from LDS for 16 rows only).
+//
+//   * A wave owns 32 rows and multiplies with v_mfma_f32_32x32x16_bf16: a key or value operand read from LDS
+//     serves twice the rows.  Four waves a workgroup (128 rows, as before), two workgroups a CU.
+//   * Tiles go from memory straight to LDS (global_load_lds_dwordx4): no staging registers, no second pass that
+//     parks them, and the loads of tile i + 1 are in flight while tile i is computed.
+//   * LDS rows carry no padding (a direct load fills 64 consecutive 16-byte pieces); instead piece c of row r
+//     lies at position c ^ (r & 7), which a lane gets by fetching the matching piece from memory, so that the
+//     operand reads of 32 rows still spread over all banks.
+//
+// Layouts (lane = 32 h + j):  scores S^T = K . Q^T per 32 keys: A lane (key j, h) = K[key][16 s + 8 h ..+7],
+// B lane (row j, h) = Q[row][16 s + 8 h ..+7], C register r = S^T[key 8 (r / 4) + 4 h + r % 4][row j].
+// Second product O^T += V^T . P^T in steps of 16 keys: lane (row j, h) offers the eight probabilities that it
+// holds anyway, registers 8 u .. 8 u + 7 of a score tile, i.e. keys 16 u + 4 h + {0..3} and 16 u + 8 + 4 h + {0..3},
+// and the value operand is read in that key order (two 8-byte reads of a d row).  Nothing moves between lanes.
+constexpr int kDmWaves = 4;
+constexpr int kDmD = 128;
+constexpr int kDmKeys = 64;
+constexpr int kDmStageBytes = kDmKeys * kDmD * 2 * 2;  // keys and values of a tile: 32 KB
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(const AttnArgs a, int min_rows, int blocks_x,
+                                                                              int segments, int listed) {
+  constexpr int D = kDmD;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  __shared__ unsigned int item_of_workgroup;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 31, h = lane >> 5;
+  const int G = a.nq / a.nkv;
+  const unsigned int nkv = static_cast<unsigned int>(a.nkv);
+  const unsigned int pairs = listed ? g_prefill_pairs : static_cast<unsigned int>(blocks_x) * segments;
+  const unsigned int parts = static_cast<unsigned int>(a.portion_splits);
+  const unsigned int items = pairs * nkv * parts;
+  const int P = a.P, ps = a.p_shift, pm = P - 1;
+  const int64_t page_elems = static_cast<int64_t>(a.nkv) * P * D;
+ for (;;) {
+  if (tid == 0) item_of_workgroup = atomicAdd(&g_prefill_next_item, 1u);
+  __syncthreads();
+  const unsigned int item = item_of_workgroup;
+  __syncthreads();
+  if (item >= items) return;
+  const unsigned int pair = item / (nkv * parts);
+  const int kvh = static_cast<int>((item / parts) % nkv);
+  const int part = static_cast<int>(item % parts);
+  int seg = static_cast<int>(pair % segments), wg_row = (blocks_x - 1 - static_cast<int>(pair / segments)) * kPfRows;
+  if (listed) {
+    const unsigned int entry = g_prefill_plan[pair];
+    seg = static_cast<int>(entry & 0xffffu);
+    wg_row = static_cast<int>(entry >> 16) * kPfRows;
+  }
+  const int row0 = a.seg_row0[seg];
+  const int qlen = a.seg_row0[seg + 1] - row0;
+  const int rows = qlen * G;
+  if (rows < min_rows) continue;
+  if (wg_row >= rows) continue;
+  const int start = a.seg_start[seg];
+  const int* table = a.block_table + static_cast<int64_t>(a.seg_slot[seg]) * a.table_stride;
+  const int64_t head_off = static_cast<int64_t>(kvh) * P * D;
+
+  const int tok_min = wg_row / G;
+  const int tok_max = (min(wg_row + kPfRows, rows) - 1) / G;
+  const int kv_total = start + qlen;
+  const int kv_hi = start + tok_max + 1;
+  const int kv_lo = a.window > 0 ? max(0, start + tok_min - a.window + 1) : 0;
+  int t0 = kv_lo / kDmKeys, t1 = (kv_hi + kDmKeys - 1) / kDmKeys;
+  if (parts > 1) {
+    const int per = (t1 - t0 + static_cast<int>(parts) - 1) / static_cast<int>(parts);
+    t0 = t0 + part * per;
+    t1 = min(t0 + per, t1);
+  }
+
+  // this wave's 32 rows; the lane's own row is row_begin + j (both halves h of a row hold the same statistics)
+  const int row_begin = wg_row + 32 * wave;
+  const bool wave_has_rows = row_begin < rows;
+  const int wave_tok_max = wave_has_rows ? (min(row_begin + 32, rows) - 1) / G : 0;
+  const int wave_kv_hi = start + wave_tok_max + 1;
+  const int wave_pos_min = start + min(row_begin, rows - 1) / G;
+  const int wave_kv_lo = a.window > 0 ? max(0, wave_pos_min - a.window + 1) : 0;
+  const int wave_win_lo = a.window > 0 ? max(0, start + wave_tok_max - a.window + 1) : 0;
+  const int row = row_begin + j;
+  const bool row_ok = row < rows;
+  const int my_tok = min(row / G, qlen - 1);
+  const int my_head = kvh * G + row % G;
+  const int my_pos = start + my_tok;
+  bf16x8 qreg[D / 16];
+  {
+    const uint16_t* qp = a.q + static_cast<int64_t>(row0 + my_tok) * a.q_stride + my_head * D + 8 * h;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) qreg[s] = load_bf16x8(qp + 16 * s);
+  }
+  f32x16 o[D / 32];
+#pragma unroll
+  for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  // page ids of 64 consecutive logical pages in one register across the wave (lane i: page pg_base + i)
+  const int pg_last = (kv_hi - 1) >> ps;
+  int pg_base = 0, pg_reg = 0;
+  auto cover = [&](int tile, bool first) {
+    const int lo = min(max(tile * kDmKeys, kv_lo), kv_hi - 1) >> ps;
+    const int hi = min(max(tile * kDmKeys + kDmKeys - 1, kv_lo), kv_hi - 1) >> ps;
+    if (first || lo < pg_base || hi >= pg_base + kWave) {
+      pg_base = lo;
+      pg_reg = table[min(lo + lane, pg_last)];
+    }
+  };
+  // what a lane fetches for a tile never changes but for the page: four pieces of keys and four of values
+  //   keys:   LDS piece q = 64 (4 wave + jj) + lane -> key q / 16 of the tile, position q % 16 in its row
+  //   values: LDS piece q                           -> d row q / 8,            position q % 8
+  int k_key[4], k_src[4], v_key[4], v_src[4];
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) {
+    const int q = 64 * (4 * wave + jj) + lane;
+    const int key = q / 16, pos = q % 16;
+    k_key[jj] = key;
+    k_src[jj] = 8 * (pos ^ (key & 7));               // element offset of the piece inside its key row
+    const int d = q / 8, vpos = q % 8;
+    v_key[jj] = 8 * (vpos ^ (d & 7));                 // first of the piece's eight keys, inside the tile
+    v_src[jj] = d * P;                                // element offset of the d row inside a page
+  }
+  auto fetch = [&](int tile, int stage) {
+    const int base = tile * kDmKeys;
+    unsigned char* at = lds_raw + stage * kDmStageBytes + (4 * wave) * 1024;
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int key = min(max(base + k_key[jj], kv_lo), kv_hi - 1);  // a key that exists; what lies outside is masked
+      const int page = __shfl(pg_reg, (key >> ps) - pg_base, kWave);
+      const uint16_t* src = a.k_pages + page * page_elems + head_off + static_cast<int64_t>(key & pm) * D + k_src[jj];
+      __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)(at + jj * 1024), 16, 0, 0);
+    }
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int key8 = min(max(base + v_key[jj], kv_lo & ~7), (kv_hi - 1) & ~7);
+      const int page = __shfl(pg_reg, (key8 >> ps) - pg_base, kWave);
+      const uint16_t* src = a.v_pages + page * page_elems + head_off + v_src[jj] + (key8 & pm);
+      __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)(at + kDmKeys * D * 2 + jj * 1024),
+                                       16, 0, 0);
+    }
+  };
+  // Slots past the request's last token may hold anything, also NaN, and 0 * NaN is NaN: in the request's last
+  // tile every lane puts the values of such keys to zero in the pieces that it fetched itself.
+  auto scrub = [&](int tile, int stage) {
+    const int base = tile * kDmKeys;
+    if (base + kDmKeys <= kv_total) return;
+    unsigned char* at = lds_raw + stage * kDmStageBytes + kDmKeys * D * 2 + (4 * wave) * 1024 + lane * 16;
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int key8 = min(max(base + v_key[jj], kv_lo & ~7), (kv_hi - 1) & ~7);  // the keys that were fetched
+      if (key8 + 8 > kv_total) {
+        u32x4 v = *reinterpret_cast<u32x4*>(at + jj * 1024);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (key8 + e >= kv_total) v[e / 2] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+        *reinterpret_cast<u32x4*>(at + jj * 1024) = v;
+      }
+    }
+  };
+
+  if (t0 < t1) {
+    cover(t0, true);
+    fetch(t0, 0);
+  }
+  for (int tile = t0; tile < t1; ++tile) {
+    const int stage = (tile - t0) & 1;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's pieces of the tile have landed
+    scrub(tile, stage);
+    __syncthreads();  // everybody's have; and everybody is done with the other stage
+    if (tile + 1 < t1) {
+      cover(tile + 1, false);
+      fetch(tile + 1, stage ^ 1);
+    }
+    const int key_base = tile * kDmKeys;
+    const bool computes = wave_has_rows && key_base < wave_kv_hi && key_base + kDmKeys > wave_kv_lo;
+    if (!computes) continue;
+    const unsigned char* ks = lds_raw + stage * kDmStageBytes;
+    const unsigned char* vs = ks + kDmKeys * D * 2;
+
+    // scores of 2 x 32 keys
+    f32x16 st[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      bf16x8 kop[D / 16];
+      const int key = 32 * t + j;
+#pragma unroll
+      for (int s = 0; s < D / 16; ++s)
+        kop[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(ks + key * (D * 2) + (((2 * s + h) ^ (key & 7)) * 16)));
+      __builtin_amdgcn_sched_barrier(0);
+      f32x16 z;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) z[r] = 0.f;
+#pragma unroll
+      for (int s = 0; s < D / 16; ++s) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kop[s], qreg[s], z, 0, 0, 0);
+      st[t] = z;
+    }
+    // st[t][r] belongs to key key_base + 32 t + 8 (r / 4) + 4 h + r % 4 and to this lane's row
+    const bool masked = key_base + kDmKeys - 1 > wave_pos_min || key_base < wave_win_lo;
+    if (masked) {
+      const int lo = a.window > 0 ? my_pos - a.window + 1 : 0;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = key_base + 32 * t + 8 * (r / 4) + 4 * h + r % 4;
+          if (!(key >= lo && key <= my_pos)) st[t][r] = -INFINITY;
+        }
+    }
+    float bmax = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) bmax = fmaxf(bmax, st[t][r]);
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave)) * a.scale_log2;  // scale > 0: the maximum commutes with it
+    const float m_new = fmaxf(m, bmax);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
+    const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+    float psum = 0.f;
+    bf16x8 pb[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        u32x4 packed;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float p0 = __builtin_amdgcn_exp2f(fmaf(st[t][8 * u + 2 * e], a.scale_log2, -m_use));
+          const float p1 = __builtin_amdgcn_exp2f(fmaf(st[t][8 * u + 2 * e + 1], a.scale_log2, -m_use));
+          psum += p0 + p1;
+          packed[e] = pack_bf16x2(p0, p1);
+        }
+        pb[t][u] = __builtin_bit_cast(bf16x8, packed);
+      }
+    psum += __shfl_xor(psum, 32, kWave);
+    l = l * alpha + psum;
+    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {  // the sums need the factor only if some row's maximum moved
+#pragma unroll
+      for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+    }
+    m = m_new;
+
+    // O^T += V^T . P^T, 16 keys a step
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int c = 4 * t + 2 * u;  // piece that holds keys 32 t + 16 u .. + 7; the next one holds .. + 8 .. + 15
+        u32x4 vop[D / 32];
+#pragma unroll
+        for (int dt = 0; dt < D / 32; ++dt) {
+          const int d = 32 * dt + j;
+          const unsigned char* vrow = vs + d * (kDmKeys * 2) + 8 * h;
+          const u32x2 va = *reinterpret_cast<const u32x2*>(vrow + ((c ^ (d & 7)) * 16));
+          const u32x2 vb = *reinterpret_cast<const u32x2*>(vrow + (((c + 1) ^ (d & 7)) * 16));
+          vop[dt][0] = va[0];
+          vop[dt][1] = va[1];
+          vop[dt][2] = vb[0];
+          vop[dt][3] = vb[1];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int dt = 0; dt < D / 32; ++dt)
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vop[dt]), pb[t][u], o[dt], 0, 0, 0);
+      }
+  }
+  __syncthreads();  // the next item's first tile goes into stage 0: everybody has to be done reading
+
+  // o[dt][r] is O^T[d = 32 dt + 8 (r / 4) + 4 h + r % 4][this lane's row]
+  if (row_ok) {
+    if (parts > 1) {
+      const int64_t slot = ((static_cast<int64_t>(row0 + my_tok) * a.nq + my_head) * parts + part);
+      float* wo = a.pws_o + slot * D;
+#pragma unroll
+      for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<float4*>(wo + 32 * dt + 8 * q + 4 * h) =
+              float4{o[dt][4 * q], o[dt][4 * q + 1], o[dt][4 * q + 2], o[dt][4 * q + 3]};
+      if (h == 0) {
+        a.pws_ml[slot * 2] = m;
+        a.pws_ml[slot * 2 + 1] = l;
+      }
+    } else {
+      const float inv_l = l > 0.f ? 1.0f / l : 0.f;
+      uint16_t* op = a.out + static_cast<int64_t>(row0 + my_tok) * a.o_stride + my_head * D;
+#pragma unroll
+      for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          uint2 w;
+          w.x = pack_bf16x2(o[dt][4 * q] * inv_l, o[dt][4 * q + 1] * inv_l);
+          w.y = pack_bf16x2(o[dt][4 * q + 2] * inv_l, o[dt][4 * q + 3] * inv_l);
+          *reinterpret_cast<uint2*>(op + 32 * dt + 8 * q + 4 * h) = w;
+        }
+    }
+  }
+ }  // next item
+}
+
 // The parts of a portion's rows put together: out = sum_p o_p 2^(m_p - m) / sum_p l_p 2^(m_p - m), in the order
 // of the parts.  Work items are (listed pair, kv head, eight rows of the row block): a workgroup of eight waves
 // takes items blockIdx.x, blockIdx.x + gridDim.x, ... and each wave one row of the item, a lane four columns
@@ -944,9 +1247,64 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
   return launch_status();
 }
 
+int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s) {
+  const size_t lds = 2 * kDmStageBytes;
+  static bool asked = false;  // dynamic LDS of 64 KiB and more has to be asked for, once
+  if (!asked) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_dma_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return static_cast<int>(e);
+    }
+    asked = true;
+  }
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cus = n;
+  }
+  const long long items = static_cast<long long>(grid.x) * grid.y * grid.z * a.portion_splits;
+  const unsigned workgroups = static_cast<unsigned>(items < 2LL * cus ? items : 2LL * cus);  // two of four waves a CU
+  const int listed = static_cast<long long>(grid.x) * grid.z <= kPfPlanMax && grid.x <= 65535 && grid.z <= 65535;
+  if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);
+  attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
+                                             a.nq / a.nkv, min_rows, listed);
+  attn_prefill_dma_kernel<<<workgroups, kDmWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
+                                                                   static_cast<int>(grid.z), listed);
+  if (a.portion_splits > 1) {
+    const long long most = static_cast<long long>(grid.x) * grid.y * grid.z * (kPfRows / kPfWaves);
+    attn_merge_portions_kernel<<<static_cast<unsigned>(most < 4LL * cus ? most : 4LL * cus), kPfWaves * kWave, 0, s>>>(a);
+  }
+  return launch_status();
+}
+
+// -1: the launcher decides (below); 1: head_dim 128 portions always run attn_prefill_dma_kernel; 0: always
+// attn_prefill_lds_kernel, as every other head_dim does.  For measurements and tests that compare the two.
+static int g_prefill_dma = -1;
+
+// The kernel with 32 rows a wave does a tile in two thirds of the time, but it occupies twice the workgroup
+// slots (two a CU), so a causal prompt from position 0 with about as many items as slots leaves each slot one
+// item, and the run lasts as long as the heaviest of them.  It pays when there are several items a slot to hand
+// out, or an item for every slot and the items are alike because a long context stands before the portion.
+inline bool prefill_dma_pays(dim3 grid, int max_qlen, int max_kv_len) {
+  if (g_prefill_dma >= 0) return g_prefill_dma != 0;
+  int dev = 0, cus = 256;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+      cus <= 0)
+    cus = 256;
+  const long long items = static_cast<long long>(grid.x) * grid.y * grid.z;
+  const int most = (max_kv_len + kDmKeys - 1) / kDmKeys, least = (max(max_kv_len - max_qlen, 0) + kDmKeys - 1) / kDmKeys;
+  return items >= 6LL * cus || (items >= 2LL * cus && 2 * least >= most);
+}
+
 }  // namespace arle
 
 using namespace arle;
+
+extern "C" void arle_attn_prefill_variant(int dma) { g_prefill_dma = dma; }
 
 // Token rows that the split-KV workspace holds for every segment: the most tokens of a segment whose rows
 // (tokens x q heads of a kv head) fit one row tile of 16.
@@ -958,7 +1316,8 @@ extern "C" int arle_attn_ws_rows(int max_qlen, int nq, int nkv) {
 // q, out: bfloat16 [token rows, nq*D] (row strides in elements).  Segments describe the packed
 // step: seg_row0[s]..seg_row0[s+1] are the token rows of segment s, whose first token sits at
 // position seg_start[s] of the request in block-table row seg_slot[s]; the cache already holds
-// the keys and values of these tokens.  max_qlen / min_qlen are the longest and shortest segment.  With splits > 1,
+// the keys and values of these tokens.  max_qlen / min_qlen are the longest and shortest segment, max_kv_len the most
+// keys any request holds after the step (it only steers the choice between kernels).  With splits > 1,
 // ws_o/ws_ml must hold [segments * ws_rows][nq][splits][D] and [..][2] floats, ws_rows = arle_attn_ws_rows(...),
 // and the merge runs after; the split is over the keys of segments of at most 16 rows (decoded tokens and
 // portions of a few tokens).  Longer portions go to the LDS kernel; when they have too few row blocks to fill
@@ -969,7 +1328,7 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
                                     const void* k_pages, const void* v_pages, const int* block_table,
                                     int table_stride, const int* seg_row0, const int* seg_slot,
                                     const int* seg_start, int segments, int max_qlen, int min_qlen,
-                                    int token_rows,
+                                    int max_kv_len, int token_rows,
                                     int nq, int nkv, int D, int page_size, float scale, int window,
                                     int splits, float* ws_o, float* ws_ml, int portion_splits, float* pws_o,
                                     float* pws_ml, void* stream) {
@@ -1018,6 +1377,8 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
     dim3 grid((max_rows + kPfRows - 1) / kPfRows, nkv, segments);
     if (D == 64)
       rc = launch_prefill_lds<64, true>(a, grid, 17, s);
+    else if (D == 128 && page_size % 8 == 0 && prefill_dma_pays(grid, max_qlen, max_kv_len))
+      rc = launch_prefill_dma(a, grid, 17, s);
     else if (D == 128)
       rc = launch_prefill_lds<128, true>(a, grid, 17, s);
     else if (D <= 64)

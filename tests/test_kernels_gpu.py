@@ -554,6 +554,59 @@ def test_attention_mfma_step_too_large_for_the_work_list():
     assert _rel(out[long_n:].cpu(), torch.cat(wants)) < 8e-3
 
 
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("nq,nkv,P", [(32, 8, 16), (8, 8, 8), (16, 1, 64), (8, 1, 32), (6, 2, 128)])
+@pytest.mark.parametrize("parts,window", [(None, 0), (1, 0), (3, 0), (8, 37), (1, 200)])
+def test_attention_mfma_both_portion_kernels_at_head_dim_128(variant, nq, nkv, P, parts, window):
+    """head_dim 128 has two kernels for prompt portions (16 rows a wave with tiles parked in LDS by the waves; 32
+    rows a wave with tiles loaded straight into LDS), chosen by the shape of the step; here each is forced in turn:
+    portions that start inside a page after a cached prefix, whole prompts of several row blocks, a single first
+    token and decoded tokens beside them, windows, and keys cut into parts."""
+    from arle_amd.kernels import lib
+    lib.function("arle_attn_prefill_variant")(variant)
+    try:
+        got, want = _mfma_case(nq, nkv, 128, P, [(300, 70), (45, 39), (0, 1), (130, 2), (0, 330), (77, 1)], window, 1,
+                               175, portion_splits=parts)
+    finally:
+        lib.function("arle_attn_prefill_variant")(-1)
+    assert torch.isfinite(got).all()
+    assert _rel(got, want) < 8e-3
+
+
+def test_attention_mfma_dma_kernel_masks_stale_slots():
+    """The kernel that loads tiles straight into LDS: pages hold NaN bits in every slot that was never written."""
+    from arle_amd.kernels import lib
+    nq, nkv, D, P = 8, 2, 128, 16
+    dt = torch.bfloat16
+    segs = [(200, 150), (17, 130), (0, 70)]
+    lengths = [a + b for a, b in segs]
+    table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, 190)
+    k_pages.fill_(float("nan"))
+    v_pages.fill_(float("nan"))
+    qs, wants, row0, starts = [], [], [0], []
+    for s, (cached, n) in enumerate(segs):
+        g = _g(191 + s)
+        q, k, v = (torch.randn(cached + n, h, D, generator=g).to(dt) for h in (nq, nkv, nkv))
+        _fill_cache(table, k_pages, v_pages, s, k, v, P)
+        qs.append(q[cached:].reshape(n, -1))
+        wants.append(plain.causal_attention(q.double(), k.double(), v.double(), nkv)[cached:].reshape(n, -1))
+        row0.append(row0[-1] + n)
+        starts.append(cached)
+    q_all = torch.cat(qs).to(DEV)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    lib.function("arle_attn_prefill_variant")(1)
+    try:
+        for parts in (1, 2):
+            out = torch.full_like(q_all, float("nan"))
+            ops.attn_paged_mfma(q_all, out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0), i32([0, 1, 2]),
+                                i32(starts), max_qlen=150, min_qlen=70, max_kv_len=max(lengths), num_q_heads=nq,
+                                num_kv_heads=nkv, head_dim=D, page_size=P, scale=1.0 / math.sqrt(D), portion_splits=parts)
+            assert torch.isfinite(out).all()
+            assert _rel(out.cpu(), torch.cat(wants)) < 8e-3
+    finally:
+        lib.function("arle_attn_prefill_variant")(-1)
+
+
 def test_attention_mfma_finds_a_far_key():
     nq, nkv, D, P, n = 4, 2, 64, 16, 900
     dt = torch.bfloat16
