@@ -843,19 +843,36 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
 //     lies at position c ^ (r & 7), which a lane gets by fetching the matching piece from memory, so that the
 //     operand reads of 32 rows still spread over all banks.
 //
-// Layouts (lane = 32 h + j):  scores S^T = K . Q^T per 32 keys: A lane (key j, h) = K[key][16 s + 8 h ..+7],
-// B lane (row j, h) = Q[row][16 s + 8 h ..+7], C register r = S^T[key 8 (r / 4) + 4 h + r % 4][row j].
+// Layouts (lane = 32 h + j):  scores S^T = K . Q^T per 32 keys: A lane (i = j, h) = K[key(i)][16 s + 8 h ..+7],
+// B lane (row j, h) = Q[row][16 s + 8 h ..+7], C register r = S^T[i = 8 (r / 4) + 4 h + r % 4][row j], where
+// key(i) is i with bits 2 and 3 exchanged: so register r is key 16 (r / 8) + 8 h + r % 8.
 // Second product O^T += V^T . P^T in steps of 16 keys: lane (row j, h) offers the eight probabilities that it
-// holds anyway, registers 8 u .. 8 u + 7 of a score tile, i.e. keys 16 u + 4 h + {0..3} and 16 u + 8 + 4 h + {0..3},
-// and the value operand is read in that key order (two 8-byte reads of a d row).  Nothing moves between lanes.
+// holds anyway, registers 8 u .. 8 u + 7 of a score tile, i.e. keys 16 u + 8 h .. + 7, and the value operand
+// of lane (d, h) is the 16-byte piece of row d with those keys.  Nothing moves between lanes.
 constexpr int kDmWaves = 4;
 constexpr int kDmD = 128;
 constexpr int kDmKeys = 64;
 constexpr int kDmStageBytes = kDmKeys * kDmD * 2 * 2;  // keys and values of a tile: 32 KB
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
+// Sixteen bytes a lane from memory straight into LDS: the wave's 64 pieces land one after the other from
+// lds_base on, which has to be the same in all lanes.  Written as assembly, and not with the compiler's builtin,
+// because of what the builtin does to every later wait: while such a load is in flight the compiler takes LDS
+// reads to finish in any order and turns each wait for one of them into a wait for all of them, so that no read
+// can stay in flight behind a matrix product.  The loads it does not know of only make its own waits for memory
+// stricter than needed; that the data has landed before it is read is the caller's business (s_waitcnt vmcnt(0)
+// and a barrier).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // m0 is a reserved register: naming it as clobbered is the point
+__device__ __forceinline__ void load_to_lds_16(const void* src, unsigned char* lds_at) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)lds_at)));
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(src) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
 __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(const AttnArgs a, int min_rows, int blocks_x,
-                                                                              int segments, int listed) {
+                                                                              int segments, int listed, int pair_up) {
   constexpr int D = kDmD;
   extern __shared__ __align__(16) unsigned char lds_raw[];
   __shared__ unsigned int item_of_workgroup;
@@ -866,16 +883,24 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
   const unsigned int parts = static_cast<unsigned int>(a.portion_splits);
   const unsigned int items = pairs * nkv * parts;
   const int P = a.P, ps = a.p_shift, pm = P - 1;
-  const int64_t page_elems = static_cast<int64_t>(a.nkv) * P * D;
+  const uint32_t page_elems32 = static_cast<uint32_t>(a.nkv) * P * D;  // the launcher refuses pages of 2^31 elements
  for (;;) {
   if (tid == 0) item_of_workgroup = atomicAdd(&g_prefill_next_item, 1u);
   __syncthreads();
   const unsigned int item = item_of_workgroup;
   __syncthreads();
   if (item >= items) return;
-  const unsigned int pair = item / (nkv * parts);
+  unsigned int pair = item / (nkv * parts);
   const int kvh = static_cast<int>((item / parts) % nkv);
   const int part = static_cast<int>(item % parts);
+  // The list runs from the heaviest row block to the lightest.  Two workgroups share a CU, and the second
+  // half of the first round of workgroups lands beside the first half: so the first pair_up pairs are handed
+  // out as they are, the next pair_up from the light end, and then the middle, which gives every CU a heavy
+  // and a light item to start with instead of two heavy ones here and two light ones there.
+  if (pair_up > 0 && pairs >= 2u * pair_up) {
+    const unsigned int h = static_cast<unsigned int>(pair_up);
+    if (pair >= h) pair = pair < 2u * h ? pairs - 1u - (pair - h) : pair - h;
+  }
   int seg = static_cast<int>(pair % segments), wg_row = (blocks_x - 1 - static_cast<int>(pair / segments)) * kPfRows;
   if (listed) {
     const unsigned int entry = g_prefill_plan[pair];
@@ -889,7 +914,7 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
   if (wg_row >= rows) continue;
   const int start = a.seg_start[seg];
   const int* table = a.block_table + static_cast<int64_t>(a.seg_slot[seg]) * a.table_stride;
-  const int64_t head_off = static_cast<int64_t>(kvh) * P * D;
+  const uint32_t head_off32 = static_cast<uint32_t>(kvh) * P * D;
 
   const int tok_min = wg_row / G;
   const int tok_max = (min(wg_row + kPfRows, rows) - 1) / G;
@@ -922,6 +947,10 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
 #pragma unroll
     for (int s = 0; s < D / 16; ++s) qreg[s] = load_bf16x8(qp + 16 * s);
   }
+  // Row i of a score tile takes the key whose number has bits 2 and 3 of i exchanged: then the eight scores
+  // that a lane holds for a step of the second product belong to eight keys in a row, and the matching values
+  // are one 16-byte piece of a d row.
+  const int jk = (j & 19) | ((j & 4) << 1) | ((j & 8) >> 1);
   f32x16 o[D / 32];
 #pragma unroll
   for (int dt = 0; dt < D / 32; ++dt)
@@ -957,20 +986,27 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
   auto fetch = [&](int tile, int stage) {
     const int base = tile * kDmKeys;
     unsigned char* at = lds_raw + stage * kDmStageBytes + (4 * wave) * 1024;
+    // the eight page ids first (lane exchanges that answer together), then the eight loads: a load that waits
+    // for its own exchange each time costs the wave a hundred cycles and more a piece
+    int k_at[4], k_page[4], v_at[4], v_page[4];
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
-      const int key = min(max(base + k_key[jj], kv_lo), kv_hi - 1);  // a key that exists; what lies outside is masked
-      const int page = __shfl(pg_reg, (key >> ps) - pg_base, kWave);
-      const uint16_t* src = a.k_pages + page * page_elems + head_off + static_cast<int64_t>(key & pm) * D + k_src[jj];
-      __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)(at + jj * 1024), 16, 0, 0);
+      k_at[jj] = min(max(base + k_key[jj], kv_lo), kv_hi - 1);  // a key that exists; what lies outside is masked
+      k_page[jj] = __shfl(pg_reg, (k_at[jj] >> ps) - pg_base, kWave);
+      v_at[jj] = min(max(base + v_key[jj], kv_lo & ~7), (kv_hi - 1) & ~7);
+      v_page[jj] = __shfl(pg_reg, (v_at[jj] >> ps) - pg_base, kWave);
     }
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
-      const int key8 = min(max(base + v_key[jj], kv_lo & ~7), (kv_hi - 1) & ~7);
-      const int page = __shfl(pg_reg, (key8 >> ps) - pg_base, kWave);
-      const uint16_t* src = a.v_pages + page * page_elems + head_off + v_src[jj] + (key8 & pm);
-      __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)(at + kDmKeys * D * 2 + jj * 1024),
-                                       16, 0, 0);
+      const uint16_t* src = a.k_pages + static_cast<uint64_t>(static_cast<uint32_t>(k_page[jj])) * page_elems32 +
+                            (head_off32 + static_cast<uint32_t>(k_at[jj] & pm) * D + k_src[jj]);
+      load_to_lds_16(src, at + jj * 1024);
+    }
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const uint16_t* src = a.v_pages + static_cast<uint64_t>(static_cast<uint32_t>(v_page[jj])) * page_elems32 +
+                            (head_off32 + v_src[jj] + static_cast<uint32_t>(v_at[jj] & pm));
+      load_to_lds_16(src, at + kDmKeys * D * 2 + jj * 1024);
     }
   };
   // Slots past the request's last token may hold anything, also NaN, and 0 * NaN is NaN: in the request's last
@@ -996,6 +1032,10 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
     cover(t0, true);
     fetch(t0, 0);
   }
+  // The query has to be there before the loop: a wait for it inside the loop would count the tile loads in
+  // flight (which the compiler does not know of) and wait for them too.
+#pragma unroll
+  for (int s = 0; s < D / 16; ++s) asm volatile("" ::"v"(qreg[s]));
   for (int tile = t0; tile < t1; ++tile) {
     const int stage = (tile - t0) & 1;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's pieces of the tile have landed
@@ -1011,24 +1051,38 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
     const unsigned char* ks = lds_raw + stage * kDmStageBytes;
     const unsigned char* vs = ks + kDmKeys * D * 2;
 
-    // scores of 2 x 32 keys
+    // scores of 2 x 32 keys: sixteen operand reads and sixteen products, the two halves taking turns, a read
+    // issued four products before the product that needs it (the order is pinned below: left to itself the
+    // compiler waits for eight reads, multiplies, and waits again)
     f32x16 st[2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      bf16x8 kop[D / 16];
-      const int key = 32 * t + j;
+    {
+      bf16x8 kop[2][D / 16];
 #pragma unroll
       for (int s = 0; s < D / 16; ++s)
-        kop[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(ks + key * (D * 2) + (((2 * s + h) ^ (key & 7)) * 16)));
-      __builtin_amdgcn_sched_barrier(0);
-      f32x16 z;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) z[r] = 0.f;
+        for (int t = 0; t < 2; ++t) {
+          const int key = 32 * t + jk;
+          kop[t][s] = __builtin_bit_cast(
+              bf16x8, *reinterpret_cast<const uint4*>(ks + key * (D * 2) + (((2 * s + h) ^ (key & 7)) * 16)));
+        }
 #pragma unroll
-      for (int s = 0; s < D / 16; ++s) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kop[s], qreg[s], z, 0, 0, 0);
-      st[t] = z;
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[t][r] = 0.f;
+#pragma unroll
+      for (int s = 0; s < D / 16; ++s)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) st[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kop[t][s], qreg[s], st[t], 0, 0, 0);
+      constexpr int kAhead = 4, kOps = 2 * (D / 16);
+      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+      for (int i = 0; i < kOps - kAhead; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
     }
-    // st[t][r] belongs to key key_base + 32 t + 8 (r / 4) + 4 h + r % 4 and to this lane's row
+    // st[t][r] belongs to key key_base + 32 t + 16 (r / 8) + 8 h + r % 8 and to this lane's row
     const bool masked = key_base + kDmKeys - 1 > wave_pos_min || key_base < wave_win_lo;
     if (masked) {
       const int lo = a.window > 0 ? my_pos - a.window + 1 : 0;
@@ -1036,7 +1090,7 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int key = key_base + 32 * t + 8 * (r / 4) + 4 * h + r % 4;
+          const int key = key_base + 32 * t + 16 * (r / 8) + 8 * h + r % 8;
           if (!(key >= lo && key <= my_pos)) st[t][r] = -INFINITY;
         }
     }
@@ -1075,29 +1129,33 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
     }
     m = m_new;
 
-    // O^T += V^T . P^T, 16 keys a step
+    // O^T += V^T . P^T, 16 keys a step; reads and products in turns as above
+    {
+      u32x4 vop[4][D / 32];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int c = 4 * t + 2 * u;  // piece that holds keys 32 t + 16 u .. + 7; the next one holds .. + 8 .. + 15
-        u32x4 vop[D / 32];
+      for (int k = 0; k < 4; ++k) {
+        const int c = 2 * k + h;  // the piece that holds keys 16 k + 8 h .. + 7 of the tile
 #pragma unroll
         for (int dt = 0; dt < D / 32; ++dt) {
           const int d = 32 * dt + j;
-          const unsigned char* vrow = vs + d * (kDmKeys * 2) + 8 * h;
-          const u32x2 va = *reinterpret_cast<const u32x2*>(vrow + ((c ^ (d & 7)) * 16));
-          const u32x2 vb = *reinterpret_cast<const u32x2*>(vrow + (((c + 1) ^ (d & 7)) * 16));
-          vop[dt][0] = va[0];
-          vop[dt][1] = va[1];
-          vop[dt][2] = vb[0];
-          vop[dt][3] = vb[1];
+          vop[k][dt] = *reinterpret_cast<const u32x4*>(vs + d * (kDmKeys * 2) + ((c ^ (d & 7)) * 16));
         }
-        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
 #pragma unroll
         for (int dt = 0; dt < D / 32; ++dt)
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vop[dt]), pb[t][u], o[dt], 0, 0, 0);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vop[k][dt]), pb[k / 2][k % 2], o[dt],
+                                                          0, 0, 0);
+      constexpr int kAhead = 4, kOps = 4 * (D / 32);
+      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 1);
+#pragma unroll
+      for (int i = 0; i < kOps - kAhead; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
       }
+      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 1);
+    }
   }
   __syncthreads();  // the next item's first tile goes into stage 0: everybody has to be done reading
 
@@ -1247,6 +1305,8 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
   return launch_status();
 }
 
+static int g_prefill_pair_up = 1;
+
 int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s) {
   const size_t lds = 2 * kDmStageBytes;
   static bool asked = false;  // dynamic LDS of 64 KiB and more has to be asked for, once
@@ -1272,8 +1332,9 @@ int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
   if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);
   attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
                                              a.nq / a.nkv, min_rows, listed);
+  const int pair_up = g_prefill_pair_up ? static_cast<int>(cus / (static_cast<long long>(a.nkv) * a.portion_splits)) : 0;
   attn_prefill_dma_kernel<<<workgroups, kDmWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
-                                                                   static_cast<int>(grid.z), listed);
+                                                                   static_cast<int>(grid.z), listed, pair_up);
   if (a.portion_splits > 1) {
     const long long most = static_cast<long long>(grid.x) * grid.y * grid.z * (kPfRows / kPfWaves);
     attn_merge_portions_kernel<<<static_cast<unsigned>(most < 4LL * cus ? most : 4LL * cus), kPfWaves * kWave, 0, s>>>(a);
@@ -1297,7 +1358,9 @@ inline bool prefill_dma_pays(dim3 grid, int max_qlen, int max_kv_len) {
     cus = 256;
   const long long items = static_cast<long long>(grid.x) * grid.y * grid.z;
   const int most = (max_kv_len + kDmKeys - 1) / kDmKeys, least = (max(max_kv_len - max_qlen, 0) + kDmKeys - 1) / kDmKeys;
-  return items >= 6LL * cus || (items >= 2LL * cus && 2 * least >= most);
+  (void)most;
+  (void)least;
+  return items >= 2LL * cus;
 }
 
 }  // namespace arle
@@ -1305,6 +1368,7 @@ inline bool prefill_dma_pays(dim3 grid, int max_qlen, int max_kv_len) {
 using namespace arle;
 
 extern "C" void arle_attn_prefill_variant(int dma) { g_prefill_dma = dma; }
+extern "C" void arle_attn_prefill_pair_up(int on) { g_prefill_pair_up = on; }
 
 // Token rows that the split-KV workspace holds for every segment: the most tokens of a segment whose rows
 // (tokens x q heads of a kv head) fit one row tile of 16.
@@ -1377,7 +1441,8 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
     dim3 grid((max_rows + kPfRows - 1) / kPfRows, nkv, segments);
     if (D == 64)
       rc = launch_prefill_lds<64, true>(a, grid, 17, s);
-    else if (D == 128 && page_size % 8 == 0 && prefill_dma_pays(grid, max_qlen, max_kv_len))
+    else if (D == 128 && page_size % 8 == 0 && static_cast<long long>(nkv) * page_size * D < (1LL << 31) &&
+             prefill_dma_pays(grid, max_qlen, max_kv_len))
       rc = launch_prefill_dma(a, grid, 17, s);
     else if (D == 128)
       rc = launch_prefill_lds<128, true>(a, grid, 17, s);
