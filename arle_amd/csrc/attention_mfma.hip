@@ -853,6 +853,7 @@ constexpr int kDmWaves = 4;
 constexpr int kDmD = 128;
 constexpr int kDmKeys = 64;
 constexpr int kDmStageBytes = kDmKeys * kDmD * 2 * 2;  // keys and values of a tile: 32 KB
+constexpr float kDmLazyBits = 8.0f;
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // Sixteen bytes a lane from memory straight into LDS: the wave's 64 pieces land one after the other from
@@ -869,8 +870,26 @@ __device__ __forceinline__ void load_to_lds_16(const void* src, unsigned char* l
       static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)lds_at)));
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(src) : "memory", "m0");
 }
+// The same with the address as a wave-wide base and a byte offset of the lane.
+__device__ __forceinline__ void load_to_lds_16(const void* base_uniform, uint32_t lane_bytes, unsigned char* lds_at) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)lds_at)));
+  const uint64_t src = reinterpret_cast<uint64_t>(base_uniform);
+  // the builtin returns a signed int: widened as it is, a low half with its top bit set would fill the high half
+  const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(src))));
+  const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(src >> 32)));
+  const uint64_t src_s = (static_cast<uint64_t>(hi) << 32) | lo;
+  // s_nop 4: a scalar register written by a vector instruction may not be a memory instruction's address for
+  // five cycles, and the compiler does not look into this text for that
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(base), "v"(lane_bytes), "s"(src_s)
+               : "memory", "m0");
+}
 #pragma clang diagnostic pop
 
+// WHOLE: the page size is a multiple of the tile's 64 keys, so a tile lies in one page: its address is a
+// matter of scalar arithmetic and a lane adds an offset that never changes.  Otherwise a lane looks up the page
+// of each of its pieces.
+template <bool WHOLE>
 __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(const AttnArgs a, int min_rows, int blocks_x,
                                                                               int segments, int listed, int pair_up) {
   constexpr int D = kDmD;
@@ -986,6 +1005,20 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
   auto fetch = [&](int tile, int stage) {
     const int base = tile * kDmKeys;
     unsigned char* at = lds_raw + stage * kDmStageBytes + (4 * wave) * 1024;
+    if constexpr (WHOLE) {
+      // keys of the tile that lie outside the request are read as they are (the page is there) and masked
+      const int page = __builtin_amdgcn_readlane(pg_reg, __builtin_amdgcn_readfirstlane((base >> ps) - pg_base));
+      const uint64_t first = static_cast<uint64_t>(static_cast<uint32_t>(page)) * page_elems32 + head_off32;
+      const uint16_t* kb = a.k_pages + first + static_cast<uint32_t>(base & pm) * D;
+      const uint16_t* vb = a.v_pages + first + static_cast<uint32_t>(base & pm);
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj)
+        load_to_lds_16(kb, 2u * static_cast<uint32_t>(k_key[jj] * D + k_src[jj]), at + jj * 1024);
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj)
+        load_to_lds_16(vb, 2u * static_cast<uint32_t>(v_src[jj] + v_key[jj]), at + kDmKeys * D * 2 + jj * 1024);
+      return;
+    }
     // the eight page ids first (lane exchanges that answer together), then the eight loads: a load that waits
     // for its own exchange each time costs the wave a hundred cycles and more a piece
     int k_at[4], k_page[4], v_at[4], v_page[4];
@@ -1017,7 +1050,7 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
     unsigned char* at = lds_raw + stage * kDmStageBytes + kDmKeys * D * 2 + (4 * wave) * 1024 + lane * 16;
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
-      const int key8 = min(max(base + v_key[jj], kv_lo & ~7), (kv_hi - 1) & ~7);  // the keys that were fetched
+      const int key8 = WHOLE ? base + v_key[jj] : min(max(base + v_key[jj], kv_lo & ~7), (kv_hi - 1) & ~7);  // as fetched
       if (key8 + 8 > kv_total) {
         u32x4 v = *reinterpret_cast<u32x4*>(at + jj * 1024);
 #pragma unroll
@@ -1100,7 +1133,10 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
 #pragma unroll
       for (int r = 0; r < 16; ++r) bmax = fmaxf(bmax, st[t][r]);
     bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave)) * a.scale_log2;  // scale > 0: the maximum commutes with it
-    const float m_new = fmaxf(m, bmax);
+    // m is the point that the row's exponentials are taken from, not its exact maximum: it moves only when
+    // the maximum has grown by more than kDmLazyBits (exponentials up to 2^8 meanwhile, nothing to a float or
+    // a bf16), which after a row's first tiles is rare, so that the 64 sums are rarely multiplied
+    const float m_new = bmax > m + kDmLazyBits ? bmax : m;
     const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
     const float alpha = __builtin_amdgcn_exp2f(m - m_use);
     float psum = 0.f;
@@ -1311,11 +1347,13 @@ int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
   const size_t lds = 2 * kDmStageBytes;
   static bool asked = false;  // dynamic LDS of 64 KiB and more has to be asked for, once
   if (!asked) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_dma_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-    if (e != hipSuccess) {
-      (void)hipGetLastError();
-      return static_cast<int>(e);
+    for (const void* kernel : {reinterpret_cast<const void*>(&attn_prefill_dma_kernel<true>),
+                               reinterpret_cast<const void*>(&attn_prefill_dma_kernel<false>)}) {
+      hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return static_cast<int>(e);
+      }
     }
     asked = true;
   }
@@ -1333,8 +1371,12 @@ int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
   attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
                                              a.nq / a.nkv, min_rows, listed);
   const int pair_up = g_prefill_pair_up ? static_cast<int>(cus / (static_cast<long long>(a.nkv) * a.portion_splits)) : 0;
-  attn_prefill_dma_kernel<<<workgroups, kDmWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
-                                                                   static_cast<int>(grid.z), listed, pair_up);
+  if (a.P % kDmKeys == 0)
+    attn_prefill_dma_kernel<true><<<workgroups, kDmWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
+                                                                           static_cast<int>(grid.z), listed, pair_up);
+  else
+    attn_prefill_dma_kernel<false><<<workgroups, kDmWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
+                                                                            static_cast<int>(grid.z), listed, pair_up);
   if (a.portion_splits > 1) {
     const long long most = static_cast<long long>(grid.x) * grid.y * grid.z * (kPfRows / kPfWaves);
     attn_merge_portions_kernel<<<static_cast<unsigned>(most < 4LL * cus ? most : 4LL * cus), kPfWaves * kWave, 0, s>>>(a);

@@ -573,10 +573,12 @@ def test_attention_mfma_both_portion_kernels_at_head_dim_128(variant, nq, nkv, P
     assert _rel(got, want) < 8e-3
 
 
-def test_attention_mfma_dma_kernel_masks_stale_slots():
-    """The kernel that loads tiles straight into LDS: pages hold NaN bits in every slot that was never written."""
+@pytest.mark.parametrize("P", [16, 64, 128])
+def test_attention_mfma_dma_kernel_masks_stale_slots(P):
+    """The kernel that loads tiles straight into LDS: pages hold NaN bits in every slot that was never written
+    (with pages of 64 keys and more it reads a tile's keys beyond the request as they lie there)."""
     from arle_amd.kernels import lib
-    nq, nkv, D, P = 8, 2, 128, 16
+    nq, nkv, D = 8, 2, 128
     dt = torch.bfloat16
     segs = [(200, 150), (17, 130), (0, 70)]
     lengths = [a + b for a, b in segs]
