@@ -188,6 +188,7 @@ def decode_32b(args) -> int:
 
 
 def main() -> int:
+    global PAGE
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
@@ -196,6 +197,7 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=8192, help="tokens of context of the qwen3-32b-decode workload")
     ap.add_argument("--layers", type=int, default=FULL_LAYERS)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--page-size", type=int, default=PAGE, help="tokens per cache page")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 decode points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiles of its kernels) and print that")
@@ -205,6 +207,7 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
         return 2
+    PAGE = args.page_size
     if args.workload == "qwen3-4b" and args.batch is None:
         args.batch = 8
     if args.workload != "qwen3-4b":
