@@ -1019,21 +1019,25 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
         load_to_lds_16(vb, 2u * static_cast<uint32_t>(v_src[jj] + v_key[jj]), at + kDmKeys * D * 2 + jj * 1024);
       return;
     }
-    // the eight page ids first (lane exchanges that answer together), then the eight loads: a load that waits
-    // for its own exchange each time costs the wave a hundred cycles and more a piece
-    int k_at[4], k_page[4], v_at[4], v_page[4];
+    // Keys: one load takes four keys in a row, which lie in one page (a page holds eight at least), so the page
+    // is the wave's and the address scalar arithmetic as above; keys outside the request are read from the
+    // nearest page that is there and masked.  Values: a lane's piece holds eight keys of its own, so a lane
+    // looks up its own page: the four page ids first (lane exchanges that answer together), then the loads.
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    int v_at[4], v_page[4];
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
-      k_at[jj] = min(max(base + k_key[jj], kv_lo), kv_hi - 1);  // a key that exists; what lies outside is masked
-      k_page[jj] = __shfl(pg_reg, (k_at[jj] >> ps) - pg_base, kWave);
       v_at[jj] = min(max(base + v_key[jj], kv_lo & ~7), (kv_hi - 1) & ~7);
       v_page[jj] = __shfl(pg_reg, (v_at[jj] >> ps) - pg_base, kWave);
     }
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
-      const uint16_t* src = a.k_pages + static_cast<uint64_t>(static_cast<uint32_t>(k_page[jj])) * page_elems32 +
-                            (head_off32 + static_cast<uint32_t>(k_at[jj] & pm) * D + k_src[jj]);
-      load_to_lds_16(src, at + jj * 1024);
+      const int first_key = base + 4 * (4 * wave_u + jj);
+      const int page_at = min(max(first_key >> ps, kv_lo >> ps), pg_last) - pg_base;
+      const int page = __builtin_amdgcn_readlane(pg_reg, __builtin_amdgcn_readfirstlane(page_at));
+      const uint16_t* kb = a.k_pages + static_cast<uint64_t>(static_cast<uint32_t>(page)) * page_elems32 + head_off32 +
+                           static_cast<uint32_t>(first_key & pm) * D;
+      load_to_lds_16(kb, 2u * static_cast<uint32_t>((lane >> 4) * D + k_src[jj]), at + jj * 1024);
     }
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
