@@ -863,6 +863,17 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // can stay in flight behind a matrix product.  The loads it does not know of only make its own waits for memory
 // stricter than needed; that the data has landed before it is read is the caller's business (s_waitcnt vmcnt(0)
 // and a barrier).
+// A value of lane i and the value of lane i ^ 32, in the same order in both lanes (v_permlane32_swap: one vector
+// instruction, where a shuffle is a trip through the LDS unit).
+struct HalfPair {
+  float lo, hi;
+};
+__device__ __forceinline__ HalfPair both_halves(float x) {
+  const unsigned bits = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+  return {__uint_as_float(r[0]), __uint_as_float(r[1])};
+}
+
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"  // m0 is a reserved register: naming it as clobbered is the point
 __device__ __forceinline__ void load_to_lds_16(const void* src, unsigned char* lds_at) {
@@ -1136,7 +1147,10 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) bmax = fmaxf(bmax, st[t][r]);
-    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave)) * a.scale_log2;  // scale > 0: the maximum commutes with it
+    {
+      const HalfPair both = both_halves(bmax);
+      bmax = fmaxf(both.lo, both.hi) * a.scale_log2;  // scale > 0: the maximum commutes with it
+    }
     // m is the point that the row's exponentials are taken from, not its exact maximum: it moves only when
     // the maximum has grown by more than kDmLazyBits (exponentials up to 2^8 meanwhile, nothing to a float or
     // a bf16), which after a row's first tiles is rare, so that the 64 sums are rarely multiplied
@@ -1159,7 +1173,10 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
         }
         pb[t][u] = __builtin_bit_cast(bf16x8, packed);
       }
-    psum += __shfl_xor(psum, 32, kWave);
+    {
+      const HalfPair both = both_halves(psum);
+      psum = both.lo + both.hi;
+    }
     l = l * alpha + psum;
     if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {  // the sums need the factor only if some row's maximum moved
 #pragma unroll
