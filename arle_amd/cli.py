@@ -48,6 +48,10 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--prefill-max-requests", type=int, default=None)
     ap.add_argument("--kv-cache-tokens", type=int, default=None, help="tokens the paged cache holds")
     ap.add_argument("--page-size", type=int, default=None)
+    ap.add_argument("--no-cuda-graph", action="store_true",
+                    help="launch every step kernel by kernel instead of replaying captured HIP graphs")
+    ap.add_argument("--no-weight-tiles", action="store_true",
+                    help="do not keep the second, decode-friendly copy of the projection weights")
     sub = ap.add_subparsers(dest="command")
     run = sub.add_parser("run", help="run a single prompt and exit")
     src = run.add_mutually_exclusive_group()
@@ -92,7 +96,8 @@ def main(argv=None) -> int:
               chunked_prefill_size=args.chunked_prefill_size,
               max_num_batched_tokens=args.max_num_batched_tokens, max_prefill_tokens=args.max_prefill_tokens,
               prefill_max_requests=args.prefill_max_requests, kv_cache_tokens=args.kv_cache_tokens,
-              page_size=args.page_size, seed=args.seed)
+              page_size=args.page_size, seed=args.seed, cuda_graph=not args.no_cuda_graph,
+              weight_tiles=False if args.no_weight_tiles else None)
     if args.prompt_ids:
         prompt = [int(t) for t in args.prompt_ids.replace(" ", "").split(",") if t]
     else:

@@ -51,7 +51,17 @@ struct RowsArgs {
   int M, N, K;
   int steps_per_split;   // k steps of 32 that one k split covers
   int64_t split_stride;  // elements between the partial products of two k splits
+  int tiled;             // w holds operand tiles (see below) instead of rows
 };
+
+// W as operand tiles: [ceil(N/16)][ceil(K/32)][64 lanes][8], tile (t, s) lane 16 g + i = W[16 t + i][32 s + 8 g .. +7],
+// zeros past N and K.  A wave's load of one k step is then one contiguous kilobyte and its stream through a
+// column tile one contiguous run, instead of sixteen 64-byte pieces a row apart: measured 4.5 against 3.6 TB/s
+// for the 100 MB gate|up matrix of the Qwen3-4B shape at 8 rows.
+__device__ __forceinline__ const uint16_t* tile_base(const RowsArgs& a, int n0, int lane) {
+  const int tile = min(n0 / 16, (a.N + 15) / 16 - 1);
+  return a.w + static_cast<int64_t>(tile) * ((a.K + 31) / 32) * 512 + lane * 8;
+}
 
 template <int MT, int WN, int WK, int PD, int XD, int EPI, typename TOut>
 __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a) {
@@ -77,9 +87,11 @@ __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a
   const int w_begin = s_begin + wk * per;
   const int n_steps = max(0, min(w_begin + per, s_end) - w_begin);
 
-  const uint16_t* wrow = a.w + static_cast<int64_t>(min(n0 + li, N - 1)) * a.ldw;
+  // rows: lane (i, g) reads 16 bytes of row n0 + i; tiles: the wave reads tile s of its column tile, lane by lane
+  const uint16_t* wrow = a.tiled ? tile_base(a, n0, lane) : a.w + static_cast<int64_t>(min(n0 + li, N - 1)) * a.ldw;
+  const int w_step = a.tiled ? 512 : 32, w_first = a.tiled ? 0 : 8 * g, w_last = a.tiled ? (steps_total - 1) * 512 : K - 8;
   auto load_w = [&](int s) {
-    const int e = min(32 * s + 8 * g, K - 8);  // clamped: always inside the row
+    const int e = min(w_step * s + w_first, w_last);  // clamped: always inside the row (the column tile)
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(wrow + e));
   };
 
@@ -264,10 +276,11 @@ __global__ __launch_bounds__(WN * 64) void gemm_stream_kernel(const RowsArgs a) 
 
   auto w_row = [&](int group) {
     const int n0 = (group * WN + wave) * 16;
-    return a.w + static_cast<int64_t>(min(n0 + li, N - 1)) * a.ldw;
+    return a.tiled ? tile_base(a, n0, lane) : a.w + static_cast<int64_t>(min(n0 + li, N - 1)) * a.ldw;
   };
+  const int w_step = a.tiled ? 512 : 32, w_first = a.tiled ? 0 : 8 * g, w_last = a.tiled ? (steps_total - 1) * 512 : K - 8;
   auto load_w = [&](const uint16_t* row, int s) {  // s: step inside the slice (may reach past it, not past K)
-    const int e = min(32 * (s_begin + s) + 8 * g, K - 8);
+    const int e = min(w_step * (s_begin + s) + w_first, w_last);
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(row + e));
   };
   const uint16_t* wcur = w_row(blockIdx.x);
@@ -453,7 +466,8 @@ extern "C" long long arle_gemm_rows_lds_max() { return static_cast<long long>(kR
 // splits == 1: out [M, N] (or [M, N/2] with the fused activation) bfloat16 or float32.
 // splits  > 1: out [splits, M, N] float32 partial products, split_stride elements apart, no activation;
 //              split s covers steps [s * steps_per_split, (s + 1) * steps_per_split) and none may be empty.
-extern "C" int arle_gemm_rows(const void* x, long long ldx, const void* w, long long ldw, void* out, long long ldo,
+// w_tiled: w holds operand tiles (RowsArgs), ldw is not used.
+extern "C" int arle_gemm_rows(const void* x, long long ldx, const void* w, long long ldw, int w_tiled, void* out, long long ldo,
                               long long split_stride, int out_dtype, int M, int N, int K, int epilogue, int variant,
                               int splits, int steps_per_split, void* stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -470,7 +484,7 @@ extern "C" int arle_gemm_rows(const void* x, long long ldx, const void* w, long 
   if (epilogue != kEpiNone && epilogue != kEpiSiluMul) return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const RowsArgs a{static_cast<const uint16_t*>(x), ldx, static_cast<const uint16_t*>(w), ldw, out, ldo, M, N, K,
-                   steps_per_split, split_stride};
+                   steps_per_split, split_stride, w_tiled ? 1 : 0};
   switch (variant) {
 #define X(ID, WN, WK, PD)                                                                       \
   case ID:                                                                                      \
@@ -540,7 +554,7 @@ int dispatch_stream(const RowsArgs& a, int splits, int workgroups, int out_dtype
 
 // The product with workgroups that stay (see gemm_stream_kernel): `workgroups` of them for every k split walk
 // the column groups.  Operands, splits and the stack of partial products as in arle_gemm_rows; no activation.
-extern "C" int arle_gemm_stream(const void* x, long long ldx, const void* w, long long ldw, void* out, long long ldo,
+extern "C" int arle_gemm_stream(const void* x, long long ldx, const void* w, long long ldw, int w_tiled, void* out, long long ldo,
                                 long long split_stride, int out_dtype, int M, int N, int K, int variant, int splits,
                                 int steps_per_split, int workgroups, void* stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -554,7 +568,7 @@ extern "C" int arle_gemm_stream(const void* x, long long ldx, const void* w, lon
   if (splits > 1 && out_dtype != kF32) return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const RowsArgs a{static_cast<const uint16_t*>(x), ldx, static_cast<const uint16_t*>(w), ldw, out, ldo, M, N, K,
-                   steps_per_split, split_stride};
+                   steps_per_split, split_stride, w_tiled ? 1 : 0};
   switch (variant) {
 #define X(ID, WN, PD) \
   case ID:            \

@@ -46,11 +46,13 @@ class LLM:
     def __init__(self, model, *, dtype="bfloat16", device=None, page_size: int | None = None,
                  kv_cache_tokens: int | None = None, num_slots: int = 4, max_seq_len: int | None = None,
                  chunked_prefill_size: int = 512, max_num_batched_tokens: int = 16384,
-                 max_prefill_tokens: int = 16384, prefill_max_requests: int | None = None, seed: int = 42):
+                 max_prefill_tokens: int = 16384, prefill_max_requests: int | None = None, seed: int = 42,
+                 cuda_graph: bool = True, weight_tiles: bool | None = None):
         """model: a model folder, or an Engine that is already built.
 
         kv_cache_tokens: tokens the paged cache holds over all live requests
         (default: num_slots * max_seq_len, max_seq_len defaulting to min(model's positions, 4096)).
+        cuda_graph, weight_tiles: as for Engine (captured steps; the decode-friendly second copy of the weights).
         """
         if isinstance(model, Engine):
             self.engine = model
@@ -66,7 +68,8 @@ class LLM:
             self.engine = Engine.from_folder(model, dtype=dtype, device=device,
                                              page_size=page_size or DEFAULT_PAGE_SIZE,
                                              max_tokens=kv_cache_tokens, max_slots=num_slots,
-                                             max_request_tokens=min(max_seq_len, positions))
+                                             max_request_tokens=min(max_seq_len, positions),
+                                             cuda_graph=cuda_graph, weight_tiles=weight_tiles)
         self.model_dir = model if isinstance(model, str) else None
         self.seed = seed
         self.sched_config = SchedulerConfig(

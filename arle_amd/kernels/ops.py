@@ -580,8 +580,27 @@ def gemm_rows_plan(M: int, N: int, K: int, fused: bool = False):
     return variant, max(want, _rows_min_splits(variant, M, K))
 
 
+def pack_weight_tiles(w: torch.Tensor) -> torch.Tensor:
+    """w [N, K] bfloat16 -> [ceil(N/16), ceil(K/32), 512]: the operand tiles that gemm_rows and gemm_stream read
+    with one contiguous kilobyte a wave and k step.  Tile (t, s), element 128 g + 8 i + e = w[16 t + i, 32 s + 8 g + e]
+    (lane 16 g + i of the wave reads its eight elements); zeros past N and K.  A rearrangement at load time, the
+    values are untouched, and the product adds them in the same order as from rows."""
+    _need(w.dim() == 2 and w.dtype == torch.bfloat16, "pack_weight_tiles takes a bfloat16 [N, K] matrix")
+    N, K = w.shape
+    Np, Kp = -(-N // 16) * 16, -(-K // 32) * 32
+    if (Np, Kp) != (N, K):
+        w = torch.nn.functional.pad(w, (0, Kp - K, 0, Np - N))
+    return w.reshape(Np // 16, 16, Kp // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(Np // 16, Kp // 32, 512)
+
+
+def _check_tiles(tiles, N: int, K: int) -> None:
+    _need(tiles.dtype == torch.bfloat16 and tiles.is_contiguous() and tiles.dim() == 3 and tiles.shape[1:] == (-(-K // 32), 512)
+          and tiles.shape[0] >= -(-N // 16) and tiles.data_ptr() % 16 == 0,
+          f"operand tiles of a [{N}, {K}] matrix have the shape [{-(-N // 16)}, {-(-K // 32)}, 512], got {tuple(tiles.shape)}")
+
+
 def gemm_rows(x, w, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, variant: int | None = None,
-              splits: int | None = None):
+              splits: int | None = None, tiles: torch.Tensor | None = None):
     """x . w^T for 1..64 rows of x, with x shared through LDS inside a workgroup.
 
     splits == 1: returns [M, N] (or [M, N/2] with EPI_SILU_MUL) in `out_dtype`.
@@ -589,6 +608,7 @@ def gemm_rows(x, w, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, varia
     no split is empty) for the consumer to add in the order of S.  With `variant` and `splits` left out
     the shape decides (gemm_rows_plan), so callers must be ready for either form.
     EPI_SILU_MUL: w holds gate and up rows interleaved in blocks of 16; out[m, j] = silu(gate_j) * up_j.
+    tiles: pack_weight_tiles(w); the kernel then streams these instead of the rows of w (same sums, bit for bit).
     """
     _gpu(x, w)
     _rows(x, "x")
@@ -622,7 +642,10 @@ def gemm_rows(x, w, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, varia
     else:
         out = torch.empty((M, N // 2 if fused else N), dtype=out_dtype, device=x.device)
         ldo, stride, code = out.stride(0), 0, _CODES[out_dtype]
-    lib.call("arle_gemm_rows", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), ldo, stride,
+    if tiles is not None:
+        _check_tiles(tiles, N, K)
+    lib.call("arle_gemm_rows", x.data_ptr(), x.stride(0), (w if tiles is None else tiles).data_ptr(), w.stride(0),
+             int(tiles is not None), out.data_ptr(), ldo, stride,
              code, M, N, K, int(epilogue), variant, splits, per_split, _stream())
     return out
 
@@ -653,7 +676,7 @@ def _stream_min_splits(variant: int, M: int, K: int) -> int:
 
 
 def gemm_stream(x, w, out_dtype=torch.bfloat16, *, variant: int = 0, splits: int | None = None,
-                workgroups: int | None = None):
+                workgroups: int | None = None, tiles: torch.Tensor | None = None):
     """x . w^T for 1..64 rows of x by workgroups that stay: each stages its slice of x once and walks several
     groups of output columns, so that w alone is streamed (see gemm_stream_kernel).
 
@@ -687,7 +710,10 @@ def gemm_stream(x, w, out_dtype=torch.bfloat16, *, variant: int = 0, splits: int
     else:
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         ldo, stride, code = out.stride(0), 0, _CODES[out_dtype]
-    lib.call("arle_gemm_stream", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), ldo, stride,
+    if tiles is not None:
+        _check_tiles(tiles, N, K)
+    lib.call("arle_gemm_stream", x.data_ptr(), x.stride(0), (w if tiles is None else tiles).data_ptr(), w.stride(0),
+             int(tiles is not None), out.data_ptr(), ldo, stride,
              code, M, N, K, variant, splits, per_split, int(workgroups), _stream())
     return out
 
@@ -707,7 +733,8 @@ def sum_partials(parts: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
-def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, partials_ok: bool = False):
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, partials_ok: bool = False,
+              tiles: torch.Tensor | None = None):
     """out[M, N] = x[M, K] . w[N, K]^T, bfloat16 operands, float32 accumulation.
 
     Few rows (decode steps, short portions) run the hand-written weight-streaming kernel.  More rows go
@@ -715,6 +742,7 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
     to a library (crates/cuda-kernels/csrc/gemm/gemv.cu:240-330).
     partials_ok: the caller adds a float32 stack [S, M, N] itself (in the order of S) if that is what the
     kernel leaves behind; otherwise the stack is added here by one more small kernel.
+    tiles: pack_weight_tiles(w), for the hand-written kernels to stream instead of w.
     """
     _gpu(x, w)
     _rows(x, "x")
@@ -723,12 +751,13 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
     _need(x.shape[1] == w.shape[1], f"gemm_bf16: inner sizes differ ({x.shape[1]} vs {w.shape[1]})")
     _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_bf16 writes bfloat16 or float32")
     if gemm_rows_preferred(x.shape[0], w.shape[0], x.shape[1], x.stride(0)) and x.data_ptr() % 16 == 0:
-        out = gemm_rows(x, w, out_dtype)
+        out = gemm_rows(x, w, out_dtype, tiles=tiles)
         if out.dim() == 3 and not partials_ok:
             out = sum_partials(out, out_dtype)
         return out
     if gemm_stream_preferred(x.shape[0], w.shape[0], x.shape[1], x.stride(0)) and x.data_ptr() % 16 == 0:
-        out = gemm_stream(x, w, out_dtype, variant=_STREAM_VARIANT, splits=_stream_splits(x.shape[0], x.shape[1]))
+        out = gemm_stream(x, w, out_dtype, variant=_STREAM_VARIANT, splits=_stream_splits(x.shape[0], x.shape[1]),
+                          tiles=tiles)
         # a large stack is added here by many workgroups; the consumer would add it with one workgroup a row
         if out.dim() == 3 and (not partials_ok or out.numel() * 4 > _STREAM_PARTIAL_BYTES):
             out = sum_partials(out, out_dtype)

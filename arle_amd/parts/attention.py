@@ -70,10 +70,11 @@ class PagedAttention(Part):
         if not (wq.dtype == wk.dtype == wv.dtype):
             raise ValueError("q, k and v projections must be stored in one type")
         self.q_width, self.kv_width = self.nq * self.D, self.nkv * self.D
-        self.qkv = Linear(torch.cat([wq, wk, wv], dim=0).contiguous())
-        # for a layer that reads another layer's cache: the q rows of the fused matrix, no copy
-        self.q_only = Linear(self.qkv.weight[: self.q_width])
-        self.o = Linear(tensors["o"])
+        self.qkv = Linear(torch.cat([wq, wk, wv], dim=0).contiguous(), rt.weight_tiles)
+        # for a layer that reads another layer's cache: the q rows of the fused matrix, no copy (head_dim is a
+        # multiple of 16, so the q rows are whole operand tiles too)
+        self.q_only = Linear(self.qkv.weight[: self.q_width], packed=self.qkv.tiles)
+        self.o = Linear(tensors["o"], rt.weight_tiles)
 
     def cache_need(self):
         return PagedNeed(num_kv_heads=self.nkv, head_dim=self.D, window=self.window)

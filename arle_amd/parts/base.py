@@ -63,6 +63,9 @@ class Runtime:
 
     device: torch.device
     act_dtype: torch.dtype  # torch.bfloat16 (serving) or torch.float32 (true 32-bit path)
+    # keep a second copy of every bfloat16 projection weight as operand tiles, the layout that the few-rows
+    # kernels stream fastest (twice the weight memory; the library keeps reading the rows)
+    weight_tiles: bool = False
 
     @property
     def is_f32(self) -> bool:

@@ -42,7 +42,7 @@ class LinearHead(Part):
 
     def __init__(self, params, tensors, rt, children=None):
         super().__init__(params, tensors, rt, children)
-        self.proj = Linear(tensors["weight"])
+        self.proj = Linear(tensors["weight"], rt.weight_tiles)
 
     def forward(self, x):
         return self.proj(x, out_dtype=torch.float32)

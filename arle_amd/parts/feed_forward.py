@@ -39,15 +39,15 @@ class SwiGLU(Part):
             fused = torch.stack([gate.view(-1, 16, h), up.view(-1, 16, h)], dim=1).reshape(2 * self.inter, h)
         else:
             fused = torch.cat([gate, up], dim=0)
-        self.gate_up = Linear(fused.contiguous())
-        self.down = Linear(tensors["down"])
+        self.gate_up = Linear(fused.contiguous(), rt.weight_tiles)
+        self.down = Linear(tensors["down"], rt.weight_tiles)
 
     def forward(self, x):
         """x [T, H] -> [T, H], or a float32 stack [S, T, H] to be added in order (see Linear)."""
         if self.block:
             w = self.gate_up.weight
             if x.shape[0] and ops.gemm_rows_preferred(x.shape[0], w.shape[0], x.shape[1], x.stride(0), fused=True):
-                act = ops.gemm_rows(x, w, x.dtype, ops.EPI_SILU_MUL)
+                act = ops.gemm_rows(x, w, x.dtype, ops.EPI_SILU_MUL, tiles=self.gate_up.tiles)
             else:
                 act = ops.silu_mul_interleaved(self.gate_up(x), self.block)
         else:

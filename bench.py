@@ -199,6 +199,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=PAGE, help="tokens per cache page")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 decode points")
+    ap.add_argument("--no-weight-tiles", action="store_true",
+                    help="without the second copy of the projection weights that the few-rows kernels stream")
     ap.add_argument("--prefill-only", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiles of its kernels) and print that")
     ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode"],
@@ -229,7 +231,7 @@ def main() -> int:
     t0 = time.time()
     engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype=args.dtype,
                                 page_size=PAGE, max_tokens=max_batch * CONTEXT, max_slots=max_batch,
-                                max_request_tokens=CONTEXT)
+                                max_request_tokens=CONTEXT, weight_tiles=False if args.no_weight_tiles else None)
     print(f"[bench] engine ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
     gen = torch.Generator().manual_seed(1234)
 
@@ -313,7 +315,7 @@ def main() -> int:
                    "kv_heads": raw["num_key_value_heads"], "head_dim": raw["head_dim"],
                    "intermediate": raw["intermediate_size"], "vocab": raw["vocab_size"],
                    "rope_theta": raw["rope_theta"], "rms_norm_eps": raw["rms_norm_eps"], "tied": True,
-                   "page_size": PAGE},
+                   "page_size": PAGE, "weight_tiles": engine.rt.weight_tiles},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},

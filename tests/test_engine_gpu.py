@@ -118,6 +118,26 @@ def test_captured_decode_steps_equal_eager_ones_on_every_replay(model, dtype):
         assert torch.equal(a[key], b[key]), f"graph replay differs from the eager step at {key}"
 
 
+def test_weights_held_as_operand_tiles_give_the_same_bits(model):
+    """The decode-friendly second copy of the projection weights changes where the few-rows kernels read
+    from, not what they add in which order."""
+    name, d, cfg, _ = model
+    reqs = _requests(cfg, [37, 20], 901)
+    steps = []
+    for rid, toks in reqs.items():
+        steps += replay.prefill_then_decode(rid, toks, 12)
+    got = []
+    for tiles in (True, False):
+        eng = Engine.from_folder(d, dtype="bfloat16", page_size=TINY[name][1], max_tokens=256, max_slots=4, weight_tiles=tiles)
+        assert eng.rt.weight_tiles == tiles
+        assert (eng.model.head.proj.tiles is not None) == tiles
+        got.append(replay.run_steps(eng, steps))
+    for key in got[0]:
+        assert torch.equal(got[0][key], got[1][key]), key
+    # the 32-bit path has no such copy
+    assert not Engine.from_folder(d, dtype="float32", page_size=TINY[name][1], max_tokens=64, weight_tiles=True).rt.weight_tiles
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_captured_steps_of_repeated_shapes_equal_eager_ones(model, dtype):
     """A step shape that repeats (equal portions of prompts, the same decoded tokens beside a portion) runs from

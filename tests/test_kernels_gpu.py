@@ -733,6 +733,49 @@ def test_gemm_rows_with_fused_activation(M, inter, K):
     assert _rel(got, want) < 1e-2
 
 
+def test_pack_weight_tiles_layout():
+    """Tile (t, s), lane 16 g + i, element e is w[16 t + i, 32 s + 8 g + e]; zeros past the matrix."""
+    N, K = 37, 72
+    w = torch.arange(N * K, dtype=torch.float32).reshape(N, K).bfloat16()
+    tiles = ops.pack_weight_tiles(w.to(DEV)).cpu()
+    assert tiles.shape == (3, 3, 512)
+    for t, s_, g, i, e in [(0, 0, 0, 0, 0), (0, 0, 1, 0, 0), (0, 0, 0, 1, 0), (1, 2, 0, 3, 7), (2, 1, 3, 4, 5), (2, 2, 1, 4, 0),
+                           (2, 0, 0, 5, 0)]:
+        n, k = 16 * t + i, 32 * s_ + 8 * g + e
+        want = w[n, k] if (n < N and k < K) else torch.tensor(0.0).bfloat16()
+        assert tiles[t, s_, (16 * g + i) * 8 + e] == want, (t, s_, g, i, e)
+
+
+@pytest.mark.parametrize("M,N,K,splits", [(1, 333, 88, 1), (5, 37, 72, 1), (16, 96, 1096, 3), (20, 200, 520, 2), (64, 72, 2056, 5),
+                                          (8, 2560, 4096, 4), (33, 1000, 2056, 3)])
+def test_gemm_rows_and_stream_from_operand_tiles_equal_rows_bit_for_bit(M, N, K, splits):
+    """Widths that end inside a tile of 16 rows and inside a k step of 32; every variant of both kernels."""
+    a = torch.randn(M, K, generator=_g(120)).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=_g(121)) * 0.1).bfloat16().to(DEV)
+    tiles = ops.pack_weight_tiles(w)
+    for variant in range(ops.ROWS_VARIANTS):
+        rows = ops.gemm_rows(a, w, torch.float32, variant=variant, splits=splits)
+        got = ops.gemm_rows(a, w, torch.float32, variant=variant, splits=splits, tiles=tiles)
+        assert torch.equal(rows, got), variant
+    assert _rel(_whole(got), a.double().cpu() @ w.double().cpu().T) < 1e-5
+    for variant in range(ops.STREAM_VARIANTS):
+        rows = ops.gemm_stream(a, w, torch.float32, variant=variant, splits=splits, workgroups=3)
+        got = ops.gemm_stream(a, w, torch.float32, variant=variant, splits=splits, workgroups=3, tiles=tiles)
+        assert torch.equal(rows, got), variant
+    assert _rel(_whole(got), a.double().cpu() @ w.double().cpu().T) < 1e-5
+    assert torch.equal(ops.gemm_bf16(a, w, torch.bfloat16), ops.gemm_bf16(a, w, torch.bfloat16, tiles=tiles))
+    with pytest.raises(ops.ShapeError, match="operand tiles"):
+        ops.gemm_rows(a, w, torch.float32, tiles=tiles[:, :-1].contiguous())
+
+
+def test_gemm_rows_fused_activation_from_operand_tiles():
+    M, inter, K = 8, 224, 96
+    x = torch.randn(M, K, generator=_g(122)).bfloat16().to(DEV)
+    fused = (torch.randn(2 * inter, K, generator=_g(123)) * 0.1).bfloat16().to(DEV)
+    rows = ops.gemm_rows(x, fused, torch.bfloat16, ops.EPI_SILU_MUL)
+    assert torch.equal(rows, ops.gemm_rows(x, fused, torch.bfloat16, ops.EPI_SILU_MUL, tiles=ops.pack_weight_tiles(fused)))
+
+
 def test_sum_partials_and_stacked_residual_add():
     parts = torch.randn(5, 7, 88, generator=_g(113))
     want = parts.double().sum(0)
