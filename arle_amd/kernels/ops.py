@@ -750,14 +750,17 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_bf16 takes bfloat16 operands")
     _need(x.shape[1] == w.shape[1], f"gemm_bf16: inner sizes differ ({x.shape[1]} vs {w.shape[1]})")
     _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_bf16 writes bfloat16 or float32")
-    if gemm_rows_preferred(x.shape[0], w.shape[0], x.shape[1], x.stride(0)) and x.data_ptr() % 16 == 0:
+    rows, n, k = x.shape[0], w.shape[0], x.shape[1]
+    aligned = x.data_ptr() % 16 == 0
+    staying = aligned and gemm_stream_preferred(rows, n, k, x.stride(0), tiled=tiles is not None)
+    if not staying and aligned and gemm_rows_preferred(rows, n, k, x.stride(0)):
         out = gemm_rows(x, w, out_dtype, tiles=tiles)
         if out.dim() == 3 and not partials_ok:
             out = sum_partials(out, out_dtype)
         return out
-    if gemm_stream_preferred(x.shape[0], w.shape[0], x.shape[1], x.stride(0)) and x.data_ptr() % 16 == 0:
-        out = gemm_stream(x, w, out_dtype, variant=_STREAM_VARIANT, splits=_stream_splits(x.shape[0], x.shape[1]),
-                          tiles=tiles)
+    if staying:
+        variant, splits = _stream_plan(rows, n, k, tiles is not None)
+        out = gemm_stream(x, w, out_dtype, variant=variant, splits=splits, tiles=tiles)
         # a large stack is added here by many workgroups; the consumer would add it with one workgroup a row
         if out.dim() == 3 and (not partials_ok or out.numel() * 4 > _STREAM_PARTIAL_BYTES):
             out = sum_partials(out, out_dtype)
@@ -780,14 +783,36 @@ _STREAM_MIN_K = 2048
 _STREAM_PARTIAL_BYTES = 6 << 20  # a larger stack of partial products is added before it is handed on
 
 
-def _stream_splits(rows: int, k: int) -> int:
-    return max(_STREAM_SPLITS, -(-k // (32 * _STREAM_STEPS_A_SPLIT)), _stream_min_splits(_STREAM_VARIANT, rows, k))
+# From operand tiles (one contiguous kilobyte a wave and k step) the staying kernel does better still, measured on
+# MI355X at the Qwen3-4B shapes: narrow outputs from 9 rows on (down at 16 rows: 12.8 us against 21.1 us of the
+# few-rows kernel, which stages x again for every column group); q|k|v (6144 columns) at 17..64 rows with eight
+# waves a workgroup and four k splits: 10.1 against the library's 11.9 us at 32 rows, 12.1 against 16.3 us at 64;
+# gate|up (19456 columns) stays level with the library, and stays there.
+_STREAM_TILED_FROM_ROWS = 8
+_STREAM_TILED_MAX_N = 8192
+_STREAM_TILED_WIDE = (1, 4)     # (variant, k splits) for outputs wider than _STREAM_MAX_N
+_STREAM_TILED_MANY_ROWS = 32    # from here on eight waves a workgroup (variant 1) for the narrow outputs too
 
 
-def gemm_stream_preferred(rows: int, n: int, k: int, x_stride: int) -> bool:
-    """Whether the kernel whose workgroups stay, not the library, should run this product: 17..64 rows, a narrow
-    output and a long K."""
-    return (_ROWS_PREFERRED < rows <= ROWS_KERNEL_MAX and n <= _STREAM_MAX_N and k >= _STREAM_MIN_K
+def _stream_splits(rows: int, k: int, variant: int = _STREAM_VARIANT) -> int:
+    return max(_STREAM_SPLITS, -(-k // (32 * _STREAM_STEPS_A_SPLIT)), _stream_min_splits(variant, rows, k))
+
+
+def _stream_plan(rows: int, n: int, k: int, tiled: bool):
+    """(variant, k splits) of the staying kernel for a product."""
+    if tiled and n > _STREAM_MAX_N:
+        variant, splits = _STREAM_TILED_WIDE
+        return variant, max(splits, _stream_min_splits(variant, rows, k))
+    variant = 1 if (tiled and rows > _STREAM_TILED_MANY_ROWS) else _STREAM_VARIANT
+    return variant, _stream_splits(rows, k, variant)
+
+
+def gemm_stream_preferred(rows: int, n: int, k: int, x_stride: int, tiled: bool = False) -> bool:
+    """Whether the kernel whose workgroups stay should run this product: a long K, and from rows: 17..64 rows and a
+    narrow output; from operand tiles: 9..64 rows and a narrow output, 17..64 rows and a middling one."""
+    least = _STREAM_TILED_FROM_ROWS if (tiled and n <= _STREAM_MAX_N) else _ROWS_PREFERRED
+    widest = _STREAM_TILED_MAX_N if tiled else _STREAM_MAX_N
+    return (least < rows <= ROWS_KERNEL_MAX and n <= widest and k >= _STREAM_MIN_K
             and gemm_rows_supported(rows, k, x_stride))
 
 
