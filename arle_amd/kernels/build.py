@@ -32,6 +32,7 @@ SOURCES = {
     "attention_simt": "attention_simt.hip",
     "attention_mfma": "attention_mfma.hip",
     "sampling": "sampling.hip",
+    "ceilings": "ceilings.hip",
     "host": "host/runtime.cpp",
 }
 HEADERS = ("common.h",)

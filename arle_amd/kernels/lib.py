@@ -45,6 +45,8 @@ SIGNATURES = {
     "arle_sample_scratch_bytes": ("sampling", [_i, _i]),
     "arle_sample_rows": ("sampling", [_p, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _p]),
     "arle_apply_penalties": ("sampling", [_p, _i, _i, _p, _p, _p, _p, _p, _p, _p]),
+    "arle_ceiling_read": ("ceilings", [_p, _ll, _i, _p, _p, _p]),
+    "arle_ceiling_mfma": ("ceilings", [_i, _i, _i, _p, _p]),
 }
 
 _libs: dict = {}

@@ -65,6 +65,23 @@ def _timed(torch, fn):
     return time.perf_counter() - t
 
 
+def ceilings() -> int:
+    """What a kernel that only reads memory and one that only multiplies reach on this GPU, against the published peaks."""
+    from arle_amd.kernels import ceilings as c
+
+    read = c.read_bandwidth()
+    small = c.read_bandwidth(launches=40)
+    m32, m16 = c.mfma_rate(shape=32), c.mfma_rate(shape=16)
+    print(json.dumps({
+        "metric": "measured ceilings of one GPU", "unit": "GB/s and TFLOP/s",
+        "hbm_read_gbs": round(read["best"] / 1e9, 1), "hbm_read_frac_of_peak": round(read["best"] / 1e9 / PEAK_HBM_GBS, 4),
+        "hbm_read_100mb_launches_gbs": round(small["best"] / 1e9, 1),
+        "hbm_read_by_workgroups_gbs": {str(k): round(v / 1e9, 1) for k, v in read["by_workgroups"].items()},
+        "mfma_bf16_32x32x16_tflops": round(m32 / 1e12, 1), "mfma_bf16_16x16x32_tflops": round(m16 / 1e12, 1),
+        "mfma_frac_of_peak": round(max(m32, m16) / PEAK_FLOPS["bf16"], 4)}))
+    return 0
+
+
 def mixed_8b(args) -> int:
     """Qwen3-8B shape: 32 requests decoding at 1,024 tokens of context beside one 2,048-token prompt
     that arrives in portions of 512: four steps of 32 + 512 rows.  Reports the mean step and the tokens a second
@@ -201,6 +218,8 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 decode points")
     ap.add_argument("--no-weight-tiles", action="store_true",
                     help="without the second copy of the projection weights that the few-rows kernels stream")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="measure what a kernel that only reads, and one that only multiplies, reach on this GPU, and exit")
     ap.add_argument("--prefill-only", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiles of its kernels) and print that")
     ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode"],
@@ -210,6 +229,8 @@ def main() -> int:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
         return 2
     PAGE = args.page_size
+    if args.ceilings:
+        return ceilings()
     if args.workload == "qwen3-4b" and args.batch is None:
         args.batch = 8
     if args.workload != "qwen3-4b":
