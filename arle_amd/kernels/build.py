@@ -28,6 +28,7 @@ SOURCES = {
     "norm": "norm.hip",
     "gemm_f32": "gemm_f32.hip",
     "gemm_rows": "gemm_rows.hip",
+    "gemm_tiles": "gemm_tiles.hip",
     "rope_kv": "rope_kv.hip",
     "attention_simt": "attention_simt.hip",
     "attention_mfma": "attention_mfma.hip",

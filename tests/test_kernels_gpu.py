@@ -776,6 +776,54 @@ def test_gemm_rows_fused_activation_from_operand_tiles():
     assert torch.equal(rows, ops.gemm_rows(x, fused, torch.bfloat16, ops.EPI_SILU_MUL, tiles=ops.pack_weight_tiles(fused)))
 
 
+@pytest.mark.parametrize("variant", ops.TILES_VARIANTS)
+@pytest.mark.parametrize("M,N,K", [(300, 200, 72), (129, 520, 264), (257, 256, 32), (1, 40, 8), (640, 1000, 1096)])
+def test_gemm_tiles_many_rows_from_operand_tiles(variant, M, N, K):
+    """Rows, columns and K that end inside a workgroup's block, inside a tile and inside a step of 32; fewer steps
+    than a ring holds; every workgroup shape and ring depth."""
+    x = torch.randn(M, K, generator=_g(130)).bfloat16()
+    w = (torch.randn(N, K, generator=_g(131)) * 0.1).bfloat16()
+    tiles = ops.pack_weight_tiles(w.to(DEV))
+    want = x.double() @ w.double().T
+    got = ops.gemm_tiles(x.to(DEV), tiles, N, torch.float32, variant=variant).cpu()
+    assert got.shape == (M, N) and _rel(got, want) < 1e-5
+    got = ops.gemm_tiles(x.to(DEV), tiles, N, torch.bfloat16, variant=variant).cpu()
+    assert got.dtype == torch.bfloat16 and _rel(got, want) < 5e-3
+    # a view with a row stride
+    wide = torch.randn(M, K + 24, generator=_g(132)).bfloat16().to(DEV)
+    got = ops.gemm_tiles(wide[:, 8:8 + K], tiles, N, torch.float32, variant=variant).cpu()
+    assert _rel(got, wide[:, 8:8 + K].double().cpu() @ w.double().T) < 1e-5
+
+
+@pytest.mark.parametrize("variant", [(4, 44), (8, 44), (4, 22)])
+@pytest.mark.parametrize("M,inter,K", [(513, 224, 136), (200, 48, 64), (2048, 1024, 256)])
+def test_gemm_tiles_with_fused_activation(variant, M, inter, K):
+    x = torch.randn(M, K, generator=_g(133)).bfloat16()
+    gate = (torch.randn(inter, K, generator=_g(134)) * 0.1).bfloat16()
+    up = (torch.randn(inter, K, generator=_g(135)) * 0.1).bfloat16()
+    fused = torch.stack([gate.view(-1, 16, K), up.view(-1, 16, K)], dim=1).reshape(2 * inter, K).contiguous()
+    want = plain.silu(x.double() @ gate.double().T) * (x.double() @ up.double().T)
+    tiles = ops.pack_weight_tiles(fused.to(DEV))
+    got = ops.gemm_tiles(x.to(DEV), tiles, 2 * inter, torch.float32, ops.EPI_SILU_MUL, variant=variant).cpu()
+    assert got.shape == (M, inter) and _rel(got, want) < 1e-5
+    got = ops.gemm_tiles(x.to(DEV), tiles, 2 * inter, torch.bfloat16, ops.EPI_SILU_MUL, variant=variant).cpu()
+    assert _rel(got, want) < 5e-3
+
+
+def test_gemm_tiles_refuses_what_it_cannot_take():
+    x = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(48, 64, dtype=torch.bfloat16, device=DEV)
+    tiles = ops.pack_weight_tiles(w)
+    with pytest.raises(ops.ShapeError, match="operand tiles"):
+        ops.gemm_tiles(x, tiles, 64)                       # tiles of another matrix
+    with pytest.raises(ops.ShapeError, match="interleaved"):
+        ops.gemm_tiles(x, tiles, 48, epilogue=ops.EPI_SILU_MUL)
+    with pytest.raises(ops.ShapeError, match="no variant"):
+        ops.gemm_tiles(x, tiles, 48, variant=(3, 3))
+    with pytest.raises(ops.ShapeError, match="bfloat16"):
+        ops.gemm_tiles(x.float(), tiles, 48)
+
+
 def test_sum_partials_and_stacked_residual_add():
     parts = torch.randn(5, 7, 88, generator=_g(113))
     want = parts.double().sum(0)
