@@ -14,16 +14,21 @@
 //     no bank conflicts, no padding, no swizzle.  Two stages.
 //   * Both streams run ahead of the products through rings of registers (PD and PX steps of 32 k).  Nothing is
 //     selected or converted behind a load: a use right behind a load is a wait for that load.
-//   * The operand reads of a step are pinned four reads ahead of the products that need them.
+//   * The operand reads of a step are pinned four reads ahead of the products that need them.  PIPE: four LDS
+//     stages, the step's barrier in mid-step, and behind it the first operands of the next step are read while
+//     the last products of this one run.
+//   * bfloat16 results leave through a wave's own part of LDS as whole rows of 128 contiguous bytes.
 //   * Workgroups are numbered so that the row blocks of a column block run on one XCD at one time: W is fetched
 //     from memory once, and X (a few megabytes) stays in the L2 of every XCD.
 //   * Epilogue kEpiSiluMul (gate and up rows interleaved in blocks of 16): the 32 columns of an accumulator are
 //     16 gate and the 16 matching up columns, registers r and r + 8 of the same lane, so silu(gate) * up happens
 //     in registers and [M, N/2] is written.
 //
-// Measured on MI355X at the Qwen3-4B shapes, weights cold: gate|up with the activation at 2,048 rows 241 us
-// against the library's 249 us and 24 us for the activation kernel; at 4,096 rows 445 against 480 us.  Plain
-// products stay with the library, which is faster there (q|k|v at 2,048 rows: 60 against 91 us), as the reference
+// Measured on MI355X at the Qwen3-4B shapes, weights cold: gate|up with the activation at 2,048 rows 248 us
+// against the library's 249 us and 22 us for the activation kernel; at 4,096 rows 451 against 494 us; at 8,192
+// rows the library is ahead.  The loop with nothing but its products runs at 1,120 TFLOP/s on q|k|v at 2,048 rows
+// (192 workgroups for 256 compute units), with everything at 760.  Plain
+// products stay with the library, which is faster there (q|k|v at 2,048 rows: 60 against 85 us), as the reference
 // leaves all of them to cuBLAS (infer/src/ops/linear.rs:921-959) and runs the activation as a kernel of its own
 // (crates/cuda-kernels/csrc/misc/split_qkv.cu:35-52).
 #include "common.h"
@@ -50,13 +55,17 @@ struct TilesArgs {
 };
 
 // MT: row tiles of 32 that a workgroup owns (4: 128 rows, two workgroups a compute unit)
-template <int MT, int PD, int PX, int EPI, typename TOut>
+template <int MT, int PD, int PX, bool PIPE, int EPI, typename TOut>
 __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_kernel(const TilesArgs a) {
   static_assert(PD % 2 == 0 && PD % PX == 0, "rounds of PD steps; the LDS stage alternates; the X ring divides the W ring");
   static_assert(MT % 2 == 0, "every wave fetches whole pieces of 16 rows");
+  static_assert(!PIPE || PD == 4, "the pipelined loop walks four LDS stages in a round of four steps");
   constexpr int kRows = 32 * MT, kStage = kRows * 32 * 2;  // bytes of one LDS stage: the rows' 32 k
   constexpr int XH = 2 * MT / kTlWaves;                    // pieces of 16 rows x 32 k that a wave fetches a step
-  __shared__ __align__(16) unsigned char lds[2 * kStage];
+  constexpr int kOutPitch = 144;  // bytes of a row of 64 bfloat16 in the epilogue's LDS, padded against bank conflicts
+  constexpr int kOutBytes = kTlWaves * 32 * kOutPitch;
+  constexpr int kLdsBytes = (PIPE ? 4 : 2) * kStage > kOutBytes ? (PIPE ? 4 : 2) * kStage : kOutBytes;
+  __shared__ __align__(16) unsigned char lds[kLdsBytes];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // known to be the same in all lanes
   const int li = lane & 15, g = lane >> 4;   // the lane as (row, 8 k) of a 16 x 32 piece: tiles in memory, fetches of X
@@ -129,9 +138,9 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
   auto multiply = [&](const bf16x8 (&wt)[2][2], int stage) {  // the step parked in `stage` with its tiles
     const unsigned char* xs = lds + stage * kStage + lane * 16;
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
+    for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
+      for (int t = 0; t < MT; ++t) {
         const bf16x8 xop = *reinterpret_cast<const bf16x8*>(xs + (2 * t + kk) * 1024);
 #pragma unroll
         for (int tn = 0; tn < 2; ++tn)
@@ -148,6 +157,49 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
     }
     __builtin_amdgcn_sched_group_barrier(0x008, 2 * kAhead, 0);
   };
+  if constexpr (PIPE) {
+    // Four stages, so that a step can be parked two steps before anybody reads its stage again, and the barrier of
+    // a step can stand in the middle of it: step s + 1 is parked first thing in step s, the barrier comes before
+    // the last kA operand reads' worth of products, and behind it the first kA operands of step s + 1 are read
+    // while the last products of step s run.  No product waits for an LDS read right behind a barrier.
+    constexpr int kA = 4, kR = 2 * MT;
+    bf16x8 pre[kA];
+#pragma unroll
+    for (int i = 0; i < kA; ++i) pre[i] = *reinterpret_cast<const bf16x8*>(lds + 2 * i * 1024 + lane * 16);  // row tiles 0 .. kA - 1, half 0
+    auto step = [&](bf16x8 (&wt)[2][2], u32x4 (&xnext)[XH], int u, int s, bool fetch) {
+      park_x((u + 1) & 3, xnext);
+      if (fetch) load_x(s + 1 + PX, xnext);
+      const unsigned char* cur = lds + (u & 3) * kStage + lane * 16;
+      const unsigned char* nxt = lds + ((u + 1) & 3) * kStage + lane * 16;
+      bf16x8 xo[kR];
+#pragma unroll
+      for (int i = 0; i < kA; ++i) xo[i] = pre[i];
+#pragma unroll
+      for (int r = 0; r < kR; ++r) {
+        if (r == kR - kA) __syncthreads();
+        // read r is the operand of row tile r % MT, half r / MT of the step: the two products into one
+        // accumulator are 2 MT products apart (a product right behind one into the same accumulator waits for it)
+        constexpr auto at = [](int q) { return (2 * (q % MT) + q / MT) * 1024; };
+        if (r + kA < kR)
+          xo[r + kA] = *reinterpret_cast<const bf16x8*>(cur + at(r + kA));
+        else
+          pre[r + kA - kR] = *reinterpret_cast<const bf16x8*>(nxt + at(r + kA - kR));
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn)
+          acc[r % MT][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wt[tn][r / MT], xo[r], acc[r % MT][tn], 0, 0, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      }
+      if (fetch) load_w(s + PD, wt);
+    };
+    for (int r = 0; r < rounds; ++r) {
+#pragma unroll
+      for (int u = 0; u < PD; ++u) step(wring[u], xring[u % PX], u, r * PD + u, true);
+    }
+#pragma unroll
+    for (int u = 0; u < PD - 1; ++u)
+      if (u < rest) step(wring[u], xring[u % PX], u, rounds * PD + u, false);
+  } else {
   for (int r = 0; r < rounds; ++r) {
 #pragma unroll
     for (int u = 0; u < PD; ++u) {
@@ -171,9 +223,64 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
       }
     }
   }
+  }
 
   // acc[t][tn][r] = C[m0 + 32 t + j][n0 + 32 tn + 8 (r / 4) + 4 h + r % 4]
   TOut* out = static_cast<TOut*>(a.out);
+  // bfloat16 results whose 64 columns all exist: a lane holds pieces of 8 bytes, and stored as they are they
+  // would reach memory as 16-byte scraps of a row (a third of the kernel's time at 2,048 x 6,144).  So every
+  // row tile goes through a part of LDS that belongs to the wave and leaves as whole rows of 128 (with the
+  // activation: 64) contiguous bytes, eight (four) lanes a row.
+  constexpr int kOutCols = EPI == kEpiSiluMul ? 32 : 64;
+  if constexpr (sizeof(TOut) == 2) {
+    const int c0 = EPI == kEpiSiluMul ? n0 / 2 : n0;          // first output column of the wave
+    const int n_out = EPI == kEpiSiluMul ? N / 2 : N;
+    if (c0 + kOutCols <= n_out && (a.ldo & 7) == 0 && (reinterpret_cast<uintptr_t>(a.out) & 15) == 0) {  // the same in all lanes
+      __syncthreads();  // every wave is done with the stages
+      unsigned char* mine = lds + wave * (32 * kOutPitch);
+      constexpr int kLanesARow = kOutCols / 8, kRowsAPass = 64 / kLanesARow;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn) {
+          if constexpr (EPI == kEpiSiluMul) {
+#pragma unroll
+            for (int q4 = 0; q4 < 2; ++q4) {
+              float v[4];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const float gate = acc[t][tn][4 * q4 + e];
+                v[e] = gate / (1.0f + expf(-gate)) * acc[t][tn][4 * q4 + e + 8];
+              }
+              *reinterpret_cast<uint2*>(mine + j * kOutPitch + (16 * tn + 8 * q4 + 4 * h) * 2) =
+                  uint2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+            }
+          } else {
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4)
+              *reinterpret_cast<uint2*>(mine + j * kOutPitch + (32 * tn + 8 * q4 + 4 * h) * 2) =
+                  uint2{pack_bf16x2(acc[t][tn][4 * q4], acc[t][tn][4 * q4 + 1]),
+                        pack_bf16x2(acc[t][tn][4 * q4 + 2], acc[t][tn][4 * q4 + 3])};
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int i = 0; i < 32 / kRowsAPass; ++i) {
+          const int rr = kRowsAPass * i + lane / kLanesARow, piece = lane % kLanesARow;
+          const u32x4 v = *reinterpret_cast<const u32x4*>(mine + rr * kOutPitch + piece * 16);
+          const int row = m0 + 32 * t + rr;
+          if (row < M)
+            *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(out) + static_cast<int64_t>(row) * a.ldo + c0 + piece * 8) = v;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int row = m0 + 32 * t + j;
@@ -227,22 +334,23 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
   }
 }
 
-template <int MT, int PD, int PX, int EPI>
+template <int MT, int PD, int PX, bool PIPE, int EPI>
 int launch_tiles(TilesArgs a, int out_dtype, hipStream_t s) {
   a.m_blocks = (a.M + 32 * MT - 1) / (32 * MT);
   const long long n_groups = (a.n_blocks + kTlXcds - 1) / kTlXcds;
   const long long grid = n_groups * a.m_blocks * kTlXcds;
   if (grid > 0x7fffffffLL) return static_cast<int>(hipErrorInvalidValue);
   if (out_dtype == kF32)
-    gemm_tiles_kernel<MT, PD, PX, EPI, float><<<static_cast<unsigned>(grid), kTlWaves * kWave, 0, s>>>(a);
+    gemm_tiles_kernel<MT, PD, PX, PIPE, EPI, float><<<static_cast<unsigned>(grid), kTlWaves * kWave, 0, s>>>(a);
   else
-    gemm_tiles_kernel<MT, PD, PX, EPI, bf16><<<static_cast<unsigned>(grid), kTlWaves * kWave, 0, s>>>(a);
+    gemm_tiles_kernel<MT, PD, PX, PIPE, EPI, bf16><<<static_cast<unsigned>(grid), kTlWaves * kWave, 0, s>>>(a);
   return launch_status();
 }
 
-template <int MT, int PD, int PX>
+template <int MT, int PD, int PX, bool PIPE = false>
 int dispatch_tiles(const TilesArgs& a, int out_dtype, int epilogue, hipStream_t s) {
-  return epilogue ? launch_tiles<MT, PD, PX, kEpiSiluMul>(a, out_dtype, s) : launch_tiles<MT, PD, PX, kEpiNone>(a, out_dtype, s);
+  return epilogue ? launch_tiles<MT, PD, PX, PIPE, kEpiSiluMul>(a, out_dtype, s)
+                  : launch_tiles<MT, PD, PX, PIPE, kEpiNone>(a, out_dtype, s);
 }
 
 }  // namespace arle
@@ -267,5 +375,7 @@ extern "C" int arle_gemm_tiles(const void* x, long long ldx, const void* w_tiles
   if (row_tiles == 8 && depth == 22) return dispatch_tiles<8, 2, 2>(a, out_dtype, epilogue, s);
   if (row_tiles == 8 && depth == 42) return dispatch_tiles<8, 4, 2>(a, out_dtype, epilogue, s);
   if (row_tiles == 8 && depth == 44) return dispatch_tiles<8, 4, 4>(a, out_dtype, epilogue, s);
+  if (row_tiles == 8 && depth == 144) return dispatch_tiles<8, 4, 4, true>(a, out_dtype, epilogue, s);
+  if (row_tiles == 8 && depth == 142) return dispatch_tiles<8, 4, 2, true>(a, out_dtype, epilogue, s);
   return static_cast<int>(hipErrorInvalidValue);
 }

@@ -722,20 +722,24 @@ _STREAM_TARGET_WORKGROUPS = 256   # staying workgroups in all: one for every com
 
 
 # The many-rows kernel that reads operand tiles takes over from the library where it was measured faster on MI355X:
-# gate|up with the activation fused, from 2,048 rows on (2,048 rows of the Qwen3-4B shape: 241 us against the
-# library's 249 + 24 us for the activation kernel; 1,024 rows and fewer: the library).  Plain products stay with
-# the library (q|k|v at 2,048 rows: 95 against 60 us).
+# gate|up with the activation fused, at 2,048 to about 6,000 rows (Qwen3-4B shape, cold weights: 248 us against the
+# library's 249 + 22 us for the activation kernel at 2,048 rows, 451 against 494 us at 4,096; at 1,024 rows the two
+# are level, at 8,192 the library is ahead, 833 against 880 us).  Plain products stay with the library (q|k|v at
+# 2,048 rows: 85 against 60 us).
 _TILES_MIN_ROWS = 2048
+_TILES_MAX_ROWS = 6144
 _TILES_MIN_N = 4096
-_TILES_BIG_ROWS = 4096      # from here on workgroups of 256 rows (917 against 873 TFLOP/s at 4,096 rows)
+_TILES_BIG_ROWS = 4096      # from here on workgroups of 256 rows with the pipelined loop
 
 
 def gemm_tiles_preferred(rows: int, n: int, k: int, x_stride: int, fused: bool = False) -> bool:
     """Whether the many-rows kernel that reads operand tiles, not the library, should run this product."""
-    return fused and rows >= _TILES_MIN_ROWS and n >= _TILES_MIN_N and k % 8 == 0 and x_stride % 8 == 0
+    return (fused and _TILES_MIN_ROWS <= rows < _TILES_MAX_ROWS and n >= _TILES_MIN_N and k % 8 == 0
+            and x_stride % 8 == 0)
 
 
-TILES_VARIANTS = ((4, 22), (4, 42), (4, 44), (8, 22), (8, 42), (8, 44))   # (row tiles of 32 a workgroup, ring depths W|X)
+# (row tiles of 32 a workgroup, ring depths W|X; 1xx: the loop with the barrier in mid-step and four LDS stages)
+TILES_VARIANTS = ((4, 22), (4, 42), (4, 44), (8, 22), (8, 42), (8, 44), (8, 144), (8, 142))
 
 
 def gemm_tiles(x, tiles, n: int, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, variant=None):
@@ -752,7 +756,7 @@ def gemm_tiles(x, tiles, n: int, out_dtype=torch.bfloat16, epilogue: int = EPI_N
     fused = epilogue == EPI_SILU_MUL
     _need(not fused or n % 32 == 0, "the fused activation needs gate/up interleaved in blocks of 16")
     if variant is None:
-        variant = (8, 44) if M >= _TILES_BIG_ROWS else (4, 44)
+        variant = (8, 144) if M >= _TILES_BIG_ROWS else (4, 44)
     _need(tuple(variant) in TILES_VARIANTS, f"gemm_tiles has no variant {variant}")
     out = torch.empty((M, n // 2 if fused else n), dtype=out_dtype, device=x.device)
     lib.call("arle_gemm_tiles", x.data_ptr(), x.stride(0), tiles.data_ptr(), out.data_ptr(), out.stride(0),
