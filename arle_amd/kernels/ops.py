@@ -823,7 +823,7 @@ _STREAM_MAX_N = 5120            # 60 against the library's 146 us there at 32 ro
 _STREAM_MIN_K = 2048
 
 
-_STREAM_PARTIAL_BYTES = 6 << 20  # a larger stack of partial products is added before it is handed on
+_STREAM_PARTIAL_BYTES = 8 << 20  # a larger stack of partial products is added before it is handed on
 
 
 # From operand tiles (one contiguous kilobyte a wave and k step) the staying kernel does better still, measured on
