@@ -359,7 +359,8 @@ using namespace arle;
 
 // x [M, K] bfloat16 (row stride ldx, a multiple of 8), w_tiles the operand tiles of W [N, K], K % 8 == 0.
 // out [M, N] (epilogue 0) or [M, N/2] (epilogue 1: N % 32 == 0, gate and up rows of W interleaved in blocks of 16),
-// bfloat16 or float32, row stride ldo.
+// bfloat16 or float32, row stride ldo.  row_tiles: row tiles of 32 a workgroup (4 or 8); depth: ring depths of W and X
+// as two digits (22, 44), + 100 for the loop with the barrier in mid-step (8 row tiles only).
 extern "C" int arle_gemm_tiles(const void* x, long long ldx, const void* w_tiles, void* out, long long ldo, int out_dtype,
                                int M, int N, int K, int epilogue, int row_tiles, int depth, void* stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -370,12 +371,8 @@ extern "C" int arle_gemm_tiles(const void* x, long long ldx, const void* w_tiles
                     0, (N + kTlCols - 1) / kTlCols};
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (row_tiles == 4 && depth == 22) return dispatch_tiles<4, 2, 2>(a, out_dtype, epilogue, s);
-  if (row_tiles == 4 && depth == 42) return dispatch_tiles<4, 4, 2>(a, out_dtype, epilogue, s);
   if (row_tiles == 4 && depth == 44) return dispatch_tiles<4, 4, 4>(a, out_dtype, epilogue, s);
-  if (row_tiles == 8 && depth == 22) return dispatch_tiles<8, 2, 2>(a, out_dtype, epilogue, s);
-  if (row_tiles == 8 && depth == 42) return dispatch_tiles<8, 4, 2>(a, out_dtype, epilogue, s);
   if (row_tiles == 8 && depth == 44) return dispatch_tiles<8, 4, 4>(a, out_dtype, epilogue, s);
   if (row_tiles == 8 && depth == 144) return dispatch_tiles<8, 4, 4, true>(a, out_dtype, epilogue, s);
-  if (row_tiles == 8 && depth == 142) return dispatch_tiles<8, 4, 2, true>(a, out_dtype, epilogue, s);
   return static_cast<int>(hipErrorInvalidValue);
 }

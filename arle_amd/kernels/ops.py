@@ -739,7 +739,7 @@ def gemm_tiles_preferred(rows: int, n: int, k: int, x_stride: int, fused: bool =
 
 
 # (row tiles of 32 a workgroup, ring depths W|X; 1xx: the loop with the barrier in mid-step and four LDS stages)
-TILES_VARIANTS = ((4, 22), (4, 42), (4, 44), (8, 22), (8, 42), (8, 44), (8, 144), (8, 142))
+TILES_VARIANTS = ((4, 22), (4, 44), (8, 44), (8, 144))
 
 
 def gemm_tiles(x, tiles, n: int, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, variant=None):

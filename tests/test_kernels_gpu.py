@@ -795,7 +795,7 @@ def test_gemm_tiles_many_rows_from_operand_tiles(variant, M, N, K):
     assert _rel(got, wide[:, 8:8 + K].double().cpu() @ w.double().T) < 1e-5
 
 
-@pytest.mark.parametrize("variant", [(4, 44), (8, 44), (4, 22), (8, 144)])
+@pytest.mark.parametrize("variant", ops.TILES_VARIANTS)
 @pytest.mark.parametrize("M,inter,K", [(513, 224, 136), (200, 48, 64), (2048, 1024, 256), (300, 128, 1096)])
 def test_gemm_tiles_with_fused_activation(variant, M, inter, K):
     x = torch.randn(M, K, generator=_g(133)).bfloat16()
