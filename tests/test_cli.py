@@ -1,0 +1,33 @@
+"""The command line's options, without a GPU: names and meanings follow the reference's `arle` and `infer`
+(crates/cli/src/args.rs:188-302, infer/src/main.rs:26-236)."""
+import pytest
+
+from arle_amd.cli import build_parser, main
+
+
+def test_global_options_and_run():
+    args = build_parser().parse_args(["--model-path", "/m", "--max-tokens", "auto", "--temperature", "0.7", "--no-cuda-graph",
+                                      "--num-slots", "8", "--chunked-prefill-size", "2048", "run", "--prompt-ids", "1, 2,3",
+                                      "--json"])
+    assert args.command == "run" and args.model_path == "/m" and args.max_tokens == 0 and args.temperature == 0.7
+    assert args.no_cuda_graph and not args.no_weight_tiles and args.num_slots == 8 and args.chunked_prefill_size == 2048
+    assert args.prompt_ids == "1, 2,3" and args.json
+
+
+def test_defaults_are_the_reference_library_defaults():
+    args = build_parser().parse_args(["--model-path", "/m", "run", "--prompt", "hi"])
+    # infer/src/scheduler/types.rs:192-238: slots 4, chunk 512, 16384 tokens a step; greedy (crates/cli/src/args.rs)
+    assert (args.num_slots, args.chunked_prefill_size, args.max_num_batched_tokens, args.max_prefill_tokens) == (4, 512, 16384, 16384)
+    assert args.temperature == 0.0 and args.top_k == -1 and args.top_p == 1.0 and args.min_p == 0.0 and args.seed == 42
+    assert not args.no_cuda_graph and not args.no_weight_tiles and args.dtype == "bfloat16"
+
+
+def test_bad_values_are_refused(capsys):
+    with pytest.raises(SystemExit):
+        build_parser().parse_args(["--max-tokens", "-3", "run", "--prompt", "x"])
+    with pytest.raises(SystemExit):
+        build_parser().parse_args(["--dtype", "float16", "run", "--prompt", "x"])
+    with pytest.raises(SystemExit):   # one source of the prompt only
+        build_parser().parse_args(["run", "--prompt", "x", "--stdin"])
+    assert main(["run", "--prompt", "x"]) == 2          # no model folder
+    assert "--model-path" in capsys.readouterr().err
