@@ -146,3 +146,40 @@ def test_step_refuses_bad_input(model_b):
     assert eng.length("a") == 0 and eng.cache.free_pages() == [4]   # nothing was changed
     out = eng.step([StepEntry("a", [1, 2, 3], [])])
     assert out.shape == (0, cfg["vocab_size"]) and eng.length("a") == 3
+
+
+def test_a_portion_of_two_thousand_rows_takes_the_many_rows_kernel(tmp_path):
+    """A feed-forward wide enough (gate|up of 4,096 rows) and a portion long enough (2,100 tokens) for
+    gemm_tiles with the fused activation: the logits of the whole prompt in one step, in portions that the
+    library takes, and of the plain implementation agree; a captured replay of the long step gives the same bits."""
+    import os
+    from arle_amd.config import Qwen3Config
+    from arle_amd.kernels import ops
+    from arle_amd.weights import write_random_model
+
+    raw = dict(num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+               intermediate_size=2048, vocab_size=300, rope_theta=10000.0, rms_norm_eps=1e-6,
+               tie_word_embeddings=True, max_position_embeddings=4096)
+    d = os.path.join(str(tmp_path), "wide_ffn")
+    write_random_model(d, "Qwen3ForCausalLM", Qwen3Config.from_dict(raw), seed=5, std=0.03, norm_std=0.02)
+    cfg, weights = read_folder(d)
+    n = 2100
+    assert ops.gemm_tiles_preferred(n, 2 * raw["intermediate_size"], raw["hidden_size"], raw["hidden_size"], fused=True)
+    toks = random_tokens(n, raw["vocab_size"], 12)
+    want_at = list(range(n))
+    eng = Engine.from_folder(d, dtype="bfloat16", page_size=16, max_tokens=3 * 2176, max_slots=3)
+    whole = replay.run_steps(eng, [{"entries": [("w", toks, want_at)], "end": ["w"]}])
+    replay.compare(whole, cfg, weights, {"w": toks}, TOL["bfloat16"], "2,100 rows in one step")
+    steps, at = [], 0
+    for size in (700, 700, 700):
+        wanted = [p - at for p in want_at if at <= p < at + size]
+        steps.append({"entries": [("p", toks[at:at + size], wanted)], "end": []})
+        at += size
+    cut = replay.run_steps(eng, steps)
+    replay.compare(cut, cfg, weights, {"p": toks}, TOL["bfloat16"], "2,100 rows in portions of 700")
+    # the same long step twice more: the third runs from a captured graph
+    again = [replay.run_steps(eng, [{"entries": [(f"g{i}", toks, want_at)], "end": [f"g{i}"]}]) for i in range(2)]
+    assert eng.graph_replays >= 1
+    for i, got in enumerate(again):
+        for (_, pos), logits in got.items():
+            assert torch.equal(logits, whole[("w", pos)]), (i, pos)
