@@ -519,6 +519,7 @@ _ROWS_MAX_SPLITS = 4             # ... the consumer pays for every part of the s
 _ROWS_PARTIAL_BYTES = 3 << 20    # ... and the float32 partial products stay below this
 _ROWS_WIDE_N = 32768             # from here on (an output head) N alone gives enough workgroups
 _ROWS_NARROW_N = 4096            # up to here N gives so few that one column tile a workgroup is best
+_ROWS_FUSED_MAX = 32             # gate|up with the activation: as many rows as fit into LDS with all of K (27 at K = 2560): 4.20 against 4.41 ms a step at batch 20
 _ROWS_PREFERRED = 16             # with more rows the library is at least as fast on MI355X
 _V_GENERAL, _V_FUSED_FEW, _V_NARROW, _V_SHARED = 0, 1, 2, 3
 ROWS_VARIANTS = 5
@@ -534,10 +535,11 @@ def _fused_variant(rows: int) -> int:
 
 def gemm_rows_preferred(rows: int, n: int, k: int, x_stride: int, fused: bool = False) -> bool:
     """Whether the hand-written kernel, not the library, should run this product."""
+    if fused:   # the activation needs whole sums: the rows of all of K in LDS at once
+        return (gemm_rows_supported(rows, k, x_stride) and rows <= _ROWS_FUSED_MAX
+                and _rows_min_splits(_fused_variant(rows), rows, k) == 1)
     if not gemm_rows_supported(rows, k, x_stride) or rows > _ROWS_PREFERRED:
         return False
-    if fused:   # the activation needs whole sums: the rows of all of K in LDS at once
-        return _rows_min_splits(_fused_variant(rows), rows, k) == 1
     return True
 
 
