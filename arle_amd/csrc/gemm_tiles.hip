@@ -235,8 +235,8 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
   if constexpr (sizeof(TOut) == 2) {
     const int c0 = EPI == kEpiSiluMul ? n0 / 2 : n0;          // first output column of the wave
     const int n_out = EPI == kEpiSiluMul ? N / 2 : N;
-    if (c0 + kOutCols <= n_out && (a.ldo & 7) == 0 && (reinterpret_cast<uintptr_t>(a.out) & 15) == 0) {  // the same in all lanes
-      __syncthreads();  // every wave is done with the stages
+    __syncthreads();  // every wave is done with the stages (all waves come here, whichever way they store)
+    if (c0 + kOutCols <= n_out && (a.ldo & 7) == 0 && (reinterpret_cast<uintptr_t>(a.out) & 15) == 0) {  // the same in all lanes of a wave
       unsigned char* mine = lds + wave * (32 * kOutPitch);
       constexpr int kLanesARow = kOutCols / 8, kRowsAPass = 64 / kLanesARow;
 #pragma unroll
