@@ -882,3 +882,16 @@ def test_split_choices_depend_on_shape_and_context_class_only():
     assert 2 <= few <= 8 and few == ops.portion_key_splits(512, 512, 1, max_kv_len=3000, **args)
     assert ops.portion_key_splits(128, 128, 1, max_kv_len=200, **args) == 1              # too few keys to cut
     assert ops.portion_key_splits(64, 64, 1, max_kv_len=65536, **args) == 8
+
+
+def test_measuring_kernels_give_plausible_ceilings():
+    """The two kernels behind `bench.py --ceilings`: a read of 256 MB and a short run of matrix-core products
+    land between a tenth of the published peaks and the peaks themselves."""
+    from arle_amd.kernels import ceilings
+
+    read = ceilings.read_bandwidth(DEV, total_bytes=256 << 20, repeats=2)
+    assert 0.8e12 < read["best"] < 8.0e12 and set(read["by_workgroups"]) and read["launches"] == 1
+    parts = ceilings.read_bandwidth(DEV, total_bytes=256 << 20, launches=4, repeats=2)
+    assert 0.5e12 < parts["best"] < 8.0e12
+    for shape in (16, 32):
+        assert 2.5e14 < ceilings.mfma_rate(DEV, shape=shape, iters=2000, repeats=1) < 2.6e15
