@@ -24,11 +24,12 @@
 //     16 gate and the 16 matching up columns, registers r and r + 8 of the same lane, so silu(gate) * up happens
 //     in registers and [M, N/2] is written.
 //
-// Measured on MI355X at the Qwen3-4B shapes, weights cold: gate|up with the activation at 2,048 rows 248 us
-// against the library's 249 us and 22 us for the activation kernel; at 4,096 rows 451 against 494 us; at 8,192
-// rows the library is ahead.  The loop with nothing but its products runs at 1,120 TFLOP/s on q|k|v at 2,048 rows
-// (192 workgroups for 256 compute units), with everything at 760.  Plain
-// products stay with the library, which is faster there (q|k|v at 2,048 rows: 60 against 85 us), as the reference
+// Measured on MI355X, weights cold: gate|up of the Qwen3-4B shape with the activation at 2,048 rows 237-255 us
+// against 234-272 us for the library's product and the activation kernel (machines differ); whole prefill steps are
+// 0.5 to 4.6 % faster with it at that shape, and 8-9 % slower at hidden sizes of 4,096 and 5,120, so the caller
+// takes it for the former only.  The loop without its global loads runs at 930 TFLOP/s on q|k|v at 2,048 rows
+// (192 workgroups for 256 compute units), with everything at 760.  Plain products stay with the library, which
+// is faster there (q|k|v at 2,048 rows: 60 against 85 us), as the reference
 // leaves all of them to cuBLAS (infer/src/ops/linear.rs:921-959) and runs the activation as a kernel of its own
 // (crates/cuda-kernels/csrc/misc/split_qkv.cu:35-52).
 #include "common.h"

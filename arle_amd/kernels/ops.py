@@ -723,21 +723,24 @@ def gemm_stream(x, w, out_dtype=torch.bfloat16, *, variant: int = 0, splits: int
 _STREAM_TARGET_WORKGROUPS = 256   # staying workgroups in all: one for every compute unit
 
 
-# The many-rows kernel that reads operand tiles takes over from the library where it was measured faster on MI355X:
-# gate|up with the activation fused, at 2,048 to about 6,000 rows (Qwen3-4B shape, cold weights: 248 us against the
-# library's 249 + 22 us for the activation kernel at 2,048 rows, 451 against 494 us at 4,096; at 1,024 rows the two
-# are level, at 8,192 the library is ahead, 833 against 880 us).  Plain products stay with the library (q|k|v at
-# 2,048 rows: 85 against 60 us).
+# The many-rows kernel that reads operand tiles takes over from the library only where whole prefill steps were
+# measured faster with it on MI355X (same machine, both ways, 12 layers): gate|up with the activation fused, a hidden
+# size of at most 2,560 and 2,048 to about 6,000 rows.  Qwen3-4B widths: 0.5 to 4.6 % of the step at 2,048 rows (the
+# gain differs from machine to machine), 1.8 % at 4,096; hidden sizes 1,024 and 2,048: level; hidden sizes 4,096 and
+# 5,120: 9 and 8 % slower, so the library keeps those.  Kernel against kernel with cold weights the library's product
+# and the activation kernel take 234-272 us at 2,048 x 19,456 x 2,560 and this kernel 237-255 us; at 8,192 rows the
+# library is ahead.  Plain products stay with the library (q|k|v at 2,048 rows: 85 against 60 us).
 _TILES_MIN_ROWS = 2048
 _TILES_MAX_ROWS = 6144
 _TILES_MIN_N = 4096
+_TILES_MAX_K = 2560
 _TILES_BIG_ROWS = 4096      # from here on workgroups of 256 rows with the pipelined loop
 
 
 def gemm_tiles_preferred(rows: int, n: int, k: int, x_stride: int, fused: bool = False) -> bool:
     """Whether the many-rows kernel that reads operand tiles, not the library, should run this product."""
-    return (fused and _TILES_MIN_ROWS <= rows < _TILES_MAX_ROWS and n >= _TILES_MIN_N and k % 8 == 0
-            and x_stride % 8 == 0)
+    return (fused and _TILES_MIN_ROWS <= rows < _TILES_MAX_ROWS and n >= _TILES_MIN_N and k <= _TILES_MAX_K
+            and k % 8 == 0 and x_stride % 8 == 0)
 
 
 # (row tiles of 32 a workgroup, ring depths W|X; 1xx: the loop with the barrier in mid-step and four LDS stages)
