@@ -426,8 +426,8 @@ using namespace arle;
 
 // Shapes of a workgroup, by `variant`: (WN, WK, PD), picked by the caller per matrix shape and row count
 // from measurements on MI355X.  The fused activation needs an even WN.
-//   0  general product               1  gate/up with the fused activation, up to 8 rows
-//   2  few output columns            3  more than 8 rows with the fused activation, or very many columns
+//   0  general product               1  gate/up with the fused activation, a few rows
+//   2  few output columns            3  more rows with the fused activation, or very many columns
 //   4  general, more columns a workgroup
 #define ARLE_ROWS_VARIANTS(X) X(0, 2, 2, 4) X(1, 2, 4, 4) X(2, 1, 4, 4) X(3, 8, 1, 4) X(4, 4, 1, 8)
 constexpr int kVariants = 5;
