@@ -15,6 +15,19 @@ from ..kernels import ops
 from .base import Part, register
 
 
+def rope_table(rotary_dim: int, theta: float, positions: int):
+    """(cos, sin), each float32 [positions, rotary_dim/2] on the CPU: angle(pos, i) = pos * theta^(-2i/rotary_dim).
+
+    float32 throughout, as the reference computes it on the host (infer/src/weight_loader.rs:963-981).
+    """
+    half = rotary_dim // 2
+    base = torch.tensor(float(theta), dtype=torch.float32)
+    exponent = torch.arange(half, dtype=torch.float32) * 2.0 / float(rotary_dim)
+    inv_freq = 1.0 / torch.pow(base, exponent)
+    angle = torch.arange(positions, dtype=torch.float32)[:, None] * inv_freq[None, :]
+    return torch.cos(angle).contiguous(), torch.sin(angle).contiguous()
+
+
 @register("position", "rope_neox")
 class RopeNeox(Part):
     """params: head_dim, rotary_dim (default head_dim), theta, max_positions."""
@@ -40,14 +53,8 @@ class RopeNeox(Part):
         return RopeNeox._shared[key]
 
     def _make_table(self, positions: int):
-        half = self.rotary_dim // 2
-        # float32 throughout, as the reference computes it on the host
-        theta = torch.tensor(self.theta, dtype=torch.float32)
-        exponent = torch.arange(half, dtype=torch.float32) * 2.0 / float(self.rotary_dim)
-        inv_freq = 1.0 / torch.pow(theta, exponent)
-        angle = torch.arange(positions, dtype=torch.float32)[:, None] * inv_freq[None, :]
-        return (torch.cos(angle).contiguous().to(self.rt.device),
-                torch.sin(angle).contiguous().to(self.rt.device))
+        cos, sin = rope_table(self.rotary_dim, self.theta, positions)
+        return cos.to(self.rt.device), sin.to(self.rt.device)
 
     def ensure_positions(self, n: int) -> None:
         """Grow the table if a request runs past what it was sized for."""

@@ -90,6 +90,15 @@ def qk_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return rms_norm(x, weight, eps)
 
 
+def prepare_heads(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, cos, sin) -> torch.Tensor:
+    """What a query or key head goes through before the scores: per-head norm first, rotation second.
+
+    Host statement infer/src/ops/tests.rs:1164-1212 (`apply_rope(&rms_norm(head, weight))` at :1202 and :1210);
+    infer/src/model/qwen3/prefill.rs:669-690 (norm and rotation in one kernel, in this order).
+    """
+    return apply_rope(qk_norm(x, norm_weight, eps), cos, sin)
+
+
 def causal_attention(q, k, v, num_kv_heads: int, window: int | None = None) -> torch.Tensor:
     """softmax(q k^T / sqrt(D) + causal mask) v with grouped heads.
 
@@ -140,11 +149,9 @@ def attention_block(x, w, prefix, cfg, positions):
     q = linear(x, w[prefix + "self_attn.q_proj.weight"]).reshape(T, nq, D)
     k = linear(x, w[prefix + "self_attn.k_proj.weight"]).reshape(T, nkv, D)
     v = linear(x, w[prefix + "self_attn.v_proj.weight"]).reshape(T, nkv, D)
-    q = qk_norm(q, w[prefix + "self_attn.q_norm.weight"], eps)
-    k = qk_norm(k, w[prefix + "self_attn.k_norm.weight"], eps)
     cos, sin = rope_cos_sin(positions, D, cfg["rope_theta"], dtype=x.dtype)
-    q = apply_rope(q, cos, sin)
-    k = apply_rope(k, cos, sin)
+    q = prepare_heads(q, w[prefix + "self_attn.q_norm.weight"], eps, cos, sin)
+    k = prepare_heads(k, w[prefix + "self_attn.k_norm.weight"], eps, cos, sin)
     a = causal_attention(q, k, v, nkv).reshape(T, nq * D)
     return linear(a, w[prefix + "self_attn.o_proj.weight"])
 

@@ -160,19 +160,111 @@ def test_model_shift_of_all_positions_changes_nothing():
     assert torch.allclose(a, b, atol=1e-4)
 
 
-def test_qk_norm_is_per_head_and_before_rope():
+def test_rope_frequencies_and_one_rotated_pair_are_the_literal_numbers():
+    # The statement of infer/src/ops/tests.rs:1090-1100: inv_freq_i = 1 / theta^(2i/D), angle = pos * inv_freq_i.
+    # D=8, theta=1e4: the exponents are 0, 1/4, 1/2, 3/4, so the frequencies are powers of ten.  theta^(-i/D)
+    # (half the exponent) would give 1, 0.316, 0.1, 0.0316; 2i/(D/2) would give 1, 0.01, ...
+    from arle_amd.parts.position import rope_table
+
+    literal = torch.tensor([1.0, 0.1, 0.01, 0.001])
+    assert torch.allclose(plain.rope_inv_freq(8, 1e4), literal, rtol=1e-6)
+    # theta=1e6, D=128 (the checkpoints' values): 10^(-6*2i/128), written out
+    inv = plain.rope_inv_freq(128, 1e6)
+    assert abs(float(inv[1]) / 0.8058421877614819 - 1) < 1e-6      # 10^-0.09375
+    assert abs(float(inv[63]) / 1.2409377607517196e-06 - 1) < 1e-5  # 10^-5.90625
+    # the engine's table holds the same angles: cos/sin(pos * inv_freq_i) at pos 7, i = 1 and 63
+    cos, sin = rope_table(128, 1e6, 8)
+    pcos, psin = plain.rope_cos_sin(range(8), 128, 1e6)
+    for i, angle in ((1, 7 * 0.8058421877614819), (63, 7 * 1.2409377607517196e-06)):
+        for table_c, table_s in ((cos, sin), (pcos, psin)):
+            assert abs(float(table_c[7, i]) - math.cos(angle)) < 1e-6
+            assert abs(float(table_s[7, i]) - math.sin(angle)) < 1e-6
+    ecos, esin = rope_table(8, 1e4, 4)
+    assert torch.allclose(torch.atan2(esin[1], ecos[1]), literal, rtol=1e-5)   # pos 1: the angles are inv_freq
+    # one pair rotated by hand at pos=3, i=1 of D=8: angle 0.3; x_1 = 1, x_5 = 2
+    #   out_1 = cos(0.3) - 2 sin(0.3) = 0.364296075,  out_5 = sin(0.3) + 2 cos(0.3) = 2.206193185
+    x = torch.zeros(1, 1, 8)
+    x[0, 0, 1], x[0, 0, 5] = 1.0, 2.0
+    for c, s in (plain.rope_cos_sin([3], 8, 1e4), (ecos[3:4], esin[3:4])):
+        y = plain.apply_rope(x, c, s)
+        assert abs(float(y[0, 0, 1]) - 0.364296075) < 1e-6 and abs(float(y[0, 0, 5]) - 2.206193185) < 1e-6
+        assert torch.count_nonzero(y[0, 0, [0, 2, 3, 4, 6, 7]]) == 0
+
+
+def test_scaling_a_query_heads_projection_changes_nothing():
+    # the per-head norm removes a head's scale (eps aside): it is per head, and it is there
     cfg = dict(TINY_A, num_hidden_layers=1)
     w = _random_weights(cfg, 5)
     p = "model.layers.0."
     x = torch.randn(6, cfg["hidden_size"], dtype=torch.float64)
     w64 = {k: t.double() for k, t in w.items()}
     base = plain.attention_block(x, w64, p, cfg, list(range(6)))
-    # scaling one q head's projection rows changes nothing: its norm removes the scale (eps aside)
     w_scaled = dict(w64)
     wq = w64[p + "self_attn.q_proj.weight"].clone()
     wq[:16] *= 7.0
     w_scaled[p + "self_attn.q_proj.weight"] = wq
     assert torch.allclose(plain.attention_block(x, w_scaled, p, cfg, list(range(6))), base, atol=1e-6)
+    # ... and scaling one head does change the others' share if the norm ran over all heads at once
+    wq2 = w64[p + "self_attn.q_proj.weight"].clone()
+    wq2[:16] *= 7.0
+    q = (x @ wq2.T).reshape(6, 4, 16)
+    over_all = plain.rms_norm(q.reshape(6, 64), torch.ones(64, dtype=torch.float64), 1e-6).reshape(6, 4, 16)
+    assert not torch.allclose(over_all[:, 1], plain.qk_norm(q, torch.ones(16, dtype=torch.float64), 1e-6)[:, 1],
+                              atol=1e-3)
+
+
+def test_qk_norm_comes_before_the_rotation():
+    # Host statement infer/src/ops/tests.rs:1164-1212, with its own weights (0.9 + (i % 13) * 0.03, :1083-1085)
+    # and head (:1074-1076): norm with a weight that differs between i and i + D/2, then the rotation.  With the
+    # order swapped the pair (i, i + D/2) would be mixed before its two different weights apply.
+    D, half, eps, pos, theta = 32, 16, 1e-6, 5, 1e6
+    head = [((i % 19) - 9.0) * 0.25 for i in range(D)]
+    weight = [0.9 + (i % 13) * 0.03 for i in range(D)]
+    assert weight[3] != weight[3 + half]
+    inv_freq = [1.0 / theta ** (i * 2.0 / D) for i in range(half)]
+
+    def norm(h, wt):
+        inv = 1.0 / math.sqrt(sum(v * v for v in h) / len(h) + eps)
+        return [v * inv * g for v, g in zip(h, wt)]
+
+    def rotate(h):
+        out = [0.0] * D
+        for i in range(half):
+            c, s = math.cos(pos * inv_freq[i]), math.sin(pos * inv_freq[i])
+            out[i] = h[i] * c - h[i + half] * s
+            out[i + half] = h[i] * s + h[i + half] * c
+        return out
+
+    norm_then_rope = torch.tensor(rotate(norm(head, weight)), dtype=torch.float64)
+    rope_then_norm = torch.tensor(norm(rotate(head), weight), dtype=torch.float64)
+    assert (norm_then_rope - rope_then_norm).abs().max() > 0.05     # the two orders are far apart here
+    cos, sin = plain.rope_cos_sin([pos], D, theta, dtype=torch.float64)
+    got = plain.prepare_heads(torch.tensor(head, dtype=torch.float64).reshape(1, 1, D),
+                              torch.tensor(weight, dtype=torch.float64), eps, cos, sin)[0, 0]
+    assert torch.allclose(got, norm_then_rope, atol=1e-6)
+    # the whole attention part uses that preparation: with v = identity-like weights its output moves when
+    # the norm weights of the two halves are exchanged (a rotation-first order would not care which half)
+    cfg = dict(TINY_A, num_hidden_layers=1)
+    w = {k: t.double() for k, t in _random_weights(cfg, 6, std=0.3).items()}
+    p = "model.layers.0."
+    w[p + "self_attn.q_norm.weight"] = torch.tensor([0.9 + (i % 13) * 0.03 for i in range(16)], dtype=torch.float64)
+    x = torch.randn(6, cfg["hidden_size"], dtype=torch.float64)
+    T, nq, nkv, Dh = 6, 4, 2, 16
+    q = plain.linear(x, w[p + "self_attn.q_proj.weight"]).reshape(T, nq, Dh)
+    k = plain.linear(x, w[p + "self_attn.k_proj.weight"]).reshape(T, nkv, Dh)
+    v = plain.linear(x, w[p + "self_attn.v_proj.weight"]).reshape(T, nkv, Dh)
+    c, s = plain.rope_cos_sin(range(T), Dh, cfg["rope_theta"], dtype=torch.float64)
+    by_hand = plain.linear(plain.causal_attention(
+        plain.apply_rope(plain.rms_norm(q, w[p + "self_attn.q_norm.weight"], cfg["rms_norm_eps"]), c, s),
+        plain.apply_rope(plain.rms_norm(k, w[p + "self_attn.k_norm.weight"], cfg["rms_norm_eps"]), c, s),
+        v, nkv).reshape(T, nq * Dh), w[p + "self_attn.o_proj.weight"])
+    swapped = plain.linear(plain.causal_attention(
+        plain.rms_norm(plain.apply_rope(q, c, s), w[p + "self_attn.q_norm.weight"], cfg["rms_norm_eps"]),
+        plain.rms_norm(plain.apply_rope(k, c, s), w[p + "self_attn.k_norm.weight"], cfg["rms_norm_eps"]),
+        v, nkv).reshape(T, nq * Dh), w[p + "self_attn.o_proj.weight"])
+    block = plain.attention_block(x, w, p, cfg, list(range(T)))
+    assert torch.allclose(block, by_hand, atol=1e-9)
+    assert (block - swapped).abs().max() > 1e-3
 
 
 def test_sampling_vectors_of_the_reference():
