@@ -3,8 +3,11 @@
 A folder holds `model.safetensors`, or `model.safetensors.index.json` whose `weight_map`
 names the shard of every tensor (infer/src/weight_loader.rs:27-84,102-120).  The model's
 spec says which tensors it needs and with which shapes; the loader compares that list with
-what the files hold and raises a single `WeightsError` listing missing tensors, unexpected
-tensors and wrong shapes.
+what the files hold and raises a single `WeightsError` listing missing tensors, wrong shapes
+and the tensors the model does not know.  Tensors the model does not know are not an error
+by themselves: the reference reads by name and never looks at the rest (a tied checkpoint
+that still stores lm_head.weight loads there: infer/src/model/qwen3/weights.rs:305-316), so
+they are reported in a warning and left in the file; `strict=True` makes them fatal.
 
 Element types: in the bfloat16 engine a tensor keeps the type it is stored in -- bfloat16
 stays bfloat16, a tensor stored in 32 bits stays float32 (float16 is widened to float32),
@@ -15,6 +18,7 @@ from __future__ import annotations
 
 import json
 import os
+import warnings
 
 import torch
 
@@ -86,14 +90,19 @@ def _engine_dtype(stored: torch.dtype, act_dtype: torch.dtype) -> torch.dtype:
     return torch.bfloat16 if stored == torch.bfloat16 else torch.float32
 
 
-def compare_with_expected(found: dict, expected: dict) -> None:
-    """found: name -> shape; expected: name -> WeightDecl.  Raises one WeightsError or returns."""
+class UnexpectedTensors(UserWarning):
+    """The checkpoint holds tensors the model does not read; they are ignored."""
+
+
+def compare_with_expected(found: dict, expected: dict, strict: bool = False) -> list:
+    """found: name -> shape; expected: name -> WeightDecl.  Raises one WeightsError, or returns the
+    names the model does not know (never fatal alone unless `strict`)."""
     missing = sorted(n for n in expected if n not in found)
     unexpected = sorted(n for n in found if n not in expected)
     wrong = sorted((n, tuple(expected[n].shape), tuple(found[n])) for n in expected
                    if n in found and tuple(found[n]) != tuple(expected[n].shape))
-    if not (missing or unexpected or wrong):
-        return
+    if not (missing or wrong or (strict and unexpected)):
+        return unexpected
     lines = ["checkpoint does not match the model:"]
     if missing:
         lines.append(f"  missing tensors ({len(missing)}): " + ", ".join(missing))
@@ -105,11 +114,15 @@ def compare_with_expected(found: dict, expected: dict) -> None:
     raise WeightsError("\n".join(lines), missing, unexpected, wrong)
 
 
-def load_weights(model_dir: str, expected: dict, device, act_dtype: torch.dtype) -> dict:
+def load_weights(model_dir: str, expected: dict, device, act_dtype: torch.dtype, strict: bool = False) -> dict:
     """name -> tensor on `device` for every expected tensor, or one WeightsError."""
     ckpt = Checkpoint(model_dir)
     try:
-        compare_with_expected({n: ckpt.info(n)[1] for n in ckpt.names()}, expected)
+        ignored = compare_with_expected({n: ckpt.info(n)[1] for n in ckpt.names()}, expected, strict)
+        if ignored:
+            shown = ", ".join(ignored[:8]) + (f", ... ({len(ignored)} in all)" if len(ignored) > 8 else "")
+            warnings.warn(f"{model_dir}: ignoring tensors the model does not read: {shown}", UnexpectedTensors,
+                          stacklevel=2)
         out = {}
         for name in expected:
             t = ckpt.read(name)

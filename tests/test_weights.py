@@ -41,6 +41,26 @@ def test_written_file_is_read_by_the_safetensors_package(tmp_path):
     assert all(torch.equal(back[k], v) for k, v in tensors.items())
 
 
+def test_file_written_by_the_safetensors_package_is_read_by_the_own_reader(tmp_path):
+    # what real checkpoints are: the package's writer (its own key order, padding of the header, alignment)
+    st = pytest.importorskip("safetensors.torch")
+    g = torch.Generator().manual_seed(3)
+    tensors = {"model.embed_tokens.weight": torch.randn(37, 24, generator=g).bfloat16(),
+               "z.norm": torch.randn(24, generator=g), "a.half": torch.randn(5, 3, generator=g).half(),
+               "ids": torch.arange(11, dtype=torch.int64), "scalar": torch.tensor(2.5),
+               "empty": torch.zeros(0, 4), "b.i32": torch.arange(6, dtype=torch.int32).reshape(2, 3),
+               "flags": torch.tensor([1, 0, 255], dtype=torch.uint8)}
+    path = str(tmp_path / "pkg.safetensors")
+    st.save_file(tensors, path, metadata={"format": "pt"})
+    f = SafetensorsFile(path)
+    assert sorted(f.names()) == sorted(tensors) and f.metadata == {"format": "pt"}
+    for name, t in tensors.items():
+        dtype, shape = f.info(name)
+        got = f.read(name)
+        assert tuple(shape) == tuple(t.shape) and got.dtype == t.dtype and torch.equal(got, t), name
+    f.close()
+
+
 def test_data_length_mismatch_names_the_tensor(tmp_path):
     path = str(tmp_path / "bad.safetensors")
     header = json.dumps({"w": {"dtype": "BF16", "shape": [2, 3], "data_offsets": [0, 8]}}).encode()
@@ -109,6 +129,31 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     text = str(err)
     for needle in ("lm_head.weight", "q_proj.bias", "expected [32], found [16]"):
         assert needle in text
+
+
+def test_tensors_the_model_does_not_know_are_ignored_with_a_warning(tmp_path):
+    # a tied checkpoint that still stores lm_head.weight loads in the reference (it reads by name:
+    # infer/src/model/qwen3/weights.rs:305-316, infer/src/weight_loader.rs:102-120) and must load here
+    from arle_amd.weights.loader import UnexpectedTensors
+
+    cfg = Qwen3Config.from_dict(TINY_A)
+    assert cfg.tie_word_embeddings
+    d = write_random_model(str(tmp_path / "m"), ARCH, cfg, seed=4)
+    path = os.path.join(d, "model.safetensors")
+    f = SafetensorsFile(path)
+    tensors = {n: f.read(n) for n in f.names()}
+    f.close()
+    tensors["lm_head.weight"] = tensors["model.embed_tokens.weight"].clone()
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.ones(8)
+    write_safetensors(path, tensors)
+    expected = expected_checkpoint_tensors(_spec(TINY_A))
+    with pytest.warns(UnexpectedTensors, match="lm_head.weight"):
+        w = load_weights(d, expected, "cpu", torch.bfloat16)
+    assert set(w) == set(expected) and "lm_head.weight" not in w
+    with pytest.raises(WeightsError) as info:
+        load_weights(d, expected, "cpu", torch.bfloat16, strict=True)
+    assert info.value.unexpected == ["lm_head.weight", "model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert not info.value.missing and not info.value.wrong_shape
 
 
 def test_sharded_folder_with_index(tmp_path):

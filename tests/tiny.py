@@ -13,7 +13,7 @@ import os
 import torch
 
 from arle_amd.config import Qwen3Config
-from arle_amd.weights import SafetensorsFile, write_random_model
+from arle_amd.weights import write_random_model
 
 ARCH = "Qwen3ForCausalLM"
 
@@ -55,12 +55,13 @@ def make_model_dir(tmp_path, name: str, std_scale: float = 1.0) -> str:
 
 
 def read_folder(model_dir: str):
-    """(config dict, {name: float32 CPU tensor}) read straight from the files."""
+    """(config dict, {name: float32 CPU tensor}) read straight from the files, with the `safetensors`
+    package's reader: the plain side shares no reader with the engine."""
+    from safetensors.torch import load_file
+
     with open(os.path.join(model_dir, "config.json")) as fh:
         cfg = json.load(fh)
-    f = SafetensorsFile(os.path.join(model_dir, "model.safetensors"))
-    weights = {n: f.read(n).to(torch.float32) for n in f.names()}
-    f.close()
+    weights = {n: t.to(torch.float32) for n, t in load_file(os.path.join(model_dir, "model.safetensors")).items()}
     return cfg, weights
 
 
