@@ -29,6 +29,10 @@
 // with exp2; probabilities are narrowed to bfloat16 before the second product, as the
 // reference does (batch_prefill_paged_hd128.py:219-225); the sum l uses the 32-bit values.
 #include "common.h"
+#include "attention_static.h"
+
+#include <cstdio>
+#include <mutex>
 
 namespace arle {
 
@@ -1440,6 +1444,40 @@ extern "C" int arle_attn_ws_rows(int max_qlen, int nq, int nkv) {
   return max(1, min(max_qlen, 16 / max(G, 1)));
 }
 
+static AttnArgs make_args(const void* q, long long q_stride, void* out, long long o_stride, const void* k_pages,
+                          const void* v_pages, const int* block_table, int table_stride, const int* seg_row0,
+                          const int* seg_slot, const int* seg_start, int max_qlen, int nq, int nkv, int D,
+                          int page_size, float scale, int window, int splits, float* ws_o, float* ws_ml) {
+  AttnArgs a;
+  a.q = static_cast<const uint16_t*>(q);
+  a.q_stride = q_stride;
+  a.out = static_cast<uint16_t*>(out);
+  a.o_stride = o_stride;
+  a.ws_o = ws_o;
+  a.ws_ml = ws_ml;
+  a.k_pages = static_cast<const uint16_t*>(k_pages);
+  a.v_pages = static_cast<const uint16_t*>(v_pages);
+  a.block_table = block_table;
+  a.table_stride = table_stride;
+  a.seg_row0 = seg_row0;
+  a.seg_slot = seg_slot;
+  a.seg_start = seg_start;
+  a.nq = nq;
+  a.nkv = nkv;
+  a.D = D;
+  a.P = page_size;
+  a.p_shift = __builtin_ctz(static_cast<unsigned>(page_size));
+  a.scale_log2 = scale * 1.4426950408889634f;
+  a.window = window;
+  a.splits = splits;
+  a.ws_rows = arle_attn_ws_rows(max_qlen, nq, nkv);
+  a.portion_splits = 1;
+  a.pws_o = nullptr;
+  a.pws_ml = nullptr;
+  a.rows_max = 0;
+  return a;
+}
+
 // q, out: bfloat16 [token rows, nq*D] (row strides in elements).  Segments describe the packed
 // step: seg_row0[s]..seg_row0[s+1] are the token rows of segment s, whose first token sits at
 // position seg_start[s] of the request in block-table row seg_slot[s]; the cache already holds
@@ -1465,33 +1503,11 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
       (portion_splits > 1 && (pws_o == nullptr || pws_ml == nullptr)))
     return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  AttnArgs a;
-  a.q = static_cast<const uint16_t*>(q);
-  a.q_stride = q_stride;
-  a.out = static_cast<uint16_t*>(out);
-  a.o_stride = o_stride;
-  a.ws_o = ws_o;
-  a.ws_ml = ws_ml;
-  a.k_pages = static_cast<const uint16_t*>(k_pages);
-  a.v_pages = static_cast<const uint16_t*>(v_pages);
-  a.block_table = block_table;
-  a.table_stride = table_stride;
-  a.seg_row0 = seg_row0;
-  a.seg_slot = seg_slot;
-  a.seg_start = seg_start;
-  a.nq = nq;
-  a.nkv = nkv;
-  a.D = D;
-  a.P = page_size;
-  a.p_shift = __builtin_ctz(static_cast<unsigned>(page_size));
-  a.scale_log2 = scale * 1.4426950408889634f;
-  a.window = window;
-  a.splits = splits;
-  a.ws_rows = arle_attn_ws_rows(max_qlen, nq, nkv);
+  AttnArgs a = make_args(q, q_stride, out, o_stride, k_pages, v_pages, block_table, table_stride, seg_row0, seg_slot,
+                         seg_start, max_qlen, nq, nkv, D, page_size, scale, window, splits, ws_o, ws_ml);
   a.portion_splits = portion_splits;
   a.pws_o = pws_o;
   a.pws_ml = pws_ml;
-  a.rows_max = 0;
   const int G = nq / nkv;
   const int max_rows = max_qlen * G, min_rows = min_qlen * G;
   const long long z = static_cast<long long>(segments) * splits;
@@ -1528,6 +1544,89 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
   const int nt = max_rows <= 16 ? 1 : 2;
   dim3 grid((max_rows + 16 * nt - 1) / (16 * nt), nkv, static_cast<unsigned>(z));
   rc = nt == 1 ? launch_attn<1>(a, grid, s) : launch_attn<2>(a, grid, s);
+  if (rc != 0 || splits == 1) return rc;
+  attn_merge_kernel<<<dim3(segments * a.ws_rows, nq), kMergeWaves * kWave, 0, s>>>(
+      ws_o, ws_ml, a.out, o_stride, seg_row0, a.ws_rows, 0, nq, nkv, D, splits);
+  return launch_status();
+}
+
+// ---- the entry point that allocates nothing (attention_static.h) ---------------------------------------------
+//
+// The split-KV partial results live in this array.  In host code its name is only a handle for
+// hipGetSymbolAddress: each GPU holds its own copy at its own address, looked up once per device below, and
+// host code uses that address wherever it needs the memory.
+static __device__ __align__(256) float scratch[kAttnStaticOFloats + kAttnStaticMlFloats];
+
+namespace {
+constexpr int kStaticDevicesMax = 64;
+float* g_static_ptr[kStaticDevicesMax];   // per device: where its copy of `scratch` lies
+std::mutex g_static_lock;
+thread_local char g_static_error[256] = "";
+
+int static_refuse(const char* what, long long got, long long most) {
+  std::snprintf(g_static_error, sizeof(g_static_error), "arle_attn_decode_static: %s %lld exceeds the maximum %lld",
+                what, got, most);
+  return static_cast<int>(hipErrorInvalidValue);
+}
+
+// The current device's address of `scratch` (looked up at the first call on that device, with it current).
+int static_scratch(float** ptr) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (dev < 0 || dev >= kStaticDevicesMax) return static_cast<int>(hipErrorInvalidDevice);
+  std::lock_guard<std::mutex> guard(g_static_lock);
+  if (g_static_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (p == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
+    g_static_ptr[dev] = static_cast<float*>(p);
+  }
+  *ptr = g_static_ptr[dev];
+  return 0;
+}
+}  // namespace
+
+extern "C" const char* arle_attn_decode_static_error() { return g_static_error; }
+
+extern "C" int arle_attn_decode_static(const void* q, long long q_stride, void* out, long long o_stride,
+                                       const void* k_pages, const void* v_pages, const int* block_table,
+                                       int table_stride, const int* seg_row0, const int* seg_slot,
+                                       const int* seg_start, int segments, int max_qlen, int nq, int nkv, int D,
+                                       int page_size, float scale, int window, int splits, void* stream) {
+  g_static_error[0] = 0;
+  if (segments == 0) return 0;
+  if (segments < 0 || max_qlen < 1 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || D % 16 != 0 || D > 256 || D <= 0 ||
+      page_size < 4 || (page_size & (page_size - 1)) != 0 || splits < 1 || splits > 64) {
+    std::snprintf(g_static_error, sizeof(g_static_error),
+                  "arle_attn_decode_static: needs head_dim %% 16 == 0 and <= 256, a power-of-two page size >= 4, "
+                  "q heads a multiple of kv heads and 1..64 splits");
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  const int G = nq / nkv;
+  if (static_cast<long long>(max_qlen) * G > 16) return static_refuse("rows of a segment (tokens x group)", static_cast<long long>(max_qlen) * G, 16);
+  const long long z = static_cast<long long>(segments) * splits;
+  if (nkv > 65535) return static_refuse("kv heads", nkv, 65535);
+  if (z > 65535) return static_refuse("segments x splits", z, 65535);
+  const long long entries = static_cast<long long>(segments) * arle_attn_ws_rows(max_qlen, nq, nkv) * nq * splits;
+  float* ws = nullptr;
+  if (splits > 1) {
+    if (entries * D > kAttnStaticOFloats) return static_refuse("partial outputs (floats)", entries * D, kAttnStaticOFloats);
+    if (entries * 2 > kAttnStaticMlFloats) return static_refuse("partial statistics (floats)", entries * 2, kAttnStaticMlFloats);
+    const int rc = static_scratch(&ws);
+    if (rc != 0) {
+      std::snprintf(g_static_error, sizeof(g_static_error),
+                    "arle_attn_decode_static: the device address of the scratch array could not be found (HIP error %d)", rc);
+      return rc;
+    }
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* ws_o = ws;
+  float* ws_ml = ws != nullptr ? ws + kAttnStaticOFloats : nullptr;
+  AttnArgs a = make_args(q, q_stride, out, o_stride, k_pages, v_pages, block_table, table_stride, seg_row0, seg_slot,
+                         seg_start, max_qlen, nq, nkv, D, page_size, scale, window, splits, ws_o, ws_ml);
+  int rc = launch_attn<1>(a, dim3(1, nkv, static_cast<unsigned>(z)), s);
   if (rc != 0 || splits == 1) return rc;
   attn_merge_kernel<<<dim3(segments * a.ws_rows, nq), kMergeWaves * kWave, 0, s>>>(
       ws_o, ws_ml, a.out, o_stride, seg_row0, a.ws_rows, 0, nq, nkv, D, splits);

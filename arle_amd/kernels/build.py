@@ -36,7 +36,7 @@ SOURCES = {
     "ceilings": "ceilings.hip",
     "host": "host/runtime.cpp",
 }
-HEADERS = ("common.h",)
+HEADERS = ("common.h", "attention_static.h")
 HOST_LIBS = ("host",)   # plain C++: page pool, block tables, step packing
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared"]
 
