@@ -1,11 +1,15 @@
 """The cache manager: paged keys/values per group of layers, and fixed-size state slots.
 
 Every schedule entry of a model that owns a cache declares its need:
-`PagedNeed` (keys and values per token: attention, possibly windowed) or `StateNeed`
-(a block of fixed size per request: recurrent or convolutional state).  Entries with
-equal paged needs form a group with one page-id space, one block table per request
-and one pair of buffers `[entries, pages, kv_heads, page_size, head_dim]`.  State needs
-get `[slots, *shape]` buffers, zeroed when a slot is assigned.  A request holds one
+`PagedNeed` (tensors that grow by one slot per token: attention, possibly windowed) or
+`StateNeed` (a block of fixed size per request: recurrent or convolutional state).  A paged
+need lists its own tensors (`PageTensor`: a name, the shape of one page with the token axis
+marked, an element type): keys and values `[kv_heads, page, head_dim]` / `[kv_heads, head_dim,
+page]` unless it says otherwise, so a mixer that caches one compressed vector per token, or
+keeps its cache in another type than the activations, declares that and nothing here
+changes.  Entries with equal paged needs form a group with one page-id space, one block
+table per request and one buffer `[entries, pages, *page shape]` per declared tensor.  State
+needs get `[slots, *shape]` buffers, zeroed when a slot is assigned.  A request holds one
 slot for its life; the slot is its row in every block table and state buffer.
 
 The bookkeeping is host-side and works without a GPU (`device=None`), which is how the
@@ -22,11 +26,52 @@ import torch
 from .pages import FREED, OutOfPages, PageGroup
 
 
+PAGE = "page"   # stands for the token axis (length page_size) in the shape of a PageTensor
+
+
+@dataclass(frozen=True)
+class PageTensor:
+    """One tensor of a paged need: `shape` is that of one page, with PAGE where the tokens of the page go."""
+
+    name: str
+    shape: tuple
+    dtype: torch.dtype | None = None   # None: the engine's activation type
+
+    def page_shape(self, page_size: int) -> tuple:
+        if sum(1 for d in self.shape if d == PAGE) != 1:
+            raise ValueError(f"page tensor {self.name!r}: the shape must hold the token axis PAGE exactly once")
+        return tuple(page_size if d == PAGE else int(d) for d in self.shape)
+
+    def bytes_per_token(self, act_dtype: torch.dtype) -> int:
+        n = 1
+        for d in self.page_shape(1):
+            n *= d
+        return n * torch.empty((), dtype=self.dtype or act_dtype).element_size()
+
+
 @dataclass(frozen=True)
 class PagedNeed:
-    num_kv_heads: int
-    head_dim: int
-    window: int | None = None  # None: every earlier key is kept
+    """Keys and values of num_kv_heads x head_dim per token, or the `tensors` the mixer lists itself."""
+
+    num_kv_heads: int = 0
+    head_dim: int = 0
+    window: int | None = None  # None: every earlier token is kept
+    tensors: tuple = ()        # of PageTensor; empty: "k" [kv_heads, PAGE, head_dim] and "v" [kv_heads, head_dim, PAGE]
+
+    def page_tensors(self) -> tuple:
+        if self.tensors:
+            names = [t.name for t in self.tensors]
+            if len(set(names)) != len(names):
+                raise ValueError(f"a paged need names a tensor twice: {names}")
+            return tuple(self.tensors)
+        if self.num_kv_heads <= 0 or self.head_dim <= 0:
+            raise ValueError("a paged need gives num_kv_heads and head_dim, or its own tensors")
+        # keys [.., slot in page, d]; values d-major inside a page [.., d, slot in page]
+        return (PageTensor("k", (self.num_kv_heads, PAGE, self.head_dim)),
+                PageTensor("v", (self.num_kv_heads, self.head_dim, PAGE)))
+
+    def bytes_per_token(self, act_dtype: torch.dtype) -> int:
+        return sum(t.bytes_per_token(act_dtype) for t in self.page_tensors())
 
 
 @dataclass(frozen=True)
@@ -34,17 +79,58 @@ class StateNeed:
     shape: tuple
     dtype: torch.dtype = torch.float32
 
+    def bytes_per_slot(self) -> int:
+        n = 1
+        for d in self.shape:
+            n *= int(d)
+        return n * torch.empty((), dtype=self.dtype).element_size()
+
+
+def cache_bytes_per_token(needs, act_dtype: torch.dtype) -> int:
+    """Bytes one token takes over every schedule entry that owns a paged cache.  For keys and values of every
+    layer this is the reference's 2 * layers * kv_heads * head_dim * element size
+    (infer/src/model/qwen3/forward.rs:777-783)."""
+    return sum(n.bytes_per_token(act_dtype) for n in needs if isinstance(n, PagedNeed))
+
+
+def state_bytes_per_slot(needs) -> int:
+    return sum(n.bytes_per_slot() for n in needs if isinstance(n, StateNeed))
+
+
+def pages_for_memory(free_bytes: int, total_bytes: int, mem_fraction_static: float, bytes_per_page: int,
+                     reserved_bytes: int = 0, most_pages: int | None = None) -> int:
+    """Pages of a pool sized from the GPU's memory, as the reference sizes its pool
+    (infer/src/scheduler/cuda/core/construction.rs:131-203): what is free now (the weights are loaded), less a
+    headroom of (1 - mem_fraction_static) of the whole memory for activations and workspaces, less what else is
+    reserved (state slots), divided by a page's bytes over all layers.  `most_pages`: what all slots can hold at
+    their longest; more would never be used, since pages are not shared between requests."""
+    if not 0.0 < mem_fraction_static <= 1.0:
+        raise ValueError("mem_fraction_static must be in (0, 1]")     # infer/src/scheduler/types.rs:407-409
+    if bytes_per_page <= 0:
+        return 0
+    headroom = int(total_bytes * (1.0 - mem_fraction_static))
+    budget = max(0, int(free_bytes) - headroom - int(reserved_bytes))
+    pages = budget // bytes_per_page
+    return int(min(pages, most_pages) if most_pages is not None else pages)
+
 
 @dataclass
 class PagedView:
     """What a mixer sees of its paged cache during a step."""
 
-    k_pages: torch.Tensor | None   # [pages, kv_heads, page_size, head_dim]
-    v_pages: torch.Tensor | None   # [pages, kv_heads, head_dim, page_size]  (d-major inside a page)
+    pages: dict                    # tensor name -> [pages, *page shape]  (None values without a device)
     block_table: torch.Tensor | None  # int32 [slots, max_pages_per_request], shared by the group
     page_size: int
     window: int | None
     writes: bool                   # False for an entry that reads another entry's cache
+
+    @property
+    def k_pages(self):             # [pages, kv_heads, page_size, head_dim]
+        return self.pages["k"]
+
+    @property
+    def v_pages(self):             # [pages, kv_heads, head_dim, page_size]  (d-major inside a page)
+        return self.pages["v"]
 
 
 @dataclass
@@ -99,15 +185,15 @@ class CacheManager:
         self._dirty = [set() for _ in self.groups]
 
         # device buffers
-        self.k_buffers, self.v_buffers, self.tables_dev, self.state_buffers = [], [], [], {}
+        self.page_buffers, self.tables_dev, self.state_buffers = [], [], {}   # page_buffers[g]: name -> tensor
+        for need in self._group_needs:
+            need.page_tensors()     # a need that is not well formed fails here, with or without a device
         if device is not None:
             for g, need in enumerate(self._group_needs):
                 n = len(self._group_entries[g])
-                # keys [.., slot in page, d]; values d-major inside a page [.., d, slot in page]
-                self.k_buffers.append(torch.zeros((n, num_pages, need.num_kv_heads, page_size, need.head_dim),
-                                                  dtype=dtype, device=device))
-                self.v_buffers.append(torch.zeros((n, num_pages, need.num_kv_heads, need.head_dim, page_size),
-                                                  dtype=dtype, device=device))
+                self.page_buffers.append({
+                    t.name: torch.zeros((n, num_pages, *t.page_shape(page_size)), dtype=t.dtype or dtype, device=device)
+                    for t in need.page_tensors()})
                 self.tables_dev.append(torch.zeros((max_slots, self.max_pages_per_request),
                                                    dtype=torch.int32, device=device))
             for entry, need in enumerate(self.needs):
@@ -201,6 +287,22 @@ class CacheManager:
         for group in self.groups:
             group.trim(key)
 
+    # -- state slots across a step that may fail ----------------------------------------
+    def snapshot_state(self, keys):
+        """A copy of the state blocks of these requests, to be handed to `restore_state` if the step that is
+        about to overwrite them fails; None when no entry keeps state.  [requests of the step, *shape] each."""
+        if not self.state_buffers:
+            return None
+        rows = torch.tensor([self.slot_of[k] for k in keys], dtype=torch.long, device=self.device)
+        return rows, {entry: buf.index_select(0, rows) for entry, buf in self.state_buffers.items()}
+
+    def restore_state(self, snapshot) -> None:
+        if snapshot is None:
+            return
+        rows, saved = snapshot
+        for entry, values in saved.items():
+            self.state_buffers[entry].index_copy_(0, rows, values)
+
     # -- views for the step -----------------------------------------------------------
     def sync_tables(self) -> None:
         """Copy block-table rows that changed since the last call to the GPU."""
@@ -221,13 +323,15 @@ class CacheManager:
         if isinstance(need, PagedNeed):
             g, idx = self._entry_place[owner]
             has = self.device is not None
-            return PagedView(k_pages=self.k_buffers[g][idx] if has else None,
-                             v_pages=self.v_buffers[g][idx] if has else None,
-                             block_table=self.tables_dev[g] if has else None,
+            pages = {t.name: (self.page_buffers[g][t.name][idx] if has else None) for t in need.page_tensors()}
+            return PagedView(pages=pages, block_table=self.tables_dev[g] if has else None,
                              page_size=self.page_size, window=need.window, writes=owner == entry)
         if isinstance(need, StateNeed):
             return StateView(state=self.state_buffers.get(owner))
         return None
+
+    def bytes_per_token(self) -> int:
+        return cache_bytes_per_token(self.needs, self.dtype)
 
     def table_of(self, key, group: int = 0) -> list:
         return list(self.groups[group].tables[key].pages)
@@ -249,5 +353,5 @@ class CacheManager:
                     raise AssertionError(f"a group disagrees on the length of {k!r}")
 
 
-__all__ = ["CacheManager", "PagedNeed", "StateNeed", "PagedView", "StateView", "OutOfPages",
-           "NoFreeSlot", "FREED"]
+__all__ = ["CacheManager", "PagedNeed", "PageTensor", "PAGE", "StateNeed", "PagedView", "StateView", "OutOfPages",
+           "NoFreeSlot", "FREED", "cache_bytes_per_token", "state_bytes_per_slot", "pages_for_memory"]

@@ -6,7 +6,8 @@ Global options and `run` follow crates/cli/src/args.rs:188-302: `--model-path`, 
 (0 or `auto`: the model's max_position_embeddings, crates/cli/src/lib.rs:240-266), `--temperature`
 (default 0.0 = greedy); `run --prompt/--stdin/--json`.  The engine options carry the names of the
 `infer` binary's flags (infer/src/main.rs:26-236): `--num-slots`, `--max-seq-len`,
-`--chunked-prefill-size`, `--max-num-batched-tokens`, `--max-prefill-tokens`, `--prefill-max-requests`.
+`--chunked-prefill-size`, `--max-num-batched-tokens`, `--max-prefill-tokens`, `--prefill-max-requests`,
+`--mem-fraction-static`.
 After the answer, one summary line goes to stderr: prompt tok/s (= prompt tokens / TTFT), TTFT and
 output tok/s (crates/cli/src/tps.rs:1-60).  `--prompt-ids` is this engine's own: folders written by
 the random-weights mode have no tokenizer.
@@ -46,7 +47,10 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--max-num-batched-tokens", type=int, default=16384)
     ap.add_argument("--max-prefill-tokens", type=int, default=16384)
     ap.add_argument("--prefill-max-requests", type=int, default=None)
-    ap.add_argument("--kv-cache-tokens", type=int, default=None, help="tokens the paged cache holds")
+    ap.add_argument("--kv-cache-tokens", type=int, default=None,
+                    help="tokens the paged cache holds (default: sized from free GPU memory, see --mem-fraction-static)")
+    ap.add_argument("--mem-fraction-static", type=float, default=0.85,
+                    help="share of the GPU's memory that weights and cache may take together; the rest is headroom")
     ap.add_argument("--page-size", type=int, default=None)
     ap.add_argument("--no-cuda-graph", action="store_true",
                     help="launch every step kernel by kernel instead of replaying captured HIP graphs")
@@ -97,6 +101,7 @@ def main(argv=None) -> int:
               max_num_batched_tokens=args.max_num_batched_tokens, max_prefill_tokens=args.max_prefill_tokens,
               prefill_max_requests=args.prefill_max_requests, kv_cache_tokens=args.kv_cache_tokens,
               page_size=args.page_size, seed=args.seed, cuda_graph=not args.no_cuda_graph,
+              mem_fraction_static=args.mem_fraction_static,
               weight_tiles=False if args.no_weight_tiles else None)
     if args.prompt_ids:
         prompt = [int(t) for t in args.prompt_ids.replace(" ", "").split(",") if t]

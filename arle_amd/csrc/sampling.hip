@@ -7,11 +7,13 @@
 // top-k -> renormalise -> top-p -> renormalise -> inverse CDF with a uniform u
 // drawn on the host); penalties infer/src/sampler.rs:100-140.
 //
-// Differences kept on purpose: thresholds are found exactly by bisection on the
-// bit pattern of the (non-negative) probabilities instead of 32 halvings of a
-// float interval, each thread owns a contiguous run of the vocabulary so the
-// inverse CDF walks tokens in index order, and one launch serves many rows with
-// per-row parameters.
+// Differences kept on purpose: the top-k and top-p thresholds are found exactly, eight
+// bits of the bit pattern of the (non-negative) probabilities at a time, from 256-bin
+// histograms filled with integer atomics, instead of 32 halvings of a float interval;
+// each thread owns a contiguous run of the vocabulary so the inverse CDF walks tokens
+// in index order; one launch serves many rows with per-row parameters; and the
+// log-probability of a chosen token (the reference has it for greedy rows only,
+// sampling.cu:252-317) is a kernel of its own that serves greedy and sampled rows.
 #include "common.h"
 
 namespace arle {
@@ -655,6 +657,34 @@ extern "C" int arle_sample_rows(const float* logits, int rows, int vocab, float*
     for (int level = 0; level < 4; ++level) sample_top_p_kernel<<<grid, kSelThreads, 0, s>>>(a, level);
   sample_mass_kernel<<<grid, kSelThreads, 0, s>>>(a);
   sample_pick_kernel<<<rows, kSelThreads, 0, s>>>(a);
+  return launch_status();
+}
+
+// out[r] = logits[r][token[r]] - logsumexp(logits[r]): the natural-log probability of the chosen token under
+// the softmax of the row (for the largest logit this is the reference's -log(sum exp(x - max)),
+// crates/cuda-kernels/csrc/misc/sampling.cu:299-316).  One workgroup a row, fixed order of additions.
+__global__ __launch_bounds__(kSampThreads) void token_logprob_kernel(const float* __restrict__ logits, int vocab,
+                                                                    const int* __restrict__ token,
+                                                                    float* __restrict__ out) {
+  __shared__ float lds[kSampWaves];
+  const float* x = logits + static_cast<int64_t>(blockIdx.x) * vocab;
+  float m = -INFINITY;
+  for (int i = threadIdx.x; i < vocab; i += kSampThreads) m = fmaxf(m, x[i]);
+  m = block_max<kSampWaves>(m, lds);
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < vocab; i += kSampThreads) sum += expf(x[i] - m);
+  sum = block_sum<kSampWaves>(sum, lds);
+  if (threadIdx.x == 0) {
+    const int t = token[blockIdx.x];
+    out[blockIdx.x] = (t >= 0 && t < vocab) ? x[t] - m - logf(sum) : -INFINITY;
+  }
+}
+
+extern "C" int arle_token_logprobs(const float* logits, int rows, int vocab, const int* token, float* out,
+                                   void* stream) {
+  if (rows == 0) return 0;
+  if (vocab <= 0) return static_cast<int>(hipErrorInvalidValue);
+  token_logprob_kernel<<<rows, kSampThreads, 0, static_cast<hipStream_t>(stream)>>>(logits, vocab, token, out);
   return launch_status();
 }
 

@@ -39,7 +39,8 @@ class CompletionOutput:
     prompt_token_ids: list
     response_token_ids: list
     ttft_s: float | None = None   # submit -> first token
-    token_logprobs: list = field(default_factory=list)
+    tpot_s: float | None = None   # mean time per output token after the first
+    token_logprobs: list = field(default_factory=list)   # log-probability of every generated token, if asked for
 
 
 class LLM:
@@ -47,11 +48,13 @@ class LLM:
                  kv_cache_tokens: int | None = None, num_slots: int = 4, max_seq_len: int | None = None,
                  chunked_prefill_size: int = 512, max_num_batched_tokens: int = 16384,
                  max_prefill_tokens: int = 16384, prefill_max_requests: int | None = None, seed: int = 42,
-                 cuda_graph: bool = True, weight_tiles: bool | None = None):
+                 cuda_graph: bool = True, weight_tiles: bool | None = None, mem_fraction_static: float = 0.85):
         """model: a model folder, or an Engine that is already built.
 
-        kv_cache_tokens: tokens the paged cache holds over all live requests
-        (default: num_slots * max_seq_len, max_seq_len defaulting to min(model's positions, 4096)).
+        kv_cache_tokens: tokens the paged cache holds over all live requests.  Default: sized from the GPU's
+        free memory after the weights are loaded, less a headroom of (1 - mem_fraction_static) of its whole
+        memory (the reference's --mem-fraction-static, default 0.85), and never more than num_slots requests
+        of max_seq_len tokens (default: the model's positions) can fill.
         cuda_graph, weight_tiles: as for Engine (captured steps; the decode-friendly second copy of the weights).
         """
         if isinstance(model, Engine):
@@ -63,13 +66,12 @@ class LLM:
 
             _, config, _ = load_model_config(model)
             positions = getattr(config, "max_position_embeddings", 4096)
-            max_seq_len = max_seq_len or min(positions, 4096)
-            kv_cache_tokens = kv_cache_tokens or num_slots * max_seq_len
+            max_seq_len = min(max_seq_len or positions, positions)
             self.engine = Engine.from_folder(model, dtype=dtype, device=device,
                                              page_size=page_size or DEFAULT_PAGE_SIZE,
                                              max_tokens=kv_cache_tokens, max_slots=num_slots,
-                                             max_request_tokens=min(max_seq_len, positions),
-                                             cuda_graph=cuda_graph, weight_tiles=weight_tiles)
+                                             max_request_tokens=max_seq_len, cuda_graph=cuda_graph,
+                                             weight_tiles=weight_tiles, mem_fraction_static=mem_fraction_static)
         self.model_dir = model if isinstance(model, str) else None
         self.seed = seed
         self.sched_config = SchedulerConfig(
@@ -99,15 +101,16 @@ class LLM:
         return self.tokenizer.encode(text).ids
 
     def generate(self, prompts, max_tokens: int = 16, temperature: float = 0.0, seed: int | None = None,
-                 ignore_eos: bool = False, sampling: SamplingParams | None = None) -> list:
+                 ignore_eos: bool = False, sampling: SamplingParams | None = None, logprobs: bool = False) -> list:
         """prompts: a list of token-id lists (or strings, with a tokenizer).  One CompletionOutput each,
-        in order.  `sampling` overrides temperature / seed / ignore_eos when given."""
+        in order.  `sampling` overrides temperature / seed / ignore_eos / logprobs when given."""
         sched = Scheduler(self.engine, self.sampler, self.sched_config, seed=self.seed,
                           stop_token_ids=self.engine.spec.stop_token_ids)
         ids = []
         for p in prompts:
             toks = self.tokenize(p) if isinstance(p, str) else list(p)
-            params = sampling or SamplingParams(temperature=temperature, seed=seed, ignore_eos=ignore_eos)
+            params = sampling or SamplingParams(temperature=temperature, seed=seed, ignore_eos=ignore_eos,
+                                                logprobs=logprobs)
             ids.append(sched.submit(toks, params, max_tokens))
         sched.run_until_done()
         self.last_stats = sched.stats
@@ -116,10 +119,12 @@ class LLM:
             r = sched.finished[rid]
             text = self.tokenizer.decode(r.generated) if self.tokenizer is not None else None
             ttft = (r.t_first_token - r.t_submit) if r.t_first_token is not None else None
+            tpot = ((r.t_tokens[-1] - r.t_tokens[0]) / (len(r.t_tokens) - 1)) if len(r.t_tokens) > 1 else None
             outs.append(CompletionOutput(text=text, finish_reason=r.finish_reason,
                                          usage=TokenUsage(len(r.prompt), len(r.generated)),
                                          prompt_token_ids=list(r.prompt),
-                                         response_token_ids=list(r.generated), ttft_s=ttft))
+                                         response_token_ids=list(r.generated), ttft_s=ttft, tpot_s=tpot,
+                                         token_logprobs=list(r.logprobs)))
         return outs
 
 

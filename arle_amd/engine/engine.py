@@ -13,7 +13,8 @@ from __future__ import annotations
 import torch
 
 from .. import models  # noqa: F401  (registers the architectures)
-from ..cache.manager import CacheManager
+from ..cache.manager import (CacheManager, PagedNeed, cache_bytes_per_token, pages_for_memory,
+                             state_bytes_per_slot)
 from ..config.registry import detect_architecture, load_model_config
 from ..models.decoder import build_model, expected_checkpoint_tensors
 from ..parts.base import Runtime
@@ -25,6 +26,7 @@ from .batch import StepEntry, build_step_batch, packed_size
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
           "fp32": torch.float32}
 DEFAULT_PAGE_SIZE = 16  # tokens per page, as the reference's bf16 pool (crates/cuda-kernels/src/kv_types.rs:53-59)
+DEFAULT_MEM_FRACTION_STATIC = 0.85   # infer/src/scheduler/types.rs:215
 
 
 class EngineError(RuntimeError):
@@ -52,10 +54,14 @@ class Engine:
                  page_size: int = DEFAULT_PAGE_SIZE, max_tokens: int | None = None,
                  num_pages: int | None = None, max_slots: int = 4,
                  max_request_tokens: int | None = None, cuda_graph: bool = True,
-                 weight_tiles: bool | None = None):
+                 weight_tiles: bool | None = None, mem_fraction_static: float = DEFAULT_MEM_FRACTION_STATIC):
         """
         max_tokens: tokens the cache holds over all live requests (num_pages = ceil(max_tokens / page_size)
-            unless num_pages is given).
+            unless num_pages is given).  With neither, the pool is sized from the GPU's memory as the
+            reference does (infer/src/scheduler/cuda/core/construction.rs:131-203): what is free once the
+            weights are loaded, less a headroom of (1 - mem_fraction_static) of the whole memory, divided by
+            the bytes of a page over all layers; never more than max_slots requests of max_request_tokens
+            (default: the model's positions) can hold, since pages are not shared.
         max_request_tokens: longest single request (default: min(model's positions, cache capacity)).
         cuda_graph: replay steps of single decoded tokens from captured HIP graphs (the reference captures
             its decode path per batch size: infer/src/model/qwen3/batch_decode.rs:1691-1730).
@@ -72,14 +78,24 @@ class Engine:
         self.rt = Runtime(device=self.device, act_dtype=self.dtype,
                           weight_tiles=bool(weight_tiles) and self.dtype == torch.bfloat16)
         self.model = build_model(spec, tensors, self.rt)
-        if num_pages is None:
-            if max_tokens is None:
-                raise EngineError("give max_tokens or num_pages to size the cache")
+        needs, readers = self.model.cache_needs()
+        self.kv_bytes_per_token = cache_bytes_per_token(needs, self.dtype)
+        if num_pages is None and max_tokens is None:
+            longest = min(max_request_tokens or spec.max_positions, spec.max_positions)
+            free, total = torch.cuda.mem_get_info(self.device)
+            num_pages = pages_for_memory(free, total, mem_fraction_static, self.kv_bytes_per_token * page_size,
+                                         reserved_bytes=max_slots * state_bytes_per_slot(needs),
+                                         most_pages=max_slots * -(-longest // page_size))
+            if num_pages < 1 and any(isinstance(n, PagedNeed) for n in needs):
+                raise EngineError(f"no memory for the cache: {free / 2**30:.1f} GiB are free, the headroom of "
+                                  f"{(1 - mem_fraction_static) * 100:.0f} % of {total / 2**30:.1f} GiB leaves less than "
+                                  f"one page of {self.kv_bytes_per_token * page_size} bytes")
+            num_pages = max(num_pages, 1)
+        elif num_pages is None:
             num_pages = -(-int(max_tokens) // page_size)
         capacity = num_pages * page_size
         if max_request_tokens is None:
             max_request_tokens = min(spec.max_positions, capacity)
-        needs, readers = self.model.cache_needs()
         self.cache = CacheManager(needs, page_size=page_size, num_pages=num_pages,
                                   max_slots=max_slots, max_request_tokens=max_request_tokens,
                                   device=self.device, dtype=self.dtype, readers=readers)
@@ -136,6 +152,8 @@ class Engine:
         Raises `OutOfPages` (nothing changed) if the cache cannot take all entries.
         """
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        if not entries:
+            raise ValueError("a step needs at least one entry")
         for e in entries:
             if not self.cache.is_live(e.request):
                 raise EngineError(f"request {e.request!r} is not live; add_request it first")
@@ -158,7 +176,10 @@ class Engine:
                     raise ValueError(f"token id {e.tokens[0]} of request {e.request!r} is outside the vocabulary "
                                      f"(size {self.spec.vocab_size})")
         self.cache.append([(e.request, len(e.tokens)) for e in entries])
+        saved_state = None
         try:
+            # a mixer with state of its own overwrites it while the step runs: keep what a failed step must leave
+            saved_state = self.cache.snapshot_state([e.request for e in entries])
             self.cache.sync_tables()
             if decode_only:
                 logits = self._decode_step_graphed(entries, before)
@@ -169,6 +190,7 @@ class Engine:
         except Exception:
             for key, n in before.items():
                 self.cache.truncate(key, n)
+            self.cache.restore_state(saved_state)
             raise
         for e in entries:
             self.cache.trim_windows(e.request)

@@ -22,7 +22,9 @@ infer/src/scheduler/cuda/execution.rs:385-425,669-800):
    where a token is sampled (the reference computes them for every portion and discards them).
 5. sampling and transitions: a stop token ends the request without being emitted
    (prefill.rs:426-479, decode.rs:784-808); `max_tokens` ends it with `length`.
-6. finished requests give their pages and slot back.
+6. finished requests give their pages and slot back.  `abort(id)` ends a request in any phase at once and
+   frees what it holds, as the reference does when a client has gone (scheduler_loop.rs:325-340: a closed
+   delta channel finishes the slot at the next cleanup); its finish reason here is `abort`.
 
 Kept differently on purpose: a preempted request keeps the tokens it has generated and
 feeds prompt + generated again when it re-enters (the reference drops them and generates
@@ -42,7 +44,7 @@ from ..cache.pages import OutOfPages
 from ..sampling.params import SamplingParams
 from .batch import StepEntry
 
-LENGTH, STOP = "length", "stop"
+LENGTH, STOP, ABORT = "length", "stop", "abort"
 REQUEST_INPUT_SLACK_TOKENS = 5      # infer/src/scheduler/types.rs:499
 DECODE_RESERVATION_CLIP = 4096      # infer/src/scheduler/cuda/budget.rs:3
 
@@ -85,12 +87,14 @@ class Request:
     feed: list = field(default_factory=list)       # tokens that have to pass through the model
     fed: int = 0                                   # how many of them have
     generated: list = field(default_factory=list)
+    logprobs: list = field(default_factory=list)   # of the generated tokens, when the request asks for them
     phase: str = "waiting"                         # waiting | prefilling | decoding | finished
     finish_reason: str | None = None
     preemptions: int = 0
     t_submit: float = 0.0
     t_first_token: float | None = None
     t_finish: float | None = None
+    t_tokens: list = field(default_factory=list)   # when each generated token arrived (for the time per output token)
 
     @property
     def remaining_prompt(self) -> int:
@@ -171,7 +175,7 @@ class Scheduler:
         self.max_request_len = min(max(context - 1, 0), max(pool_tokens - 1, 0))
         self.max_request_input_len = max(self.max_request_len - REQUEST_INPUT_SLACK_TOKENS, 0)
         self.stats = {"steps": {"decode": 0, "prefill": 0, "mixed": 0}, "tokens_prefilled": 0,
-                      "tokens_decoded": 0, "preemptions": 0, "rejected": 0, "pages_high_water": 0}
+                      "tokens_decoded": 0, "preemptions": 0, "rejected": 0, "aborted": 0, "pages_high_water": 0}
 
     # -- intake ---------------------------------------------------------------------------
     def submit(self, prompt_tokens, sampling: SamplingParams | None = None,
@@ -196,6 +200,26 @@ class Scheduler:
         req.max_tokens = min(req.max_tokens, max(self.max_request_len - len(prompt) - 1, 0))
         self.waiting.append(req)
         return rid
+
+    def abort(self, rid: int) -> bool:
+        """End request `rid` now, whatever its phase: out of the queue, or its pages and slot given back.
+        True if it was still running or waiting; False if it had finished already or was never submitted.
+        The tokens it has generated so far stay on its record (finish reason `abort`)."""
+        for req in self.waiting:
+            if req.id == rid:
+                self.waiting.remove(req)
+                self._finish(req, ABORT)
+                self.finished[rid] = req
+                self.stats["aborted"] += 1
+                return True
+        for group in (self.prefilling, self.decoding):
+            for req in group:
+                if req.id == rid and req.phase != "finished":
+                    self._finish(req, ABORT)
+                    self.stats["aborted"] += 1
+                    self._cleanup()
+                    return True
+        return False
 
     # -- one iteration ------------------------------------------------------------------------
     def has_work(self) -> bool:
@@ -291,6 +315,9 @@ class Scheduler:
             # planning said it fits; if the pool disagrees, nothing was changed: skip the portions
             if not plan.prefill:
                 raise
+            if not plan.decode:
+                self.stats["steps_skipped"] = self.stats.get("steps_skipped", 0) + 1
+                return None      # nothing else to run: this iteration idles, the next one plans anew
             return self._run(StepPlan(plan.decode, []))
         self.stats["steps"][plan.kind] += 1
         self.stats["tokens_decoded"] += len(plan.decode)
@@ -302,12 +329,13 @@ class Scheduler:
         if not sampled:
             return
         rows = [(r.sampling, r.seed, len(r.generated), r.generated) for r in sampled]
-        tokens = self.sampler.sample(logits, rows)
+        tokens, logprobs = self.sampler.sample_with_logprobs(logits, rows)
         now = time.perf_counter()
-        for r, tok in zip(sampled, tokens):
-            self._apply_token(r, int(tok), now)
+        for i, (r, tok) in enumerate(zip(sampled, tokens)):
+            wants = logprobs is not None and r.sampling.logprobs
+            self._apply_token(r, int(tok), now, float(logprobs[i]) if wants else None)
 
-    def _apply_token(self, r: Request, tok: int, now: float) -> None:
+    def _apply_token(self, r: Request, tok: int, now: float, logprob: float | None = None) -> None:
         if r.phase == "prefilling":
             self.prefilling.remove(r)
             r.phase = "decoding"
@@ -319,6 +347,9 @@ class Scheduler:
             self._finish(r, STOP)  # the stop token is not emitted
             return
         r.generated.append(tok)
+        r.t_tokens.append(now)
+        if logprob is not None:
+            r.logprobs.append(logprob)
         r.feed.append(tok)
         r.fed = len(r.feed) - 1  # the new token is fed by the next decode row
         if len(r.generated) >= r.max_tokens:

@@ -46,6 +46,9 @@ SIGNATURES = {
     "arle_sample_scratch_bytes": ("sampling", [_i, _i]),
     "arle_sample_rows": ("sampling", [_p, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _p]),
     "arle_apply_penalties": ("sampling", [_p, _i, _i, _p, _p, _p, _p, _p, _p, _p]),
+    "arle_token_logprobs": ("sampling", [_p, _i, _i, _p, _p, _p]),
+    "arle_attn_decode_static": ("attention_mfma", [_p, _ll, _p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i,
+                                                   _i, _f, _i, _i, _p]),
     "arle_ceiling_read": ("ceilings", [_p, _ll, _i, _p, _p, _p]),
     "arle_ceiling_mfma": ("ceilings", [_i, _i, _i, _p, _p]),
 }
@@ -89,6 +92,14 @@ def function(name: str):
         fn.argtypes = argtypes
         fn.restype = ctypes.c_int
         _funcs[name] = fn
+    return fn
+
+
+def function_raw(name: str, restype, library_name: str = "attention_mfma", argtypes=()):
+    """A function outside the `int f(...)` convention (one that returns text, say)."""
+    fn = getattr(library(library_name), name)
+    fn.argtypes = list(argtypes)
+    fn.restype = restype
     return fn
 
 

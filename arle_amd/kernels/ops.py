@@ -435,6 +435,38 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
     return out
 
 
+def attn_decode_static(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *, max_qlen: int,
+                       num_q_heads: int, num_kv_heads: int, head_dim: int, page_size: int, scale: float,
+                       window: int = 0, splits: int = 1):
+    """attn_paged_mfma for steps whose every segment fits one row tile of 16, with the split-KV partial results
+    in the library's fixed device array: the call allocates nothing (for code under graph capture and other
+    callers that cannot allocate).  Steps too large for the array raise with the library's reason; calls that
+    overlap on one GPU race on the array."""
+    _gpu(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start)
+    tokens = q.shape[0]
+    _rows(q, "q")
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "the MFMA attention takes bfloat16")
+    _need(q.shape == (tokens, num_q_heads * head_dim) and out.shape == q.shape and out.is_contiguous(),
+          "q must be [T, nq*D] and out contiguous [T, nq*D]")
+    _need(q.data_ptr() % 16 == 0 and (q.stride(0) * 2) % 16 == 0, "q rows must be 16-byte aligned")
+    _check_pages(k_pages, v_pages, num_kv_heads, page_size, head_dim, q.dtype)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "block_table must be contiguous int32 [slots, pages]")
+    segments = seg_slot.numel()
+    _i32(seg_row0, "seg_row0", segments + 1)
+    _i32(seg_slot, "seg_slot")
+    _i32(seg_start, "seg_start", segments)
+    status = lib.function("arle_attn_decode_static")(
+        q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
+        block_table.data_ptr(), block_table.shape[1], seg_row0.data_ptr(), seg_slot.data_ptr(), seg_start.data_ptr(),
+        segments, int(max_qlen), num_q_heads, num_kv_heads, head_dim, page_size, float(scale), int(window), int(splits),
+        _stream())
+    if status != 0:
+        why = lib.function_raw("arle_attn_decode_static_error", ctypes.c_char_p)().decode()
+        raise lib.KernelError(why or f"arle_attn_decode_static failed with HIP error {status}")
+    return out
+
+
 # ------------------------------------------------------------------- sampling
 
 
@@ -458,6 +490,16 @@ def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
     parts = torch.empty((rows, chunks, 2), dtype=torch.int32, device=logits.device) if chunks > 1 else None
     lib.call("arle_argmax_rows", logits.data_ptr(), rows, vocab, out.data_ptr(),
              parts.data_ptr() if parts is not None else 0, _stream())
+    return out
+
+
+def token_logprobs(logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
+    """float32 [rows]: log softmax(logits[r])[tokens[r]], natural logarithm (tokens int32 [rows])."""
+    rows, vocab = _logits(logits)
+    _gpu(tokens)
+    _i32(tokens, "tokens", rows)
+    out = torch.empty((rows,), dtype=torch.float32, device=logits.device)
+    lib.call("arle_token_logprobs", logits.data_ptr(), rows, vocab, tokens.data_ptr(), out.data_ptr(), _stream())
     return out
 
 

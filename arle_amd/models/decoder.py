@@ -34,6 +34,27 @@ def expected_checkpoint_tensors(spec: ModelSpec) -> dict:
     return out
 
 
+def declared_cache_needs(spec: ModelSpec) -> list:
+    """The cache need of every schedule entry as its mixer's class declares it from the spec alone (no
+    weights, no GPU): what a shape summary and a memory plan are made from."""
+    needs = []
+    for entry in spec.schedule:
+        if entry.cache_from is not None:
+            needs.append(None)
+        else:
+            mixer = spec.layers[entry.layer].mixer
+            needs.append(lookup("mixer", mixer.kind).declare_cache(mixer.params))
+    return needs
+
+
+def kv_cache_bytes_per_token(spec: ModelSpec, act_dtype) -> int:
+    """Bytes of cache one token takes over all layers; for Qwen3 2 * layers * kv_heads * head_dim * element size
+    (infer/src/model/qwen3/forward.rs:777-783)."""
+    from ..cache.manager import cache_bytes_per_token
+
+    return cache_bytes_per_token(declared_cache_needs(spec), act_dtype)
+
+
 class DecoderModel:
     def __init__(self, spec: ModelSpec, fetch, rt: Runtime):
         spec.validate()

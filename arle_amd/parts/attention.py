@@ -57,9 +57,11 @@ class PagedAttention(Part):
         self.D = int(params["head_dim"])
         if self.nq % self.nkv:
             raise ValueError("num_q_heads must be a multiple of num_kv_heads")
-        if self.D % 16 or not 0 < self.D <= ops.MAX_HEAD_DIM:
-            raise ValueError(f"head_dim {self.D} is not supported: the attention kernels take "
-                             f"multiples of 16 up to {ops.MAX_HEAD_DIM}")
+        if not 0 < self.D <= ops.MAX_HEAD_DIM:
+            raise ValueError(f"head_dim {self.D} is not supported: the attention kernels take 1..{ops.MAX_HEAD_DIM}")
+        if self.D % 16 and not rt.is_f32:
+            raise ValueError(f"head_dim {self.D} is not supported in bfloat16: its kernels take multiples of 16 "
+                             f"(dtype float32 runs any head_dim up to {ops.MAX_HEAD_DIM})")
         self.eps = float(params.get("eps", 0.0))
         self.window = params.get("window")
         self.scale = float(params["scale"]) if params.get("scale") is not None else 1.0 / math.sqrt(self.D)
@@ -76,8 +78,13 @@ class PagedAttention(Part):
         self.q_only = Linear(self.qkv.weight[: self.q_width], packed=self.qkv.tiles)
         self.o = Linear(tensors["o"], rt.weight_tiles)
 
+    @classmethod
+    def declare_cache(cls, params):
+        return PagedNeed(num_kv_heads=int(params["num_kv_heads"]), head_dim=int(params["head_dim"]),
+                         window=params.get("window"))
+
     def cache_need(self):
-        return PagedNeed(num_kv_heads=self.nkv, head_dim=self.D, window=self.window)
+        return self.declare_cache(self.params)
 
     def forward(self, x, batch, cache):
         """x [T, H] -> [T, H], or a float32 stack [S, T, H] to be added in order (see Linear)."""

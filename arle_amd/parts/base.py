@@ -12,7 +12,8 @@ Interfaces (T = tokens of the packed step, H = hidden size, A = activation dtype
                 A delta is A[T,H], or a float32 stack [S,T,H] of partial sums to be added in the order
                 of S (what a matrix product with K split over workgroups leaves behind).
 * position      `fused_rotary() -> (cos, sin, rotary_dim) | None`;  `apply(q, k, positions)` in place.
-* mixer         `cache_need() -> PagedNeed | StateNeed | None`;
+* mixer         `cache_need() -> PagedNeed | StateNeed | None` (and, so that a model's cache can be sized
+                from its description alone, the class method `declare_cache(params)` with the same answer);
                 `forward(x A[T,H], batch: StepBatch, cache_view) -> delta`.
 * feed_forward  `forward(x A[T,H]) -> delta`.
 * block         `forward(residual f32[T,H], delta | None, batch, cache_view) -> (residual, delta)`;
@@ -89,6 +90,12 @@ class Part:
     def children(cls, params: dict) -> dict:
         """child name -> (role, PartSpec) of parts nested in this one."""
         return {}
+
+    @classmethod
+    def declare_cache(cls, params: dict):
+        """What a mixer of these sizes keeps between steps (PagedNeed | StateNeed | None), known without building
+        it.  A mixer that only answers `cache_need()` on a built instance is sized from the built model."""
+        return None
 
     def __init__(self, params: dict, tensors: dict, rt: Runtime, children: dict | None = None):
         self.params = params

@@ -18,6 +18,7 @@ class SamplingParams:
     stop_token_ids: list = field(default_factory=list)
     seed: int | None = None           # None = the engine's seed
     max_new_tokens: int | None = None
+    logprobs: bool = False            # report log softmax(logits)[chosen token] of every generated token
 
     def is_greedy(self) -> bool:
         """(temperature <= 0 or top_k == 1) and no stochastic filter (infer/src/sampler.rs:82-84)."""

@@ -40,15 +40,28 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, rows) -> list:
         """rows: one (SamplingParams, seed, draw_index, generated_tokens) per row of `logits`."""
+        return self.sample_with_logprobs(logits, rows)[0]
+
+    def sample_with_logprobs(self, logits: torch.Tensor, rows):
+        """(token ids, log-probabilities): the second is None unless a row asks for `logprobs`; then it holds,
+        for every row, log softmax(logits)[token] of the (penalised) logits, before temperature and truncation
+        (for a greedy row: the reference's -log(sum exp(x - max)), crates/cuda-kernels/csrc/misc/sampling.cu:252-317)."""
         if logits.shape[0] != len(rows):
             raise ValueError("one sampling row per row of logits is needed")
         if not rows:
-            return []
+            return [], None
         if any(p.has_penalties() and gen for p, _, _, gen in rows):
             logits = logits.clone()
             self._penalise(logits, rows)
+        chosen = self._choose(logits, rows)
+        if not any(p.logprobs for p, _, _, _ in rows):
+            return chosen.tolist(), None
+        logprobs = ops.token_logprobs(logits, chosen)
+        return chosen.tolist(), logprobs.tolist()
+
+    def _choose(self, logits: torch.Tensor, rows) -> torch.Tensor:
         if all(p.is_greedy() for p, _, _, _ in rows):
-            return ops.argmax_rows(logits).tolist()
+            return ops.argmax_rows(logits)
         # one host->device copy for the five per-row arrays (top_k travels as the bits of an int32)
         n, vocab = len(rows), logits.shape[1]
         packed = np.empty((5, n), dtype=np.float32)
@@ -61,7 +74,7 @@ class Sampler:
         out = ops.sample_rows(logits, dev[0], dev[4].view(torch.int32), dev[1], dev[2], dev[3],
                               use_top_k=any(0 < p.top_k < vocab for p, _, _, _ in rows),
                               use_top_p=any(p.top_p < 1.0 for p, _, _, _ in rows))
-        return out.tolist()
+        return out
 
     def _penalise(self, logits, rows) -> None:
         indptr, toks, counts = [0], [], []

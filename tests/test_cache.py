@@ -159,3 +159,59 @@ def test_random_orders_lose_nothing(seed):
         m.release(k)
     m.check()
     assert m.free_pages() == [g.pool.num_pages for g in m.groups]
+
+
+def test_bytes_per_token_and_the_pool_sized_from_memory():
+    # infer/src/model/qwen3/forward.rs:777-783: 2 (K+V) * layers * kv heads * head_dim * 2 bytes;
+    # Qwen3-4B: 2 * 36 * 8 * 128 * 2 = 147,456
+    import torch
+
+    import arle_amd.models  # noqa: F401
+    from arle_amd.cache import PAGE, PageTensor, cache_bytes_per_token, pages_for_memory, state_bytes_per_slot
+    from arle_amd.config import Qwen3Config
+    from arle_amd.models import declared_cache_needs, kv_cache_bytes_per_token
+    from arle_amd.models.qwen3 import qwen3_spec
+
+    cfg = Qwen3Config.from_dict(dict(num_hidden_layers=36, hidden_size=2560, num_attention_heads=32,
+                                     num_key_value_heads=8, head_dim=128, intermediate_size=9728, vocab_size=151936,
+                                     rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=True,
+                                     max_position_embeddings=40960))
+    spec = qwen3_spec(cfg)
+    assert kv_cache_bytes_per_token(spec, torch.bfloat16) == 147456
+    assert kv_cache_bytes_per_token(spec, torch.float32) == 294912
+    needs = declared_cache_needs(spec)
+    assert len(needs) == 36 and needs[0] == PagedNeed(8, 128)
+    # a need with tensors of its own: one compressed vector of 72 per token in float16, and an index in int8
+    latent = PagedNeed(tensors=(PageTensor("latent", (PAGE, 72), torch.float16), PageTensor("tag", (PAGE,), torch.int8)))
+    assert latent.bytes_per_token(torch.bfloat16) == 72 * 2 + 1
+    assert cache_bytes_per_token([latent, None, PagedNeed(2, 16), StateNeed((4, 4))], torch.bfloat16) == 145 + 2 * 2 * 16 * 2
+    assert state_bytes_per_slot([StateNeed((4, 4)), StateNeed((3,), torch.bfloat16), latent]) == 64 + 6
+    with pytest.raises(ValueError, match="PAGE exactly once"):
+        PagedNeed(tensors=(PageTensor("x", (4, 4)),)).bytes_per_token(torch.float32)
+    # infer/src/scheduler/cuda/core/construction.rs:131-203: free - headroom, headroom = (1 - fraction) * total
+    gib = 1 << 30
+    page = 147456 * 16
+    assert pages_for_memory(200 * gib, 288 * gib, 0.85, page) == int((200 - 288 * 0.15) * gib) // page
+    assert pages_for_memory(200 * gib, 288 * gib, 0.85, page, most_pages=1000) == 1000
+    assert pages_for_memory(10 * gib, 288 * gib, 0.85, page) == 0          # less free than the headroom
+    assert pages_for_memory(100 * gib, 288 * gib, 1.0, page, reserved_bytes=gib) == (99 * gib) // page
+    with pytest.raises(ValueError):
+        pages_for_memory(1, 1, 0.0, 1)
+
+
+def test_a_group_with_tensors_of_its_own_keeps_its_bookkeeping():
+    import torch
+
+    from arle_amd.cache import PAGE, PageTensor
+
+    latent = PagedNeed(tensors=(PageTensor("latent", (PAGE, 24), torch.float32),), window=None)
+    m = CacheManager([latent, PagedNeed(1, 16), latent], page_size=4, num_pages=6, max_slots=2, max_request_tokens=16)
+    assert len(m.groups) == 2                      # the two latent entries share pages and a block table
+    m.admit("a")
+    m.append([("a", 9)])
+    assert m.free_pages() == [3, 3]
+    view = m.view(2)
+    assert set(view.pages) == {"latent"} and view.writes and m.view(1).pages.keys() == {"k", "v"}
+    m.release("a")
+    m.check()
+    assert m.free_pages() == [6, 6]

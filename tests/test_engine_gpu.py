@@ -189,3 +189,15 @@ def test_captured_steps_are_kept_least_recently_used(model):
     assert len(graphed._graphs) <= 2 and graphed.graph_replays >= 4
     for key in a:
         assert torch.equal(a[key], b[key]), key
+
+
+def test_head_dim_that_is_no_multiple_of_16_runs_in_float32_and_is_refused_in_bfloat16(tmp_path):
+    d = make_model_dir(tmp_path, "F")
+    cfg, weights = read_folder(d)
+    assert cfg["head_dim"] == 24
+    reqs = {f"r{i}": random_tokens(n, cfg["vocab_size"], 900 + i) for i, n in enumerate([40, 23, 57, 31, 18])}
+    eng = Engine.from_folder(d, dtype="float32", page_size=TINY["F"][1], max_tokens=3 * 64, max_slots=3)
+    got = replay.run_steps(eng, replay.mixed(reqs, max_live=3, seed=11))
+    replay.compare(got, cfg, weights, reqs, TOL["float32"], "head_dim 24 / float32")
+    with pytest.raises(ValueError, match="multiples of 16"):
+        Engine.from_folder(d, dtype="bfloat16", page_size=8, max_tokens=64)

@@ -197,3 +197,95 @@ def test_many_requests_through_the_scheduler_with_and_without_captured_steps(fol
     if dtype == "float32":
         for p, b, got in list(zip(prompts, budgets, results[True]))[::5]:
             assert got == _plain_greedy(cfg, weights, p, b)
+
+
+def test_command_line_run_with_a_text_prompt_and_a_tokenizer(folders, tmp_path):
+    """`run --prompt TEXT`: text -> tokenizer.json of the folder -> ids -> generation -> text again.  The test writes a
+    small word-level tokenizer (word "t<i>" is id i), so the ids are known."""
+    import shutil
+
+    tokenizers = pytest.importorskip("tokenizers")
+    cfg, weights = read_folder(folders["A"])
+    d = str(tmp_path / "with_tokenizer")
+    shutil.copytree(folders["A"], d)
+    tok = tokenizers.Tokenizer(tokenizers.models.WordLevel({f"t{i}": i for i in range(cfg["vocab_size"])}, unk_token="t0"))
+    tok.pre_tokenizer = tokenizers.pre_tokenizers.Whitespace()
+    tok.decoder = tokenizers.decoders.WordPiece(prefix="##", cleanup=False)     # joins words with a blank
+    tok.save(os.path.join(d, "tokenizer.json"))
+    prompt = random_tokens(6, cfg["vocab_size"], 31)
+    want = _plain_greedy(cfg, weights, prompt, 4)
+    text = " ".join(f"t{t}" for t in prompt)
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "arle-amd"), "--model-path", d, "--max-tokens", "4",
+           "--dtype", "float32", "--max-seq-len", "64", "run", "--prompt", text, "--json"]
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr[-2000:]
+    doc = json.loads(res.stdout.strip().splitlines()[-1])
+    assert doc["token_ids"] == want and doc["usage"]["prompt_tokens"] == 6
+    assert doc["text"].split() == [f"t{t}" for t in want]
+    # the same through --stdin, as plain text on stdout
+    cmd = cmd[:-3] + ["--stdin"]
+    res = subprocess.run(cmd, input=text, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert res.stdout.strip().splitlines()[-1].split() == [f"t{t}" for t in want]
+
+
+def test_log_probabilities_of_the_chosen_tokens(folders):
+    """token_logprobs = log softmax(logits)[token] of every generated token, greedy and sampled rows in one batch
+    (greedy: the reference's -log(sum exp(x - max)), crates/cuda-kernels/csrc/misc/sampling.cu:252-317)."""
+    cfg, weights = read_folder(folders["B"])
+    prompts = [random_tokens(n, cfg["vocab_size"], 40 + n) for n in (7, 12)]
+    llm = LLM(folders["B"], dtype="float32", page_size=TINY["B"][1], kv_cache_tokens=256, max_seq_len=64)
+    from arle_amd.engine.scheduler import Scheduler
+
+    sched = Scheduler(llm.engine, llm.sampler, llm.sched_config, seed=3)
+    a = sched.submit(prompts[0], SamplingParams(logprobs=True), max_tokens=5)
+    b = sched.submit(prompts[1], SamplingParams(temperature=0.9, seed=77, logprobs=True), max_tokens=5)
+    c = sched.submit(prompts[1], SamplingParams(), max_tokens=5)
+    sched.run_until_done()
+    assert sched.finished[c].logprobs == []
+    for rid, p in ((a, prompts[0]), (b, prompts[1])):
+        r = sched.finished[rid]
+        assert len(r.logprobs) == len(r.generated) == 5
+        hist = list(p)
+        for t, lp in zip(r.generated, r.logprobs):
+            ref = torch.log_softmax(plain.forward_logits(weights, cfg, hist, dtype=torch.float64)[-1], dim=-1)
+            assert abs(lp - float(ref[t])) < 1e-4
+            hist.append(t)
+    greedy = sched.finished[a]
+    assert all(lp <= 0.0 for lp in greedy.logprobs)
+    out = llm.generate([prompts[0]], max_tokens=5, logprobs=True)[0]
+    assert out.response_token_ids == greedy.generated and out.token_logprobs == pytest.approx(greedy.logprobs, abs=1e-6)
+    assert out.tpot_s is not None and out.tpot_s > 0
+
+
+def test_abort_on_the_real_engine_gives_pages_back(folders):
+    from arle_amd.engine.scheduler import ABORT, Scheduler
+
+    cfg, weights = read_folder(folders["A"])
+    llm = LLM(folders["A"], dtype="float32", page_size=4, kv_cache_tokens=256, max_seq_len=64, chunked_prefill_size=8)
+    sched = Scheduler(llm.engine, llm.sampler, llm.sched_config, seed=1)
+    keep_prompt = random_tokens(9, cfg["vocab_size"], 21)
+    keep = sched.submit(keep_prompt, max_tokens=10)
+    gone = sched.submit(random_tokens(30, cfg["vocab_size"], 22), max_tokens=10)
+    sched.iteration()
+    sched.iteration()
+    assert sched.abort(gone) and sched.finished[gone].finish_reason == ABORT
+    sched.run_until_done()
+    assert sched.finished[keep].generated == _plain_greedy(cfg, weights, keep_prompt, 10)
+    assert llm.engine.cache.free_pages() == [64] and not llm.engine.cache.slot_of
+
+
+def test_the_pool_is_sized_from_free_memory_when_no_size_is_given(folders):
+    """No kv_cache_tokens: pages for what is free less the headroom, but never more than the slots can fill."""
+    cfg, weights = read_folder(folders["A"])
+    llm = LLM(folders["A"], dtype="bfloat16", page_size=16, num_slots=3, max_seq_len=200)
+    cache = llm.engine.cache
+    assert cache.groups[0].pool.num_pages == 3 * 13          # 3 slots x ceil(200 / 16) pages: the cap
+    assert llm.engine.kv_bytes_per_token == 2 * cfg["num_hidden_layers"] * cfg["num_key_value_heads"] * cfg["head_dim"] * 2
+    out = llm.generate([random_tokens(5, cfg["vocab_size"], 2)], max_tokens=3)[0]
+    assert len(out.response_token_ids) == 3
+    from arle_amd.engine import Engine
+    from arle_amd.engine.engine import EngineError
+
+    with pytest.raises(EngineError, match="no memory for the cache"):
+        Engine.from_folder(folders["A"], dtype="bfloat16", mem_fraction_static=1e-6)

@@ -355,6 +355,25 @@ def test_sampling_vectors_of_the_reference():
     assert _sample(x, 0.0, 0.3) == [2]
 
 
+@pytest.mark.parametrize("rows,vocab", [(1, 151936), (5, 333), (9, 4099), (64, 1031)])
+def test_token_logprobs_are_the_log_softmax_of_the_chosen_tokens(rows, vocab):
+    # for the largest logit: -log(sum exp(x - max)), crates/cuda-kernels/csrc/misc/sampling.cu:299-316
+    g = _g(61)
+    x = (torch.randn(rows, vocab, generator=g) * 4.0).contiguous()
+    x[0, vocab // 2] = 40.0                       # a row with one dominant logit: its log-probability is about 0
+    tokens = torch.randint(0, vocab, (rows,), generator=g).to(torch.int32)
+    tokens[0] = vocab // 2
+    if rows > 1:
+        tokens[1] = int(x[1].argmax())
+    got = ops.token_logprobs(x.to(DEV), tokens.to(DEV)).cpu().double()
+    want = torch.log_softmax(x.double(), dim=-1)[torch.arange(rows), tokens.long()]
+    assert torch.allclose(got, want, atol=2e-5, rtol=1e-5)
+    assert abs(float(got[0])) < 1e-3
+    if rows > 1:
+        m = x[1].double().max()
+        assert abs(float(got[1]) + float(torch.log(torch.exp(x[1].double() - m).sum()))) < 2e-5
+
+
 @pytest.mark.parametrize("vocab", [5, 333, 4099])
 def test_sampling_against_plain_inverse_cdf(vocab):
     g = _g(60)

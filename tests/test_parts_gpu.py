@@ -175,5 +175,10 @@ def test_unknown_part_and_bad_head_dim_are_refused():
                                         "qk_norm": False, "position": pos_spec},
                     {"q": "q", "k": "k", "v": "v", "o": "o"})
     w = _tensors({"q": (48, 48), "k": (24, 48), "v": (24, 48), "o": (48, 48)}, torch.float32)
-    with pytest.raises(ValueError, match="head_dim 24 is not supported"):
+    build_part("mixer", spec, lambda n: w[n].to(DEV), _rt(torch.float32))     # float32 takes any head_dim
+    wb = {k: v.bfloat16() for k, v in w.items()}
+    with pytest.raises(ValueError, match="head_dim 24 is not supported in bfloat16"):
+        build_part("mixer", spec, lambda n: wb[n].to(DEV), _rt(torch.bfloat16))
+    spec.params["head_dim"] = 1024
+    with pytest.raises(ValueError, match="head_dim 1024 is not supported"):
         build_part("mixer", spec, lambda n: w[n].to(DEV), _rt(torch.float32))

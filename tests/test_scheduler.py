@@ -6,7 +6,7 @@ from types import SimpleNamespace
 import pytest
 
 from arle_amd.cache import CacheManager, OutOfPages, PagedNeed
-from arle_amd.engine.scheduler import (LENGTH, STOP, Request, Scheduler, SchedulerConfig, plan_prefill,
+from arle_amd.engine.scheduler import (ABORT, LENGTH, STOP, Request, Scheduler, SchedulerConfig, plan_prefill,
                                        retract_victim)
 from arle_amd.sampling import SamplingParams
 
@@ -53,9 +53,10 @@ class FakeEngine:
 
 
 class FakeSampler:
-    def sample(self, logits, rows):
+    def sample_with_logprobs(self, logits, rows):
         assert len(logits) == len(rows)
-        return list(logits)
+        wanted = any(p.logprobs for p, _, _, _ in rows)
+        return list(logits), ([-0.5 - t for t in logits] if wanted else None)
 
 
 def expected_output(prompt, n):
@@ -244,3 +245,64 @@ def test_sampling_params_greedy_rule():
     assert not SamplingParams(temperature=0.0, top_p=0.9).is_greedy()
     assert not SamplingParams(temperature=0.0, min_p=0.1).is_greedy()
     assert SamplingParams(repetition_penalty=1.1).has_penalties() and not SamplingParams().has_penalties()
+
+
+def test_abort_frees_a_request_in_any_phase():
+    # the reference finishes a slot whose client has gone at the next cleanup
+    # (infer/src/scheduler/cuda/runtime/scheduler_loop.rs:325-340); here by an explicit call
+    eng, s = make(num_pages=64, slots=2, chunked_prefill_size=8)
+    a = s.submit(prompt(20), max_tokens=50)          # will be prefilling (three portions)
+    b = s.submit(prompt(5, 1), max_tokens=50)        # will be decoding
+    c = s.submit(prompt(6, 2), max_tokens=50)        # waits: no slot
+    s.iteration()
+    assert [r.id for r in s.prefilling] == [a] and [r.id for r in s.decoding] == [b] and [r.id for r in s.waiting] == [c]
+    free_before = eng.cache.free_pages()[0]
+    assert s.abort(c) and s.finished[c].finish_reason == ABORT and not s.waiting
+    assert eng.cache.free_pages()[0] == free_before          # a waiting request held nothing
+    assert s.abort(a)                                         # mid-prefill: pages and slot come back
+    assert not eng.cache.is_live(a) and s.finished[a].finish_reason == ABORT and not s.prefilling
+    assert eng.cache.free_pages()[0] > free_before and eng.cache.free_slot_count == 1
+    s.iteration()
+    kept = list(s.decoding[0].generated)
+    assert s.abort(b)                                         # decoding: what it generated stays on the record
+    assert s.finished[b].generated == kept == expected_output(prompt(5, 1), len(kept)) and len(kept) >= 2
+    assert not s.abort(b) and not s.abort(12345)              # finished already / never submitted
+    eng.cache.check()
+    assert eng.cache.free_pages()[0] == 64 and eng.cache.free_slot_count == 2 and not s.has_work()
+    assert s.stats["aborted"] == 3
+    # the scheduler goes on with new work in the freed slots
+    d = s.submit(prompt(9, 3), max_tokens=4)
+    s.run_until_done()
+    assert s.finished[d].generated == expected_output(prompt(9, 3), 4)
+
+
+def test_out_of_pages_on_a_prefill_only_step_idles_instead_of_running_an_empty_step():
+    eng, s = make(num_pages=64, slots=2)
+
+    calls = {"n": 0}
+    real_step = eng.step
+
+    def step(entries):
+        calls["n"] += 1
+        assert entries, "an empty step was run"
+        if calls["n"] == 1:
+            raise OutOfPages("the pool disagrees with the plan")
+        return real_step(entries)
+
+    eng.step = step
+    rid = s.submit(prompt(7), max_tokens=3)
+    plan = s.iteration()                      # the step is refused; nothing else to run: the iteration idles
+    assert plan.kind == "prefill" and s.stats["steps"]["prefill"] == 0 and s.stats["steps_skipped"] == 1
+    assert eng.cache.length(rid) == 0
+    s.run_until_done()
+    assert s.finished[rid].generated == expected_output(prompt(7), 3)
+
+
+def test_logprobs_reach_the_request_only_when_asked_for():
+    eng, s = make()
+    a = s.submit(prompt(6), SamplingParams(logprobs=True), max_tokens=4)
+    b = s.submit(prompt(7, 1), SamplingParams(), max_tokens=4)
+    s.run_until_done()
+    ra, rb = s.finished[a], s.finished[b]
+    assert ra.logprobs == [-0.5 - t for t in ra.generated] and rb.logprobs == []
+    assert len(ra.t_tokens) == 4 and ra.t_tokens == sorted(ra.t_tokens)

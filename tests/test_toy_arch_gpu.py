@@ -178,3 +178,37 @@ def test_windowed_group_needs_fewer_pages(toy_folder):
     full = [g for g in eng.cache.groups if not g.window][0]
     assert full.pool.num_pages - full.pool.free_count == 15
     assert windowed.pool.num_pages - windowed.pool.free_count <= 3
+
+
+def test_a_failed_step_leaves_state_slots_and_pages_as_they_were(toy_folder):
+    """A step that fails after its mixers ran must not leave a request with the state of tokens it does not
+    hold: the state blocks of the step's slots are put back, like the lengths and pages."""
+    _, weights = read_folder(toy_folder)
+    eng = Engine.from_folder(toy_folder, dtype="float32", page_size=4, max_tokens=256, max_slots=2, cuda_graph=False)
+    toks = random_tokens(21, TOY.vocab_size, 8)
+    other = random_tokens(9, TOY.vocab_size, 9)
+    eng.add_request("a")
+    eng.add_request("b")
+    eng.step([("a", toks[:8], []), ("b", other[:4], [])])
+    state_before = {e: buf.clone() for e, buf in eng.cache.state_buffers.items()}
+    free_before, len_before = eng.cache.free_pages(), (eng.length("a"), eng.length("b"))
+    real_forward = eng.model.forward
+
+    def forward_then_fail(batch, cache):
+        real_forward(batch, cache)          # every mixer has run: the state blocks are overwritten
+        torch.cuda.synchronize()
+        raise RuntimeError("planted failure after the layers")
+
+    eng.model.forward = forward_then_fail
+    with pytest.raises(RuntimeError, match="planted"):
+        eng.step([("a", toks[8:15], [6]), ("b", other[4:6], [])])
+    eng.model.forward = real_forward
+    assert (eng.length("a"), eng.length("b")) == len_before and eng.cache.free_pages() == free_before
+    for e, buf in eng.cache.state_buffers.items():
+        assert torch.equal(buf, state_before[e])
+    # the requests go on as if nothing had happened
+    got = eng.step([("a", toks[8:], list(range(13))), ("b", other[4:], [4])])
+    ref = toy_plain_logits(TOY, weights, toks)
+    assert float((got[:13].cpu().double() - ref[8:]).abs().max() / ref.abs().max()) <= 1e-5
+    ref_b = toy_plain_logits(TOY, weights, other)
+    assert float((got[13].cpu().double() - ref_b[8]).abs().max() / ref_b.abs().max()) <= 1e-5

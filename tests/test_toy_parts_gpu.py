@@ -259,3 +259,116 @@ def test_toy_parts_run_in_bfloat16_too(folder):
         outs[dtype] = rows
     agree = (outs["float32"].argmax(-1) == outs["bfloat16"].argmax(-1)).float().mean()
     assert float(agree) >= 0.8
+
+
+# ---- a mixer whose paged cache is not keys and values ---------------------------------------------------------
+
+from arle_amd.cache import PAGE, PagedNeed, PageTensor  # noqa: E402
+
+
+@register("mixer", "toy_latent_mean")
+class LatentMean(Part):
+    """Caches one compressed float32 vector per token, c_t = W_down x_t (in a tensor of its own, float32 even in a
+    bfloat16 engine, beside a one-byte tag per token), and returns W_up applied to the mean of c_0..c_t."""
+
+    @classmethod
+    def declare_weights(cls, params):
+        return {"down": WeightDecl((params["latent"], params["hidden_size"])),
+                "up": WeightDecl((params["hidden_size"], params["latent"]))}
+
+    @classmethod
+    def declare_cache(cls, params):
+        return PagedNeed(tensors=(PageTensor("latent", (PAGE, int(params["latent"])), torch.float32),
+                                  PageTensor("tag", (PAGE,), torch.uint8)))
+
+    def __init__(self, params, tensors, rt, children=None):
+        super().__init__(params, tensors, rt, children)
+        self.down, self.up = tensors["down"].float(), tensors["up"].float()
+
+    def cache_need(self):
+        return self.declare_cache(self.params)
+
+    def forward(self, x, batch, cache):
+        c = x.float() @ self.down.T
+        latent, tag, P = cache.pages["latent"], cache.pages["tag"], cache.page_size
+        assert latent.dtype == torch.float32 and tag.dtype == torch.uint8
+        out = torch.empty_like(c)
+        for seg in batch.segments:
+            table = cache.block_table[seg.slot].long()
+            pos = torch.arange(seg.start, seg.start + seg.length, device=x.device)
+            latent[table[pos // P], pos % P] = c[seg.row0:seg.row0 + seg.length]
+            tag[table[pos // P], pos % P] = 1
+            every = torch.arange(0, seg.start + seg.length, device=x.device)
+            assert bool((tag[table[every // P], every % P] == 1).all())      # every earlier token was written
+            sums = latent[table[every // P], every % P].cumsum(0)[seg.start:]
+            out[seg.row0:seg.row0 + seg.length] = sums / (pos + 1).float()[:, None]
+        return (out @ self.up.T).to(x.dtype)
+
+
+@dataclass(frozen=True)
+class LatentConfig:
+    hidden_size: int
+    intermediate_size: int
+    latent: int
+    vocab_size: int
+    eps: float
+    max_position_embeddings: int = 256
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(**{k: raw[k] for k in cls.__dataclass_fields__})
+
+    def to_dict(self):
+        return dict(asdict(self), architectures=["ToyLatentLM"])
+
+
+def latent_spec(c: LatentConfig, stop_token_ids=()):
+    norm = lambda name: PartSpec("rmsnorm", {"width": c.hidden_size, "eps": c.eps}, {"weight": name})
+    layers = [LayerSpec("pre_norm",
+                        PartSpec("toy_latent_mean", {"hidden_size": c.hidden_size, "latent": c.latent},
+                                 {"down": f"l{i}.down", "up": f"l{i}.up"}),
+                        PartSpec("swiglu", {"hidden_size": c.hidden_size, "intermediate_size": c.intermediate_size},
+                                 {"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}),
+                        {"mixer_in": norm(f"l{i}.n1"), "ffn_in": norm(f"l{i}.n2")}) for i in range(2)]
+    sizes = {"vocab_size": c.vocab_size, "hidden_size": c.hidden_size}
+    return ModelSpec(hidden_size=c.hidden_size, vocab_size=c.vocab_size, max_positions=c.max_position_embeddings,
+                     embedding=PartSpec("token_table", sizes, {"table": "embed"}), layers=layers,
+                     schedule=[ScheduleEntry(0), ScheduleEntry(1)], final_norm=norm("fn"),
+                     head=PartSpec("linear", sizes, {"weight": "embed"}), stop_token_ids=tuple(stop_token_ids))
+
+
+register_architecture("ToyLatentLM", LatentConfig, latent_spec)
+LATENT = LatentConfig(hidden_size=40, intermediate_size=72, latent=12, vocab_size=90, eps=1e-5)
+
+
+def latent_plain_logits(c, w, tokens):
+    w = {k: v.double() for k, v in w.items()}
+    h = plain.embedding(w["embed"], tokens)
+    for i in range(2):
+        a = plain.rms_norm(h, w[f"l{i}.n1"], c.eps)
+        lat = a @ w[f"l{i}.down"].T
+        mean = lat.cumsum(0) / torch.arange(1, len(tokens) + 1, dtype=torch.float64)[:, None]
+        h = h + mean @ w[f"l{i}.up"].T
+        b = plain.rms_norm(h, w[f"l{i}.n2"], c.eps)
+        h = h + plain.swiglu_mlp(b, w[f"l{i}.g"], w[f"l{i}.u"], w[f"l{i}.d"])
+    return plain.linear(plain.rms_norm(h, w["fn"], c.eps), w["embed"])
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-5), ("bfloat16", 2.5e-2)])
+def test_a_mixer_declares_the_tensors_and_types_of_its_own_paged_cache(tmp_path, dtype, tol):
+    d = str(tmp_path / "latent")
+    write_random_model(d, "ToyLatentLM", LATENT, seed=5, std=0.1, norm_std=0.05)
+    _, weights = read_folder(d)
+    eng = Engine.from_folder(d, dtype=dtype, page_size=4, max_tokens=3 * 64, max_slots=4)
+    group = eng.cache.page_buffers[0]
+    assert set(group) == {"latent", "tag"} and group["latent"].dtype == torch.float32
+    assert group["latent"].shape == (2, 48, 4, 12) and group["tag"].shape == (2, 48, 4)
+    assert eng.kv_bytes_per_token == 2 * (12 * 4 + 1)
+    reqs = {f"q{i}": random_tokens(n, LATENT.vocab_size, 60 + i) for i, n in enumerate([33, 50, 19, 41])}
+    got = replay.run_steps(eng, replay.mixed(reqs, max_live=3, seed=4))
+    for rid, toks in reqs.items():
+        ref = latent_plain_logits(LATENT, weights, toks)
+        for p in range(len(toks)):
+            err = float((got[(rid, p)].double() - ref[p]).abs().max() / ref.abs().max())
+            assert err <= tol, f"{dtype}: request {rid} position {p}: {err:.3e}"
+    assert eng.cache.free_pages() == [48]

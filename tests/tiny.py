@@ -36,6 +36,11 @@ TINY_E = dict(num_hidden_layers=2, hidden_size=104, num_attention_heads=6, num_k
               head_dim=96, intermediate_size=168, vocab_size=517, rope_theta=20000.0,
               rms_norm_eps=1e-5, tie_word_embeddings=False, max_position_embeddings=1024)
 
+# F: a head_dim that is even but no multiple of 16: the float32 kernels take it, the bfloat16 ones refuse it
+TINY_F = dict(num_hidden_layers=2, hidden_size=56, num_attention_heads=4, num_key_value_heads=2,
+              head_dim=24, intermediate_size=100, vocab_size=211, rope_theta=30000.0,
+              rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=512)
+
 # name -> (config, page size, weight std, norm std, seed)
 TINY = {
     "A": (TINY_A, 4, 0.02, 0.02, 11),
@@ -43,6 +48,7 @@ TINY = {
     "C": (TINY_C, 16, 0.08, 0.1, 33),
     "D": (TINY_D, 32, 0.06, 0.05, 44),
     "E": (TINY_E, 16, 0.07, 0.08, 55),
+    "F": (TINY_F, 8, 0.07, 0.06, 66),
 }
 
 
