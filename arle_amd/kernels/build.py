@@ -187,7 +187,15 @@ def ensure(name: str) -> str:
 
 
 def build_all(names=None, jobs: int = 4) -> dict:
-    """Compile every library (always), a few at a time; returns name -> path."""
+    """Compile every library (always), a few at a time; returns name -> path.  Libraries of sources that no
+    longer exist are removed from the folder."""
+    if not names:
+        known = {f"libarle_{n}.so" for n in SOURCES}
+        folder = lib_dir()
+        for fname in os.listdir(folder):
+            base = fname[:-len(".srchash")] if fname.endswith(".srchash") else fname
+            if base.startswith("libarle_") and base.endswith(".so") and base not in known:
+                os.remove(os.path.join(folder, fname))
     names = list(names or SOURCES)
     results: dict = {}
     errors: list = []

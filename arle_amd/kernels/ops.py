@@ -910,7 +910,9 @@ _MM_OUT_DTYPE_OK = None
 
 
 def _library_mm_f32out(x, w):
-    """bfloat16 x bfloat16 -> float32 through the library, without rounding the result to bfloat16."""
+    """bfloat16 x bfloat16 -> float32 through the library.  With a torch that takes `out_dtype` the 32-bit
+    accumulators are returned as they are; an older one hands back bfloat16, which is then only widened (the
+    result has been rounded once)."""
     global _MM_OUT_DTYPE_OK
     if _MM_OUT_DTYPE_OK is None:
         try:
