@@ -57,6 +57,149 @@ def prefill_flops(c, tokens: int) -> float:
     return gemm + attn + head
 
 
+# ---- where a step's time goes: kernels of a profiled step, sorted into the parts of a layer -------------------------
+
+GEMM_NAMES = ("gemm_rows", "gemm_stream", "gemm_tiles", "gemm_f32", "Cijk_", "sum_partials", "silu_mul")
+PARTS = ("qkv", "o", "gate_up", "down", "head", "attention", "qk_prep", "norm", "other")
+
+
+def _template_args(name: str) -> list:
+    return name[name.index("<") + 1:name.rindex(">")].replace(" ", "").split(",") if "<" in name and ">" in name else []
+
+
+def _completes_gate_up(name: str) -> bool:
+    """Whether this kernel leaves gate|up complete: a product with the activation fused (gemm_rows_kernel<MT, WN,
+    WK, PD, XD, EPI, out> / gemm_tiles_kernel<MT, PD, PX, PIPE, EPI, out> with EPI = 1), or the activation kernel
+    behind a plain product."""
+    if "silu_mul" in name:
+        return True
+    args = _template_args(name)
+    if "gemm_rows_kernel" in name:
+        return len(args) > 5 and args[5] == "1"
+    if "gemm_tiles_kernel" in name:
+        return len(args) > 4 and args[4] == "1"
+    return False
+
+
+def classify_step(names, layers: int) -> list:
+    """The part of the model that each kernel of one step belongs to, from the order in which a layer launches
+    them: norm, q|k|v product, q/k preparation, attention (+ merges), o product, norm, gate|up (+ activation),
+    down product; after the last layer the final norm and the head."""
+    out, phase, layers_done = [], "qkv", 0
+    for name in names:
+        if "qk_prep" in name:
+            part, phase = "qk_prep", "o"
+        elif "attn_" in name:
+            part = "attention"
+        elif "rmsnorm" in name:
+            part = "norm"
+            if phase == "o":
+                phase = "gate_up"
+            elif phase == "down":
+                layers_done += 1
+                phase = "head" if layers_done >= layers else "qkv"
+        elif any(g in name for g in GEMM_NAMES):
+            part = phase
+            if phase == "gate_up" and _completes_gate_up(name):
+                phase = "down"
+        else:
+            part = "other"
+        out.append(part)
+    return out
+
+
+def profiled_steps(torch, fns) -> list:
+    """The kernels of every call in `fns`, run one after the other inside ONE profiler session (a second session
+    in a process has crashed the profiler here): a list, one entry a call, of (name, microseconds) in launch
+    order.  A step begins with the embedding kernel, which is how the session's kernels are cut into calls."""
+    from torch.profiler import ProfilerActivity, profile
+
+    torch.cuda.synchronize()
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        for fn in fns:
+            fn()
+            torch.cuda.synchronize()
+    evs = [e for e in prof.events() if e.device_type == torch.autograd.DeviceType.CUDA and "Memcpy" not in e.name
+           and "Memset" not in e.name]
+    evs.sort(key=lambda e: e.time_range.start)
+    steps, early = [], []
+    for e in evs:
+        item = (e.name, e.time_range.end - e.time_range.start)
+        if "embed_gather" in e.name:
+            steps.append(early + [item])     # what ran before the first step's embedding is counted with it
+            early = []
+        elif steps:
+            steps[-1].append(item)
+        else:
+            early.append(item)
+    if len(steps) != len(fns):
+        raise RuntimeError(f"the profiler saw {len(steps)} steps for {len(fns)} calls")
+    return steps
+
+
+def part_times(steps, layers: int) -> dict:
+    """part -> microseconds a step (mean over `steps`, lists of (kernel name, microseconds)), plus "kernels".
+    The profiler now and then loses kernels of a step; only the steps with the most kernels are counted, and
+    those must show every layer."""
+    most = max(len(k) for k in steps)
+    steps = [k for k in steps if len(k) == most]
+    for kernels in steps:
+        seen = sum(1 for n, _ in kernels if "qk_prep" in n)
+        if seen != layers:
+            raise RuntimeError(f"a profiled step shows {seen} of {layers} layers")
+    total = {p: 0.0 for p in PARTS}
+    for kernels in steps:
+        for part, (_, us) in zip(classify_step([n for n, _ in kernels], layers), kernels):
+            total[part] += us
+    out = {p: t / len(steps) for p, t in total.items()}
+    out["kernels"] = sum(len(k) for k in steps) / len(steps)
+    return out
+
+
+def part_bytes_decode(c, batch: int, context: float, elt: int = 2) -> dict:
+    """Bytes that each part of a decode step has to read: its weights once, and for attention the cache."""
+    L, h, i = c["num_hidden_layers"], c["hidden_size"], c["intermediate_size"]
+    q, kv = c["num_attention_heads"] * c["head_dim"], c["num_key_value_heads"] * c["head_dim"]
+    return {"qkv": L * h * (q + 2 * kv) * elt, "o": L * q * h * elt, "gate_up": L * 2 * i * h * elt,
+            "down": L * h * i * elt, "head": c["vocab_size"] * h * elt, "attention": batch * context * 2 * L * kv * elt}
+
+
+def part_flops_prefill(c, tokens: int) -> dict:
+    L, h, i = c["num_hidden_layers"], c["hidden_size"], c["intermediate_size"]
+    q, kv = c["num_attention_heads"] * c["head_dim"], c["num_key_value_heads"] * c["head_dim"]
+    return {"qkv": 2.0 * tokens * L * h * (q + 2 * kv), "o": 2.0 * tokens * L * q * h,
+            "gate_up": 2.0 * tokens * L * 2 * i * h, "down": 2.0 * tokens * L * h * i,
+            "head": 2.0 * c["vocab_size"] * h, "attention": 4.0 * q * (tokens * (tokens + 1) / 2) * L}
+
+
+def part_report(times: dict, work: dict, peak: float, ceiling: float) -> tuple:
+    """(microseconds a step by part, fraction of the published peak, fraction of the measured ceiling)."""
+    us = {p: round(times[p], 1) for p in PARTS if times.get(p)}
+    us["kernels"] = round(times["kernels"], 1)
+    of_peak = {p: round(work[p] / (times[p] * 1e-6) / peak, 4) for p in work if times.get(p)}
+    of_ceiling = {p: round(work[p] / (times[p] * 1e-6) / ceiling, 4) for p in work if times.get(p)}
+    return us, of_peak, of_ceiling
+
+
+def parts_in_a_child_process(args) -> dict:
+    """The breakdown by part of the model, measured by a second run of this program under the profiler: the
+    profiler stays out of the process whose steps are timed, and a fault of its own costs only the breakdown."""
+    import os
+    import subprocess
+
+    cmd = [sys.executable, os.path.abspath(__file__), "--parts-only", "--batch", str(args.batch), "--layers", str(args.layers),
+           "--page-size", str(PAGE), "--dtype", args.dtype]
+    cmd += ["--no-weight-tiles"] if args.no_weight_tiles else []
+    try:
+        res = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+        lines = [ln for ln in res.stdout.splitlines() if ln.startswith("{")]
+        if res.returncode != 0 or not lines:
+            return {"parts": f"not measured: the profiled run ended with code {res.returncode}"}
+        return json.loads(lines[-1])
+    except (subprocess.TimeoutExpired, OSError, ValueError) as exc:
+        return {"parts": f"not measured: {type(exc).__name__}"}
+
+
 def _timed(torch, fn):
     torch.cuda.synchronize()
     t = time.perf_counter()
@@ -218,6 +361,10 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 decode points")
     ap.add_argument("--no-weight-tiles", action="store_true",
                     help="without the second copy of the projection weights that the few-rows kernels stream")
+    ap.add_argument("--no-parts", action="store_true",
+                    help="skip the breakdown of the step's time by part of the model (a profiled step)")
+    ap.add_argument("--parts-only", action="store_true",
+                    help="print only that breakdown (what the default run starts as a child process, after its own timing)")
     ap.add_argument("--ceilings", action="store_true",
                     help="measure what a kernel that only reads, and one that only multiplies, reach on this GPU, and exit")
     ap.add_argument("--prefill-only", action="store_true",
@@ -248,10 +395,10 @@ def main() -> int:
     config = Qwen3Config.from_dict(raw)
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
     elt = 2 if dkey == "bf16" else 4
-    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    max_batch = args.batch if (args.no_points or args.parts_only) else max(args.batch, 64)
     t0 = time.time()
     engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype=args.dtype,
-                                page_size=PAGE, max_tokens=max_batch * CONTEXT, max_slots=max_batch,
+                                page_size=PAGE, max_tokens=(max_batch + 1) * CONTEXT, max_slots=max_batch + 1,
                                 max_request_tokens=CONTEXT, weight_tiles=False if args.no_weight_tiles else None)
     print(f"[bench] engine ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
     gen = torch.Generator().manual_seed(1234)
@@ -274,6 +421,7 @@ def main() -> int:
         engine.end_request(key)
         return dt
 
+
     for i in range(2):
         prefill_once(("warm", i))
     prefill_s = min(prefill_once(("prefill", i)) for i in range(3))
@@ -287,7 +435,8 @@ def main() -> int:
         return 0
 
     # ---- decode ---------------------------------------------------------------------------------
-    def decode_run(batch, steps, warmup):
+    def decode_run(batch, steps, warmup, parts=False):
+        """(seconds of `steps` timed steps, mean context); with `parts` instead the breakdown of a step's time."""
         keys = [("d", batch, i) for i in range(batch)]
         last = []
         for k in keys:
@@ -308,10 +457,32 @@ def main() -> int:
         ctx0 = engine.length(keys[0])
         dt = timed(lambda: [one_step() for _ in range(steps)])
         ctx_mean = ctx0 + (steps - 1) / 2.0 + 1
+        if parts:
+            from arle_amd.kernels import ceilings as measured
+
+            read_ceiling = measured.read_bandwidth(total_bytes=1 << 30, repeats=3)["best"]
+            mfma_ceiling = max(measured.mfma_rate(shape=32, iters=4000, repeats=2),
+                               measured.mfma_rate(shape=16, iters=4000, repeats=2))
+            ctx_now = engine.length(keys[0]) + 2
+            calls = [lambda: prefill_once(("parts", 0))] * 3 + [one_step] * 5
+            traced = profiled_steps(torch, calls)
+            out = {"ceilings": {"hbm_read_gbs": round(read_ceiling / 1e9, 1), "mfma_tflops": round(mfma_ceiling / 1e12, 1)}}
+            us, of_peak, of_ceiling = part_report(part_times(traced[:3], args.layers), part_flops_prefill(raw, PROMPT),
+                                                  PEAK_FLOPS[dkey], mfma_ceiling)
+            out.update(prefill_parts_us=us, prefill_parts_frac_peak=of_peak, prefill_parts_frac_ceiling=of_ceiling)
+            us, of_peak, of_ceiling = part_report(part_times(traced[3:], args.layers),
+                                                  part_bytes_decode(raw, batch, ctx_now, elt), PEAK_HBM_GBS * 1e9, read_ceiling)
+            out.update(decode_parts_us=us, decode_parts_frac_peak=of_peak, decode_parts_frac_ceiling=of_ceiling)
+            for k in keys:
+                engine.end_request(k)
+            return out
         for k in keys:
             engine.end_request(k)
         return dt, ctx_mean
 
+    if args.parts_only:
+        print(json.dumps(decode_run(args.batch, 4, 6, parts=True)))
+        return 0
     dt, ctx_mean = decode_run(args.batch, args.steps, args.warmup)
     ms_per_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
@@ -342,6 +513,8 @@ def main() -> int:
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
         "points": points,
     }
+    if not args.no_parts and dkey == "bf16":
+        line.update(parts_in_a_child_process(args))
     if args.batch != 8:
         line["metric"] = line["metric"].replace("batch 8", f"batch {args.batch}")
     print(json.dumps(line))
