@@ -354,9 +354,11 @@ def portion_key_splits(tokens: int, max_qlen: int, long_segments: int, num_q_hea
 
     The portions kernel gives a row block of 128 rows (tokens x q heads of a kv head) to a workgroup.  A short
     portion has fewer row blocks than the chip has compute units, however long its context: then the keys are
-    cut too, each part at least 256 keys long, and the parts are merged afterwards.  The number depends on the
-    shape of the step and on the power-of-two class of the longest context only, like the split of decoded
-    tokens, so that a captured step and an eager one choose alike.
+    cut too, each part about a thousand keys long at least (the parts are merged by a kernel of its own, which
+    writes and reads every part's rows: for a fresh 512-token prompt two parts cost more than they save), and
+    the parts are merged afterwards.  The number depends on the shape of the step and on the power-of-two class of
+    the longest context only, like the split of decoded tokens, so that a captured step and an eager one choose
+    alike.
     """
     group = num_q_heads // num_kv_heads
     blocks = -(-max_qlen * group // _PORTION_ROWS)
@@ -364,8 +366,8 @@ def portion_key_splits(tokens: int, max_qlen: int, long_segments: int, num_q_hea
     units = _compute_units(device.index if device.index is not None else torch.cuda.current_device())
     if items >= units or blocks * max(1, long_segments) > _PORTION_LIST_MAX:
         return 1
-    most = max(1, decode_split_cap(max_kv_len) // 4)
-    parts = min(-(-units // items), _PORTION_SPLITS_MAX, most)
+    most = max(1, (1 << (max(int(max_kv_len), 1).bit_length() - 1)) // 1024)    # 2 from 2,048 keys on, 4 from 4,096, ...
+    parts = min(-(-2 * units // items), _PORTION_SPLITS_MAX, most)    # up to two items a compute unit
     while parts > 1 and tokens * num_q_heads * parts * (head_dim + 2) * 4 > _PORTION_WS_BYTES:
         parts -= 1
     return parts
@@ -855,9 +857,62 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
         if out.dim() == 3 and (not partials_ok or out.numel() * 4 > _STREAM_PARTIAL_BYTES):
             out = sum_partials(out, out_dtype)
         return out
+    if partials_ok:
+        splits = library_k_splits(rows, n, k)
+        if splits > 1:
+            stack = _library_mm_split_k(x, w, splits)
+            if stack is not None:
+                return stack
     if out_dtype == torch.float32:
         return _library_mm_f32out(x, w)
     return torch.matmul(x, w.t())
+
+
+# The library runs a product with a narrow output and a long K (o and down: 2,560 columns) as a few dozen
+# workgroups that each walk all of K, and takes as long for 128 rows as for 1,024 (down of the Qwen3-4B shape: 60 us
+# at 512 rows, where reading the weights takes 10 and the products 17).  Cut into parts along K, as one batched
+# product of the parts, it fills the chip: 33 us at 512 rows, 29 at 128.  The parts come back as a float32 stack
+# for the consumer to add in order, like the stacks of the few-rows kernels (added in float32, where the single
+# product rounds its sum to bfloat16).  More parts make a larger stack to write and read, so wide outputs and
+# rows beyond 1,024 stay whole.
+_LIB_SPLIT_MAX_N = 4096
+_LIB_SPLIT_MIN_K = 2048
+_LIB_SPLIT_MAX_ROWS = 1024
+_BMM_OUT_DTYPE_OK = None
+
+
+def library_k_splits(rows: int, n: int, k: int) -> int:
+    """Into how many parts along K the library's product is cut (1: not at all)."""
+    if not (ROWS_KERNEL_MAX < rows <= _LIB_SPLIT_MAX_ROWS and n <= _LIB_SPLIT_MAX_N and k >= _LIB_SPLIT_MIN_K):
+        return 1
+    if k >= 8192:
+        splits = 8 if rows <= 256 else 4
+    else:
+        splits = 4 if rows <= 512 else 2
+    while splits > 1 and k % (32 * splits):
+        splits //= 2
+    return splits
+
+
+def _library_mm_split_k(x, w, splits: int):
+    """float32 [splits, M, N]: part s is x[:, s-th part of K] . w[:, s-th part of K]^T; None if this torch cannot
+    give a batched product float32 results."""
+    global _BMM_OUT_DTYPE_OK
+    if _BMM_OUT_DTYPE_OK is False:
+        return None
+    m, k = x.shape
+    n, part = w.shape[0], k // splits
+    xs = x.as_strided((splits, m, part), (part, x.stride(0), 1))
+    ws = w.as_strided((splits, part, n), (part, 1, k))
+    try:
+        out = torch.bmm(xs, ws, out_dtype=torch.float32)
+        _BMM_OUT_DTYPE_OK = True
+        return out
+    except (TypeError, RuntimeError):
+        if _BMM_OUT_DTYPE_OK:
+            raise
+        _BMM_OUT_DTYPE_OK = False
+        return None
 
 
 # 17..64 rows: the kernel whose workgroups stay beats the library where the output is narrow and K long (the

@@ -347,6 +347,106 @@ def decode_32b(args) -> int:
     return 0
 
 
+def sweep(args) -> int:
+    """Further sizes of the Qwen3-4B shape, one JSON line each with its fraction of the roofline: decode at batch 16
+    and 32 (2,048-token prompts), at batch 8 with 8,192 and 32,768 tokens of context, a prefill of 8,192 tokens, and
+    a 512-token prompt portion beside 8 decoding requests."""
+    import torch
+
+    from arle_amd.config import Qwen3Config
+    from arle_amd.engine import Engine, StepEntry
+    from arle_amd.kernels import ops
+
+    raw = dict(QWEN3_4B, num_hidden_layers=args.layers)
+    config = Qwen3Config.from_dict(raw)
+    longest = 32768 + 64
+    engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype="bfloat16", page_size=PAGE,
+                                max_tokens=8 * longest + 40 * 4096, max_slots=33, max_request_tokens=longest)
+    gen = torch.Generator().manual_seed(1234)
+    rand = lambda n: torch.randint(0, config.vocab_size, (n,), generator=gen).tolist()
+    base = {"n_gpus": 1, "dtype": "bf16", "higher_is_better": True, "data": "synthetic", "layers": args.layers}
+
+    def fill(keys, context, portion=8192):
+        last = []
+        for k in keys:
+            engine.add_request(k)
+            toks = rand(context)
+            for a in range(0, context, portion):
+                piece = toks[a:a + portion]
+                out = engine.step([StepEntry(k, piece, [len(piece) - 1] if a + portion >= context else [])])
+            last.append(int(ops.argmax_rows(out)[0]))
+        return last
+
+    def decode_point(batch, context, steps):
+        keys = [("s", batch, context, i) for i in range(batch)]
+        state = {"last": fill(keys, context)}
+
+        def one_step():
+            out = engine.step([StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])])
+            state["last"] = ops.argmax_rows(out).tolist()
+
+        for _ in range(6):
+            one_step()
+        dt = _timed(torch, lambda: [one_step() for _ in range(steps)]) / steps
+        ctx = engine.length(keys[0]) - steps / 2.0
+        for k in keys:
+            engine.end_request(k)
+        got = decode_bytes(raw, batch, ctx) / dt / 1e9
+        print(json.dumps(dict(base, metric=f"decode tok/s at batch {batch}, {context}-token context (Qwen3-4B shape)",
+                              value=round(batch / dt, 1), unit="tok/s", ms_per_step=round(dt * 1e3, 4), steps=steps,
+                              roofline={"bound": "hbm", "achieved": round(got, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                        "frac": round(got / PEAK_HBM_GBS, 4)})), flush=True)
+
+    def prefill_point(tokens):
+        def once(tag):
+            engine.add_request(tag)
+            toks = rand(tokens)
+            dt = _timed(torch, lambda: ops.argmax_rows(engine.step([StepEntry(tag, toks, [tokens - 1])])))
+            engine.end_request(tag)
+            return dt
+
+        once(("w", tokens, 0)), once(("w", tokens, 1))
+        dt = min(once(("p", tokens, i)) for i in range(3))
+        print(json.dumps(dict(base, metric=f"prefill tok/s at {tokens} tokens (Qwen3-4B shape)", value=round(tokens / dt, 1),
+                              unit="tok/s", ms=round(dt * 1e3, 3),
+                              frac=round(prefill_flops(raw, tokens) / dt / PEAK_FLOPS["bf16"], 4))), flush=True)
+
+    def mixed_point(decoders, context, portion, prompt):
+        keys = [("m", i) for i in range(decoders)]
+        state = {"last": fill(keys, context)}
+
+        def one_prompt(tag):
+            engine.add_request(tag)
+            toks = rand(prompt)
+            for a in range(0, prompt, portion):
+                entries = [StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])]
+                entries.append(StepEntry(tag, toks[a:a + portion], [portion - 1] if a + portion == prompt else []))
+                state["last"] = ops.argmax_rows(engine.step(entries)).tolist()[:decoders]
+            engine.end_request(tag)
+
+        one_prompt(("mw", 0)), one_prompt(("mw", 1))
+        reps, per = 4, prompt // portion
+        dt = _timed(torch, lambda: [one_prompt(("mp", i)) for i in range(reps)]) / (reps * per)
+        for k in keys:
+            engine.end_request(k)
+        flops = 2.0 * (decoders + portion) * (raw["num_hidden_layers"] * layer_params(raw) ) + 2.0 * raw["vocab_size"] * raw["hidden_size"] * (decoders + 1)
+        print(json.dumps(dict(base, metric=f"mixed step: {decoders} decoding requests at {context} tokens + a {portion}-token "
+                                           f"prompt portion (Qwen3-4B shape)", value=round((decoders + portion) / dt, 1),
+                              unit="tok/s", ms_per_step=round(dt * 1e3, 4), decode_tok_s=round(decoders / dt, 1),
+                              prefill_tok_s=round(portion / dt, 1), frac_of_matrix_peak=round(flops / dt / PEAK_FLOPS["bf16"], 4),
+                              frac_of_hbm_peak=round(decode_bytes(raw, decoders, context + 64) / dt / 1e9 / PEAK_HBM_GBS, 4))),
+              flush=True)
+
+    for batch in (16, 32):
+        decode_point(batch, 2048, args.steps)
+    for context in (8192, 32768):
+        decode_point(8, context, args.steps)
+    prefill_point(8192)
+    prefill_point(512)
+    mixed_point(8, 2048, 512, 2048)
+    return 0
+
+
 def main() -> int:
     global PAGE
     ap = argparse.ArgumentParser()
@@ -369,6 +469,9 @@ def main() -> int:
                     help="measure what a kernel that only reads, and one that only multiplies, reach on this GPU, and exit")
     ap.add_argument("--prefill-only", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiles of its kernels) and print that")
+    ap.add_argument("--sweep", action="store_true",
+                    help="further sizes of the Qwen3-4B shape (batch 16/32, 8k/32k context, 8,192-token prefill, portions "
+                         "beside decoding requests), one JSON line each")
     ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode"],
                     help="qwen3-4b is the default run; the other two are further workloads at larger shapes")
     args = ap.parse_args()
@@ -378,6 +481,8 @@ def main() -> int:
     PAGE = args.page_size
     if args.ceilings:
         return ceilings()
+    if args.sweep:
+        return sweep(args)
     if args.workload == "qwen3-4b" and args.batch is None:
         args.batch = 8
     if args.workload != "qwen3-4b":

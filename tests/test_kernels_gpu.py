@@ -752,6 +752,32 @@ def test_gemm_rows_with_fused_activation(M, inter, K):
     assert _rel(got, want) < 1e-2
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 2560, 4096), (200, 333, 2048), (512, 2560, 9728), (1024, 96, 8192), (300, 2560, 2080)])
+def test_library_product_cut_along_k_for_narrow_outputs(M, N, K):
+    """65 to 1,024 rows, a narrow output and a long K: the library's product is run as a batched product of parts
+    of K, and the parts come back as a float32 stack whose sum, in order, is the product."""
+    x = torch.randn(M, K, generator=_g(150)).bfloat16()
+    w = (torch.randn(N, K, generator=_g(151)) * 0.05).bfloat16()
+    want = x.double() @ w.double().T
+    splits = ops.library_k_splits(M, N, K)
+    assert splits == {4096: 4 if M <= 512 else 2, 2048: 4, 9728: 4, 8192: 4, 2080: 1}[K] or (K == 4096 and M == 65 and splits == 4)
+    got = ops.gemm_bf16(x.to(DEV), w.to(DEV), torch.bfloat16, partials_ok=True)
+    if splits > 1:
+        assert got.dtype == torch.float32 and got.shape == (splits, M, N)
+        part = K // splits
+        assert _rel(got[1].cpu(), x[:, part:2 * part].double() @ w[:, part:2 * part].double().T) < 1e-5
+        assert _rel(got.sum(0).cpu(), want) < 1e-5           # float32 parts: no rounding to bfloat16 in between
+    else:
+        assert got.shape == (M, N) and _rel(got.cpu(), want) < 8e-3
+    whole = ops.gemm_bf16(x.to(DEV), w.to(DEV), torch.bfloat16)           # a caller that cannot add a stack gets none
+    assert whole.shape == (M, N) and whole.dtype == torch.bfloat16 and _rel(whole.cpu(), want) < 8e-3
+    # a strided x (a view of wider rows)
+    wide = torch.randn(M, K + 64, generator=_g(152)).bfloat16().to(DEV)
+    got = ops.gemm_bf16(wide[:, :K], w.to(DEV), torch.bfloat16, partials_ok=True)
+    got = got.sum(0) if got.dim() == 3 else got
+    assert _rel(got.cpu(), wide[:, :K].cpu().double() @ w.double().T) < 8e-3
+
+
 def test_pack_weight_tiles_layout():
     """Tile (t, s), lane 16 g + i, element e is w[16 t + i, 32 s + 8 g + e]; zeros past the matrix."""
     N, K = 37, 72
