@@ -10,13 +10,15 @@ is an entry of one token and there is one call.
 """
 from __future__ import annotations
 
+import os
+
 import torch
 
 from .. import models  # noqa: F401  (registers the architectures)
 from ..cache.manager import (CacheManager, PagedNeed, cache_bytes_per_token, pages_for_memory,
                              state_bytes_per_slot)
 from ..config.registry import detect_architecture, load_model_config
-from ..models.decoder import build_model, expected_checkpoint_tensors
+from ..models.decoder import DEBUG_DUMP_ENV, build_model, expected_checkpoint_tensors
 from ..parts.base import Runtime
 from ..weights.loader import load_weights
 from ..weights.random_init import random_weights
@@ -102,7 +104,8 @@ class Engine:
         self.page_size = page_size
         self.max_request_tokens = max_request_tokens
         self.steps_run = 0
-        self.use_graphs = bool(cuda_graph) and self.model.graph_safe
+        # the debugging dump of hidden states reads them on the host after every layer: such steps are not captured
+        self.use_graphs = bool(cuda_graph) and self.model.graph_safe and os.environ.get(DEBUG_DUMP_ENV) is None
         self._graphs: dict = {}       # (rows, split cap) or a step shape -> (graph, input buffer, logits)
         self._shapes_seen: set = set()
         self.max_graphs = 64          # captured steps kept (each holds its activations)

@@ -7,6 +7,9 @@ layers, then norm and project only the rows whose logits are wanted
 """
 from __future__ import annotations
 
+import os
+import sys
+
 from ..parts import base  # noqa: F401  (registries)
 from ..parts import attention, block, embedding, feed_forward, norm, position  # noqa: F401  registers the stock parts
 from ..parts.base import Runtime, build_part, expected_tensors, lookup
@@ -25,10 +28,14 @@ def expected_checkpoint_tensors(spec: ModelSpec) -> dict:
 
     merge(expected_tensors("embedding", spec.embedding))
     for layer in spec.layers:
-        merge(expected_tensors("mixer", layer.mixer))
-        merge(expected_tensors("feed_forward", layer.feed_forward))
+        if layer.mixer is not None:
+            merge(expected_tensors("mixer", layer.mixer))
+        if layer.feed_forward is not None:
+            merge(expected_tensors("feed_forward", layer.feed_forward))
         for norm_spec in layer.norms.values():
             merge(expected_tensors("norm", norm_spec))
+        for role, part_spec in layer.parts.values():
+            merge(expected_tensors(role, part_spec))
     merge(expected_tensors("norm", spec.final_norm))
     merge(expected_tensors("head", spec.head))
     return out
@@ -43,7 +50,7 @@ def declared_cache_needs(spec: ModelSpec) -> list:
             needs.append(None)
         else:
             mixer = spec.layers[entry.layer].mixer
-            needs.append(lookup("mixer", mixer.kind).declare_cache(mixer.params))
+            needs.append(None if mixer is None else lookup("mixer", mixer.kind).declare_cache(mixer.params))
     return needs
 
 
@@ -55,6 +62,24 @@ def kv_cache_bytes_per_token(spec: ModelSpec, act_dtype) -> int:
     return cache_bytes_per_token(declared_cache_needs(spec), act_dtype)
 
 
+DEBUG_DUMP_ENV = "ARLE_AMD_DEBUG_DUMP"
+
+
+def debug_dump(residual, delta, label: str) -> None:
+    """With ARLE_AMD_DEBUG_DUMP set: one line to stderr about the hidden state of the step's last row after every
+    schedule entry (first and last values, minimum, maximum, root mean square, NaN or infinity anywhere), as the
+    reference prints with INFER_DEBUG_DUMP (infer/src/model/common.rs:85-124).  Synchronises; steps are then not
+    captured."""
+    row = residual[-1].float()
+    if delta is not None:
+        row = row + (delta.float().sum(0) if delta.dim() == 3 else delta.float())[-1]
+    row = row.cpu()
+    fmt = lambda vals: "[" + ", ".join(f"{v:+.5f}" for v in vals.tolist()) + "]"
+    print(f"[debug-dump] {label}: head={fmt(row[:8])} tail={fmt(row[-4:])} min={float(row.min()):.4f} "
+          f"max={float(row.max()):.4f} rms={float(row.pow(2).mean().sqrt()):.4f} nan={bool(row.isnan().any())} "
+          f"inf={bool(row.isinf().any())}", file=sys.stderr, flush=True)
+
+
 class DecoderModel:
     def __init__(self, spec: ModelSpec, fetch, rt: Runtime):
         spec.validate()
@@ -62,17 +87,23 @@ class DecoderModel:
         self.rt = rt
         self.embedding = build_part("embedding", spec.embedding, fetch, rt)
         self.blocks = []
+        self._extra_parts = []
         for layer in spec.layers:
-            mixer = build_part("mixer", layer.mixer, fetch, rt)
-            ffn = build_part("feed_forward", layer.feed_forward, fetch, rt)
+            mixer = build_part("mixer", layer.mixer, fetch, rt) if layer.mixer is not None else None
+            ffn = build_part("feed_forward", layer.feed_forward, fetch, rt) if layer.feed_forward is not None else None
             norms = {role: build_part("norm", s, fetch, rt) for role, s in layer.norms.items()}
-            self.blocks.append(lookup("block", layer.block)(mixer, ffn, norms))
+            if layer.parts:     # an arrangement with further parts takes them as a fourth argument
+                extra = {name: build_part(role, s, fetch, rt) for name, (role, s) in layer.parts.items()}
+                self._extra_parts.extend(extra.values())
+                self.blocks.append(lookup("block", layer.block)(mixer, ffn, norms, extra))
+            else:
+                self.blocks.append(lookup("block", layer.block)(mixer, ffn, norms))
         self.schedule = list(spec.schedule)
         self.final_norm = build_part("norm", spec.final_norm, fetch, rt)
         self.head = build_part("head", spec.head, fetch, rt)
-        parts = [self.embedding, self.final_norm, self.head]
+        parts = [self.embedding, self.final_norm, self.head, *self._extra_parts]
         for b in self.blocks:
-            parts += [b.mixer, b.feed_forward, *getattr(b, "norms", {}).values()]
+            parts += [p for p in (b.mixer, b.feed_forward) if p is not None] + list(getattr(b, "norms", {}).values())
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in parts)
 
     def cache_needs(self):
@@ -83,15 +114,21 @@ class DecoderModel:
                 needs.append(None)
                 readers[i] = entry.cache_from
             else:
-                needs.append(self.blocks[entry.layer].mixer.cache_need())
+                mixer = self.blocks[entry.layer].mixer
+                needs.append(mixer.cache_need() if mixer is not None else None)
         return needs, readers
 
     def forward(self, batch, cache):
         """Logits float32 [len(batch.want_rows), vocab] of one packed step."""
         residual = self.embedding.forward(batch.token_ids)
         delta = None
+        dump = os.environ.get(DEBUG_DUMP_ENV) is not None
+        if dump:
+            debug_dump(residual, None, "embedding")
         for i, entry in enumerate(self.schedule):
             residual, delta = self.blocks[entry.layer].forward(residual, delta, batch, cache.view(i))
+            if dump:
+                debug_dump(residual, delta, f"schedule entry {i} (layer {entry.layer})")
         wanted = self.final_norm.add_norm(residual, delta, rows=batch.want_rows)
         return self.head.forward(wanted)
 

@@ -23,7 +23,7 @@ class WeightDecl:
     """What a part expects of one parameter: its shape and how random weights fill it."""
 
     shape: tuple
-    init: str = "normal"  # "normal": N(0, std);  "ones": 1 + N(0, norm_std)
+    init: str = "normal"  # a name known to weights.random_init: "normal" N(0, std), "ones" 1 + N(0, norm_std), "zeros", ...
 
 
 @dataclass
@@ -35,10 +35,15 @@ class PartSpec:
 
 @dataclass
 class LayerSpec:
-    block: str        # arrangement, a name in the "block" registry
-    mixer: PartSpec
-    feed_forward: PartSpec
-    norms: dict       # role in the arrangement -> PartSpec of a norm
+    """One block.  Most arrangements hold one mixer, one feed-forward and their norms; an arrangement may also do
+    without one of the two (None), and may name further parts of any role in `parts`, which it is handed built
+    (a second feed-forward beside the routed one, a gate, a norm of another kind)."""
+
+    block: str                          # arrangement, a name in the "block" registry
+    mixer: PartSpec | None = None
+    feed_forward: PartSpec | None = None
+    norms: dict = field(default_factory=dict)   # role in the arrangement -> PartSpec of a norm
+    parts: dict = field(default_factory=dict)   # name -> (role, PartSpec) of further parts of the arrangement
 
 
 @dataclass(frozen=True)

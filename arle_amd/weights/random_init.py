@@ -24,17 +24,39 @@ def _tensor_seed(seed: int, name: str) -> int:
     return int.from_bytes(digest[:8], "little") & 0x7FFFFFFFFFFFFFFF
 
 
+def _init_normal(shape, gen, std, norm_std, device):
+    return torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * std
+
+
+def _init_ones(shape, gen, std, norm_std, device):
+    t = torch.ones(shape, dtype=torch.float32, device=device)
+    if norm_std:
+        t += torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * norm_std
+    return t
+
+
+def _init_zeros(shape, gen, std, norm_std, device):
+    return torch.zeros(shape, dtype=torch.float32, device=device)
+
+
+# WeightDecl.init -> how a random tensor of that kind is filled: f(shape, generator, std, norm_std, device) -> float32
+INITS = {"normal": _init_normal, "ones": _init_ones, "zeros": _init_zeros}
+
+
+def register_init(name: str, fill) -> None:
+    """Make `name` usable as WeightDecl.init: fill(shape, generator, std, norm_std, device) -> float32 tensor."""
+    INITS[name] = fill
+
+
 def random_tensor(name: str, decl, seed: int, std: float, norm_std: float, dtype, device="cpu"):
     gen = torch.Generator(device=device)
     gen.manual_seed(_tensor_seed(seed, name))
-    shape = tuple(decl.shape)
-    if decl.init == "ones":
-        t = torch.ones(shape, dtype=torch.float32, device=device)
-        if norm_std:
-            t += torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * norm_std
-    else:
-        t = torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * std
-    return t.to(dtype)
+    try:
+        fill = INITS[decl.init]
+    except KeyError:
+        raise ValueError(f"tensor '{name}': no way to fill a weight of kind {decl.init!r} is registered "
+                         f"(known: {', '.join(sorted(INITS))})") from None
+    return fill(tuple(decl.shape), gen, std, norm_std, device).to(dtype)
 
 
 def random_weights(spec, seed: int, std: float = 0.02, norm_std: float = 0.0,

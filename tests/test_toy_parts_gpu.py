@@ -372,3 +372,98 @@ def test_a_mixer_declares_the_tensors_and_types_of_its_own_paged_cache(tmp_path,
             err = float((got[(rid, p)].double() - ref[p]).abs().max() / ref.abs().max())
             assert err <= tol, f"{dtype}: request {rid} position {p}: {err:.3e}"
     assert eng.cache.free_pages() == [48]
+
+
+# ---- an arrangement without a mixer, with a further part of its own, and weights filled in other ways --------------
+
+from arle_amd.weights import register_init  # noqa: E402
+
+register_init("toy_uniform", lambda shape, gen, std, norm_std, device:
+              (torch.rand(shape, generator=gen, dtype=torch.float32, device=device) - 0.5) * 4.0 * std)
+
+
+@register("feed_forward", "toy_biased_linear")
+class BiasedLinear(Part):
+    """x W^T + b: the bias starts at zero ("zeros"), the matrix is filled uniformly ("toy_uniform")."""
+
+    @classmethod
+    def declare_weights(cls, params):
+        h = params["hidden_size"]
+        return {"w": WeightDecl((h, h), init="toy_uniform"), "b": WeightDecl((h,), init="zeros")}
+
+    def __init__(self, params, tensors, rt, children=None):
+        super().__init__(params, tensors, rt, children)
+        self.w, self.b = tensors["w"].float(), tensors["b"].float()
+
+    def forward(self, x):
+        return (x.float() @ self.w.T + self.b).to(x.dtype)
+
+
+@register("block", "toy_two_branches")
+class TwoBranches:
+    """h += feed_forward(norm(h)) + extra["second"](norm(h)): no mixer, no cache, one further part."""
+
+    def __init__(self, mixer, feed_forward, norms, extra):
+        assert mixer is None
+        self.mixer, self.feed_forward, self.norms, self.second = None, feed_forward, norms, extra["second"]
+
+    def forward(self, residual, delta, batch, cache_view):
+        assert cache_view is None
+        a = self.norms["in"].add_norm(residual, delta)
+        return residual, _whole(self.feed_forward.forward(a)) + _whole(self.second.forward(a))
+
+
+@dataclass(frozen=True)
+class BranchConfig:
+    hidden_size: int
+    intermediate_size: int
+    vocab_size: int
+    eps: float
+    max_position_embeddings: int = 64
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(**{k: raw[k] for k in cls.__dataclass_fields__})
+
+    def to_dict(self):
+        return dict(asdict(self), architectures=["ToyBranchLM"])
+
+
+def branch_spec(c: BranchConfig, stop_token_ids=()):
+    norm = lambda name: PartSpec("rmsnorm", {"width": c.hidden_size, "eps": c.eps}, {"weight": name})
+    layers = [LayerSpec("toy_two_branches",
+                        feed_forward=PartSpec("swiglu", {"hidden_size": c.hidden_size, "intermediate_size": c.intermediate_size},
+                                              {"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}),
+                        norms={"in": norm(f"l{i}.n")},
+                        parts={"second": ("feed_forward", PartSpec("toy_biased_linear", {"hidden_size": c.hidden_size},
+                                                                   {"w": f"l{i}.w", "b": f"l{i}.b"}))})
+              for i in range(2)]
+    sizes = {"vocab_size": c.vocab_size, "hidden_size": c.hidden_size}
+    return ModelSpec(hidden_size=c.hidden_size, vocab_size=c.vocab_size, max_positions=c.max_position_embeddings,
+                     embedding=PartSpec("token_table", sizes, {"table": "embed"}), layers=layers,
+                     schedule=[ScheduleEntry(0), ScheduleEntry(1)], final_norm=norm("fn"),
+                     head=PartSpec("linear", sizes, {"weight": "head"}), stop_token_ids=tuple(stop_token_ids))
+
+
+register_architecture("ToyBranchLM", BranchConfig, branch_spec)
+
+
+def test_an_arrangement_without_a_mixer_with_a_further_part_and_other_weight_fills(tmp_path):
+    c = BranchConfig(hidden_size=24, intermediate_size=40, vocab_size=50, eps=1e-5)
+    d = str(tmp_path / "branch")
+    write_random_model(d, "ToyBranchLM", c, seed=9, std=0.2, norm_std=0.05)
+    _, w = read_folder(d)
+    assert torch.count_nonzero(w["l0.b"]) == 0 and float(w["l0.w"].abs().max()) <= 0.4 + 1e-3     # the two fills
+    assert float(w["l0.w"].abs().max()) > 0.3
+    eng = Engine.from_folder(d, dtype="float32", page_size=4, max_tokens=64, max_slots=2)
+    assert eng.cache.groups == [] and eng.kv_bytes_per_token == 0                                   # no layer keeps anything
+    toks = random_tokens(19, c.vocab_size, 3)
+    got = replay.run_steps(eng, replay.portions("x", toks, sizes=(4, 1, 7, 2)))
+    wd = {k: v.double() for k, v in w.items()}
+    h = plain.embedding(wd["embed"], toks)
+    for i in range(2):
+        a = plain.rms_norm(h, wd[f"l{i}.n"], c.eps)
+        h = h + plain.swiglu_mlp(a, wd[f"l{i}.g"], wd[f"l{i}.u"], wd[f"l{i}.d"]) + a @ wd[f"l{i}.w"].T + wd[f"l{i}.b"]
+    ref = plain.linear(plain.rms_norm(h, wd["fn"], c.eps), wd["head"])
+    for pos in range(len(toks)):
+        assert float((got[("x", pos)].double() - ref[pos]).abs().max() / ref.abs().max()) <= 1e-5

@@ -175,3 +175,16 @@ def test_sharded_folder_with_index(tmp_path):
     json.dump({}, open(os.path.join(d, "model.safetensors.index.json"), "w"))
     with pytest.raises(WeightsError, match="missing weight_map"):
         load_weights(d, expected_checkpoint_tensors(_spec(TINY_A)), "cpu", torch.bfloat16)
+
+
+def test_weight_fills_are_a_registry():
+    from arle_amd.parts import WeightDecl
+    from arle_amd.weights import register_init
+    from arle_amd.weights.random_init import random_tensor
+
+    z = random_tensor("any", WeightDecl((3, 2), init="zeros"), 1, 0.5, 0.1, torch.float32)
+    assert torch.count_nonzero(z) == 0
+    register_init("test_sevens", lambda shape, gen, std, norm_std, device: torch.full(shape, 7.0, device=device))
+    assert float(random_tensor("x", WeightDecl((2,), init="test_sevens"), 1, 0.5, 0.1, torch.bfloat16).float().sum()) == 14.0
+    with pytest.raises(ValueError, match="no way to fill a weight of kind 'nope'"):
+        random_tensor("w", WeightDecl((2,), init="nope"), 1, 0.5, 0.1, torch.float32)
