@@ -448,7 +448,7 @@ def sweep(args) -> int:
 
 
 def main() -> int:
-    global PAGE
+    global PAGE, PROMPT
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
@@ -467,6 +467,8 @@ def main() -> int:
                     help="print only that breakdown (what the default run starts as a child process, after its own timing)")
     ap.add_argument("--ceilings", action="store_true",
                     help="measure what a kernel that only reads, and one that only multiplies, reach on this GPU, and exit")
+    ap.add_argument("--prompt-len", type=int, default=PROMPT,
+                    help="tokens of the prefill that --prefill-only measures (the default run's is 2,048)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiles of its kernels) and print that")
     ap.add_argument("--sweep", action="store_true",
@@ -479,6 +481,8 @@ def main() -> int:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
         return 2
     PAGE = args.page_size
+    if args.prefill_only:
+        PROMPT = args.prompt_len
     if args.ceilings:
         return ceilings()
     if args.sweep:
@@ -534,7 +538,7 @@ def main() -> int:
                "frac": round(prefill_flops(raw, PROMPT) / prefill_s / PEAK_FLOPS[dkey], 4)}
     print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
     if args.prefill_only:
-        print(json.dumps({"metric": "prefill tok/s at 2,048 tokens (Qwen3-4B shape, random weights)",
+        print(json.dumps({"metric": f"prefill tok/s at {PROMPT} tokens (Qwen3-4B shape, random weights)",
                           "value": prefill["value"], "unit": "tok/s", "n_gpus": 1, "dtype": dkey,
                           "higher_is_better": True, "prefill": prefill}))
         return 0
