@@ -904,13 +904,22 @@ __device__ __forceinline__ void load_to_lds_16(const void* base_uniform, uint32_
 // WHOLE: the page size is a multiple of the tile's 64 keys, so a tile lies in one page: its address is a
 // matter of scalar arithmetic and a lane adds an offset that never changes.  Otherwise a lane looks up the page
 // of each of its pieces.
-template <bool WHOLE>
-__global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(const AttnArgs a, int min_rows, int blocks_x,
-                                                                              int segments, int listed, int pair_up) {
+//
+// GROUPS == 2: eight waves, two groups of four that take the same 128 rows and every other tile of keys each, with
+// tiles of their own in LDS, and put their sums together through LDS at the end.  One such workgroup a CU instead
+// of two of four waves: a row block is done in half the time, which is what a launch waits for when it has about
+// as many row blocks as the chip has places for them (a causal prompt of 2,048 tokens: 512 row blocks from 1 to 32
+// tiles of keys, and the launch lasts as long as the heaviest).
+template <bool WHOLE, int GROUPS>
+__global__ __launch_bounds__(GROUPS* kDmWaves* kWave, GROUPS == 1 ? 2 : 1) void attn_prefill_dma_kernel(
+    const AttnArgs a, int min_rows, int blocks_x, int segments, int listed, int pair_up) {
   constexpr int D = kDmD;
-  extern __shared__ __align__(16) unsigned char lds_raw[];
+  extern __shared__ __align__(16) unsigned char lds_all[];
   __shared__ unsigned int item_of_workgroup;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 31, h = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, j = lane & 31, h = lane >> 5;
+  const int grp = GROUPS == 1 ? 0 : __builtin_amdgcn_readfirstlane(tid >> 8);   // the group of this wave
+  const int wave = __builtin_amdgcn_readfirstlane((tid >> 6) & 3);              // the wave inside its group
+  unsigned char* const lds_raw = lds_all + grp * (2 * kDmStageBytes);
   const int G = a.nq / a.nkv;
   const unsigned int nkv = static_cast<unsigned int>(a.nkv);
   const unsigned int pairs = listed ? g_prefill_pairs : static_cast<unsigned int>(blocks_x) * segments;
@@ -1012,9 +1021,9 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
     const int q = 64 * (4 * wave + jj) + lane;
     const int key = q / 16, pos = q % 16;
     k_key[jj] = key;
-    k_src[jj] = 8 * (pos ^ (key & 7));               // element offset of the piece inside its key row
+    k_src[jj] = 8 * (pos ^ (key & 15));              // element offset of the piece inside its key row
     const int d = q / 8, vpos = q % 8;
-    v_key[jj] = 8 * (vpos ^ (d & 7));                 // first of the piece's eight keys, inside the tile
+    v_key[jj] = 8 * (vpos ^ ((d >> 1) & 7));               // first of the piece's eight keys, inside the tile
     v_src[jj] = d * P;                                // element offset of the d row inside a page
   }
   auto fetch = [&](int tile, int stage) {
@@ -1080,25 +1089,28 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
     }
   };
 
-  if (t0 < t1) {
-    cover(t0, true);
-    fetch(t0, 0);
+  if (t0 + grp < t1) {
+    cover(t0 + grp, true);
+    fetch(t0 + grp, 0);
   }
   // The query has to be there before the loop: a wait for it inside the loop would count the tile loads in
   // flight (which the compiler does not know of) and wait for them too.
 #pragma unroll
   for (int s = 0; s < D / 16; ++s) asm volatile("" ::"v"(qreg[s]));
-  for (int tile = t0; tile < t1; ++tile) {
-    const int stage = (tile - t0) & 1;
+  // group g takes the tiles t0 + g, t0 + g + GROUPS, ...; both groups walk the loop as often as group 0 does (the
+  // barriers are the workgroup's), a group without a tile in its last round does nothing there
+  for (int first = t0; first < t1; first += GROUPS) {
+    const int tile = first + grp;
+    const int stage = ((first - t0) / GROUPS) & 1;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's pieces of the tile have landed
-    scrub(tile, stage);
+    if (tile < t1) scrub(tile, stage);
     __syncthreads();  // everybody's have; and everybody is done with the other stage
-    if (tile + 1 < t1) {
-      cover(tile + 1, false);
-      fetch(tile + 1, stage ^ 1);
+    if (tile + GROUPS < t1) {
+      cover(tile + GROUPS, false);
+      fetch(tile + GROUPS, stage ^ 1);
     }
     const int key_base = tile * kDmKeys;
-    const bool computes = wave_has_rows && key_base < wave_kv_hi && key_base + kDmKeys > wave_kv_lo;
+    const bool computes = tile < t1 && wave_has_rows && key_base < wave_kv_hi && key_base + kDmKeys > wave_kv_lo;
     if (!computes) continue;
     const unsigned char* ks = lds_raw + stage * kDmStageBytes;
     const unsigned char* vs = ks + kDmKeys * D * 2;
@@ -1115,7 +1127,7 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
         for (int t = 0; t < 2; ++t) {
           const int key = 32 * t + jk;
           kop[t][s] = __builtin_bit_cast(
-              bf16x8, *reinterpret_cast<const uint4*>(ks + key * (D * 2) + (((2 * s + h) ^ (key & 7)) * 16)));
+              bf16x8, *reinterpret_cast<const uint4*>(ks + key * (D * 2) + (((2 * s + h) ^ (key & 15)) * 16)));
         }
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -1199,7 +1211,7 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
 #pragma unroll
         for (int dt = 0; dt < D / 32; ++dt) {
           const int d = 32 * dt + j;
-          vop[k][dt] = *reinterpret_cast<const u32x4*>(vs + d * (kDmKeys * 2) + ((c ^ (d & 7)) * 16));
+          vop[k][dt] = *reinterpret_cast<const u32x4*>(vs + d * (kDmKeys * 2) + ((c ^ ((d >> 1) & 7)) * 16));
         }
       }
 #pragma unroll
@@ -1219,6 +1231,39 @@ __global__ __launch_bounds__(kDmWaves* kWave, 2) void attn_prefill_dma_kernel(co
     }
   }
   __syncthreads();  // the next item's first tile goes into stage 0: everybody has to be done reading
+
+  if constexpr (GROUPS == 2) {
+    // group 1 hands its sums to group 0 through LDS (a lane to the same lane of the same wave: 66 floats, laid out
+    // so that the 64 lanes of a wave write and read 16 contiguous bytes each): out = o_0 2^(m_0 - m) + o_1 2^(m_1 - m)
+    float* mine = reinterpret_cast<float*>(lds_all) + wave * (D / 2 + 2) * kWave;   // [wave][D / 8 + 1 pieces][lane][4]
+    if (grp == 1) {
+#pragma unroll
+      for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<float4*>(mine + ((4 * dt + q) * kWave + lane) * 4) =
+              float4{o[dt][4 * q], o[dt][4 * q + 1], o[dt][4 * q + 2], o[dt][4 * q + 3]};
+      *reinterpret_cast<float2*>(mine + (D / 8) * kWave * 4 + lane * 2) = float2{m, l};
+    }
+    __syncthreads();
+    if (grp == 1) continue;  // the barriers at the head of the loop hold it until group 0 has read
+    const float2 other = *reinterpret_cast<const float2*>(mine + (D / 8) * kWave * 4 + lane * 2);
+    const float m_all = fmaxf(m, other.x);
+    const float m_ref = m_all == -INFINITY ? 0.f : m_all;
+    const float f0 = __builtin_amdgcn_exp2f(m - m_ref), f1 = __builtin_amdgcn_exp2f(other.x - m_ref);
+    l = l * f0 + other.y * f1;
+    m = m_all;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float4 v = *reinterpret_cast<const float4*>(mine + ((4 * dt + q) * kWave + lane) * 4);
+        o[dt][4 * q] = o[dt][4 * q] * f0 + v.x * f1;
+        o[dt][4 * q + 1] = o[dt][4 * q + 1] * f0 + v.y * f1;
+        o[dt][4 * q + 2] = o[dt][4 * q + 2] * f0 + v.z * f1;
+        o[dt][4 * q + 3] = o[dt][4 * q + 3] * f0 + v.w * f1;
+      }
+  }
 
   // o[dt][r] is O^T[d = 32 dt + 8 (r / 4) + 4 h + r % 4][this lane's row]
   if (row_ok) {
@@ -1368,12 +1413,15 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
 
 static int g_prefill_pair_up = 1;
 
-int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s) {
-  const size_t lds = 2 * kDmStageBytes;
+static int g_prefill_groups = -1;  // -1: the launcher decides; 1, 2: forced (measurements and tests)
+
+template <int GROUPS>
+int launch_prefill_dma_groups(const AttnArgs& a, dim3 grid, int min_rows, int cus, hipStream_t s) {
+  const size_t lds = GROUPS * 2 * kDmStageBytes;
   static bool asked = false;  // dynamic LDS of 64 KiB and more has to be asked for, once
   if (!asked) {
-    for (const void* kernel : {reinterpret_cast<const void*>(&attn_prefill_dma_kernel<true>),
-                               reinterpret_cast<const void*>(&attn_prefill_dma_kernel<false>)}) {
+    for (const void* kernel : {reinterpret_cast<const void*>(&attn_prefill_dma_kernel<true, GROUPS>),
+                               reinterpret_cast<const void*>(&attn_prefill_dma_kernel<false, GROUPS>)}) {
       hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
       if (e != hipSuccess) {
         (void)hipGetLastError();
@@ -1382,6 +1430,28 @@ int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
     }
     asked = true;
   }
+  const long long items = static_cast<long long>(grid.x) * grid.y * grid.z * a.portion_splits;
+  const long long places = (GROUPS == 1 ? 2LL : 1LL) * cus;  // two workgroups of four waves a CU, or one of eight
+  const unsigned workgroups = static_cast<unsigned>(items < places ? items : places);
+  const int listed = static_cast<long long>(grid.x) * grid.z <= kPfPlanMax && grid.x <= 65535 && grid.z <= 65535;
+  if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);
+  attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
+                                             a.nq / a.nkv, min_rows, listed);
+  const int pair_up = GROUPS == 1 && g_prefill_pair_up ? static_cast<int>(cus / (static_cast<long long>(a.nkv) * a.portion_splits)) : 0;
+  if (a.P % kDmKeys == 0)
+    attn_prefill_dma_kernel<true, GROUPS><<<workgroups, GROUPS * kDmWaves * kWave, lds, s>>>(
+        a, min_rows, static_cast<int>(grid.x), static_cast<int>(grid.z), listed, pair_up);
+  else
+    attn_prefill_dma_kernel<false, GROUPS><<<workgroups, GROUPS * kDmWaves * kWave, lds, s>>>(
+        a, min_rows, static_cast<int>(grid.x), static_cast<int>(grid.z), listed, pair_up);
+  if (a.portion_splits > 1) {
+    const long long most = static_cast<long long>(grid.x) * grid.y * grid.z * (kPfRows / kPfWaves);
+    attn_merge_portions_kernel<<<static_cast<unsigned>(most < 4LL * cus ? most : 4LL * cus), kPfWaves * kWave, 0, s>>>(a);
+  }
+  return launch_status();
+}
+
+int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s) {
   static int cus = 0;
   if (cus == 0) {
     int dev = 0, n = 0;
@@ -1389,24 +1459,14 @@ int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
       n = 256;
     cus = n;
   }
+  // With about as many row blocks as the chip has places for workgroups of four waves (more than one for every
+  // second CU, no more than two a CU) the launch lasts as long as its heaviest row block: then every row block goes
+  // to two groups of waves.  Measured on MI355X (32 q heads over 8 kv heads, pages of 16): a fresh prompt of 2,048
+  // tokens 62 against 72 us, 1,024 tokens behind 3,072 cached 87 against 111 us; with fewer or more row blocks the
+  // one group is level or ahead (512 tokens behind 3,584: 67 against 79 us; 8,192 tokens: 590 against 608 us).
   const long long items = static_cast<long long>(grid.x) * grid.y * grid.z * a.portion_splits;
-  const unsigned workgroups = static_cast<unsigned>(items < 2LL * cus ? items : 2LL * cus);  // two of four waves a CU
-  const int listed = static_cast<long long>(grid.x) * grid.z <= kPfPlanMax && grid.x <= 65535 && grid.z <= 65535;
-  if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);
-  attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
-                                             a.nq / a.nkv, min_rows, listed);
-  const int pair_up = g_prefill_pair_up ? static_cast<int>(cus / (static_cast<long long>(a.nkv) * a.portion_splits)) : 0;
-  if (a.P % kDmKeys == 0)
-    attn_prefill_dma_kernel<true><<<workgroups, kDmWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
-                                                                           static_cast<int>(grid.z), listed, pair_up);
-  else
-    attn_prefill_dma_kernel<false><<<workgroups, kDmWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
-                                                                            static_cast<int>(grid.z), listed, pair_up);
-  if (a.portion_splits > 1) {
-    const long long most = static_cast<long long>(grid.x) * grid.y * grid.z * (kPfRows / kPfWaves);
-    attn_merge_portions_kernel<<<static_cast<unsigned>(most < 4LL * cus ? most : 4LL * cus), kPfWaves * kWave, 0, s>>>(a);
-  }
-  return launch_status();
+  const bool two = g_prefill_groups >= 0 ? g_prefill_groups == 2 : (2 * items > cus && items <= 2LL * cus);
+  return two ? launch_prefill_dma_groups<2>(a, grid, min_rows, cus, s) : launch_prefill_dma_groups<1>(a, grid, min_rows, cus, s);
 }
 
 // -1: the launcher decides (below); 1: head_dim 128 portions always run attn_prefill_dma_kernel; 0: always
@@ -1430,6 +1490,7 @@ using namespace arle;
 
 extern "C" void arle_attn_prefill_variant(int dma) { g_prefill_dma = dma; }
 extern "C" void arle_attn_prefill_pair_up(int on) { g_prefill_pair_up = on; }
+extern "C" void arle_attn_prefill_groups(int groups) { g_prefill_groups = groups; }
 
 // Token rows that the split-KV workspace holds for every segment: the most tokens of a segment whose rows
 // (tokens x q heads of a kv head) fit one row tile of 16.

@@ -573,21 +573,24 @@ def test_attention_mfma_step_too_large_for_the_work_list():
     assert _rel(out[long_n:].cpu(), torch.cat(wants)) < 8e-3
 
 
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 2])
 @pytest.mark.parametrize("nq,nkv,P", [(32, 8, 16), (8, 8, 8), (16, 1, 64), (8, 1, 32), (6, 2, 128)])
 @pytest.mark.parametrize("parts,window", [(None, 0), (1, 0), (3, 0), (8, 37), (1, 200)])
 def test_attention_mfma_both_portion_kernels_at_head_dim_128(variant, nq, nkv, P, parts, window):
     """head_dim 128 has two kernels for prompt portions (16 rows a wave with tiles parked in LDS by the waves; 32
-    rows a wave with tiles loaded straight into LDS), chosen by the shape of the step; here each is forced in turn:
-    portions that start inside a page after a cached prefix, whole prompts of several row blocks, a single first
-    token and decoded tokens beside them, windows, and keys cut into parts."""
+    rows a wave with tiles loaded straight into LDS, by one group of four waves or by two that take every other
+    tile of keys each), chosen by the shape of the step; here each is forced in turn: portions that start inside a
+    page after a cached prefix, whole prompts of several row blocks, a single first token and decoded tokens
+    beside them, windows, and keys cut into parts."""
     from arle_amd.kernels import lib
-    lib.function("arle_attn_prefill_variant")(variant)
+    lib.function("arle_attn_prefill_variant")(min(variant, 1))
+    lib.function("arle_attn_prefill_groups")(variant if variant else -1)
     try:
         got, want = _mfma_case(nq, nkv, 128, P, [(300, 70), (45, 39), (0, 1), (130, 2), (0, 330), (77, 1)], window, 1,
                                175, portion_splits=parts)
     finally:
         lib.function("arle_attn_prefill_variant")(-1)
+        lib.function("arle_attn_prefill_groups")(-1)
     assert torch.isfinite(got).all()
     assert _rel(got, want) < 8e-3
 
@@ -617,7 +620,8 @@ def test_attention_mfma_dma_kernel_masks_stale_slots(P):
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
     lib.function("arle_attn_prefill_variant")(1)
     try:
-        for parts in (1, 2):
+        for parts, groups in ((1, 1), (2, 1), (1, 2), (2, 2)):
+            lib.function("arle_attn_prefill_groups")(groups)
             out = torch.full_like(q_all, float("nan"))
             ops.attn_paged_mfma(q_all, out, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0), i32([0, 1, 2]),
                                 i32(starts), max_qlen=150, min_qlen=70, max_kv_len=max(lengths), num_q_heads=nq,
@@ -626,6 +630,7 @@ def test_attention_mfma_dma_kernel_masks_stale_slots(P):
             assert _rel(out.cpu(), torch.cat(wants)) < 8e-3
     finally:
         lib.function("arle_attn_prefill_variant")(-1)
+        lib.function("arle_attn_prefill_groups")(-1)
 
 
 def test_attention_mfma_finds_a_far_key():
