@@ -6,7 +6,11 @@
 //                       sixteen loads in flight a lane, each workgroup one contiguous part: the fastest way
 //                       found to pull bytes out of HBM3E (6.3 TB/s measured).
 //   arle_ceiling_mfma:  every wave issues `iters` rounds of eight independent v_mfma_f32_32x32x16_bf16 (or
-//                       sixteen v_mfma_f32_16x16x32_bf16) on registers; 2 * 32 * 32 * 16 flops each.
+//                       sixteen v_mfma_f32_16x16x32_bf16) on registers; 2 * 32 * 32 * 16 flops each.  The operands
+//                       are either all the same value near 1.0 or pseudo-random bits with exponents around 1.0:
+//                       the chip's clock follows its power, and products of operands whose bits differ draw more
+//                       (with all 256 compute units busy 1.65 GHz instead of 2.2 and more, measured), so the second
+//                       is the ceiling for real data.
 #include "common.h"
 
 namespace arle {
@@ -32,10 +36,13 @@ __global__ __launch_bounds__(256) void ceiling_read_kernel(const uint4* __restri
 }
 
 template <int SHAPE>
-__global__ __launch_bounds__(256) void ceiling_mfma_kernel(int iters, float* sink) {
+__global__ __launch_bounds__(256) void ceiling_mfma_kernel(int iters, int random_operands, float* sink) {
   const uint32_t seed = 0x3f803f80u + threadIdx.x;  // bfloat16 pairs near 1.0
-  const uint4 raw = {seed, seed, seed, seed};
-  const bf16x8 a = __builtin_bit_cast(bf16x8, raw), b = a;
+  // random: every 16-bit half keeps a random sign and mantissa and an exponent of 0x30..0x3f or 0xb0..0xbf
+  auto bits = [&](uint32_t mul) { return random_operands ? ((seed * mul) & 0xbfffbfffu) | 0x30003000u : seed; };
+  const uint4 raw = {bits(2654435761u), bits(40503u), bits(69069u), bits(1664525u)};
+  const uint4 raw_b = {bits(22695477u), bits(134775813u), bits(1103515245u), bits(214013u)};
+  const bf16x8 a = __builtin_bit_cast(bf16x8, raw), b = __builtin_bit_cast(bf16x8, raw_b);
   float total = 0.f;
   if constexpr (SHAPE == 32) {
     f32x16 acc[8];
@@ -82,12 +89,12 @@ extern "C" int arle_ceiling_read(const void* p, long long bytes, int workgroups,
 
 // shape 32: v_mfma_f32_32x32x16_bf16, eight a round; shape 16: v_mfma_f32_16x16x32_bf16, sixteen a round.  Either
 // way a wave does iters * 262144 flops; workgroups of four waves.
-extern "C" int arle_ceiling_mfma(int shape, int iters, int workgroups, void* sink, void* stream) {
+extern "C" int arle_ceiling_mfma(int shape, int iters, int workgroups, int random_operands, void* sink, void* stream) {
   if (workgroups < 1 || iters < 1 || (shape != 16 && shape != 32)) return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (shape == 32)
-    ceiling_mfma_kernel<32><<<workgroups, 256, 0, s>>>(iters, static_cast<float*>(sink));
+    ceiling_mfma_kernel<32><<<workgroups, 256, 0, s>>>(iters, random_operands, static_cast<float*>(sink));
   else
-    ceiling_mfma_kernel<16><<<workgroups, 256, 0, s>>>(iters, static_cast<float*>(sink));
+    ceiling_mfma_kernel<16><<<workgroups, 256, 0, s>>>(iters, random_operands, static_cast<float*>(sink));
   return launch_status();
 }

@@ -40,17 +40,20 @@ def read_bandwidth(device="cuda:0", total_bytes: int = 4 << 30, launches: int = 
     return {"bytes": total_bytes, "launches": launches, "by_workgroups": out, "best": max(out.values())}
 
 
-def mfma_rate(device="cuda:0", shape: int = 32, iters: int = 20000, repeats: int = 3) -> float:
-    """Flops a second of waves that do nothing but bfloat16 matrix-core products (16 waves a compute unit)."""
+def mfma_rate(device="cuda:0", shape: int = 32, iters: int = 20000, repeats: int = 3, random_operands: bool = True,
+              workgroups: int | None = None) -> float:
+    """Flops a second of waves that do nothing but bfloat16 matrix-core products (16 waves a compute unit, or
+    `workgroups` of four waves over the chip).  `random_operands`: operands whose bits differ, as real data's do;
+    the chip clocks lower under them than under operands that are all alike."""
     dev = torch.device(device)
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     sink = torch.zeros(4, dtype=torch.float32, device=dev)
-    wgs = cus * 4
+    wgs = workgroups or cus * 4
     best = float("inf")
     for _ in range(repeats + 1):
         torch.cuda.synchronize(dev)
         t = time.perf_counter()
-        lib.call("arle_ceiling_mfma", shape, iters, wgs, sink.data_ptr(), _stream())
+        lib.call("arle_ceiling_mfma", shape, iters, wgs, 1 if random_operands else 0, sink.data_ptr(), _stream())
         torch.cuda.synchronize(dev)
         best = min(best, time.perf_counter() - t)
     return wgs * 4 * iters * 262144.0 / best

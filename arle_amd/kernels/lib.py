@@ -51,7 +51,7 @@ SIGNATURES = {
     "arle_attn_decode_static": ("attention_mfma", [_p, _ll, _p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i,
                                                    _i, _f, _i, _i, _p]),
     "arle_ceiling_read": ("ceilings", [_p, _ll, _i, _p, _p, _p]),
-    "arle_ceiling_mfma": ("ceilings", [_i, _i, _i, _p, _p]),
+    "arle_ceiling_mfma": ("ceilings", [_i, _i, _i, _i, _p, _p]),
 }
 
 _libs: dict = {}

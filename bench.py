@@ -210,18 +210,26 @@ def _timed(torch, fn):
 
 def ceilings() -> int:
     """What a kernel that only reads memory and one that only multiplies reach on this GPU, against the published peaks."""
+    import torch
+
     from arle_amd.kernels import ceilings as c
 
     read = c.read_bandwidth()
     small = c.read_bandwidth(launches=40)
     m32, m16 = c.mfma_rate(shape=32), c.mfma_rate(shape=16)
+    same32 = c.mfma_rate(shape=32, random_operands=False)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    # one workgroup of four waves a busy compute unit: what a product costs in time says what the clock is (32 cycles)
+    by_busy = {n: c.mfma_rate(shape=32, workgroups=n, repeats=2) for n in (cus // 8, cus // 2, 3 * cus // 4, cus)}
     print(json.dumps({
         "metric": "measured ceilings of one GPU", "unit": "GB/s and TFLOP/s",
         "hbm_read_gbs": round(read["best"] / 1e9, 1), "hbm_read_frac_of_peak": round(read["best"] / 1e9 / PEAK_HBM_GBS, 4),
         "hbm_read_100mb_launches_gbs": round(small["best"] / 1e9, 1),
         "hbm_read_by_workgroups_gbs": {str(k): round(v / 1e9, 1) for k, v in read["by_workgroups"].items()},
         "mfma_bf16_32x32x16_tflops": round(m32 / 1e12, 1), "mfma_bf16_16x16x32_tflops": round(m16 / 1e12, 1),
-        "mfma_frac_of_peak": round(max(m32, m16) / PEAK_FLOPS["bf16"], 4)}))
+        "mfma_frac_of_peak": round(max(m32, m16) / PEAK_FLOPS["bf16"], 4),
+        "mfma_bf16_32x32x16_same_operands_tflops": round(same32 / 1e12, 1),
+        "mfma_clock_ghz_by_busy_cus": {str(n): round(v / (n * 4 * 32768.0 / 32.0) / 1e9, 2) for n, v in by_busy.items()}}))
     return 0
 
 

@@ -944,4 +944,6 @@ def test_measuring_kernels_give_plausible_ceilings():
     parts = ceilings.read_bandwidth(DEV, total_bytes=256 << 20, launches=4, repeats=2)
     assert 0.5e12 < parts["best"] < 8.0e12
     for shape in (16, 32):
-        assert 2.5e14 < ceilings.mfma_rate(DEV, shape=shape, iters=2000, repeats=1) < 2.6e15
+        for random_operands in (False, True):
+            rate = ceilings.mfma_rate(DEV, shape=shape, iters=2000, repeats=1, random_operands=random_operands)
+            assert 2.5e14 < rate < 2.6e15
