@@ -9,9 +9,9 @@
 // the matrix cores, 2.4 PFLOP/s measured over the chip, the latter at 1.4.)
 //
 //   * X goes through registers into LDS in operand order: a lane fetches 16 bytes of a (16 rows x 32 k) piece,
-//     64 contiguous bytes a row, and parks them where the lane (row j, half h) of the 32 x 16 operand will read
-//     them, at (operand * 64 + 32 h + j) * 16.  Reads are linear in the lane, writes linear in runs of 16 lanes:
-//     no bank conflicts, no padding, no swizzle.  Two stages.
+//     four neighbouring lanes the 64 contiguous bytes of a row, and parks them where the lane (row j, half h) of
+//     the 32 x 16 operand will read them.  Reads are linear in the lane inside a half; the halves are padded so that
+//     the writes of neighbouring lanes meet different banks.  Two stages.
 //   * Both streams run ahead of the products through rings of registers (PD and PX steps of 32 k).  Nothing is
 //     selected or converted behind a load: a use right behind a load is a wait for that load.
 //   * The operand reads of a step are pinned four reads ahead of the products that need them.  PIPE: four LDS
@@ -61,7 +61,8 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
   static_assert(PD % 2 == 0 && PD % PX == 0, "rounds of PD steps; the LDS stage alternates; the X ring divides the W ring");
   static_assert(MT % 2 == 0, "every wave fetches whole pieces of 16 rows");
   static_assert(!PIPE || PD == 4, "the pipelined loop walks four LDS stages in a round of four steps");
-  constexpr int kRows = 32 * MT, kStage = kRows * 32 * 2;  // bytes of one LDS stage: the rows' 32 k
+  constexpr int kHalf = 576, kPiece = 2 * kHalf;             // an operand's two halves of 512 bytes, 64 bytes of padding behind each
+  constexpr int kRows = 32 * MT, kStage = 2 * MT * kPiece;  // bytes of one LDS stage: the rows' 32 k
   constexpr int XH = 2 * MT / kTlWaves;                    // pieces of 16 rows x 32 k that a wave fetches a step
   constexpr int kOutPitch = 144;  // bytes of a row of 64 bfloat16 in the epilogue's LDS, padded against bank conflicts
   constexpr int kOutBytes = kTlWaves * 32 * kOutPitch;
@@ -94,26 +95,32 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) dst[tn][kk] = *reinterpret_cast<const bf16x8*>(wptr[tn] + off + kk * 256);
   };
-  // X: wave w fetches row tile w as two pieces of 16 rows x 32 k, lane (li, g) the 16 bytes of row li, k 8 g .. + 7,
-  // and parks them where the lane (j = 16 half + li, h = g % 2) of the operand of half kk = g / 2 will read them.
+  // X: a fetch is 16 rows x 32 k, four lanes a row (64 contiguous bytes), so that four neighbouring lanes ask for one
+  // piece of a cache line (the memory pipeline takes the lanes of a load four at a time: with a lane a row it had
+  // four times the requests).  Lane 4 r + c holds row r, k 8 c .. + 7 and parks it where lane (j = 16 half + r,
+  // h = c % 2) of the operand of half kk = c / 2 reads it.  An operand in LDS is its two halves h of 512 bytes with 64
+  // bytes of padding behind each: the four pieces that four neighbouring lanes park (c = 0 .. 3) then fall into
+  // different banks, and sixteen lanes in a row of either access never share one.
   // A piece past K is fetched from a place that exists and meets the zeros that the tiles hold there.
+  const int fr = lane >> 2, fc = lane & 3;
   const uint16_t* xptr[XH];
 #pragma unroll
   for (int p = 0; p < XH; ++p)
-    xptr[p] = a.x + static_cast<int64_t>(min(m0 + 16 * (XH * wave + p) + li, M - 1)) * a.ldx;
+    xptr[p] = a.x + static_cast<int64_t>(min(m0 + 16 * (XH * wave + p) + fr, M - 1)) * a.ldx;
   auto load_x = [&](int s, u32x4 (&dst)[XH]) {
-    const int col = 32 * s + 8 * g;
+    const int col = 32 * s + 8 * fc;
     const int at = col < K ? col : 0;
 #pragma unroll
     for (int p = 0; p < XH; ++p) dst[p] = *reinterpret_cast<const u32x4*>(xptr[p] + at);
   };
   // piece p of the wave is half (XH wave + p) % 2 of row tile (XH wave + p) / 2; XH is even, so p / 2 and p % 2 do
-  const int park_at = ((XH / 2 * wave) * 2 + (g >> 1)) * 1024 + (32 * (g & 1) + li) * 16;
+  const int park_at = ((XH / 2 * wave) * 2 + (fc >> 1)) * kPiece + (fc & 1) * kHalf + fr * 16;
   auto park_x = [&](int stage, const u32x4 (&src)[XH]) {
 #pragma unroll
     for (int p = 0; p < XH; ++p)
-      *reinterpret_cast<u32x4*>(lds + stage * kStage + park_at + (p / 2) * 2048 + (p % 2) * 256) = src[p];
+      *reinterpret_cast<u32x4*>(lds + stage * kStage + park_at + (p / 2) * 2 * kPiece + (p % 2) * 256) = src[p];
   };
+  const int read_at = h * kHalf + j * 16;   // this lane's place in an operand
 
   f32x16 acc[MT][2];
 #pragma unroll
@@ -137,12 +144,12 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
   __syncthreads();
 
   auto multiply = [&](const bf16x8 (&wt)[2][2], int stage) {  // the step parked in `stage` with its tiles
-    const unsigned char* xs = lds + stage * kStage + lane * 16;
+    const unsigned char* xs = lds + stage * kStage + read_at;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        const bf16x8 xop = *reinterpret_cast<const bf16x8*>(xs + (2 * t + kk) * 1024);
+        const bf16x8 xop = *reinterpret_cast<const bf16x8*>(xs + (2 * t + kk) * kPiece);
 #pragma unroll
         for (int tn = 0; tn < 2; ++tn)
           acc[t][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wt[tn][kk], xop, acc[t][tn], 0, 0, 0);
@@ -166,12 +173,24 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
     constexpr int kA = 4, kR = 2 * MT;
     bf16x8 pre[kA];
 #pragma unroll
-    for (int i = 0; i < kA; ++i) pre[i] = *reinterpret_cast<const bf16x8*>(lds + 2 * i * 1024 + lane * 16);  // row tiles 0 .. kA - 1, half 0
-    auto step = [&](bf16x8 (&wt)[2][2], u32x4 (&xnext)[XH], int u, int s, bool fetch) {
+    for (int i = 0; i < kA; ++i) pre[i] = *reinterpret_cast<const bf16x8*>(lds + 2 * i * kPiece + read_at);  // row tiles 0 .. kA - 1, half 0
+    // The step's eight loads go out one at a time between the products, two operand reads and four products
+    // apart (sent together they queue in the memory pipeline, and a wave that cannot send a load cannot send the
+    // product behind it either): first the halves kk = 1 of the step before, whose registers are free since its
+    // last product, then the four pieces of X, then the halves kk = 0 of this step, free after its first half.
+    auto load_w1 = [&](int s, bf16x8& dst, int tn, int kk) {
+      const int64_t off = static_cast<int64_t>(min(s, steps - 1)) * 512;
+      dst = *reinterpret_cast<const bf16x8*>(wptr[tn] + off + kk * 256);
+    };
+    auto load_x1 = [&](int s, u32x4& dst, int p) {
+      const int col = 32 * s + 8 * fc;
+      dst = *reinterpret_cast<const u32x4*>(xptr[p] + (col < K ? col : 0));
+    };
+    static_assert(2 + XH + 2 <= MT, "a load behind every second operand read of a step");
+    auto step = [&](bf16x8 (&wt)[2][2], bf16x8 (&wprev)[2][2], u32x4 (&xnext)[XH], int u, int s, bool fetch) {
       park_x((u + 1) & 3, xnext);
-      if (fetch) load_x(s + 1 + PX, xnext);
-      const unsigned char* cur = lds + (u & 3) * kStage + lane * 16;
-      const unsigned char* nxt = lds + ((u + 1) & 3) * kStage + lane * 16;
+      const unsigned char* cur = lds + (u & 3) * kStage + read_at;
+      const unsigned char* nxt = lds + ((u + 1) & 3) * kStage + read_at;
       bf16x8 xo[kR];
 #pragma unroll
       for (int i = 0; i < kA; ++i) xo[i] = pre[i];
@@ -180,26 +199,35 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
         if (r == kR - kA) __syncthreads();
         // read r is the operand of row tile r % MT, half r / MT of the step: the two products into one
         // accumulator are 2 MT products apart (a product right behind one into the same accumulator waits for it)
-        constexpr auto at = [](int q) { return (2 * (q % MT) + q / MT) * 1024; };
+        constexpr auto at = [](int q) { return (2 * (q % MT) + q / MT) * kPiece; };
         if (r + kA < kR)
           xo[r + kA] = *reinterpret_cast<const bf16x8*>(cur + at(r + kA));
         else
           pre[r + kA - kR] = *reinterpret_cast<const bf16x8*>(nxt + at(r + kA - kR));
+        if (fetch && (r & 1)) {
+          const int q = r >> 1;
+          if (q < 2)
+            load_w1(s - 1 + PD, wprev[q][1], q, 1);   // in the first step: the same tiles as before the loop, again
+          else if (q < 2 + XH)
+            load_x1(s + 1 + PX, xnext[q - 2], q - 2);
+          else
+            load_w1(s + PD, wt[q - 2 - XH][0], q - 2 - XH, 0);
+        }
 #pragma unroll
         for (int tn = 0; tn < 2; ++tn)
           acc[r % MT][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wt[tn][r / MT], xo[r], acc[r % MT][tn], 0, 0, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (r & 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
       }
-      if (fetch) load_w(s + PD, wt);
     };
     for (int r = 0; r < rounds; ++r) {
 #pragma unroll
-      for (int u = 0; u < PD; ++u) step(wring[u], xring[u % PX], u, r * PD + u, true);
+      for (int u = 0; u < PD; ++u) step(wring[u], wring[(u + PD - 1) % PD], xring[u % PX], u, r * PD + u, true);
     }
 #pragma unroll
     for (int u = 0; u < PD - 1; ++u)
-      if (u < rest) step(wring[u], xring[u % PX], u, rounds * PD + u, false);
+      if (u < rest) step(wring[u], wring[(u + PD - 1) % PD], xring[u % PX], u, rounds * PD + u, false);
   } else {
   for (int r = 0; r < rounds; ++r) {
 #pragma unroll
