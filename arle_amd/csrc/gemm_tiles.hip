@@ -40,8 +40,6 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // a plain vector: arrays of HIP's uint4 structs end up in scratch memory
 
-constexpr int kTlWaves = 4;
-constexpr int kTlCols = 64 * kTlWaves;  // columns a workgroup owns
 constexpr int kTlXcds = 8;
 constexpr int kEpiNone = 0, kEpiSiluMul = 1;
 
@@ -53,18 +51,28 @@ struct TilesArgs {
   int64_t ldo;
   int M, N, K;
   int m_blocks, n_blocks;
+  int steps_per_split;    // steps of 32 k that one workgroup walks: blockIdx.y picks the part of K
+  int64_t split_stride;   // elements between the parts' results in `out` (a float32 stack [parts][M][N])
 };
 
-// MT: row tiles of 32 that a workgroup owns (4: 128 rows, two workgroups a compute unit)
-template <int MT, int PD, int PX, bool PIPE, int EPI, typename TOut>
-__global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_kernel(const TilesArgs a) {
+// MT: row tiles of 32 that a workgroup owns (4: 128 rows); TN: column tiles of 32 that a wave owns (2: 256
+// columns a workgroup; 1: 128, for products with so few rows that they are a matter of streaming W, where more and
+// smaller workgroups keep more loads in flight; kTlWaves = 2 halves the workgroup once more).  gridDim.y parts of K,
+// each leaving a result of its own.
+template <int MT, int TN, int PD, int PX, bool PIPE, int EPI, typename TOut, int kTlWaves = 4>
+// (the second figure is waves a SIMD: the registers a wave may have)
+__global__ __launch_bounds__(kTlWaves* kWave, MT* TN >= 16 ? 1 : (MT * TN >= 8 || PD >= 8 ? 2 : 3))
+void gemm_tiles_kernel(const TilesArgs a) {
+  static_assert(kTlWaves == 4 || kTlWaves == 2, "four waves a workgroup, or two");
+  static_assert(!PIPE || TN == 2, "the pipelined loop is written for two column tiles a wave");
+  constexpr int kTlCols = 32 * TN * kTlWaves;  // columns a workgroup owns
   static_assert(PD % 2 == 0 && PD % PX == 0, "rounds of PD steps; the LDS stage alternates; the X ring divides the W ring");
   static_assert(MT % 2 == 0, "every wave fetches whole pieces of 16 rows");
   static_assert(!PIPE || PD == 4, "the pipelined loop walks four LDS stages in a round of four steps");
   constexpr int kHalf = 576, kPiece = 2 * kHalf;             // an operand's two halves of 512 bytes, 64 bytes of padding behind each
   constexpr int kRows = 32 * MT, kStage = 2 * MT * kPiece;  // bytes of one LDS stage: the rows' 32 k
   constexpr int XH = 2 * MT / kTlWaves;                    // pieces of 16 rows x 32 k that a wave fetches a step
-  constexpr int kOutPitch = 144;  // bytes of a row of 64 bfloat16 in the epilogue's LDS, padded against bank conflicts
+  constexpr int kOutPitch = 64 * TN + 16;  // bytes of a wave's row of bfloat16 in the epilogue's LDS, padded against bank conflicts
   constexpr int kOutBytes = kTlWaves * 32 * kOutPitch;
   constexpr int kLdsBytes = (PIPE ? 4 : 2) * kStage > kOutBytes ? (PIPE ? 4 : 2) * kStage : kOutBytes;
   __shared__ __align__(16) unsigned char lds[kLdsBytes];
@@ -77,21 +85,23 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
   const int xcd = blockIdx.x % kTlXcds, q = blockIdx.x / kTlXcds;
   const int mb = q % a.m_blocks, nb = (q / a.m_blocks) * kTlXcds + xcd;
   if (nb >= a.n_blocks) return;  // the whole workgroup
-  const int m0 = mb * kRows, n0 = nb * kTlCols + wave * 64;
+  const int m0 = mb * kRows, n0 = nb * kTlCols + wave * (32 * TN);
   const int M = a.M, N = a.N, K = a.K;
   const int steps = (K + 31) / 32, n_tiles = (N + 15) / 16;
-  const int rounds = steps / PD, rest = steps % PD;  // whole rounds of the rings, and the steps after them
+  const int s_begin = blockIdx.y * a.steps_per_split;                 // this workgroup's part of K
+  const int n_steps = min(a.steps_per_split, steps - s_begin);
+  const int rounds = n_steps / PD, rest = n_steps % PD;  // whole rounds of the rings, and the steps after them
 
   // W operand of column tile tn (32 columns), half kk of a step: lane (j, h) takes the piece that lane
   // 16 (2 kk + h) + j % 16 of the 16-column tile 2 tn + j / 16 holds: k = 32 s + 16 kk + 8 h .. + 7
-  const uint16_t* wptr[2];
+  const uint16_t* wptr[TN];
 #pragma unroll
-  for (int tn = 0; tn < 2; ++tn)
+  for (int tn = 0; tn < TN; ++tn)
     wptr[tn] = a.w + static_cast<int64_t>(min(n0 / 16 + 2 * tn + (j >> 4), n_tiles - 1)) * steps * 512 + (16 * h + (j & 15)) * 8;
-  auto load_w = [&](int s, bf16x8 (&dst)[2][2]) {
-    const int64_t off = static_cast<int64_t>(min(s, steps - 1)) * 512;  // a step past K is fetched and never multiplied
+  auto load_w = [&](int s, bf16x8 (&dst)[TN][2]) {   // s: step inside this workgroup's part
+    const int64_t off = static_cast<int64_t>(min(s_begin + s, steps - 1)) * 512;  // a step past K is fetched and never multiplied
 #pragma unroll
-    for (int tn = 0; tn < 2; ++tn)
+    for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) dst[tn][kk] = *reinterpret_cast<const bf16x8*>(wptr[tn] + off + kk * 256);
   };
@@ -108,7 +118,7 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
   for (int p = 0; p < XH; ++p)
     xptr[p] = a.x + static_cast<int64_t>(min(m0 + 16 * (XH * wave + p) + fr, M - 1)) * a.ldx;
   auto load_x = [&](int s, u32x4 (&dst)[XH]) {
-    const int col = 32 * s + 8 * fc;
+    const int col = 32 * (s_begin + s) + 8 * fc;
     const int at = col < K ? col : 0;
 #pragma unroll
     for (int p = 0; p < XH; ++p) dst[p] = *reinterpret_cast<const u32x4*>(xptr[p] + at);
@@ -122,15 +132,15 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
   };
   const int read_at = h * kHalf + j * 16;   // this lane's place in an operand
 
-  f32x16 acc[MT][2];
+  f32x16 acc[MT][TN];
 #pragma unroll
   for (int t = 0; t < MT; ++t)
 #pragma unroll
-    for (int tn = 0; tn < 2; ++tn)
+    for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[t][tn][r] = 0.f;
 
-  bf16x8 wring[PD][2][2];
+  bf16x8 wring[PD][TN][2];
   u32x4 xring[PX][XH];  // slot u % PX holds step (round * PD + u) + 1: the one parked while step u is multiplied
 #pragma unroll
   for (int u = 0; u < PD; ++u) load_w(u, wring[u]);
@@ -143,7 +153,7 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
   }
   __syncthreads();
 
-  auto multiply = [&](const bf16x8 (&wt)[2][2], int stage) {  // the step parked in `stage` with its tiles
+  auto multiply = [&](const bf16x8 (&wt)[TN][2], int stage) {  // the step parked in `stage` with its tiles
     const unsigned char* xs = lds + stage * kStage + read_at;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
@@ -151,7 +161,7 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
       for (int t = 0; t < MT; ++t) {
         const bf16x8 xop = *reinterpret_cast<const bf16x8*>(xs + (2 * t + kk) * kPiece);
 #pragma unroll
-        for (int tn = 0; tn < 2; ++tn)
+        for (int tn = 0; tn < TN; ++tn)
           acc[t][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wt[tn][kk], xop, acc[t][tn], 0, 0, 0);
       }
     // operand reads run kAhead reads (2 kAhead products) ahead of the products that need them; left to itself the
@@ -160,10 +170,10 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
     __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
 #pragma unroll
     for (int i = 0; i < kReads - kAhead; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, TN, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 2 * kAhead, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, TN * kAhead, 0);
   };
   if constexpr (PIPE) {
     // Four stages, so that a step can be parked two steps before anybody reads its stage again, and the barrier of
@@ -179,11 +189,11 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
     // product behind it either): first the halves kk = 1 of the step before, whose registers are free since its
     // last product, then the four pieces of X, then the halves kk = 0 of this step, free after its first half.
     auto load_w1 = [&](int s, bf16x8& dst, int tn, int kk) {
-      const int64_t off = static_cast<int64_t>(min(s, steps - 1)) * 512;
+      const int64_t off = static_cast<int64_t>(min(s_begin + s, steps - 1)) * 512;
       dst = *reinterpret_cast<const bf16x8*>(wptr[tn] + off + kk * 256);
     };
     auto load_x1 = [&](int s, u32x4& dst, int p) {
-      const int col = 32 * s + 8 * fc;
+      const int col = 32 * (s_begin + s) + 8 * fc;
       dst = *reinterpret_cast<const u32x4*>(xptr[p] + (col < K ? col : 0));
     };
     static_assert(2 + XH + 2 <= MT, "a load behind every second operand read of a step");
@@ -255,12 +265,12 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
   }
 
   // acc[t][tn][r] = C[m0 + 32 t + j][n0 + 32 tn + 8 (r / 4) + 4 h + r % 4]
-  TOut* out = static_cast<TOut*>(a.out);
-  // bfloat16 results whose 64 columns all exist: a lane holds pieces of 8 bytes, and stored as they are they
+  TOut* out = static_cast<TOut*>(a.out) + static_cast<int64_t>(blockIdx.y) * a.split_stride;
+  // bfloat16 results whose columns (64 a wave, or 32) all exist: a lane holds pieces of 8 bytes, and stored as they are they
   // would reach memory as 16-byte scraps of a row (a third of the kernel's time at 2,048 x 6,144).  So every
   // row tile goes through a part of LDS that belongs to the wave and leaves as whole rows of 128 (with the
   // activation: 64) contiguous bytes, eight (four) lanes a row.
-  constexpr int kOutCols = EPI == kEpiSiluMul ? 32 : 64;
+  constexpr int kOutCols = EPI == kEpiSiluMul ? 16 * TN : 32 * TN;
   if constexpr (sizeof(TOut) == 2) {
     const int c0 = EPI == kEpiSiluMul ? n0 / 2 : n0;          // first output column of the wave
     const int n_out = EPI == kEpiSiluMul ? N / 2 : N;
@@ -271,7 +281,7 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
 #pragma unroll
-        for (int tn = 0; tn < 2; ++tn) {
+        for (int tn = 0; tn < TN; ++tn) {
           if constexpr (EPI == kEpiSiluMul) {
 #pragma unroll
             for (int q4 = 0; q4 < 2; ++q4) {
@@ -315,7 +325,7 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
     const int row = m0 + 32 * t + j;
     if (row >= M) continue;
 #pragma unroll
-    for (int tn = 0; tn < 2; ++tn) {
+    for (int tn = 0; tn < TN; ++tn) {
       if constexpr (EPI == kEpiSiluMul) {
         // the 32 columns are 16 gate and the 16 matching up columns: registers r and r + 8
 #pragma unroll
@@ -363,23 +373,25 @@ __global__ __launch_bounds__(kTlWaves* kWave, MT == 4 ? 2 : 1) void gemm_tiles_k
   }
 }
 
-template <int MT, int PD, int PX, bool PIPE, int EPI>
-int launch_tiles(TilesArgs a, int out_dtype, hipStream_t s) {
+template <int MT, int TN, int PD, int PX, bool PIPE, int EPI, int kTlWaves = 4>
+int launch_tiles(TilesArgs a, int splits, int out_dtype, hipStream_t s) {
   a.m_blocks = (a.M + 32 * MT - 1) / (32 * MT);
+  a.n_blocks = (a.N + 32 * TN * kTlWaves - 1) / (32 * TN * kTlWaves);
   const long long n_groups = (a.n_blocks + kTlXcds - 1) / kTlXcds;
   const long long grid = n_groups * a.m_blocks * kTlXcds;
   if (grid > 0x7fffffffLL) return static_cast<int>(hipErrorInvalidValue);
+  const dim3 blocks(static_cast<unsigned>(grid), static_cast<unsigned>(splits));
   if (out_dtype == kF32)
-    gemm_tiles_kernel<MT, PD, PX, PIPE, EPI, float><<<static_cast<unsigned>(grid), kTlWaves * kWave, 0, s>>>(a);
+    gemm_tiles_kernel<MT, TN, PD, PX, PIPE, EPI, float, kTlWaves><<<blocks, kTlWaves * kWave, 0, s>>>(a);
   else
-    gemm_tiles_kernel<MT, PD, PX, PIPE, EPI, bf16><<<static_cast<unsigned>(grid), kTlWaves * kWave, 0, s>>>(a);
+    gemm_tiles_kernel<MT, TN, PD, PX, PIPE, EPI, bf16, kTlWaves><<<blocks, kTlWaves * kWave, 0, s>>>(a);
   return launch_status();
 }
 
-template <int MT, int PD, int PX, bool PIPE = false>
-int dispatch_tiles(const TilesArgs& a, int out_dtype, int epilogue, hipStream_t s) {
-  return epilogue ? launch_tiles<MT, PD, PX, PIPE, kEpiSiluMul>(a, out_dtype, s)
-                  : launch_tiles<MT, PD, PX, PIPE, kEpiNone>(a, out_dtype, s);
+template <int MT, int TN, int PD, int PX, bool PIPE = false, int kTlWaves = 4>
+int dispatch_tiles(const TilesArgs& a, int splits, int out_dtype, int epilogue, hipStream_t s) {
+  return epilogue ? launch_tiles<MT, TN, PD, PX, PIPE, kEpiSiluMul, kTlWaves>(a, splits, out_dtype, s)
+                  : launch_tiles<MT, TN, PD, PX, PIPE, kEpiNone, kTlWaves>(a, splits, out_dtype, s);
 }
 
 }  // namespace arle
@@ -388,20 +400,35 @@ using namespace arle;
 
 // x [M, K] bfloat16 (row stride ldx, a multiple of 8), w_tiles the operand tiles of W [N, K], K % 8 == 0.
 // out [M, N] (epilogue 0) or [M, N/2] (epilogue 1: N % 32 == 0, gate and up rows of W interleaved in blocks of 16),
-// bfloat16 or float32, row stride ldo.  row_tiles: row tiles of 32 a workgroup (4 or 8); depth: ring depths of W and X
-// as two digits (22, 44), + 100 for the loop with the barrier in mid-step (8 row tiles only).
+// bfloat16 or float32, row stride ldo.  row_tiles: row tiles of 32 a workgroup (4 or 8); col_tiles: column tiles of
+// 32 a wave (2, or 1 with 4 row tiles); depth: ring depths of W and X as two digits (22, 44, 84), + 100 for the loop
+// with the barrier in mid-step (8 row tiles only), + 200 for workgroups of two waves (one column tile a wave only).  splits > 1: K is cut into parts of steps_per_split steps of 32
+// (splits of them cover it), and part p leaves its product at out + p * split_stride as float32, no epilogue.
 extern "C" int arle_gemm_tiles(const void* x, long long ldx, const void* w_tiles, void* out, long long ldo, int out_dtype,
-                               int M, int N, int K, int epilogue, int row_tiles, int depth, void* stream) {
+                               int M, int N, int K, int epilogue, int row_tiles, int col_tiles, int depth, int splits,
+                               int steps_per_split, long long split_stride, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || K % 8 != 0 || ldx % 8 != 0 || (epilogue != kEpiNone && epilogue != kEpiSiluMul) ||
-      (epilogue == kEpiSiluMul && N % 32 != 0))
+      (epilogue == kEpiSiluMul && N % 32 != 0) || splits < 1 || splits > 65535 || steps_per_split < 1)
     return static_cast<int>(hipErrorInvalidValue);
+  const int steps = (K + 31) / 32;
+  if (static_cast<long long>(splits - 1) * steps_per_split >= steps || static_cast<long long>(splits) * steps_per_split < steps)
+    return static_cast<int>(hipErrorInvalidValue);
+  if (splits > 1 && (out_dtype != kF32 || epilogue != kEpiNone)) return static_cast<int>(hipErrorInvalidValue);
   const TilesArgs a{static_cast<const uint16_t*>(x), ldx, static_cast<const uint16_t*>(w_tiles), out, ldo, M, N, K,
-                    0, (N + kTlCols - 1) / kTlCols};
+                    0, 0, steps_per_split, split_stride};
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (row_tiles == 4 && depth == 22) return dispatch_tiles<4, 2, 2>(a, out_dtype, epilogue, s);
-  if (row_tiles == 4 && depth == 44) return dispatch_tiles<4, 4, 4>(a, out_dtype, epilogue, s);
-  if (row_tiles == 8 && depth == 44) return dispatch_tiles<8, 4, 4>(a, out_dtype, epilogue, s);
-  if (row_tiles == 8 && depth == 144) return dispatch_tiles<8, 4, 4, true>(a, out_dtype, epilogue, s);
+  if (col_tiles == 2) {
+    if (row_tiles == 4 && depth == 22) return dispatch_tiles<4, 2, 2, 2>(a, splits, out_dtype, epilogue, s);
+    if (row_tiles == 4 && depth == 44) return dispatch_tiles<4, 2, 4, 4>(a, splits, out_dtype, epilogue, s);
+    if (row_tiles == 8 && depth == 44) return dispatch_tiles<8, 2, 4, 4>(a, splits, out_dtype, epilogue, s);
+    if (row_tiles == 8 && depth == 144) return dispatch_tiles<8, 2, 4, 4, true>(a, splits, out_dtype, epilogue, s);
+  } else if (col_tiles == 1) {
+    if (row_tiles == 4 && depth == 44) return dispatch_tiles<4, 1, 4, 4>(a, splits, out_dtype, epilogue, s);
+    if (row_tiles == 4 && depth == 84) return dispatch_tiles<4, 1, 8, 4>(a, splits, out_dtype, epilogue, s);
+    if (row_tiles == 4 && depth == 66) return dispatch_tiles<4, 1, 6, 6>(a, splits, out_dtype, epilogue, s);
+    if (row_tiles == 4 && depth == 88) return dispatch_tiles<4, 1, 8, 8>(a, splits, out_dtype, epilogue, s);
+    if (row_tiles == 4 && depth == 288) return dispatch_tiles<4, 1, 8, 8, false, 2>(a, splits, out_dtype, epilogue, s);
+  }
   return static_cast<int>(hipErrorInvalidValue);
 }

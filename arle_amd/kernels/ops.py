@@ -787,14 +787,18 @@ def gemm_tiles_preferred(rows: int, n: int, k: int, x_stride: int, fused: bool =
             and k % 8 == 0 and x_stride % 8 == 0)
 
 
-# (row tiles of 32 a workgroup, ring depths W|X; 1xx: the loop with the barrier in mid-step and four LDS stages)
-TILES_VARIANTS = ((4, 22), (4, 44), (8, 44), (8, 144))
+# (row tiles of 32 a workgroup, ring depths W|X; 1xx: the loop with the barrier in mid-step and four LDS stages;
+#  2xx: workgroups of two waves[,
+#  column tiles of 32 a wave: 2 unless given])
+TILES_VARIANTS = ((4, 22), (4, 44), (8, 44), (8, 144), (4, 44, 1), (4, 84, 1), (4, 66, 1), (4, 88, 1), (4, 288, 1))
 
 
-def gemm_tiles(x, tiles, n: int, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, variant=None):
+def gemm_tiles(x, tiles, n: int, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, variant=None, splits: int = 1):
     """x [M, K] . W^T for many rows, W [n, K] given as its operand tiles (pack_weight_tiles): workgroups of
-    128 or 256 rows x 256 columns, W straight from memory into the matrix cores, x through LDS.
-    EPI_SILU_MUL: gate and up rows of W interleaved in blocks of 16; returns [M, n/2]."""
+    128 or 256 rows x 256 (or 128) columns, W straight from memory into the matrix cores, x through LDS.
+    EPI_SILU_MUL: gate and up rows of W interleaved in blocks of 16; returns [M, n/2].
+    splits > 1: K cut into that many parts (of whole steps of 32), one workgroup each; returns the float32 stack
+    [splits, M, n] for the caller to add in order."""
     _gpu(x, tiles)
     _rows(x, "x")
     _need(x.dtype == torch.bfloat16, "gemm_tiles takes bfloat16 operands")
@@ -807,9 +811,20 @@ def gemm_tiles(x, tiles, n: int, out_dtype=torch.bfloat16, epilogue: int = EPI_N
     if variant is None:
         variant = (8, 144) if M >= _TILES_BIG_ROWS else (4, 44)
     _need(tuple(variant) in TILES_VARIANTS, f"gemm_tiles has no variant {variant}")
-    out = torch.empty((M, n // 2 if fused else n), dtype=out_dtype, device=x.device)
-    lib.call("arle_gemm_tiles", x.data_ptr(), x.stride(0), tiles.data_ptr(), out.data_ptr(), out.stride(0),
-             _CODES[out_dtype], M, n, K, int(epilogue), variant[0], variant[1], _stream())
+    col_tiles = variant[2] if len(variant) > 2 else 2
+    steps = -(-K // 32)
+    _need(1 <= splits <= steps, f"gemm_tiles cannot cut {steps} steps of K into {splits} parts")
+    per = -(-steps // splits)
+    splits = -(-steps // per)   # parts of `per` steps cover K; the last one may be shorter
+    if splits > 1:
+        _need(not fused and out_dtype == torch.float32, "parts of K come back as a float32 stack without an epilogue")
+        out = torch.empty((splits, M, n), dtype=torch.float32, device=x.device)
+        ldo, stride = out.stride(1), out.stride(0)
+    else:
+        out = torch.empty((M, n // 2 if fused else n), dtype=out_dtype, device=x.device)
+        ldo, stride = out.stride(0), 0
+    lib.call("arle_gemm_tiles", x.data_ptr(), x.stride(0), tiles.data_ptr(), out.data_ptr(), ldo,
+             _CODES[out_dtype], M, n, K, int(epilogue), variant[0], col_tiles, variant[1], splits, per, stride, _stream())
     return out
 
 
@@ -857,6 +872,10 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
         if out.dim() == 3 and (not partials_ok or out.numel() * 4 > _STREAM_PARTIAL_BYTES):
             out = sum_partials(out, out_dtype)
         return out
+    if partials_ok and tiles is not None and aligned:
+        splits = narrow_tiles_splits(rows, n, k, x.stride(0))
+        if splits:
+            return gemm_tiles(x, tiles, n, torch.float32, variant=_NARROW_TILES_VARIANT, splits=splits)
     if partials_ok:
         splits = library_k_splits(rows, n, k)
         if splits > 1:
@@ -879,6 +898,32 @@ _LIB_SPLIT_MAX_N = 4096
 _LIB_SPLIT_MIN_K = 2048
 _LIB_SPLIT_MAX_ROWS = 1024
 _BMM_OUT_DTYPE_OK = None
+
+
+# A product with a narrow output and 65 to 256 rows (o and down of a large decode batch or a short portion) is a
+# matter of streaming W, and the library gives it a few dozen workgroups.  gemm_tiles with workgroups of 128 rows x
+# 128 columns and K cut into parts, so that about 160 to 200 workgroups stream at once, leaves a float32 stack like
+# the few-rows kernels.  Measured on MI355X at the Qwen3-4B shape, in us: o (2,560 x 4,096) at 96 / 128 / 256 rows
+# 13.0 / 14.7 / 19.3 against 23.4 / 23.8 / 22.0 for the library's batched parts; down (2,560 x 9,728) at 96 / 128 /
+# 192 rows 20.7 / 23.7 / 30.2 against 28.4 / 30.1 / 33.7, and behind at 256 (34.7 against 25.8).  For q|k|v the
+# larger stack costs the consumer what the product gains, and gate|up needs whole sums for its activation.
+_NARROW_TILES_VARIANT = (4, 44, 1)
+_NARROW_TILES_MAX_N = 4096
+_NARROW_TILES_MIN_K = 2048
+_NARROW_TILES_WORKGROUPS = 200
+
+
+def narrow_tiles_splits(rows: int, n: int, k: int, x_stride: int) -> int:
+    """Into how many parts along K gemm_tiles' narrow workgroups cut such a product; 0: they do not take it."""
+    most_rows = 256 if k < 8192 else 192
+    if not (ROWS_KERNEL_MAX < rows <= most_rows and n <= _NARROW_TILES_MAX_N and k >= _NARROW_TILES_MIN_K
+            and k % 8 == 0 and x_stride % 8 == 0):
+        return 0
+    blocks = -(-n // 128) * -(-rows // 128)
+    splits = 8
+    while splits > 1 and (blocks * splits > _NARROW_TILES_WORKGROUPS or k < 320 * splits):
+        splits //= 2
+    return splits if splits > 1 else 0
 
 
 def library_k_splits(rows: int, n: int, k: int) -> int:

@@ -783,6 +783,26 @@ def test_library_product_cut_along_k_for_narrow_outputs(M, N, K):
     assert _rel(got.cpu(), wide[:, :K].cpu().double() @ w.double().T) < 8e-3
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 2560, 4096), (128, 2560, 9728), (200, 333, 2048), (256, 2560, 4096), (96, 136, 2056)])
+def test_narrow_products_of_65_to_256_rows_go_to_the_tiles_kernel_when_tiles_are_given(M, N, K):
+    """With operand tiles at hand a narrow product of 65 to 256 rows is cut along K for gemm_tiles' workgroups of
+    128 x 128: a float32 stack whose parts add up to the product; without tiles, or for a caller that cannot add a
+    stack, nothing changes."""
+    x = torch.randn(M, K, generator=_g(153)).bfloat16()
+    w = (torch.randn(N, K, generator=_g(154)) * 0.05).bfloat16()
+    want = x.double() @ w.double().T
+    tiles = ops.pack_weight_tiles(w.to(DEV))
+    splits = ops.narrow_tiles_splits(M, N, K, K)
+    assert splits in (2, 4, 8) and -(-N // 128) * -(-M // 128) * splits <= 200
+    got = ops.gemm_bf16(x.to(DEV), w.to(DEV), torch.bfloat16, partials_ok=True, tiles=tiles)
+    assert got.dtype == torch.float32 and got.dim() == 3 and got.shape[1:] == (M, N) and got.shape[0] <= splits
+    assert _rel(got.sum(0).cpu(), want) < 1e-5
+    whole = ops.gemm_bf16(x.to(DEV), w.to(DEV), torch.bfloat16, tiles=tiles)
+    assert whole.shape == (M, N) and whole.dtype == torch.bfloat16 and _rel(whole.cpu(), want) < 8e-3
+    assert ops.narrow_tiles_splits(64, N, K, K) == 0 and ops.narrow_tiles_splits(257, N, K, K) == 0
+    assert ops.narrow_tiles_splits(M, 6144, K, K) == 0 and ops.narrow_tiles_splits(256, 2560, 9728, 9728) == 0
+
+
 def test_pack_weight_tiles_layout():
     """Tile (t, s), lane 16 g + i, element e is w[16 t + i, 32 s + 8 g + e]; zeros past the matrix."""
     N, K = 37, 72
@@ -858,6 +878,26 @@ def test_gemm_tiles_with_fused_activation(variant, M, inter, K):
     assert got.shape == (M, inter) and _rel(got, want) < 1e-5
     got = ops.gemm_tiles(x.to(DEV), tiles, 2 * inter, torch.bfloat16, ops.EPI_SILU_MUL, variant=variant).cpu()
     assert _rel(got, want) < 5e-3
+
+
+@pytest.mark.parametrize("variant", ops.TILES_VARIANTS)
+@pytest.mark.parametrize("M,N,K,splits", [(100, 200, 1096, 3), (129, 136, 264, 9), (65, 2560, 4096, 8), (300, 72, 96, 2)])
+def test_gemm_tiles_parts_of_k_as_a_stack(variant, M, N, K, splits):
+    """K cut into parts that end inside a step of 32 and inside a ring: part p of the stack is the product over
+    the p-th part of K alone, and the parts add up to the product."""
+    x = torch.randn(M, K, generator=_g(136)).bfloat16()
+    w = (torch.randn(N, K, generator=_g(137)) * 0.1).bfloat16()
+    tiles = ops.pack_weight_tiles(w.to(DEV))
+    got = ops.gemm_tiles(x.to(DEV), tiles, N, torch.float32, variant=variant, splits=splits).cpu()
+    steps = -(-K // 32)
+    per = -(-steps // splits)
+    assert got.shape == (-(-steps // per), M, N)
+    for part in range(got.shape[0]):
+        k0, k1 = part * per * 32, min((part + 1) * per * 32, K)
+        assert _rel(got[part], x[:, k0:k1].double() @ w[:, k0:k1].double().T) < 1e-5, f"part {part}"
+    assert _rel(got.double().sum(0), x.double() @ w.double().T) < 1e-5
+    with pytest.raises(ops.ShapeError, match="float32 stack"):
+        ops.gemm_tiles(x.to(DEV), tiles, N, torch.bfloat16, variant=variant, splits=splits)
 
 
 def test_gemm_tiles_refuses_what_it_cannot_take():
