@@ -40,6 +40,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // a plain vector: arrays of HIP's uint4 structs end up in scratch memory
 
+constexpr int kTlWaves = 4;
 constexpr int kTlXcds = 8;
 constexpr int kEpiNone = 0, kEpiSiluMul = 1;
 
@@ -57,13 +58,11 @@ struct TilesArgs {
 
 // MT: row tiles of 32 that a workgroup owns (4: 128 rows); TN: column tiles of 32 that a wave owns (2: 256
 // columns a workgroup; 1: 128, for products with so few rows that they are a matter of streaming W, where more and
-// smaller workgroups keep more loads in flight; kTlWaves = 2 halves the workgroup once more).  gridDim.y parts of K,
-// each leaving a result of its own.
-template <int MT, int TN, int PD, int PX, bool PIPE, int EPI, typename TOut, int kTlWaves = 4>
+// smaller workgroups keep more loads in flight).  gridDim.y parts of K, each leaving a result of its own.
+template <int MT, int TN, int PD, int PX, bool PIPE, int EPI, typename TOut>
 // (the second figure is waves a SIMD: the registers a wave may have)
 __global__ __launch_bounds__(kTlWaves* kWave, MT* TN >= 16 ? 1 : (MT * TN >= 8 || PD >= 8 ? 2 : 3))
 void gemm_tiles_kernel(const TilesArgs a) {
-  static_assert(kTlWaves == 4 || kTlWaves == 2, "four waves a workgroup, or two");
   static_assert(!PIPE || TN == 2, "the pipelined loop is written for two column tiles a wave");
   constexpr int kTlCols = 32 * TN * kTlWaves;  // columns a workgroup owns
   static_assert(PD % 2 == 0 && PD % PX == 0, "rounds of PD steps; the LDS stage alternates; the X ring divides the W ring");
@@ -373,7 +372,7 @@ void gemm_tiles_kernel(const TilesArgs a) {
   }
 }
 
-template <int MT, int TN, int PD, int PX, bool PIPE, int EPI, int kTlWaves = 4>
+template <int MT, int TN, int PD, int PX, bool PIPE, int EPI>
 int launch_tiles(TilesArgs a, int splits, int out_dtype, hipStream_t s) {
   a.m_blocks = (a.M + 32 * MT - 1) / (32 * MT);
   a.n_blocks = (a.N + 32 * TN * kTlWaves - 1) / (32 * TN * kTlWaves);
@@ -382,16 +381,16 @@ int launch_tiles(TilesArgs a, int splits, int out_dtype, hipStream_t s) {
   if (grid > 0x7fffffffLL) return static_cast<int>(hipErrorInvalidValue);
   const dim3 blocks(static_cast<unsigned>(grid), static_cast<unsigned>(splits));
   if (out_dtype == kF32)
-    gemm_tiles_kernel<MT, TN, PD, PX, PIPE, EPI, float, kTlWaves><<<blocks, kTlWaves * kWave, 0, s>>>(a);
+    gemm_tiles_kernel<MT, TN, PD, PX, PIPE, EPI, float><<<blocks, kTlWaves * kWave, 0, s>>>(a);
   else
-    gemm_tiles_kernel<MT, TN, PD, PX, PIPE, EPI, bf16, kTlWaves><<<blocks, kTlWaves * kWave, 0, s>>>(a);
+    gemm_tiles_kernel<MT, TN, PD, PX, PIPE, EPI, bf16><<<blocks, kTlWaves * kWave, 0, s>>>(a);
   return launch_status();
 }
 
-template <int MT, int TN, int PD, int PX, bool PIPE = false, int kTlWaves = 4>
+template <int MT, int TN, int PD, int PX, bool PIPE = false>
 int dispatch_tiles(const TilesArgs& a, int splits, int out_dtype, int epilogue, hipStream_t s) {
-  return epilogue ? launch_tiles<MT, TN, PD, PX, PIPE, kEpiSiluMul, kTlWaves>(a, splits, out_dtype, s)
-                  : launch_tiles<MT, TN, PD, PX, PIPE, kEpiNone, kTlWaves>(a, splits, out_dtype, s);
+  return epilogue ? launch_tiles<MT, TN, PD, PX, PIPE, kEpiSiluMul>(a, splits, out_dtype, s)
+                  : launch_tiles<MT, TN, PD, PX, PIPE, kEpiNone>(a, splits, out_dtype, s);
 }
 
 }  // namespace arle
@@ -402,7 +401,7 @@ using namespace arle;
 // out [M, N] (epilogue 0) or [M, N/2] (epilogue 1: N % 32 == 0, gate and up rows of W interleaved in blocks of 16),
 // bfloat16 or float32, row stride ldo.  row_tiles: row tiles of 32 a workgroup (4 or 8); col_tiles: column tiles of
 // 32 a wave (2, or 1 with 4 row tiles); depth: ring depths of W and X as two digits (22, 44, 84), + 100 for the loop
-// with the barrier in mid-step (8 row tiles only), + 200 for workgroups of two waves (one column tile a wave only).  splits > 1: K is cut into parts of steps_per_split steps of 32
+// with the barrier in mid-step (8 row tiles only).  splits > 1: K is cut into parts of steps_per_split steps of 32
 // (splits of them cover it), and part p leaves its product at out + p * split_stride as float32, no epilogue.
 extern "C" int arle_gemm_tiles(const void* x, long long ldx, const void* w_tiles, void* out, long long ldo, int out_dtype,
                                int M, int N, int K, int epilogue, int row_tiles, int col_tiles, int depth, int splits,
@@ -426,9 +425,6 @@ extern "C" int arle_gemm_tiles(const void* x, long long ldx, const void* w_tiles
   } else if (col_tiles == 1) {
     if (row_tiles == 4 && depth == 44) return dispatch_tiles<4, 1, 4, 4>(a, splits, out_dtype, epilogue, s);
     if (row_tiles == 4 && depth == 84) return dispatch_tiles<4, 1, 8, 4>(a, splits, out_dtype, epilogue, s);
-    if (row_tiles == 4 && depth == 66) return dispatch_tiles<4, 1, 6, 6>(a, splits, out_dtype, epilogue, s);
-    if (row_tiles == 4 && depth == 88) return dispatch_tiles<4, 1, 8, 8>(a, splits, out_dtype, epilogue, s);
-    if (row_tiles == 4 && depth == 288) return dispatch_tiles<4, 1, 8, 8, false, 2>(a, splits, out_dtype, epilogue, s);
   }
   return static_cast<int>(hipErrorInvalidValue);
 }

@@ -787,10 +787,9 @@ def gemm_tiles_preferred(rows: int, n: int, k: int, x_stride: int, fused: bool =
             and k % 8 == 0 and x_stride % 8 == 0)
 
 
-# (row tiles of 32 a workgroup, ring depths W|X; 1xx: the loop with the barrier in mid-step and four LDS stages;
-#  2xx: workgroups of two waves[,
+# (row tiles of 32 a workgroup, ring depths W|X; 1xx: the loop with the barrier in mid-step and four LDS stages[,
 #  column tiles of 32 a wave: 2 unless given])
-TILES_VARIANTS = ((4, 22), (4, 44), (8, 44), (8, 144), (4, 44, 1), (4, 84, 1), (4, 66, 1), (4, 88, 1), (4, 288, 1))
+TILES_VARIANTS = ((4, 22), (4, 44), (8, 44), (8, 144), (4, 44, 1), (4, 84, 1))
 
 
 def gemm_tiles(x, tiles, n: int, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, variant=None, splits: int = 1):
