@@ -69,7 +69,7 @@ def _template_args(name: str) -> list:
 
 def _completes_gate_up(name: str) -> bool:
     """Whether this kernel leaves gate|up complete: a product with the activation fused (gemm_rows_kernel<MT, WN,
-    WK, PD, XD, EPI, out> / gemm_tiles_kernel<MT, PD, PX, PIPE, EPI, out> with EPI = 1), or the activation kernel
+    WK, PD, XD, EPI, out> / gemm_tiles_kernel<MT, TN, PD, PX, PIPE, EPI, out> with EPI = 1), or the activation kernel
     behind a plain product."""
     if "silu_mul" in name:
         return True
@@ -77,7 +77,7 @@ def _completes_gate_up(name: str) -> bool:
     if "gemm_rows_kernel" in name:
         return len(args) > 5 and args[5] == "1"
     if "gemm_tiles_kernel" in name:
-        return len(args) > 4 and args[4] == "1"
+        return len(args) > 5 and args[5] == "1"
     return False
 
 
@@ -152,6 +152,9 @@ def part_times(steps, layers: int) -> dict:
         for part, (_, us) in zip(classify_step([n for n, _ in kernels], layers), kernels):
             total[part] += us
     out = {p: t / len(steps) for p, t in total.items()}
+    missing = [p for p in ("qkv", "o", "gate_up", "down", "head") if not out.get(p)]
+    if missing:  # a kernel's name no longer says what the sorting reads from it
+        raise RuntimeError(f"no kernel of a profiled step was sorted into {', '.join(missing)}")
     out["kernels"] = sum(len(k) for k in steps) / len(steps)
     return out
 

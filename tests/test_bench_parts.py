@@ -22,9 +22,24 @@ def test_kernels_of_a_step_are_sorted_into_the_parts_of_a_layer():
             + ["norm", "head", "other"])
     assert bench.classify_step(names, layers=2) == want
     tiles = ["rmsnorm", "Cijk_a", "qk_prep", "attn_prefill_lds_kernel<128>", "Cijk_b", "rmsnorm",
-             "gemm_tiles_kernel<4, 4, 4, false, 1, arle::bf16>", "Cijk_c", "rmsnorm", "Cijk_head"]
+             "gemm_tiles_kernel<4, 2, 4, 4, false, 1, arle::bf16>", "Cijk_c", "rmsnorm", "Cijk_head"]
     assert bench.classify_step(tiles, layers=1) == ["norm", "qkv", "qk_prep", "attention", "o", "norm", "gate_up", "down",
                                                     "norm", "head"]
+
+
+def test_a_step_whose_kernels_are_not_all_sorted_is_refused():
+    """A kernel whose name no longer says what the sorting reads from it (here: an activation that never ends
+    gate|up, so that down and the head stay empty) must not end up as figures in the record."""
+    import pytest
+
+    layer = ["rmsnorm", "Cijk_a", "qk_prep", "attn_prefill_dma_kernel<false, 1>", "Cijk_b", "rmsnorm",
+             "gemm_tiles_kernel<4, 2, 4, 4, false, 7, arle::bf16>", "Cijk_c"]
+    step = [("embed_gather_kernel", 1.0)] + [(n, 2.0) for n in layer] + [("rmsnorm", 1.0), ("Cijk_head", 3.0)]
+    with pytest.raises(RuntimeError, match="down"):
+        bench.part_times([step], layers=1)
+    good = [(n.replace("false, 7", "false, 1"), us) for n, us in step]
+    times = bench.part_times([good], layers=1)
+    assert times["down"] == 2.0 and times["head"] == 3.0 and times["gate_up"] == 2.0 and times["kernels"] == len(good)
 
 
 def test_bytes_and_flops_of_the_parts_add_up_to_the_step():

@@ -300,3 +300,24 @@ def test_four_layers_at_the_widths_of_qwen3_4b(four_layers, dtype, tol):
     got = replay.run_steps(eng, replay.mixed(requests, max_live=3, seed=5, max_portion=40))
     assert len(got) == sum(len(t) for t in requests.values())
     check(got, "mixed")
+
+
+def test_bench_sorts_the_kernels_of_real_steps_into_every_part_of_a_layer():
+    """`bench.py --parts-only` on two layers of the benchmark's shape: the kernel names that the profiler reports
+    today are sorted into all parts of a prefill and of a decode step (a renamed kernel or a changed list of
+    template arguments would leave a part empty, which the program refuses)."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..")
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--parts-only", "--layers", "2", "--batch", "2"],
+                         capture_output=True, text=True, timeout=400, cwd=root)
+    lines = [ln for ln in res.stdout.splitlines() if ln.startswith("{")]
+    assert res.returncode == 0 and lines, res.stderr[-2000:]
+    line = json.loads(lines[-1])
+    for step in ("prefill_parts_us", "decode_parts_us"):
+        for part in ("qkv", "o", "gate_up", "down", "head", "attention", "qk_prep", "norm"):
+            assert line[step][part] > 0, (step, part, line[step])
+    assert line["prefill_parts_us"]["gate_up"] > line["prefill_parts_us"]["qkv"] > line["prefill_parts_us"]["head"] / 100
