@@ -360,8 +360,8 @@ def decode_32b(args) -> int:
 
 def sweep(args) -> int:
     """Further sizes of the Qwen3-4B shape, one JSON line each with its fraction of the roofline: decode at batch 16
-    and 32 (2,048-token prompts), at batch 8 with 8,192 and 32,768 tokens of context, a prefill of 8,192 tokens, and
-    a 512-token prompt portion beside 8 decoding requests."""
+    and 32 (2,048-token prompts), at batch 128 (1,024 tokens of context), at batch 8 with 8,192 and 32,768 tokens of
+    context, prefills of 8,192, 512 and 128 tokens, and a 512-token prompt portion beside 8 decoding requests."""
     import torch
 
     from arle_amd.config import Qwen3Config
@@ -372,7 +372,7 @@ def sweep(args) -> int:
     config = Qwen3Config.from_dict(raw)
     longest = 32768 + 64
     engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype="bfloat16", page_size=PAGE,
-                                max_tokens=8 * longest + 40 * 4096, max_slots=33, max_request_tokens=longest)
+                                max_tokens=8 * longest + 40 * 4096, max_slots=129, max_request_tokens=longest)
     gen = torch.Generator().manual_seed(1234)
     rand = lambda n: torch.randint(0, config.vocab_size, (n,), generator=gen).tolist()
     base = {"n_gpus": 1, "dtype": "bf16", "higher_is_better": True, "data": "synthetic", "layers": args.layers}
@@ -450,10 +450,12 @@ def sweep(args) -> int:
 
     for batch in (16, 32):
         decode_point(batch, 2048, args.steps)
+    decode_point(128, 1024, args.steps)
     for context in (8192, 32768):
         decode_point(8, context, args.steps)
     prefill_point(8192)
     prefill_point(512)
+    prefill_point(128)
     mixed_point(8, 2048, 512, 2048)
     return 0
 
