@@ -65,6 +65,7 @@ struct AttnArgs {
   float* pws_o;        // [token row][q head][part][D]   (portion_splits > 1)
   float* pws_ml;       // [token row][q head][part][2]
   int rows_max;  // the streaming kernel skips segments with more rows than this (0: takes all)
+  long long plan_token;  // names the step for the portions kernels' list of work (0: no name, plan every time)
 };
 
 __device__ __forceinline__ bf16x8 load_bf16x8(const uint16_t* p) {
@@ -422,8 +423,8 @@ constexpr int kPfVPad = 4;              // padding of a value row in LDS: 34 dwo
 // the keys of the first 128, and a fixed assignment of row blocks to workgroups leaves most of the chip idle
 // while the heaviest ones finish.  So the launch has one workgroup per CU and every workgroup takes the next
 // item (row block, kv head, segment), heaviest row blocks first, from a counter until none is left.  The counter
-// is a device variable of this module, put to zero by the planning kernel before every launch: launches of this
-// kernel on one device must not overlap (they never do on one stream).
+// is a device variable of this module, put to zero by the planning kernel and again by the last workgroup that
+// leaves a launch: launches of this kernel on one device must not overlap (they never do on one stream).
 //
 // The planning kernel (one workgroup) also lists the live (row block, segment) pairs in that order: a step
 // that mixes a few portions with many decoded tokens has far more pairs that are dead (segments left to the
@@ -431,6 +432,7 @@ constexpr int kPfVPad = 4;              // padding of a value row in LDS: 34 dwo
 // costs a round trip to the counter each time.  Steps with more pairs than the list holds go without it.
 constexpr int kPfPlanMax = 16384;
 __device__ unsigned int g_prefill_next_item;
+__device__ unsigned int g_prefill_left;               // workgroups of the running launch that have found the list empty
 __device__ unsigned int g_prefill_pairs;              // entries of g_prefill_plan
 __device__ unsigned int g_prefill_plan[kPfPlanMax];   // (row block << 16) | segment
 
@@ -442,6 +444,7 @@ __global__ __launch_bounds__(256) void attn_prefill_plan_kernel(const int* __res
   if (tid == 0) {
     base = 0u;
     g_prefill_next_item = 0u;
+    g_prefill_left = 0u;
   }
   if (!listed) return;  // the whole workgroup
   __syncthreads();
@@ -494,7 +497,15 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
   __syncthreads();
   const unsigned int item = item_of_workgroup;
   __syncthreads();  // everyone has read it before thread 0 asks for the next
-  if (item >= items) return;
+  if (item >= items) {
+    // The last workgroup to leave puts the counters back to zero: the layers of a step hand out the same list one
+    // after the other, and only the first of them runs the planning kernel.
+    if (tid == 0 && atomicAdd(&g_prefill_left, 1u) == gridDim.x - 1) {
+      g_prefill_next_item = 0u;
+      g_prefill_left = 0u;
+    }
+    return;
+  }
   const unsigned int pair = item / (nkv * parts);
   const int kvh = static_cast<int>((item / parts) % nkv);
   const int part = static_cast<int>(item % parts);
@@ -932,7 +943,15 @@ __global__ __launch_bounds__(GROUPS* kDmWaves* kWave, GROUPS == 1 ? 2 : 1) void 
   __syncthreads();
   const unsigned int item = item_of_workgroup;
   __syncthreads();
-  if (item >= items) return;
+  if (item >= items) {
+    // The last workgroup to leave puts the counters back to zero: the layers of a step hand out the same list one
+    // after the other, and only the first of them runs the planning kernel.
+    if (tid == 0 && atomicAdd(&g_prefill_left, 1u) == gridDim.x - 1) {
+      g_prefill_next_item = 0u;
+      g_prefill_left = 0u;
+    }
+    return;
+  }
   unsigned int pair = item / (nkv * parts);
   const int kvh = static_cast<int>((item / parts) % nkv);
   const int part = static_cast<int>(item % parts);
@@ -1378,6 +1397,27 @@ inline size_t prefill_lds_bytes(int D) {
   return 2 * (static_cast<size_t>(kPfKeys) * (D + 8) + static_cast<size_t>(D) * (kPfKeys + kPfVPad)) * sizeof(uint16_t);
 }
 
+// The list of live (row block, segment) pairs depends on the step, not on the layer: a caller that names the step
+// (plan_token != 0, a number that no other step of the process has) gets the planning kernel for the first launch
+// of the step only.  What the list was made from is kept here, on the host, and compared.
+struct PlanMade {
+  long long token = 0;
+  const int* seg_row0 = nullptr;
+  unsigned blocks = 0, segments = 0;
+  int group = 0, min_rows = 0, listed = 0;
+  void* stream = nullptr;
+};
+static PlanMade g_plan_made;
+
+inline bool plan_is_current(const AttnArgs& a, dim3 grid, int min_rows, int listed) {
+  const PlanMade now{a.plan_token, a.seg_row0, grid.x, grid.z, a.nq / a.nkv, min_rows, listed, nullptr};
+  const bool same = a.plan_token != 0 && now.token == g_plan_made.token && now.seg_row0 == g_plan_made.seg_row0 &&
+                    now.blocks == g_plan_made.blocks && now.segments == g_plan_made.segments &&
+                    now.group == g_plan_made.group && now.min_rows == g_plan_made.min_rows && now.listed == g_plan_made.listed;
+  g_plan_made = now;
+  return same;
+}
+
 template <int DMAX, bool EXACT>
 int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s) {
   const size_t lds = prefill_lds_bytes(a.D);
@@ -1399,8 +1439,9 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
   const int per_cu = 1;  // eight waves: two on every SIMD, with all the registers they want
   const unsigned workgroups = static_cast<unsigned>(items < static_cast<long long>(per_cu) * cus ? items : per_cu * cus);
   const int listed = static_cast<long long>(grid.x) * grid.z <= kPfPlanMax && grid.x <= 65535 && grid.z <= 65535;
-  attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
-                                             a.nq / a.nkv, min_rows, listed);
+  if (!plan_is_current(a, grid, min_rows, listed))
+    attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
+                                               a.nq / a.nkv, min_rows, listed);
   if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);  // the merge walks the list
   attn_prefill_lds_kernel<DMAX, EXACT><<<workgroups, kPfWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
                                                                                 static_cast<int>(grid.z), listed);
@@ -1435,8 +1476,9 @@ int launch_prefill_dma_groups(const AttnArgs& a, dim3 grid, int min_rows, int cu
   const unsigned workgroups = static_cast<unsigned>(items < places ? items : places);
   const int listed = static_cast<long long>(grid.x) * grid.z <= kPfPlanMax && grid.x <= 65535 && grid.z <= 65535;
   if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);
-  attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
-                                             a.nq / a.nkv, min_rows, listed);
+  if (!plan_is_current(a, grid, min_rows, listed))
+    attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
+                                               a.nq / a.nkv, min_rows, listed);
   const int pair_up = GROUPS == 1 && g_prefill_pair_up ? static_cast<int>(cus / (static_cast<long long>(a.nkv) * a.portion_splits)) : 0;
   if (a.P % kDmKeys == 0)
     attn_prefill_dma_kernel<true, GROUPS><<<workgroups, GROUPS * kDmWaves * kWave, lds, s>>>(
@@ -1527,6 +1569,7 @@ static AttnArgs make_args(const void* q, long long q_stride, void* out, long lon
   a.splits = splits;
   a.ws_rows = arle_attn_ws_rows(max_qlen, nq, nkv);
   a.portion_splits = 1;
+  a.plan_token = 0;
   a.pws_o = nullptr;
   a.pws_ml = nullptr;
   a.rows_max = 0;
@@ -1543,6 +1586,8 @@ static AttnArgs make_args(const void* q, long long q_stride, void* out, long lon
 // portions of a few tokens).  Longer portions go to the LDS kernel; when they have too few row blocks to fill
 // the chip, portion_splits > 1 cuts the keys of every row block into that many parts (at most 8), pws_o/pws_ml
 // must hold [token rows][nq][portion_splits][D] and [..][2] floats, and a merge of their own runs after.
+// plan_token: 0, or a number that names the step (the same for every layer of it, another for every other step of
+// the process): the portions kernels then list their work once a step instead of once a call.
 // Requires D % 16 == 0, D <= 256, page_size a power of two >= 4.
 extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out, long long o_stride,
                                     const void* k_pages, const void* v_pages, const int* block_table,
@@ -1551,7 +1596,7 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
                                     int max_kv_len, int token_rows,
                                     int nq, int nkv, int D, int page_size, float scale, int window,
                                     int splits, float* ws_o, float* ws_ml, int portion_splits, float* pws_o,
-                                    float* pws_ml, void* stream) {
+                                    float* pws_ml, long long plan_token, void* stream) {
   if (segments == 0 || token_rows == 0) return 0;
   if (D % 16 != 0 || D > 256 || D <= 0 || page_size < 4 || (page_size & (page_size - 1)) != 0 || nq % nkv != 0 ||
       splits < 1 || splits > 64 || portion_splits < 1 || portion_splits > kPortionPartsMax ||
@@ -1563,6 +1608,7 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
   a.portion_splits = portion_splits;
   a.pws_o = pws_o;
   a.pws_ml = pws_ml;
+  a.plan_token = plan_token;
   const int G = nq / nkv;
   const int max_rows = max_qlen * G, min_rows = min_qlen * G;
   const long long z = static_cast<long long>(segments) * splits;

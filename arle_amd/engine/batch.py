@@ -49,6 +49,7 @@ class StepBatch:
     host: dict                   # the same arrays as numpy, for parts that plan on the host
     single_segments: int = 0     # segments of one token (decoded tokens)
     kv_splits: int | None = None  # split-KV factor fixed by the caller (a captured graph), else chosen per call
+    plan_token: int = 0          # names one pass over the layers (set by the model): what parts plan once a pass
 
 
 def packed_size(num_tokens: int, num_segments: int, num_wanted: int) -> int:

@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import ctypes
 import functools
+import itertools
 import math
 
 import torch
@@ -376,7 +377,8 @@ def portion_key_splits(tokens: int, max_qlen: int, long_segments: int, num_q_hea
 def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *,
                     max_qlen: int, max_kv_len: int, num_q_heads: int, num_kv_heads: int, head_dim: int,
                     page_size: int, scale: float, window: int = 0, splits: int | None = None,
-                    min_qlen: int = 1, short_segments: int | None = None, portion_splits: int | None = None):
+                    min_qlen: int = 1, short_segments: int | None = None, portion_splits: int | None = None,
+                    plan_token: int = 0):
     """Causal attention of a packed step on the matrix cores (bfloat16).
 
     Segments: rows seg_row0[s]..seg_row0[s+1] belong to block-table row seg_slot[s] and start at
@@ -384,7 +386,8 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
     decoded tokens above all, are split over the keys (split-KV), also beside longer portions in one
     step; `short_segments` says how many there are (default: all), which sets the number of splits.
     Longer portions that are too few to fill the chip have their keys cut into `portion_splits` parts
-    (default: portion_key_splits).
+    (default: portion_key_splits).  `plan_token` (new_plan_token()) names the step: with the same token and the
+    same segments the portions kernels list their work once, for the first layer, and not once a layer.
     """
     _gpu(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start)
     tokens = q.shape[0]
@@ -433,8 +436,16 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
              seg_row0.data_ptr(), seg_slot.data_ptr(), seg_start.data_ptr(), segments, int(max_qlen),
              int(min_qlen), int(max_kv_len), tokens,
              num_q_heads, num_kv_heads, head_dim, page_size, float(scale), int(window), int(splits),
-             _ptr(ws_o), _ptr(ws_ml), int(portion_splits), _ptr(pws_o), _ptr(pws_ml), _stream())
+             _ptr(ws_o), _ptr(ws_ml), int(portion_splits), _ptr(pws_o), _ptr(pws_ml), int(plan_token), _stream())
     return out
+
+
+_plan_tokens = itertools.count(1)
+
+
+def new_plan_token() -> int:
+    """A number that no other step of this process has (attn_paged_mfma's plan_token)."""
+    return next(_plan_tokens)
 
 
 def attn_decode_static(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *, max_qlen: int,

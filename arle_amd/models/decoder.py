@@ -10,6 +10,7 @@ from __future__ import annotations
 import os
 import sys
 
+from ..kernels import ops
 from ..parts import base  # noqa: F401  (registries)
 from ..parts import attention, block, embedding, feed_forward, norm, position  # noqa: F401  registers the stock parts
 from ..parts.base import Runtime, build_part, expected_tensors, lookup
@@ -120,6 +121,9 @@ class DecoderModel:
 
     def forward(self, batch, cache):
         """Logits float32 [len(batch.want_rows), vocab] of one packed step."""
+        # every pass over the layers gets a name of its own (a pass that is being captured into a graph too: its
+        # first layer has to plan inside the graph): parts that prepare something once a step key it with this
+        batch.plan_token = ops.new_plan_token()
         residual = self.embedding.forward(batch.token_ids)
         delta = None
         dump = os.environ.get(DEBUG_DUMP_ENV) is not None

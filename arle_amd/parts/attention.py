@@ -140,7 +140,8 @@ def paged_attention(q, out, cache, batch, *, num_q_heads, num_kv_heads, head_dim
                             max_kv_len=batch.max_position + 1, num_q_heads=num_q_heads,
                             num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=cache.page_size,
                             scale=scale, window=window, splits=getattr(batch, "kv_splits", None),
-                            short_segments=getattr(batch, "single_segments", 0) or None)
+                            short_segments=getattr(batch, "single_segments", 0) or None,
+                            plan_token=getattr(batch, "plan_token", 0))
     else:
         ops.attn_paged_simt(q, out, cache.k_pages, cache.v_pages, cache.block_table, batch.positions,
                             batch.slot_of_token, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads,

@@ -595,6 +595,50 @@ def test_attention_mfma_both_portion_kernels_at_head_dim_128(variant, nq, nkv, P
     assert _rel(got, want) < 8e-3
 
 
+@pytest.mark.parametrize("variant", [0, 1])
+def test_attention_portions_list_their_work_once_for_calls_that_name_the_same_step(variant):
+    """Calls with one plan_token and the same segments (the layers of a step) run the planning kernel once; the
+    results are those of calls without a token.  Another step under the same token by mistake (other segments)
+    is planned anew, and so is the same step under another token."""
+    from arle_amd.kernels import lib
+    nq, nkv, D, P = 8, 2, 128, 16
+    lib.function("arle_attn_prefill_variant")(variant)
+    try:
+        def case(segs, seed, token):
+            lengths = [a + b for a, b in segs]
+            table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, torch.bfloat16, seed)
+            qs, wants, row0, starts = [], [], [0], []
+            for s_, (cached, n) in enumerate(segs):
+                g = _g(seed + 1 + s_)
+                q, k, v = (torch.randn(cached + n, h, D, generator=g).to(torch.bfloat16) for h in (nq, nkv, nkv))
+                _fill_cache(table, k_pages, v_pages, s_, k, v, P)
+                qs.append(q[cached:].reshape(n, -1))
+                wants.append(plain.causal_attention(q.double(), k.double(), v.double(), nkv)[cached:].reshape(n, -1))
+                row0.append(row0[-1] + n)
+                starts.append(cached)
+            i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+            args = (torch.cat(qs).to(DEV), k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0),
+                    i32(list(range(len(segs)))), i32(starts))
+            kw = dict(max_qlen=max(n for _, n in segs), min_qlen=min(n for _, n in segs), max_kv_len=max(lengths),
+                      num_q_heads=nq, num_kv_heads=nkv, head_dim=D, page_size=P, scale=1.0 / math.sqrt(D))
+            outs = []
+            for tok in token:
+                out = torch.full_like(args[0], float("nan"))
+                ops.attn_paged_mfma(args[0], out, *args[1:], plan_token=tok, **kw)
+                outs.append(out.cpu())
+            return outs, torch.cat(wants)
+
+        first = ops.new_plan_token()
+        outs, want = case([(40, 300), (0, 170), (7, 1)], 300, [0, first, first, first, ops.new_plan_token()])
+        for out in outs:
+            assert torch.equal(out, outs[0]) and _rel(out, want) < 8e-3
+        outs, want = case([(0, 50), (90, 420), (3, 33), (0, 200)], 310, [first, first, 0])   # the old token, other segments
+        for out in outs:
+            assert torch.equal(out, outs[-1]) and _rel(out, want) < 8e-3
+    finally:
+        lib.function("arle_attn_prefill_variant")(-1)
+
+
 @pytest.mark.parametrize("P", [16, 64, 128])
 def test_attention_mfma_dma_kernel_masks_stale_slots(P):
     """The kernel that loads tiles straight into LDS: pages hold NaN bits in every slot that was never written
