@@ -435,8 +435,11 @@ __device__ unsigned int g_prefill_next_item;
 __device__ unsigned int g_prefill_left;               // workgroups of the running launch that have found the list empty
 __device__ unsigned int g_prefill_pairs;              // entries of g_prefill_plan
 __device__ unsigned int g_prefill_plan[kPfPlanMax];   // (row block << 16) | segment
+__device__ int4 g_prefill_seg[kPfPlanMax];            // the entry's segment: first row, rows, first position, table row
 
-__global__ __launch_bounds__(256) void attn_prefill_plan_kernel(const int* __restrict__ seg_row0, int segments,
+__global__ __launch_bounds__(256) void attn_prefill_plan_kernel(const int* __restrict__ seg_row0,
+                                                                 const int* __restrict__ seg_start,
+                                                                 const int* __restrict__ seg_slot, int segments,
                                                                  int blocks_x, int G, int min_rows, int listed) {
   __shared__ unsigned int wave_count[4];
   __shared__ unsigned int base;
@@ -453,11 +456,15 @@ __global__ __launch_bounds__(256) void attn_prefill_plan_kernel(const int* __res
     const int i = i0 + tid;
     bool live = false;
     unsigned int entry = 0u;
+    int4 of_seg = {0, 0, 0, 0};
     if (i < total) {
       const int seg = i % segments, rb = blocks_x - 1 - i / segments;  // the last rows see the most keys: first
-      const int rows = (seg_row0[seg + 1] - seg_row0[seg]) * G;
+      const int row0 = seg_row0[seg], qlen = seg_row0[seg + 1] - row0;
+      const int rows = qlen * G;
       live = rows >= min_rows && rb * kPfRows < rows;
       entry = (static_cast<unsigned int>(rb) << 16) | static_cast<unsigned int>(seg);
+      // what a workgroup needs to know of the segment, beside the entry: one load instead of a chain of them
+      if (live) of_seg = int4{row0, qlen, seg_start[seg], seg_slot[seg]};
     }
     const unsigned long long votes = __ballot(live);
     const unsigned int before = __popcll(votes & ((1ull << lane) - 1ull));
@@ -465,7 +472,10 @@ __global__ __launch_bounds__(256) void attn_prefill_plan_kernel(const int* __res
     __syncthreads();
     unsigned int offset = base;
     for (int w = 0; w < wave; ++w) offset += wave_count[w];
-    if (live) g_prefill_plan[offset + before] = entry;
+    if (live) {
+      g_prefill_plan[offset + before] = entry;
+      g_prefill_seg[offset + before] = of_seg;
+    }
     __syncthreads();
     if (tid == 0) base += wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
     __syncthreads();
@@ -511,18 +521,23 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
   const int part = static_cast<int>(item % parts);
   // the last rows of a segment see the most keys: they are handed out first
   int seg = static_cast<int>(pair % segments), wg_row = (blocks_x - 1 - static_cast<int>(pair / segments)) * kPfRows;
-  if (listed) {
+  int row0, qlen, start, slot;
+  if (listed) {  // the entry and what the list holds of its segment: two loads side by side
     const unsigned int entry = g_prefill_plan[pair];
+    const int4 of_seg = g_prefill_seg[pair];
     seg = static_cast<int>(entry & 0xffffu);
     wg_row = static_cast<int>(entry >> 16) * kPfRows;
+    row0 = of_seg.x, qlen = of_seg.y, start = of_seg.z, slot = of_seg.w;
+  } else {
+    row0 = a.seg_row0[seg];
+    qlen = a.seg_row0[seg + 1] - row0;
+    start = a.seg_start[seg];
+    slot = a.seg_slot[seg];
   }
-  const int row0 = a.seg_row0[seg];
-  const int qlen = a.seg_row0[seg + 1] - row0;
   const int rows = qlen * G;
   if (rows < min_rows) continue;  // short segments (decoded tokens) belong to the other kernel
   if (wg_row >= rows) continue;
-  const int start = a.seg_start[seg];
-  const int* table = a.block_table + static_cast<int64_t>(a.seg_slot[seg]) * a.table_stride;
+  const int* table = a.block_table + static_cast<int64_t>(slot) * a.table_stride;
   const int D = EXACT ? DMAX : a.D, P = a.P;
   const int n_dch = EXACT ? DCH : (D + 31) / 32, n_dt = EXACT ? DTL : D / 16;
 
@@ -964,18 +979,23 @@ __global__ __launch_bounds__(GROUPS* kDmWaves* kWave, GROUPS == 1 ? 2 : 1) void 
     if (pair >= h) pair = pair < 2u * h ? pairs - 1u - (pair - h) : pair - h;
   }
   int seg = static_cast<int>(pair % segments), wg_row = (blocks_x - 1 - static_cast<int>(pair / segments)) * kPfRows;
-  if (listed) {
+  int row0, qlen, start, slot;
+  if (listed) {  // the entry and what the list holds of its segment: two loads side by side
     const unsigned int entry = g_prefill_plan[pair];
+    const int4 of_seg = g_prefill_seg[pair];
     seg = static_cast<int>(entry & 0xffffu);
     wg_row = static_cast<int>(entry >> 16) * kPfRows;
+    row0 = of_seg.x, qlen = of_seg.y, start = of_seg.z, slot = of_seg.w;
+  } else {
+    row0 = a.seg_row0[seg];
+    qlen = a.seg_row0[seg + 1] - row0;
+    start = a.seg_start[seg];
+    slot = a.seg_slot[seg];
   }
-  const int row0 = a.seg_row0[seg];
-  const int qlen = a.seg_row0[seg + 1] - row0;
   const int rows = qlen * G;
   if (rows < min_rows) continue;
   if (wg_row >= rows) continue;
-  const int start = a.seg_start[seg];
-  const int* table = a.block_table + static_cast<int64_t>(a.seg_slot[seg]) * a.table_stride;
+  const int* table = a.block_table + static_cast<int64_t>(slot) * a.table_stride;
   const uint32_t head_off32 = static_cast<uint32_t>(kvh) * P * D;
 
   const int tok_min = wg_row / G;
@@ -1403,6 +1423,8 @@ inline size_t prefill_lds_bytes(int D) {
 struct PlanMade {
   long long token = 0;
   const int* seg_row0 = nullptr;
+  const int* seg_start = nullptr;
+  const int* seg_slot = nullptr;
   unsigned blocks = 0, segments = 0;
   int group = 0, min_rows = 0, listed = 0;
   void* stream = nullptr;
@@ -1410,8 +1432,9 @@ struct PlanMade {
 static PlanMade g_plan_made;
 
 inline bool plan_is_current(const AttnArgs& a, dim3 grid, int min_rows, int listed) {
-  const PlanMade now{a.plan_token, a.seg_row0, grid.x, grid.z, a.nq / a.nkv, min_rows, listed, nullptr};
+  const PlanMade now{a.plan_token, a.seg_row0, a.seg_start, a.seg_slot, grid.x, grid.z, a.nq / a.nkv, min_rows, listed, nullptr};
   const bool same = a.plan_token != 0 && now.token == g_plan_made.token && now.seg_row0 == g_plan_made.seg_row0 &&
+                    now.seg_start == g_plan_made.seg_start && now.seg_slot == g_plan_made.seg_slot &&
                     now.blocks == g_plan_made.blocks && now.segments == g_plan_made.segments &&
                     now.group == g_plan_made.group && now.min_rows == g_plan_made.min_rows && now.listed == g_plan_made.listed;
   g_plan_made = now;
@@ -1440,8 +1463,8 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
   const unsigned workgroups = static_cast<unsigned>(items < static_cast<long long>(per_cu) * cus ? items : per_cu * cus);
   const int listed = static_cast<long long>(grid.x) * grid.z <= kPfPlanMax && grid.x <= 65535 && grid.z <= 65535;
   if (!plan_is_current(a, grid, min_rows, listed))
-    attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
-                                               a.nq / a.nkv, min_rows, listed);
+    attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, a.seg_start, a.seg_slot, static_cast<int>(grid.z),
+                                               static_cast<int>(grid.x), a.nq / a.nkv, min_rows, listed);
   if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);  // the merge walks the list
   attn_prefill_lds_kernel<DMAX, EXACT><<<workgroups, kPfWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
                                                                                 static_cast<int>(grid.z), listed);
@@ -1477,8 +1500,8 @@ int launch_prefill_dma_groups(const AttnArgs& a, dim3 grid, int min_rows, int cu
   const int listed = static_cast<long long>(grid.x) * grid.z <= kPfPlanMax && grid.x <= 65535 && grid.z <= 65535;
   if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);
   if (!plan_is_current(a, grid, min_rows, listed))
-    attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, static_cast<int>(grid.z), static_cast<int>(grid.x),
-                                               a.nq / a.nkv, min_rows, listed);
+    attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, a.seg_start, a.seg_slot, static_cast<int>(grid.z),
+                                               static_cast<int>(grid.x), a.nq / a.nkv, min_rows, listed);
   const int pair_up = GROUPS == 1 && g_prefill_pair_up ? static_cast<int>(cus / (static_cast<long long>(a.nkv) * a.portion_splits)) : 0;
   if (a.P % kDmKeys == 0)
     attn_prefill_dma_kernel<true, GROUPS><<<workgroups, GROUPS * kDmWaves * kWave, lds, s>>>(
@@ -1493,7 +1516,7 @@ int launch_prefill_dma_groups(const AttnArgs& a, dim3 grid, int min_rows, int cu
   return launch_status();
 }
 
-int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s) {
+int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, int max_qlen, int max_kv_len, hipStream_t s) {
   static int cus = 0;
   if (cus == 0) {
     int dev = 0, n = 0;
@@ -1501,13 +1524,19 @@ int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
       n = 256;
     cus = n;
   }
-  // With about as many row blocks as the chip has places for workgroups of four waves (more than one for every
-  // second CU, no more than two a CU) the launch lasts as long as its heaviest row block: then every row block goes
-  // to two groups of waves.  Measured on MI355X (32 q heads over 8 kv heads, pages of 16): a fresh prompt of 2,048
-  // tokens 62 against 72 us, 1,024 tokens behind 3,072 cached 87 against 111 us; with fewer or more row blocks the
-  // one group is level or ahead (512 tokens behind 3,584: 67 against 79 us; 8,192 tokens: 590 against 608 us).
+  // Every row block goes to two groups of waves where workgroups of four waves would leave the chip part empty:
+  // with more than one item for every fourth CU and no more than three for every two (two such workgroups fit a
+  // CU), or with up to two a CU when the items are unequal (a fresh prompt, whose last rows see all keys and whose
+  // first rows few: the launch lasts as long as its heaviest item).  Items of about one length, two a CU, fill the
+  // chip best with four waves each.  Measured on MI355X (32 q heads over 8 kv heads, pages of 16), two groups
+  // against one: a fresh prompt of 2,048 tokens 60 against 65 us, of 1,024 tokens 31 against 35, 1,024 tokens
+  // behind 3,072 cached 87 against 111; but 512 tokens behind 3,584 (keys in four parts) 79 against 68, eight
+  // portions of 256 behind 1,024 each 69 against 62, 8,192 fresh tokens 633 against 604; 512 tokens behind 512
+  // cached (one item for every second CU) 27 against 33, a fresh prompt of 128 tokens 12.6 against 11.2.
   const long long items = static_cast<long long>(grid.x) * grid.y * grid.z * a.portion_splits;
-  const bool two = g_prefill_groups >= 0 ? g_prefill_groups == 2 : (2 * items > cus && items <= 2LL * cus);
+  const bool unequal = 2LL * max_qlen > max_kv_len;  // the first rows see less than half of what the last see
+  const bool two = g_prefill_groups >= 0 ? g_prefill_groups == 2
+                                         : (4 * items > cus && (2 * items <= 3LL * cus || (unequal && items <= 2LL * cus)));
   return two ? launch_prefill_dma_groups<2>(a, grid, min_rows, cus, s) : launch_prefill_dma_groups<1>(a, grid, min_rows, cus, s);
 }
 
@@ -1623,7 +1652,7 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
       rc = launch_prefill_lds<64, true>(a, grid, 17, s);
     else if (D == 128 && page_size % 8 == 0 && static_cast<long long>(nkv) * page_size * D < (1LL << 31) &&
              prefill_dma_pays(grid, max_qlen, max_kv_len))
-      rc = launch_prefill_dma(a, grid, 17, s);
+      rc = launch_prefill_dma(a, grid, 17, max_qlen, max_kv_len, s);
     else if (D == 128)
       rc = launch_prefill_lds<128, true>(a, grid, 17, s);
     else if (D <= 64)
