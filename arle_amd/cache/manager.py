@@ -23,6 +23,7 @@ from dataclasses import dataclass
 import numpy as np
 import torch
 
+from ..kernels.upload import upload
 from .pages import FREED, OutOfPages, PageGroup
 
 
@@ -312,8 +313,11 @@ class CacheManager:
             if not self._dirty[g]:
                 continue
             rows = sorted(self._dirty[g])
-            host = torch.from_numpy(self._tables_host[g][rows])
-            self.tables_dev[g][torch.tensor(rows, device=self.device)] = host.to(self.device)
+            # row numbers and rows in one staged copy that the host does not wait for
+            staged = np.concatenate([np.asarray(rows, dtype=np.int32),
+                                     self._tables_host[g][rows].astype(np.int32, copy=False).reshape(-1)])
+            both = upload(staged, self.device)
+            self.tables_dev[g].index_copy_(0, both[:len(rows)].long(), both[len(rows):].view(len(rows), -1))
             self._dirty[g].clear()
 
     def view(self, entry: int):

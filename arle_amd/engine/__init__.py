@@ -1,4 +1,4 @@
-from .batch import StepBatch, StepEntry
+from .batch import DeviceToken, StepBatch, StepEntry
 from .engine import Engine, EngineError
 
-__all__ = ["Engine", "EngineError", "StepBatch", "StepEntry"]
+__all__ = ["DeviceToken", "Engine", "EngineError", "StepBatch", "StepEntry"]

@@ -48,7 +48,8 @@ class LLM:
                  kv_cache_tokens: int | None = None, num_slots: int = 4, max_seq_len: int | None = None,
                  chunked_prefill_size: int = 512, max_num_batched_tokens: int = 16384,
                  max_prefill_tokens: int = 16384, prefill_max_requests: int | None = None, seed: int = 42,
-                 cuda_graph: bool = True, weight_tiles: bool | None = None, mem_fraction_static: float = 0.85):
+                 cuda_graph: bool = True, weight_tiles: bool | None = None, mem_fraction_static: float = 0.85,
+                 async_overlap: bool = True):
         """model: a model folder, or an Engine that is already built.
 
         kv_cache_tokens: tokens the paged cache holds over all live requests.  Default: sized from the GPU's
@@ -56,6 +57,8 @@ class LLM:
         memory (the reference's --mem-fraction-static, default 0.85), and never more than num_slots requests
         of max_seq_len tokens (default: the model's positions) can fill.
         cuda_graph, weight_tiles: as for Engine (captured steps; the decode-friendly second copy of the weights).
+        async_overlap: decode steps are launched from the last step's tokens on the GPU, and those are read back
+        while the new step runs (SchedulerConfig.async_overlap); the tokens are the same either way.
         """
         if isinstance(model, Engine):
             self.engine = model
@@ -77,7 +80,7 @@ class LLM:
         self.sched_config = SchedulerConfig(
             num_slots=self.engine.cache.max_slots, chunked_prefill_size=chunked_prefill_size,
             max_num_batched_tokens=max_num_batched_tokens, max_prefill_tokens=max_prefill_tokens,
-            prefill_max_requests=prefill_max_requests, max_seq_len=max_seq_len)
+            prefill_max_requests=prefill_max_requests, max_seq_len=max_seq_len, async_overlap=async_overlap)
         self.sampler = Sampler(self.engine.device)
         self.tokenizer = self._load_tokenizer()
         self.last_stats: dict = {}

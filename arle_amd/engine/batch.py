@@ -14,12 +14,23 @@ import numpy as np
 import torch
 
 from ..cache import native
+from ..kernels.upload import staging_for, upload
+
+
+@dataclass(frozen=True)
+class DeviceToken:
+    """A token that the host does not know yet: element `row` of an int32 tensor on the GPU, which a sampling
+    kernel of the step before wrote (or will have written when this step's kernels run: same stream).  As the one
+    token of an entry it lets the next decode step be launched before the last one's tokens are read back, as the
+    reference hands its argmax output to the next step on the device (infer/src/model/qwen3/batch_decode.rs:683-774)."""
+    source: object
+    row: int
 
 
 @dataclass
 class StepEntry:
     request: object          # key of a live request
-    tokens: list             # its next token ids (>= 1)
+    tokens: list             # its next token ids (>= 1), or [DeviceToken]
     want: list = field(default_factory=list)  # places among `tokens` whose logits are wanted
 
 
@@ -68,12 +79,15 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device, into=
         raise ValueError("a step needs at least one entry")
     seen = set()
     segments, row = [], 0
+    fed = []     # (row of the step, DeviceToken): token ids that come from GPU memory
     for e in entries:
         if e.request in seen:
             raise ValueError(f"request {e.request!r} appears twice in one step")
         seen.add(e.request)
         if len(e.tokens) == 0:
             raise ValueError(f"request {e.request!r} brings no tokens")
+        if len(e.tokens) == 1 and isinstance(e.tokens[0], DeviceToken):
+            fed.append((row, e.tokens[0]))
         segments.append(Segment(e.request, slot_of(e.request), length_of(e.request), len(e.tokens), row))
         row += len(e.tokens)
     # the arrays themselves are laid out by the native runtime core, which also checks ids and places;
@@ -83,11 +97,20 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device, into=
     staged += [s.start for s in segments]
     staged += [s.length for s in segments]
     staged += [len(e.want) for e in entries]
-    for e in entries:
-        staged += e.tokens
+    if fed:
+        device_rows = {r for r, _ in fed}
+        for seg, e in zip(segments, entries):
+            staged += [0] if seg.row0 in device_rows and seg.length == 1 else e.tokens   # 0 until the GPU fills it in
+    else:
+        for e in entries:
+            staged += e.tokens
     for e in entries:
         staged += e.want
-    wide = np.array(staged, dtype=np.int64)
+    try:
+        wide = np.array(staged, dtype=np.int64)
+    except (TypeError, ValueError):
+        raise ValueError("token ids and wanted places are integers (a DeviceToken only as the one token of an "
+                         "entry)") from None
     np.clip(wide, -1, 2**31 - 1, out=wide)     # what is out of range stays out of range
     inputs = wide.astype(np.int32)
     num_wanted = inputs.size - 4 * S - row
@@ -121,12 +144,35 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device, into=
     else:
         if into.numel() != flat.numel():
             raise ValueError("the fixed step buffer does not fit this step")
-        into.copy_(flat)
+        staging_for(device).copy_into(into, flat_np)
         packed = into
     dev, off = {}, 0
     for k, n in zip(order, sizes):
         dev[k] = packed[off:off + n]
         off += n
+    if fed:
+        feed_device_tokens(dev["token_ids"], fed)
     return StepBatch(num_tokens=row, segments=segments, max_position=meta[2], max_qlen=meta[3], min_qlen=meta[4],
                      single_segments=meta[5],
                      host=host, **dev)
+
+
+def feed_device_tokens(token_ids: torch.Tensor, fed) -> None:
+    """token_ids[row] = source[source_row] for every (row, DeviceToken(source, source_row)), on the GPU."""
+    by_source: dict = {}
+    for row, tok in fed:
+        by_source.setdefault(id(tok.source), (tok.source, [], []))
+        by_source[id(tok.source)][1].append(row)
+        by_source[id(tok.source)][2].append(int(tok.row))
+    for source, rows, source_rows in by_source.values():
+        if source.device != token_ids.device or source.dim() != 1:
+            raise ValueError("a DeviceToken names a one-dimensional tensor on the engine's GPU")
+        if min(source_rows) < 0 or max(source_rows) >= source.numel():
+            raise ValueError("a DeviceToken names a row outside its tensor")
+        n = len(rows)
+        if rows == list(range(rows[0], rows[0] + n)) and source_rows == list(range(source_rows[0], source_rows[0] + n)):
+            token_ids[rows[0]:rows[0] + n].copy_(source[source_rows[0]:source_rows[0] + n])     # the usual case: one copy
+            continue
+        index = upload(np.array([rows, source_rows], dtype=np.int32), token_ids.device).long()
+        token_ids.index_copy_(0, index[0], source.index_select(0, index[1]).to(torch.int32))
+

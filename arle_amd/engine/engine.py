@@ -23,7 +23,7 @@ from ..parts.base import Runtime
 from ..weights.loader import load_weights
 from ..weights.random_init import random_weights
 from ..kernels import ops
-from .batch import StepEntry, build_step_batch, packed_size
+from .batch import DeviceToken, StepEntry, build_step_batch, packed_size
 
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
           "fp32": torch.float32}
@@ -175,7 +175,7 @@ class Engine:
             for e in entries:
                 if any(int(w) != 0 for w in e.want):
                     raise ValueError(f"wanted place outside the one token of request {e.request!r}")
-                if not 0 <= int(e.tokens[0]) < self.spec.vocab_size:
+                if not isinstance(e.tokens[0], DeviceToken) and not 0 <= int(e.tokens[0]) < self.spec.vocab_size:
                     raise ValueError(f"token id {e.tokens[0]} of request {e.request!r} is outside the vocabulary "
                                      f"(size {self.spec.vocab_size})")
         self.cache.append([(e.request, len(e.tokens)) for e in entries])

@@ -65,6 +65,7 @@ class SchedulerConfig:
     long_prefill_token_threshold: int = 512
     max_waiting_requests: int = 256
     max_seq_len: int | None = None
+    async_overlap: bool = True   # launch a decode step from the last one's tokens on the GPU, read those back after
 
     def validate(self) -> None:
         for name in ("num_slots", "chunked_prefill_size", "max_num_batched_tokens",
@@ -95,6 +96,7 @@ class Request:
     t_first_token: float | None = None
     t_finish: float | None = None
     t_tokens: list = field(default_factory=list)   # when each generated token arrived (for the time per output token)
+    pending: int = 0                               # tokens that a launched step has chosen and the host has not read yet
 
     @property
     def remaining_prompt(self) -> int:
@@ -111,6 +113,19 @@ class StepPlan:
         if self.decode and self.prefill:
             return "mixed"
         return "decode" if self.decode else ("prefill" if self.prefill else "idle")
+
+
+class _ChosenNow:
+    """What a sampler that answers at once chose, in the shape of the sampler's `Chosen`."""
+
+    def __init__(self, tokens, logprobs):
+        self._tokens, self._logprobs = list(tokens), logprobs
+
+    def tokens(self):
+        return self._tokens
+
+    def logprobs(self):
+        return self._logprobs
 
 
 def retract_victim(decoding: list):
@@ -168,6 +183,7 @@ class Scheduler:
         self.decoding: list = []
         self.finished: dict = {}
         self._next_id = 0
+        self._pending = None    # (requests, Chosen) of the step whose tokens have not been read back
         pool_tokens = min((g.pool.num_pages for g in self.cache.groups), default=1 << 30) * self.cache.page_size
         context = self.cfg.max_seq_len or pool_tokens
         context = min(context, self.cache.max_pages_per_request * self.cache.page_size)
@@ -223,13 +239,26 @@ class Scheduler:
 
     # -- one iteration ------------------------------------------------------------------------
     def has_work(self) -> bool:
-        return bool(self.waiting or self.prefilling or self.decoding)
+        return bool(self.waiting or self.prefilling or self.decoding or self._pending is not None)
 
     def iteration(self) -> StepPlan:
-        self._admit()
-        plan = self._plan()
-        if plan.kind != "idle":
-            self._run(plan)
+        """One step.  The tokens that a step chooses stay on the GPU until the next iteration reads them
+        (the reference launches in iteration i and reads back in i + 1: infer/src/scheduler/cuda/execution.rs:676-708).
+        While nothing but the same requests' next decode step can follow, that step is launched first, from
+        the tokens on the GPU, and the last step's tokens are read while it runs; anything else (a portion to
+        plan, a request about to reach its length, pages running out, penalties that need the token's value)
+        reads them first and plans as usual."""
+        if self._pending is not None and self._can_run_ahead():
+            plan = self._run_ahead()
+        else:
+            self._settle()
+            self._cleanup()     # what the read tokens finished gives its slot and pages back before the plan
+            self._admit()
+            plan = self._plan()
+            if plan.kind != "idle":
+                self._run(plan)
+            if not self.cfg.async_overlap or (self._pending is not None and not hasattr(self._pending[1], "feed")):
+                self._settle()      # nothing to gain from waiting: the tokens are on the host already
         self._cleanup()
         return plan
 
@@ -328,12 +357,68 @@ class Scheduler:
             r.fed += n
         if not sampled:
             return
-        rows = [(r.sampling, r.seed, len(r.generated), r.generated) for r in sampled]
-        tokens, logprobs = self.sampler.sample_with_logprobs(logits, rows)
+        self._choose(logits, sampled, plan)
+
+    def _choose(self, logits, sampled: list, plan: StepPlan) -> None:
+        """Queue the sampling of a step's wanted rows; what it chooses is read by `_settle`."""
+        rows = [(r.sampling, r.seed, len(r.generated) + r.pending, r.generated) for r in sampled]
+        if hasattr(self.sampler, "choose"):
+            chosen = self.sampler.choose(logits, rows)
+        else:   # a sampler that answers at once
+            chosen = _ChosenNow(*self.sampler.sample_with_logprobs(logits, rows))
+        for r in sampled:
+            r.pending += 1
+        self._pending = (sampled, chosen, plan)
+
+    def _settle(self) -> None:
+        """Read the pending step's tokens and apply them: a request that has finished meanwhile (a stop token
+        one step earlier, an abort) takes none."""
+        if self._pending is None:
+            return
+        sampled, chosen, _ = self._pending
+        self._pending = None
+        tokens, logprobs = chosen.tokens(), chosen.logprobs()
         now = time.perf_counter()
         for i, (r, tok) in enumerate(zip(sampled, tokens)):
+            r.pending -= 1
+            if r.phase == "finished":
+                continue
             wants = logprobs is not None and r.sampling.logprobs
             self._apply_token(r, int(tok), now, float(logprobs[i]) if wants else None)
+
+    # -- a decode step launched before the last one's tokens are known ------------------------------
+    def _can_run_ahead(self) -> bool:
+        if not self.cfg.async_overlap:
+            return False
+        sampled, chosen, plan = self._pending
+        if plan.prefill or self.prefilling or not hasattr(chosen, "feed"):
+            return False
+        if self.waiting and self.cache.free_slot_count > 0:
+            return False    # an admission may change the next step
+        rows = [r for r in sampled if r.phase == "decoding"]
+        if not rows or len(rows) != len(self.decoding):
+            return False
+        for r in rows:
+            if r.sampling.has_penalties() or len(r.generated) + r.pending >= r.max_tokens:
+                return False    # the token's value is needed, or it is the request's last
+        return self.cache.can_append([(r.id, 1) for r in rows])
+
+    def _run_ahead(self) -> StepPlan:
+        sampled, chosen, _ = self._pending
+        rows = [(i, r) for i, r in enumerate(sampled) if r.phase == "decoding"]
+        plan = StepPlan([r for _, r in rows], [])
+        logits = self.engine.step([StepEntry(r.id, [chosen.feed(i)], [0]) for i, r in rows])
+        self.stats["steps"]["decode"] += 1
+        self.stats["steps_ahead"] = self.stats.get("steps_ahead", 0) + 1
+        self.stats["tokens_decoded"] += len(rows)
+        held = max((g.pool.num_pages - g.pool.free_count for g in self.cache.groups), default=0)
+        self.stats["pages_high_water"] = max(self.stats["pages_high_water"], held)
+        before = self._pending
+        self._choose(logits, plan.decode, plan)     # queued behind the step; _pending is the new step now
+        ahead, self._pending = self._pending, before
+        self._settle()                              # the step before: its tokens are there by now
+        self._pending = ahead
+        return plan
 
     def _apply_token(self, r: Request, tok: int, now: float, logprob: float | None = None) -> None:
         if r.phase == "prefilling":

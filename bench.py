@@ -375,6 +375,8 @@ def sweep(args) -> int:
                                 max_tokens=8 * longest + 40 * 4096, max_slots=129, max_request_tokens=longest)
     gen = torch.Generator().manual_seed(1234)
     rand = lambda n: torch.randint(0, config.vocab_size, (n,), generator=gen).tolist()
+    from arle_amd.sampling import Sampler, SamplingParams
+    sampler, greedy_rows = Sampler(engine.device), [(SamplingParams(), 0, 0, [])] * 129
     base = {"n_gpus": 1, "dtype": "bf16", "higher_is_better": True, "data": "synthetic", "layers": args.layers}
 
     def fill(keys, context, portion=8192):
@@ -392,13 +394,23 @@ def sweep(args) -> int:
         keys = [("s", batch, context, i) for i in range(batch)]
         state = {"last": fill(keys, context)}
 
-        def one_step():
-            out = engine.step([StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])])
-            state["last"] = ops.argmax_rows(out).tolist()
+        def one_step():     # as the headline run: launched from the last step's tokens on the GPU, those read meanwhile
+            before = state.get("chosen")
+            if before is None:
+                entries = [StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])]
+            else:
+                entries = [StepEntry(k, [before.feed(i)], [0]) for i, k in enumerate(keys)]
+            state["chosen"] = sampler.choose(engine.step(entries), greedy_rows[:batch])
+            if before is not None:
+                state["last"] = before.tokens()
+
+        def settle():
+            state["last"] = state.pop("chosen").tokens()
 
         for _ in range(6):
             one_step()
-        dt = _timed(torch, lambda: [one_step() for _ in range(steps)]) / steps
+        settle()
+        dt = _timed(torch, lambda: ([one_step() for _ in range(steps)], settle())) / steps
         ctx = engine.length(keys[0]) - steps / 2.0
         for k in keys:
             engine.end_request(k)
@@ -472,6 +484,9 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=PAGE, help="tokens per cache page")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 decode points")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="decode steps wait for their tokens on the host before the next is prepared (default: the "
+                         "next step is launched from the tokens on the GPU, as the scheduler does)")
     ap.add_argument("--no-weight-tiles", action="store_true",
                     help="without the second copy of the projection weights that the few-rows kernels stream")
     ap.add_argument("--no-parts", action="store_true",
@@ -512,6 +527,7 @@ def main() -> int:
     from arle_amd.config import Qwen3Config
     from arle_amd.engine import Engine, StepEntry
     from arle_amd.kernels import ops
+    from arle_amd.sampling import Sampler, SamplingParams
 
     raw = dict(QWEN3_4B, num_hidden_layers=args.layers)
     config = Qwen3Config.from_dict(raw)
@@ -524,6 +540,8 @@ def main() -> int:
                                 max_request_tokens=CONTEXT, weight_tiles=False if args.no_weight_tiles else None)
     print(f"[bench] engine ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
     gen = torch.Generator().manual_seed(1234)
+    sampler = Sampler(engine.device)       # the product's sampler: greedy rows are one argmax kernel, read back on its own stream
+    greedy_rows = [(SamplingParams(), 0, 0, [])] * (max_batch + 1)
 
     def prompt_tokens(n):
         return torch.randint(0, config.vocab_size, (n,), generator=gen).tolist()
@@ -568,16 +586,35 @@ def main() -> int:
             group = keys[i:i + per_step]
             out = engine.step([StepEntry(k, prompt_tokens(PROMPT), [PROMPT - 1]) for k in group])
             last.extend(ops.argmax_rows(out).tolist())
-        state = {"last": last}
+        state = {"last": last, "chosen": None}
 
         def one_step():
-            out = engine.step([StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])])
-            state["last"] = ops.argmax_rows(out).tolist()   # the host needs the token to go on
+            """A decode step as the scheduler runs it (Scheduler._run_ahead): launched from the tokens that the
+            step before left on the GPU, which the host reads back while this step runs.  --no-overlap: every
+            step waits for its tokens on the host before the next is prepared."""
+            if args.no_overlap or parts:
+                out = engine.step([StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])])
+                state["last"] = ops.argmax_rows(out).tolist()   # the host needs the token to go on
+                return
+            before = state["chosen"]
+            if before is None:
+                entries = [StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])]
+            else:
+                entries = [StepEntry(k, [before.feed(i)], [0]) for i, k in enumerate(keys)]
+            state["chosen"] = sampler.choose(engine.step(entries), greedy_rows[:batch])
+            if before is not None:
+                state["last"] = before.tokens()                 # the step before: every token reaches the host
+
+        def settle():
+            if state["chosen"] is not None:
+                state["last"] = state["chosen"].tokens()
+                state["chosen"] = None
 
         for _ in range(warmup):
             one_step()
         ctx0 = engine.length(keys[0])
-        dt = timed(lambda: [one_step() for _ in range(steps)])
+        settle()
+        dt = timed(lambda: ([one_step() for _ in range(steps)], settle()))   # the last step's tokens are read inside
         ctx_mean = ctx0 + (steps - 1) / 2.0 + 1
         if parts:
             from arle_amd.kernels import ceilings as measured
@@ -629,7 +666,8 @@ def main() -> int:
                    "kv_heads": raw["num_key_value_heads"], "head_dim": raw["head_dim"],
                    "intermediate": raw["intermediate_size"], "vocab": raw["vocab_size"],
                    "rope_theta": raw["rope_theta"], "rms_norm_eps": raw["rms_norm_eps"], "tied": True,
-                   "page_size": PAGE, "weight_tiles": engine.rt.weight_tiles},
+                   "page_size": PAGE, "weight_tiles": engine.rt.weight_tiles,
+                   "readback_lag_steps": 0 if args.no_overlap else 1},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},

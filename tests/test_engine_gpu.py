@@ -201,3 +201,45 @@ def test_head_dim_that_is_no_multiple_of_16_runs_in_float32_and_is_refused_in_bf
     replay.compare(got, cfg, weights, reqs, TOL["float32"], "head_dim 24 / float32")
     with pytest.raises(ValueError, match="multiples of 16"):
         Engine.from_folder(d, dtype="bfloat16", page_size=8, max_tokens=64)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_tokens_fed_from_gpu_memory_give_the_bits_of_tokens_fed_from_the_host(model, dtype):
+    """An entry's one token may be a DeviceToken, an element of an int32 tensor on the GPU: eager steps, captured
+    decode steps and a decoded token beside a prompt portion must give the same logits as with the id itself,
+    whatever the order of the rows in the tensor."""
+    from arle_amd.engine import DeviceToken, StepEntry
+
+    name, d, cfg, _ = model
+    reqs = _requests(cfg, [37, 52, 44], 1200)
+    outs = {}
+    for fed in (False, True):
+        eng = Engine.from_folder(d, dtype=dtype, page_size=TINY[name][1], max_tokens=320, max_slots=4)
+        got = []
+        for rid, toks in reqs.items():
+            eng.add_request(rid)
+            eng.step([StepEntry(rid, toks[:20], [])])
+        for i in range(20, 30):                                     # decode steps of three rows: captured from the second on
+            ids = [toks[i] for toks in reqs.values()]
+            if fed:
+                source = torch.tensor(ids[::-1] + [0], dtype=torch.int32, device=eng.device)    # reversed, and one more
+                entries = [StepEntry(rid, [DeviceToken(source, 2 - j)], [0]) for j, rid in enumerate(reqs)]
+            else:
+                entries = [StepEntry(rid, [t], [0]) for rid, t in zip(reqs, ids)]
+            got.append(eng.step(entries).clone())
+        rid0, rid1 = list(reqs)[:2]                                # a decoded token beside a portion of another request
+        t0 = reqs[rid0][30]
+        first = [DeviceToken(torch.tensor([t0], dtype=torch.int32, device=eng.device), 0)] if fed else [t0]
+        got.append(eng.step([StepEntry(rid0, first, [0]), StepEntry(rid1, reqs[rid1][30:37], [6])]).clone())
+        assert eng.graph_replays >= 8
+        outs[fed] = got
+    for a, b in zip(outs[False], outs[True]):
+        assert torch.equal(a, b)
+    eng = Engine.from_folder(d, dtype=dtype, page_size=TINY[name][1], max_tokens=64, max_slots=2)
+    eng.add_request(0)
+    source = torch.zeros(2, dtype=torch.int32, device=eng.device)
+    with pytest.raises(ValueError, match="DeviceToken"):
+        eng.step([StepEntry(0, [DeviceToken(source, 0), 3], [1])])       # only as the one token of an entry
+    with pytest.raises(ValueError, match="outside its tensor"):
+        eng.step([StepEntry(0, [DeviceToken(source, 2)], [0])])
+    assert eng.length(0) == 0

@@ -289,3 +289,39 @@ def test_the_pool_is_sized_from_free_memory_when_no_size_is_given(folders):
 
     with pytest.raises(EngineError, match="no memory for the cache"):
         Engine.from_folder(folders["A"], dtype="bfloat16", mem_fraction_static=1e-6)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_launched_ahead_give_the_tokens_of_steps_that_wait(folders, dtype):
+    """Decode steps fed from the last step's tokens on the GPU, read back one step late, against steps that
+    read every token before they go on: greedy and seeded sampling with log-probabilities, requests that end by
+    a stop token (one row runs in vain), by their length, and arrive in waves."""
+    from arle_amd.engine import Engine
+
+    cfg, weights = read_folder(folders["B"])
+    rng = np.random.default_rng(11)
+    prompts = [random_tokens(int(n), cfg["vocab_size"], 700 + i) for i, n in enumerate(rng.integers(2, 40, size=12))]
+    free_run = _plain_greedy(cfg, weights, prompts[0], 12) if dtype == "float32" else None
+    results = {}
+    for overlap in (False, True):
+        eng = Engine.from_folder(folders["B"], dtype=dtype, page_size=TINY["B"][1], max_tokens=400, max_slots=4,
+                                 max_request_tokens=96)
+        llm = LLM(eng, num_slots=4, chunked_prefill_size=16, max_num_batched_tokens=48, max_seq_len=96,
+                  async_overlap=overlap)
+        greedy = llm.generate(prompts[:6], max_tokens=12, sampling=SamplingParams(temperature=0.0, ignore_eos=True))
+        ahead = llm.last_stats.get("steps_ahead", 0)
+        drawn = llm.generate(prompts[6:], max_tokens=9, sampling=SamplingParams(temperature=0.8, top_p=0.9, seed=3,
+                                                                                 ignore_eos=True, logprobs=True))
+        stop = greedy[0].response_token_ids[5]
+        stopped = llm.generate(prompts[:3], max_tokens=12, sampling=SamplingParams(stop_token_ids=[stop]))
+        results[overlap] = ([o.response_token_ids for o in greedy], [o.response_token_ids for o in drawn],
+                            [o.token_logprobs for o in drawn], [(o.response_token_ids, o.finish_reason) for o in stopped])
+        assert (ahead >= 8) == overlap and (llm.last_stats.get("steps_ahead", 0) > 0) == overlap
+        assert stopped[0].finish_reason == "stop" and stop not in stopped[0].response_token_ids
+        assert not eng.cache.slot_of
+        for g in eng.cache.groups:
+            g.check()
+            assert g.pool.free_count == g.pool.num_pages
+    assert results[False] == results[True]
+    if free_run is not None:
+        assert results[True][0][0] == free_run

@@ -306,3 +306,135 @@ def test_logprobs_reach_the_request_only_when_asked_for():
     ra, rb = s.finished[a], s.finished[b]
     assert ra.logprobs == [-0.5 - t for t in ra.generated] and rb.logprobs == []
     assert len(ra.t_tokens) == 4 and ra.t_tokens == sorted(ra.t_tokens)
+
+
+# -- decode steps launched before the last step's tokens are read ---------------------------------------------
+from arle_amd.engine.batch import DeviceToken
+
+
+class LazyChosen:
+    """What the GPU sampler's `Chosen` is to the scheduler: tokens that can be fed on without being read."""
+
+    def __init__(self, tokens, logprobs, log):
+        self._tokens, self._logprobs, self.log = list(tokens), logprobs, log
+
+    def feed(self, row):
+        return DeviceToken(self._tokens, row)
+
+    def tokens(self):
+        self.log.append("read")
+        return self._tokens
+
+    def logprobs(self):
+        return self._logprobs
+
+
+class LazySampler(FakeSampler):
+    def __init__(self):
+        self.log = []
+
+    def choose(self, logits, rows):
+        self.draw_indices = [idx for _, _, idx, _ in rows]
+        return LazyChosen(*self.sample_with_logprobs(logits, rows), self.log)
+
+
+class LazyEngine(FakeEngine):
+    """Takes a DeviceToken where a token id stands, as the real step does."""
+
+    def step(self, entries):
+        from arle_amd.engine.batch import StepEntry
+        self.sampler_log.append("step")
+        plain = [StepEntry(e.request, [t.source[t.row] if isinstance(t, DeviceToken) else t for t in e.tokens], e.want)
+                 for e in entries]
+        self.fed_from_device = sum(isinstance(e.tokens[0], DeviceToken) for e in entries)
+        return super().step(plain)
+
+
+def make_lazy(num_pages=64, page_size=4, slots=4, stop=(), **cfg):
+    eng, sampler = LazyEngine(num_pages, page_size, slots), LazySampler()
+    eng.sampler_log = sampler.log
+    return eng, Scheduler(eng, sampler, SchedulerConfig(num_slots=slots, **cfg), stop_token_ids=stop), sampler
+
+
+def run_both(submit, **kw):
+    """The same requests with and without steps launched ahead: (records, scheduler) each."""
+    out = []
+    for overlap in (True, False):
+        eng, s, _ = make_lazy(async_overlap=overlap, **kw)
+        ids = submit(s)
+        s.run_until_done()
+        eng.cache.check()
+        assert not eng.cache.slot_of and eng.cache.free_pages() == [kw.get("num_pages", 64)]
+        out.append(([(s.finished[i].generated, s.finished[i].finish_reason, s.finished[i].logprobs) for i in ids], s))
+    return out
+
+
+def test_steps_launched_ahead_give_the_same_tokens():
+    def submit(s):
+        return [s.submit(prompt(10, k), SamplingParams(logprobs=k == 1), max_tokens=5 + 3 * k) for k in range(3)]
+    (ahead, s_ahead), (plain, s_plain) = run_both(submit)
+    assert ahead == plain
+    assert [g for g, _, _ in ahead] == [expected_output(prompt(10, k), 5 + 3 * k) for k in range(3)]
+    assert s_ahead.stats["steps_ahead"] >= 6 and "steps_ahead" not in s_plain.stats
+    # no token is computed twice or in vain when requests end by their length
+    assert s_ahead.stats["tokens_decoded"] == s_plain.stats["tokens_decoded"]
+
+
+def test_a_step_ahead_is_launched_before_the_last_tokens_are_read():
+    eng, s, sampler = make_lazy()
+    s.submit(prompt(6), max_tokens=6)
+    s.iteration()                        # the prompt; its token stays with the sampler
+    assert sampler.log == ["step"]
+    s.iteration()                        # a portion came before: read first, then the first decode step
+    assert sampler.log == ["step", "read", "step"] and eng.fed_from_device == 0
+    s.iteration()                        # decode follows decode: launched from the tokens not yet read
+    assert sampler.log == ["step", "read", "step", "step", "read"] and eng.fed_from_device == 1
+    assert sampler.draw_indices == [2]   # the third draw of the request, though the host knows one token only
+    s.run_until_done()
+    assert s.finished[0].generated == expected_output(prompt(6), 6)
+
+
+def test_a_stop_token_one_step_late_wastes_one_row_and_nothing_else():
+    full = expected_output(prompt(8, 3), 12)
+    stop = full[5]
+    assert stop not in full[:5]
+    def submit(s):
+        return [s.submit(prompt(8, 3), max_tokens=12), s.submit(prompt(9, 1), max_tokens=12)]
+    (ahead, s_ahead), (plain, s_plain) = run_both(submit, stop=(stop,))
+    assert ahead == plain
+    assert ahead[0][0] == full[:5] and ahead[0][1] == STOP      # the stop token is not emitted, nor what came after
+    # the row that was launched for the stopped request before its stop token was read
+    assert s_ahead.stats["tokens_decoded"] == s_plain.stats["tokens_decoded"] + 1
+
+
+def test_arrivals_preemptions_and_penalties_fall_back_to_reading_first():
+    def submit(s):
+        ids = [s.submit(prompt(7, 1), max_tokens=20), s.submit(prompt(5, 2), SamplingParams(repetition_penalty=1.2), max_tokens=6)]
+        for _ in range(4):
+            s.iteration()
+        ids.append(s.submit(prompt(12, 4), max_tokens=9))       # arrives while the others decode
+        return ids
+    (ahead, s_ahead), (plain, _) = run_both(submit, chunked_prefill_size=8)
+    assert ahead == plain
+    assert s_ahead.stats["steps_ahead"] > 0
+    # a pool so small that decoding requests have to give pages back
+    def crowd(s):
+        return [s.submit(prompt(6, k), max_tokens=14) for k in range(3)]
+    (ahead, s_ahead), (plain, s_plain) = run_both(crowd, num_pages=10, slots=3)
+    assert ahead == plain and s_ahead.stats["preemptions"] > 0
+    assert [g for g, _, _ in ahead] == [expected_output(prompt(6, k), 14) for k in range(3)]
+
+
+def test_abort_while_a_step_is_pending():
+    eng, s, _ = make_lazy()
+    a, b = s.submit(prompt(6, 1), max_tokens=30), s.submit(prompt(7, 2), max_tokens=10)
+    for _ in range(5):
+        s.iteration()
+    assert s.stats["steps_ahead"] >= 2
+    kept = list(s.finished.get(a, s.decoding[0]).generated)
+    assert s.abort(a)
+    assert s.finished[a].generated == kept == expected_output(prompt(6, 1), len(kept))
+    s.run_until_done()
+    eng.cache.check()
+    assert s.finished[b].generated == expected_output(prompt(7, 2), 10)
+    assert not eng.cache.slot_of and eng.cache.free_pages() == [64] and not s.has_work()
