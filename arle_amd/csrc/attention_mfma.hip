@@ -1609,7 +1609,7 @@ static AttnArgs make_args(const void* q, long long q_stride, void* out, long lon
 // step: seg_row0[s]..seg_row0[s+1] are the token rows of segment s, whose first token sits at
 // position seg_start[s] of the request in block-table row seg_slot[s]; the cache already holds
 // the keys and values of these tokens.  max_qlen / min_qlen are the longest and shortest segment, max_kv_len the most
-// keys any request holds after the step (it only steers the choice between kernels).  With splits > 1,
+// keys that a segment of more than one token holds after the step (it only steers choices of the portions kernels).  With splits > 1,
 // ws_o/ws_ml must hold [segments * ws_rows][nq][splits][D] and [..][2] floats, ws_rows = arle_attn_ws_rows(...),
 // and the merge runs after; the split is over the keys of segments of at most 16 rows (decoded tokens and
 // portions of a few tokens).  Longer portions go to the LDS kernel; when they have too few row blocks to fill

@@ -61,6 +61,7 @@ class StepBatch:
     single_segments: int = 0     # segments of one token (decoded tokens)
     kv_splits: int | None = None  # split-KV factor fixed by the caller (a captured graph), else chosen per call
     plan_token: int = 0          # names one pass over the layers (set by the model): what parts plan once a pass
+    max_portion_kv: int = 0      # longest context (cached + new) among the segments of more than one token; 0: none
 
 
 def packed_size(num_tokens: int, num_segments: int, num_wanted: int) -> int:
@@ -154,6 +155,7 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device, into=
         feed_device_tokens(dev["token_ids"], fed)
     return StepBatch(num_tokens=row, segments=segments, max_position=meta[2], max_qlen=meta[3], min_qlen=meta[4],
                      single_segments=meta[5],
+                     max_portion_kv=max((s.start + s.length for s in segments if s.length > 1), default=0),
                      host=host, **dev)
 
 

@@ -66,6 +66,8 @@ class SchedulerConfig:
     max_waiting_requests: int = 256
     max_seq_len: int | None = None
     async_overlap: bool = True   # launch a decode step from the last one's tokens on the GPU, read those back after
+    step_row_alignment: int = 128  # a portion that does not end its prompt is shortened until the step's rows are a
+                                   # multiple of this, if at least as many tokens stay (0: portions as the reference cuts them)
 
     def validate(self) -> None:
         for name in ("num_slots", "chunked_prefill_size", "max_num_batched_tokens",
@@ -157,6 +159,14 @@ def plan_prefill(queue, decode_rows: int, cfg: SchedulerConfig, fits) -> list:
         n = min(remaining, max(cap, 1))
         if n > tokens_left or requests_left <= 0:
             continue  # skipped whole, never shrunk; a later, smaller one may still fit
+        # The matrix products of a step run in tiles of 128 and 256 rows: 8 decoded tokens beside a portion of 512
+        # are 520 rows and cost a tenth more than 512 (measured on MI355X, Qwen3-4B shape: 9.8 against 8.7 ms).  A
+        # portion that is cut anyway gives up the few tokens that stand over; they come with the next one.
+        align = cfg.step_row_alignment
+        if align > 0 and n < remaining:
+            over = (decode_rows + sum(m for _, m in picked) + n) % align
+            if over and n - over >= align:
+                n -= over
         completes = n == remaining
         first_decode = 1 if completes and req.max_tokens - len(req.generated) > 0 else 0
         if not fits(reserved, req, n + first_decode):

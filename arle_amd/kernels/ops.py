@@ -378,7 +378,7 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
                     max_qlen: int, max_kv_len: int, num_q_heads: int, num_kv_heads: int, head_dim: int,
                     page_size: int, scale: float, window: int = 0, splits: int | None = None,
                     min_qlen: int = 1, short_segments: int | None = None, portion_splits: int | None = None,
-                    plan_token: int = 0):
+                    plan_token: int = 0, max_portion_kv_len: int | None = None):
     """Causal attention of a packed step on the matrix cores (bfloat16).
 
     Segments: rows seg_row0[s]..seg_row0[s+1] belong to block-table row seg_slot[s] and start at
@@ -388,6 +388,9 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
     Longer portions that are too few to fill the chip have their keys cut into `portion_splits` parts
     (default: portion_key_splits).  `plan_token` (new_plan_token()) names the step: with the same token and the
     same segments the portions kernels list their work once, for the first layer, and not once a layer.
+    `max_portion_kv_len`: the longest context among the segments of more than one token (default: max_kv_len); what
+    the portions kernels plan by, so that a fresh portion beside requests that decode deep into their contexts is
+    not cut into parts for the decoders' sake.
     """
     _gpu(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start)
     tokens = q.shape[0]
@@ -423,7 +426,7 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
     if portion_splits is None:
         long_segments = segments if short_segments is None else max(1, segments - short_segments)
         portion_splits = portion_key_splits(tokens, max_qlen, long_segments, num_q_heads, num_kv_heads, head_dim,
-                                            max_kv_len, q.device)
+                                            max_portion_kv_len or max_kv_len, q.device)
     if max_qlen * group <= _ATTN_ROW_TILE:
         portion_splits = 1              # no portion for the kernel that they are for
     _need(1 <= portion_splits <= _PORTION_SPLITS_MAX, f"portion_splits must be 1..{_PORTION_SPLITS_MAX}")
@@ -434,7 +437,7 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
     lib.call("arle_attn_paged_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
              k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
              seg_row0.data_ptr(), seg_slot.data_ptr(), seg_start.data_ptr(), segments, int(max_qlen),
-             int(min_qlen), int(max_kv_len), tokens,
+             int(min_qlen), int(max_portion_kv_len or max_kv_len), tokens,
              num_q_heads, num_kv_heads, head_dim, page_size, float(scale), int(window), int(splits),
              _ptr(ws_o), _ptr(ws_ml), int(portion_splits), _ptr(pws_o), _ptr(pws_ml), int(plan_token), _stream())
     return out

@@ -141,7 +141,8 @@ def paged_attention(q, out, cache, batch, *, num_q_heads, num_kv_heads, head_dim
                             num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=cache.page_size,
                             scale=scale, window=window, splits=getattr(batch, "kv_splits", None),
                             short_segments=getattr(batch, "single_segments", 0) or None,
-                            plan_token=getattr(batch, "plan_token", 0))
+                            plan_token=getattr(batch, "plan_token", 0),
+                            max_portion_kv_len=getattr(batch, "max_portion_kv", 0) or None)
     else:
         ops.attn_paged_simt(q, out, cache.k_pages, cache.v_pages, cache.block_table, batch.positions,
                             batch.slot_of_token, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads,

@@ -361,7 +361,7 @@ def decode_32b(args) -> int:
 def sweep(args) -> int:
     """Further sizes of the Qwen3-4B shape, one JSON line each with its fraction of the roofline: decode at batch 16
     and 32 (2,048-token prompts), at batch 128 (1,024 tokens of context), at batch 8 with 8,192 and 32,768 tokens of
-    context, prefills of 8,192, 512 and 128 tokens, and a 512-token prompt portion beside 8 decoding requests."""
+    context, prefills of 8,192, 512 and 128 tokens, and a 504-token prompt portion beside 8 decoding requests."""
     import torch
 
     from arle_amd.config import Qwen3Config
@@ -370,7 +370,7 @@ def sweep(args) -> int:
 
     raw = dict(QWEN3_4B, num_hidden_layers=args.layers)
     config = Qwen3Config.from_dict(raw)
-    longest = 32768 + 64
+    longest = 32768 + args.steps + 16     # the longest context, its warm-up and timed steps
     engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype="bfloat16", page_size=PAGE,
                                 max_tokens=8 * longest + 40 * 4096, max_slots=129, max_request_tokens=longest)
     gen = torch.Generator().manual_seed(1234)
@@ -468,7 +468,7 @@ def sweep(args) -> int:
     prefill_point(8192)
     prefill_point(512)
     prefill_point(128)
-    mixed_point(8, 2048, 512, 2048)
+    mixed_point(8, 2048, 504, 2016)      # as the scheduler cuts a long prompt beside 8 decoding requests: 512 rows a step
     return 0
 
 

@@ -149,7 +149,7 @@ def test_a_portion_that_does_not_fit_is_skipped_whole_not_shrunk():
     # pages: the finishing portion asks for one token more (the first decoded token)
     asked = []
     plan_prefill([_req(0, 8), _req(1, 600)], 0, SchedulerConfig(), lambda res, r, n: asked.append((r.id, n)) or True)
-    assert asked == [(0, 9), (1, 512)]
+    assert asked == [(0, 9), (1, 504)]     # the cut portion stops where the step has 8 + 504 = 512 rows
 
 
 def test_retract_victim_is_least_progress_then_longest_prompt():
@@ -438,3 +438,20 @@ def test_abort_while_a_step_is_pending():
     eng.cache.check()
     assert s.finished[b].generated == expected_output(prompt(7, 2), 10)
     assert not eng.cache.slot_of and eng.cache.free_pages() == [64] and not s.has_work()
+
+
+def test_a_cut_portion_gives_up_the_tokens_that_stand_over_a_multiple_of_128_rows():
+    cfg = SchedulerConfig(num_slots=16, chunked_prefill_size=512, long_prefill_token_threshold=512)
+    long_one = Request(0, prompt(2000), SamplingParams(), 8, 0, feed=prompt(2000))
+    fits = lambda reserved, req, n: True
+    assert plan_prefill([long_one], 8, cfg, fits) == [(long_one, 504)]          # 8 + 504 = 512 rows
+    assert plan_prefill([long_one], 0, cfg, fits) == [(long_one, 512)]
+    assert plan_prefill([long_one], 130, cfg, fits) == [(long_one, 510)]        # 130 + 510 = 640
+    short = Request(1, prompt(300), SamplingParams(), 8, 0, feed=prompt(300))
+    assert plan_prefill([short], 8, cfg, fits) == [(short, 300)]                # the end of a prompt is never cut
+    two = plan_prefill([short, long_one], 8, cfg, fits)
+    assert two == [(short, 300), (long_one, 460)] and (8 + 300 + 460) % 128 == 0
+    small = SchedulerConfig(num_slots=16, chunked_prefill_size=200, long_prefill_token_threshold=200)
+    assert plan_prefill([long_one], 8, small, fits) == [(long_one, 200)]        # fewer than 128 tokens would stay
+    off = SchedulerConfig(num_slots=16, chunked_prefill_size=512, long_prefill_token_threshold=512, step_row_alignment=0)
+    assert plan_prefill([long_one], 8, off, fits) == [(long_one, 512)]
