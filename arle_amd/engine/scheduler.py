@@ -254,21 +254,22 @@ class Scheduler:
     def iteration(self) -> StepPlan:
         """One step.  The tokens that a step chooses stay on the GPU until the next iteration reads them
         (the reference launches in iteration i and reads back in i + 1: infer/src/scheduler/cuda/execution.rs:676-708).
-        While nothing but the same requests' next decode step can follow, that step is launched first, from
-        the tokens on the GPU, and the last step's tokens are read while it runs; anything else (a portion to
-        plan, a request about to reach its length, pages running out, penalties that need the token's value)
-        reads them first and plans as usual."""
-        if self._pending is not None and self._can_run_ahead():
-            plan = self._run_ahead()
-        else:
+        The next step is planned and launched first, its decode rows fed from the tokens on the GPU, and the last
+        step's tokens are read while it runs; a request that met a stop token is found out one step late, and
+        the row launched for it has run in vain.  Where the plan needs a token's value or a request's true end
+        (a request about to reach its length, pages running out and somebody to preempt, penalties over the
+        tokens so far), the tokens are read first and the step follows."""
+        if self._pending is not None and not self._can_plan_ahead():
             self._settle()
             self._cleanup()     # what the read tokens finished gives its slot and pages back before the plan
-            self._admit()
-            plan = self._plan()
-            if plan.kind != "idle":
-                self._run(plan)
-            if not self.cfg.async_overlap or (self._pending is not None and not hasattr(self._pending[1], "feed")):
-                self._settle()      # nothing to gain from waiting: the tokens are on the host already
+        self._admit()
+        plan = self._plan()
+        if plan.kind != "idle":
+            self._run(plan)     # launches, then reads what was pending before
+        else:
+            self._settle()
+        if not self.cfg.async_overlap or (self._pending is not None and not hasattr(self._pending[1], "feed")):
+            self._settle()      # nothing to gain from waiting: the tokens are on the host already
         self._cleanup()
         return plan
 
@@ -340,8 +341,12 @@ class Scheduler:
     # -- execution --------------------------------------------------------------------------------
     def _run(self, plan: StepPlan) -> None:
         entries, sampled = [], []
+        before = self._pending
+        fed_from = {id(r): i for i, r in enumerate(before[0])} if before is not None else {}
         for r in plan.decode:
-            entries.append(StepEntry(r.id, [r.generated[-1]], [0]))
+            # the request's last token: known, or still on the GPU where the step before chose it
+            last = before[1].feed(fed_from[id(r)]) if r.pending else r.generated[-1]
+            entries.append(StepEntry(r.id, [last], [0]))
             sampled.append(r)
         for r, n in plan.prefill:
             completes = n == r.remaining_prompt
@@ -365,9 +370,15 @@ class Scheduler:
         self.stats["pages_high_water"] = max(self.stats["pages_high_water"], held)
         for r, n in plan.prefill:
             r.fed += n
-        if not sampled:
-            return
-        self._choose(logits, sampled, plan)
+        if before is not None:
+            self.stats["steps_ahead"] = self.stats.get("steps_ahead", 0) + 1
+        self._pending = None
+        if sampled:
+            self._choose(logits, sampled, plan)     # queued behind the step
+        if before is not None:                      # the step before: its tokens are there by now
+            ahead, self._pending = self._pending, before
+            self._settle()
+            self._pending = ahead
 
     def _choose(self, logits, sampled: list, plan: StepPlan) -> None:
         """Queue the sampling of a step's wanted rows; what it chooses is read by `_settle`."""
@@ -378,6 +389,10 @@ class Scheduler:
             chosen = _ChosenNow(*self.sampler.sample_with_logprobs(logits, rows))
         for r in sampled:
             r.pending += 1
+            if r.phase == "prefilling":     # its prompt is through: the next step decodes it, whatever the token is
+                self.prefilling.remove(r)
+                r.phase = "decoding"
+                self.decoding.append(r)
         self._pending = (sampled, chosen, plan)
 
     def _settle(self) -> None:
@@ -396,45 +411,22 @@ class Scheduler:
             wants = logprobs is not None and r.sampling.logprobs
             self._apply_token(r, int(tok), now, float(logprobs[i]) if wants else None)
 
-    # -- a decode step launched before the last one's tokens are known ------------------------------
-    def _can_run_ahead(self) -> bool:
+    # -- planning before the last step's tokens are known -------------------------------------------
+    def _can_plan_ahead(self) -> bool:
         if not self.cfg.async_overlap:
             return False
-        sampled, chosen, plan = self._pending
-        if plan.prefill or self.prefilling or not hasattr(chosen, "feed"):
+        sampled, chosen, _ = self._pending
+        if not hasattr(chosen, "feed"):
             return False
-        if self.waiting and self.cache.free_slot_count > 0:
-            return False    # an admission may change the next step
-        rows = [r for r in sampled if r.phase == "decoding"]
-        if not rows or len(rows) != len(self.decoding):
-            return False
-        for r in rows:
+        for r in sampled:
+            if r.phase != "decoding":
+                continue
             if r.sampling.has_penalties() or len(r.generated) + r.pending >= r.max_tokens:
                 return False    # the token's value is needed, or it is the request's last
-        return self.cache.can_append([(r.id, 1) for r in rows])
-
-    def _run_ahead(self) -> StepPlan:
-        sampled, chosen, _ = self._pending
-        rows = [(i, r) for i, r in enumerate(sampled) if r.phase == "decoding"]
-        plan = StepPlan([r for _, r in rows], [])
-        logits = self.engine.step([StepEntry(r.id, [chosen.feed(i)], [0]) for i, r in rows])
-        self.stats["steps"]["decode"] += 1
-        self.stats["steps_ahead"] = self.stats.get("steps_ahead", 0) + 1
-        self.stats["tokens_decoded"] += len(rows)
-        held = max((g.pool.num_pages - g.pool.free_count for g in self.cache.groups), default=0)
-        self.stats["pages_high_water"] = max(self.stats["pages_high_water"], held)
-        before = self._pending
-        self._choose(logits, plan.decode, plan)     # queued behind the step; _pending is the new step now
-        ahead, self._pending = self._pending, before
-        self._settle()                              # the step before: its tokens are there by now
-        self._pending = ahead
-        return plan
+        # one more token of every decoding request must fit without anybody giving pages back
+        return self.cache.can_append([(r.id, 1) for r in self.decoding if r.phase == "decoding"])
 
     def _apply_token(self, r: Request, tok: int, now: float, logprob: float | None = None) -> None:
-        if r.phase == "prefilling":
-            self.prefilling.remove(r)
-            r.phase = "decoding"
-            self.decoding.append(r)
         if r.t_first_token is None:
             r.t_first_token = now
         stops = self.stop_token_ids | set(r.sampling.stop_token_ids)

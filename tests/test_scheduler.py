@@ -385,11 +385,12 @@ def test_a_step_ahead_is_launched_before_the_last_tokens_are_read():
     s.submit(prompt(6), max_tokens=6)
     s.iteration()                        # the prompt; its token stays with the sampler
     assert sampler.log == ["step"]
-    s.iteration()                        # a portion came before: read first, then the first decode step
-    assert sampler.log == ["step", "read", "step"] and eng.fed_from_device == 0
-    s.iteration()                        # decode follows decode: launched from the tokens not yet read
-    assert sampler.log == ["step", "read", "step", "step", "read"] and eng.fed_from_device == 1
-    assert sampler.draw_indices == [2]   # the third draw of the request, though the host knows one token only
+    s.iteration()                        # the first decode step: launched from the token not yet read
+    assert sampler.log == ["step", "step", "read"] and eng.fed_from_device == 1
+    assert sampler.draw_indices == [1]   # the second draw of the request, though the host knew no token yet
+    s.iteration()
+    assert sampler.log == ["step", "step", "read", "step", "read"] and eng.fed_from_device == 1
+    assert sampler.draw_indices == [2]
     s.run_until_done()
     assert s.finished[0].generated == expected_output(prompt(6), 6)
 
@@ -455,3 +456,54 @@ def test_a_cut_portion_gives_up_the_tokens_that_stand_over_a_multiple_of_128_row
     assert plan_prefill([long_one], 8, small, fits) == [(long_one, 200)]        # fewer than 128 tokens would stay
     off = SchedulerConfig(num_slots=16, chunked_prefill_size=512, long_prefill_token_threshold=512, step_row_alignment=0)
     assert plan_prefill([long_one], 8, off, fits) == [(long_one, 512)]
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_traffic_gives_the_same_tokens_with_and_without_steps_launched_ahead(seed):
+    """Requests of random lengths and budgets arriving while others run, stop tokens that some of them meet, a few
+    with penalties, pools from generous to so small that requests are preempted, aborts in between: every request
+    ends with the same tokens and reason whether steps are launched ahead or wait for their tokens, nothing is
+    held at the end, and the cache's books are right after every iteration."""
+    import random
+
+    rng = random.Random(seed)
+    slots, page_size = rng.choice([2, 3, 5]), rng.choice([2, 4])
+    num_pages = rng.choice([12, 20, 64])
+    chunk = rng.choice([3, 8, 16])
+    arrivals = []
+    for i in range(rng.randint(4, 10)):
+        plen, budget = rng.randint(1, 18), rng.randint(1, 12)
+        if -(-(plen + budget + 1) // page_size) > num_pages - 1:
+            budget = 1
+        params = SamplingParams(repetition_penalty=1.3) if rng.random() < 0.15 else SamplingParams(logprobs=rng.random() < 0.3)
+        arrivals.append((rng.randint(0, 25), prompt(plen, i), params, budget))
+    stops = {next_token(prompt(5, 1) + [3]), rng.randrange(VOCAB), rng.randrange(VOCAB), rng.randrange(VOCAB)}
+    abort_at = rng.choice([None, 6, 11])
+    results = []
+    for overlap in (True, False):
+        eng, s, _ = make_lazy(num_pages=num_pages, page_size=page_size, slots=slots, stop=tuple(stops),
+                              async_overlap=overlap, chunked_prefill_size=chunk, max_num_batched_tokens=max(24, slots))
+        ids, it = {}, 0
+        while it < 400 and (s.has_work() or len(ids) < len(arrivals)):
+            for j, (when, toks, params, budget) in enumerate(arrivals):
+                if when == it:
+                    ids[j] = s.submit(toks, params, max_tokens=budget)
+            if abort_at == it and ids:
+                s.abort(ids[min(ids)])
+            s.iteration()
+            eng.cache.check()
+            it += 1
+        assert not s.has_work() and len(ids) == len(arrivals)
+        assert not eng.cache.slot_of and eng.cache.free_pages() == [num_pages]
+        results.append({j: (s.finished[i].generated, s.finished[i].finish_reason, s.finished[i].logprobs)
+                        for j, i in ids.items()})
+        if overlap:
+            ahead = s.stats.get("steps_ahead", 0)
+    aborted = {j for j, r in results[1].items() if r[1] == ABORT}
+    for j in results[1]:
+        if j in aborted:     # an abort drops the token that was on its way: a prefix of what the waiting run kept
+            a, b = results[0][j][0], results[1][j][0]
+            assert a == b[:len(a)] or b == a[:len(b)]
+        else:
+            assert results[0][j] == results[1][j], j
+    assert ahead > 0
