@@ -138,12 +138,11 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device, into=
     for k, n in zip(order, sizes):
         host[k] = flat_np[off:off + n]
         off += n
-    # one host->device copy for all arrays
-    flat = torch.from_numpy(flat_np)
+    # one host->device copy for all arrays, through pinned memory: the host does not wait for the stream
     if into is None:
-        packed = flat.to(device, non_blocking=False)
+        packed = upload(flat_np, device) if torch.device(device).type == "cuda" else torch.from_numpy(flat_np)
     else:
-        if into.numel() != flat.numel():
+        if into.numel() != flat_np.size:
             raise ValueError("the fixed step buffer does not fit this step")
         staging_for(device).copy_into(into, flat_np)
         packed = into
