@@ -358,6 +358,81 @@ def decode_32b(args) -> int:
     return 0
 
 
+def step_gaps(args) -> int:
+    """Decode steps of the Qwen3-4B shape both ways, steps that wait for their tokens on the host and steps launched
+    from the last one's tokens on the GPU: milliseconds a step, and from a kernel timeline of six steps how long
+    the GPU works and how long it idles between kernels in a step.  One JSON line a batch size."""
+    import torch
+    from torch.profiler import ProfilerActivity, profile
+
+    from arle_amd.config import Qwen3Config
+    from arle_amd.engine import Engine, StepEntry
+    from arle_amd.kernels import ops
+    from arle_amd.sampling import Sampler, SamplingParams
+
+    raw = dict(QWEN3_4B, num_hidden_layers=args.layers)
+    config = Qwen3Config.from_dict(raw)
+    batches = [args.batch] if args.batch else [1, 8, 64]
+    most = max(batches)
+    engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype="bfloat16", page_size=PAGE,
+                                max_tokens=most * (PROMPT + 256), max_slots=most, max_request_tokens=PROMPT + 256)
+    sampler = Sampler(engine.device)
+    gen = torch.Generator().manual_seed(1234)
+    for batch in batches:
+        keys, last = [("g", batch, i) for i in range(batch)], []
+        rows = [(SamplingParams(), 0, 0, [])] * batch
+        for k in keys:
+            engine.add_request(k)
+            toks = torch.randint(0, config.vocab_size, (PROMPT,), generator=gen).tolist()
+            last.append(int(ops.argmax_rows(engine.step([StepEntry(k, toks, [PROMPT - 1])]))[0]))
+        state = {"last": last, "chosen": None}
+
+        def waiting():
+            out = engine.step([StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])])
+            state["last"] = sampler.choose(out, rows).tokens()
+
+        def ahead():
+            before = state["chosen"]
+            if before is None:
+                entries = [StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])]
+            else:
+                entries = [StepEntry(k, [before.feed(i)], [0]) for i, k in enumerate(keys)]
+            state["chosen"] = sampler.choose(engine.step(entries), rows)
+            if before is not None:
+                state["last"] = before.tokens()
+
+        def settle():
+            if state["chosen"] is not None:
+                state["last"], state["chosen"] = state["chosen"].tokens(), None
+
+        line = {"metric": f"decode step at batch {batch}, {PROMPT}-token prompts (Qwen3-4B shape): steps that wait "
+                          f"for their tokens and steps launched ahead", "unit": "ms a step", "n_gpus": 1, "dtype": "bf16",
+                "layers": args.layers}
+        for name, fn in (("waiting", waiting), ("ahead", ahead)):
+            for _ in range(8):
+                fn()
+            settle()
+            wall = _timed(torch, lambda: ([fn() for _ in range(args.steps)], settle())) / args.steps
+            with profile(activities=[ProfilerActivity.CUDA]) as prof:
+                for _ in range(7):
+                    fn()
+                settle()
+                torch.cuda.synchronize()
+            evs = sorted((e for e in prof.events() if e.device_type == torch.autograd.DeviceType.CUDA),
+                         key=lambda e: e.time_range.start)
+            first = [i for i, e in enumerate(evs) if "embed_gather" in e.name]
+            evs = evs[first[1]:first[-1]]          # whole steps 2..6: the first carries the profiler's start
+            n = len(first) - 2
+            busy = sum(e.time_range.end - e.time_range.start for e in evs) / n
+            span = (evs[-1].time_range.end - evs[0].time_range.start) / n
+            line[name] = {"ms_per_step": round(wall * 1e3, 4), "gpu_busy_us": round(busy, 1), "gpu_idle_us": round(span - busy, 1),
+                          "kernels": round(len(evs) / n, 1)}
+        print(json.dumps(line), flush=True)
+        for k in keys:
+            engine.end_request(k)
+    return 0
+
+
 def sweep(args) -> int:
     """Further sizes of the Qwen3-4B shape, one JSON line each with its fraction of the roofline: decode at batch 16
     and 32 (2,048-token prompts), at batch 128 (1,024 tokens of context), at batch 8 with 8,192 and 32,768 tokens of
@@ -499,6 +574,8 @@ def main() -> int:
                     help="tokens of the prefill that --prefill-only measures (the default run's is 2,048)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiles of its kernels) and print that")
+    ap.add_argument("--gaps", action="store_true",
+                    help="decode steps that wait for their tokens against steps launched ahead: time a step, GPU busy and idle")
     ap.add_argument("--sweep", action="store_true",
                     help="further sizes of the Qwen3-4B shape (batch 16/32, 8k/32k context, 8,192-token prefill, portions "
                          "beside decoding requests), one JSON line each")
@@ -515,6 +592,8 @@ def main() -> int:
         return ceilings()
     if args.sweep:
         return sweep(args)
+    if args.gaps:
+        return step_gaps(args)
     if args.workload == "qwen3-4b" and args.batch is None:
         args.batch = 8
     if args.workload != "qwen3-4b":
