@@ -66,8 +66,8 @@ class SchedulerConfig:
     max_waiting_requests: int = 256
     max_seq_len: int | None = None
     async_overlap: bool = True   # launch a decode step from the last one's tokens on the GPU, read those back after
-    step_row_alignment: int = 128  # a portion that does not end its prompt is shortened until the step's rows are a
-                                   # multiple of this, if at least as many tokens stay (0: portions as the reference cuts them)
+    step_row_alignment: int = 128  # a portion that does not end its prompt stops where the step's rows are a multiple
+                                   # of this (aligned_portion; 0: portions as the reference cuts them)
 
     def validate(self) -> None:
         for name in ("num_slots", "chunked_prefill_size", "max_num_batched_tokens",
@@ -139,6 +139,22 @@ def retract_victim(decoding: list):
     return decoding[native.lib().arle_retract_victim(n, generated, prompts)]
 
 
+def aligned_portion(n: int, remaining: int, rows_before: int, align: int) -> int:
+    """How many of the n tokens that a prompt with `remaining` tokens could bring to a step of `rows_before` rows it
+    brings.  The matrix products of a step run in tiles of 128 and 256 rows: 8 decoded tokens beside a portion of 512
+    are 520 rows and cost a tenth more than 512 (measured on MI355X, Qwen3-4B shape: 9.8 against 8.7 ms).  So a
+    portion that is cut anyway gives up the few tokens that stand over a multiple of `align` rows, if at least
+    `align` tokens stay and the prompt does not need one more step for it (a 2,048-token prompt in portions of 512
+    stays at four steps)."""
+    if align <= 0 or n >= remaining:
+        return n
+    over = (rows_before + n) % align
+    m = n - over
+    if over == 0 or m < align or -(-remaining // m) != -(-remaining // n):
+        return n
+    return m
+
+
 def plan_prefill(queue, decode_rows: int, cfg: SchedulerConfig, fits) -> list:
     """Pick portions of queued prompts for this step: [(request, tokens)].
 
@@ -159,14 +175,7 @@ def plan_prefill(queue, decode_rows: int, cfg: SchedulerConfig, fits) -> list:
         n = min(remaining, max(cap, 1))
         if n > tokens_left or requests_left <= 0:
             continue  # skipped whole, never shrunk; a later, smaller one may still fit
-        # The matrix products of a step run in tiles of 128 and 256 rows: 8 decoded tokens beside a portion of 512
-        # are 520 rows and cost a tenth more than 512 (measured on MI355X, Qwen3-4B shape: 9.8 against 8.7 ms).  A
-        # portion that is cut anyway gives up the few tokens that stand over; they come with the next one.
-        align = cfg.step_row_alignment
-        if align > 0 and n < remaining:
-            over = (decode_rows + sum(m for _, m in picked) + n) % align
-            if over and n - over >= align:
-                n -= over
+        n = aligned_portion(n, remaining, decode_rows + sum(m for _, m in picked), cfg.step_row_alignment)
         completes = n == remaining
         first_decode = 1 if completes and req.max_tokens - len(req.generated) > 0 else 0
         if not fits(reserved, req, n + first_decode):

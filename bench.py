@@ -238,13 +238,17 @@ def ceilings() -> int:
 
 def mixed_8b(args) -> int:
     """Qwen3-8B shape: 32 requests decoding at 1,024 tokens of context beside one 2,048-token prompt
-    that arrives in portions of 512: four steps of 32 + 512 rows.  Reports the mean step and the tokens a second
-    of both kinds."""
+    that arrives in portions of 512, cut as the scheduler cuts them (aligned_portion: four steps of 32 + 512
+    rows, since stopping at 480 would cost this prompt a fifth step).  Every step is launched from the last one's
+    tokens on the GPU; --no-overlap: each waits for its tokens on the host.
+    Reports the mean step and the tokens a second of both kinds."""
     import torch
 
     from arle_amd.config import Qwen3Config
     from arle_amd.engine import Engine, StepEntry
+    from arle_amd.engine.scheduler import SchedulerConfig, aligned_portion
     from arle_amd.kernels import ops
+    from arle_amd.sampling import Sampler, SamplingParams
 
     raw = dict(QWEN3_8B, num_hidden_layers=args.layers or QWEN3_8B["num_hidden_layers"])
     config = Qwen3Config.from_dict(raw)
@@ -261,32 +265,56 @@ def mixed_8b(args) -> int:
     for i in range(0, decoders, 8):
         out = engine.step([StepEntry(k, rand(context - 1), [context - 2]) for k in keys[i:i + 8]])
         last.extend(ops.argmax_rows(out).tolist())
-    state = {"last": last}
+    state = {"last": last, "chosen": None}
+    sampler = Sampler(engine.device)
+    greedy = [(SamplingParams(), 0, 0, [])] * (decoders + 1)
+    align = 0 if args.no_overlap else SchedulerConfig().step_row_alignment
+    cuts, a = [], 0
+    while a < prompt:       # the portions as Scheduler.plan_prefill cuts them
+        n = aligned_portion(min(prompt - a, portion), prompt - a, decoders, align)
+        cuts.append((a, n))
+        a += n
 
     def one_prompt(tag):
         engine.add_request(tag)
         toks = rand(prompt)
-        for a in range(0, prompt, portion):
-            entries = [StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])]
-            entries.append(StepEntry(tag, toks[a:a + portion], [portion - 1] if a + portion == prompt else []))
-            out = engine.step(entries)
-            state["last"] = ops.argmax_rows(out).tolist()[:decoders]
+        for a, n in cuts:
+            before = state["chosen"]
+            if before is None:
+                entries = [StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])]
+            else:
+                entries = [StepEntry(k, [before.feed(i)], [0]) for i, k in enumerate(keys)]
+            last_piece = a + n == prompt
+            entries.append(StepEntry(tag, toks[a:a + n], [n - 1] if last_piece else []))
+            chosen = sampler.choose(engine.step(entries), greedy[:decoders + (1 if last_piece else 0)])
+            if args.no_overlap:
+                state["last"] = chosen.tokens()[:decoders]
+            else:
+                state["chosen"] = chosen
+                if before is not None:
+                    state["last"] = before.tokens()[:decoders]
         engine.end_request(tag)
 
-    for i in range(2):          # the second pass captures the four step shapes, later ones replay them
+    def settle():
+        if state["chosen"] is not None:
+            state["last"], state["chosen"] = state["chosen"].tokens()[:decoders], None
+
+    for i in range(2):          # the second pass captures the step shapes, later ones replay them
         one_prompt(("warm", i))
-    # the decoders have grown by 8 tokens; the timed prompts run at 1,032..1,048 tokens of context
-    reps = max(1, args.steps // 4)
-    dt = _timed(torch, lambda: [one_prompt(("p", i)) for i in range(reps)])
-    steps = 4 * reps
+    settle()
+    # the decoders have grown by a few tokens; the timed prompts run just above 1,024 tokens of context
+    reps = max(1, args.steps // len(cuts))
+    dt = _timed(torch, lambda: ([one_prompt(("p", i)) for i in range(reps)], settle()))
+    steps = len(cuts) * reps
     ms = dt / steps * 1e3
-    flops = sum(prefill_flops_portion(raw, a, portion) for a in range(0, prompt, portion)) / 4.0
+    flops = sum(prefill_flops_portion(raw, a, n) for a, n in cuts) / len(cuts)
+    portion = prompt / len(cuts)     # mean tokens of a portion
     line = {"metric": "mixed step: 32 decoding requests at 1,024 tokens + a 512-token prompt portion (Qwen3-8B shape)",
             "value": round(steps * (decoders + portion) / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps,
             "warmup": 8, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16", "data": "synthetic: seeded random weights N(0,0.02), uniform random token ids",
             "config": {"model": "Qwen3-8B shape", "decoding_requests": decoders, "decode_context": context,
-                       "prompt_len": prompt, "portion": portion, "layers": raw["num_hidden_layers"],
+                       "prompt_len": prompt, "portions": " ".join(str(n) for _, n in cuts), "layers": raw["num_hidden_layers"],
                        "hidden": raw["hidden_size"], "q_heads": 32, "kv_heads": 8, "head_dim": 128,
                        "intermediate": raw["intermediate_size"], "vocab": raw["vocab_size"], "tied": False,
                        "page_size": PAGE},
@@ -332,16 +360,33 @@ def decode_32b(args) -> int:
         last.extend(ops.argmax_rows(out).tolist())
         if i % 8 == 7:
             print(f"[bench] prefilled {i + 1} of {batch} requests ({time.time() - t0:.0f} s)", file=sys.stderr, flush=True)
-    state = {"last": last}
+    state = {"last": last, "chosen": None}
+    from arle_amd.sampling import Sampler, SamplingParams
+    sampler, greedy = Sampler(engine.device), [(SamplingParams(), 0, 0, [])] * batch
 
-    def one_step():
-        out = engine.step([StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])])
-        state["last"] = ops.argmax_rows(out).tolist()
+    def one_step():     # launched from the last step's tokens on the GPU, those read meanwhile; --no-overlap: waiting
+        before = state["chosen"]
+        if before is None:
+            entries = [StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])]
+        else:
+            entries = [StepEntry(k, [before.feed(i)], [0]) for i, k in enumerate(keys)]
+        chosen = sampler.choose(engine.step(entries), greedy)
+        if args.no_overlap:
+            state["last"] = chosen.tokens()
+        else:
+            state["chosen"] = chosen
+            if before is not None:
+                state["last"] = before.tokens()
+
+    def settle():
+        if state["chosen"] is not None:
+            state["last"], state["chosen"] = state["chosen"].tokens(), None
 
     for _ in range(warmup):
         one_step()
+    settle()
     ctx0 = engine.length(keys[0])
-    dt = _timed(torch, lambda: [one_step() for _ in range(steps)])
+    dt = _timed(torch, lambda: ([one_step() for _ in range(steps)], settle()))
     ctx_mean = ctx0 + (steps - 1) / 2.0 + 1
     achieved = decode_bytes(raw, batch, ctx_mean) / (dt / steps) / 1e9
     line = {"metric": f"decode tok/s at batch {batch}, {context:,} tokens of context (Qwen3-32B shape, random weights)",
@@ -543,7 +588,7 @@ def sweep(args) -> int:
     prefill_point(8192)
     prefill_point(512)
     prefill_point(128)
-    mixed_point(8, 2048, 504, 2016)      # as the scheduler cuts a long prompt beside 8 decoding requests: 512 rows a step
+    mixed_point(8, 2048, 504, 2016)      # the first four portions of a long prompt as the scheduler cuts it beside 8 decoding requests: 512 rows a step
     return 0
 
 

@@ -450,8 +450,12 @@ def test_a_cut_portion_gives_up_the_tokens_that_stand_over_a_multiple_of_128_row
     assert plan_prefill([long_one], 130, cfg, fits) == [(long_one, 510)]        # 130 + 510 = 640
     short = Request(1, prompt(300), SamplingParams(), 8, 0, feed=prompt(300))
     assert plan_prefill([short], 8, cfg, fits) == [(short, 300)]                # the end of a prompt is never cut
-    two = plan_prefill([short, long_one], 8, cfg, fits)
-    assert two == [(short, 300), (long_one, 460)] and (8 + 300 + 460) % 128 == 0
+    # 460 tokens would make 768 rows, but the prompt would then need five steps instead of four
+    assert plan_prefill([short, long_one], 8, cfg, fits) == [(short, 300), (long_one, 512)]
+    even = Request(2, prompt(2048), SamplingParams(), 8, 0, feed=prompt(2048))
+    assert plan_prefill([even], 32, cfg, fits) == [(even, 512)]                # 480 would add a fifth step
+    longer = Request(3, prompt(3600), SamplingParams(), 8, 0, feed=prompt(3600))
+    assert plan_prefill([short, longer], 8, cfg, fits) == [(short, 300), (longer, 460)]     # 768 rows; eight steps either way
     small = SchedulerConfig(num_slots=16, chunked_prefill_size=200, long_prefill_token_threshold=200)
     assert plan_prefill([long_one], 8, small, fits) == [(long_one, 200)]        # fewer than 128 tokens would stay
     off = SchedulerConfig(num_slots=16, chunked_prefill_size=512, long_prefill_token_threshold=512, step_row_alignment=0)
