@@ -1031,3 +1031,55 @@ def test_measuring_kernels_give_plausible_ceilings():
         for random_operands in (False, True):
             rate = ceilings.mfma_rate(DEV, shape=shape, iters=2000, repeats=1, random_operands=random_operands)
             assert 2.5e14 < rate < 2.6e15
+
+
+@pytest.mark.parametrize("nq,nkv,D,P,splits", [(32, 8, 128, 16, 3), (4, 2, 16, 4, 1), (6, 2, 64, 8, 2)])
+def test_attention_decoded_tokens_on_a_side_branch_give_the_bits_of_one_stream(nq, nkv, D, P, splits):
+    """In a mixed step the split-KV kernel of the decoded tokens and its merge run on a second stream beside the
+    portions kernel (forked and joined by events).  With the branch and without it the result is the same bit for
+    bit and right; a graph captured with the branch in it gives the same again on every replay, with eager calls
+    and synchronisations between the replays."""
+    from arle_amd.kernels import lib
+    segs = [(300, 70), (45, 1), (0, 1), (130, 2), (0, 200), (77, 1), (511, 1)]
+    results = {}
+    try:
+        for side in (0, 1):
+            lib.function("arle_attn_side_branch")(side)
+            results[side], want = _mfma_case(nq, nkv, D, P, segs, 0, splits, 410)
+        assert torch.isfinite(results[1]).all() and _rel(results[1], want) < 8e-3
+        assert torch.equal(results[0], results[1])
+
+        # the same call captured with the branch in it
+        dt = torch.bfloat16
+        lengths = [a + b for a, b in segs]
+        table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, 410)
+        qs, row0, starts = [], [0], []
+        for s, (cached, n) in enumerate(segs):
+            g = _g(411 + s)
+            q, k, v = (torch.randn(cached + n, h, D, generator=g).to(dt) for h in (nq, nkv, nkv))
+            _fill_cache(table, k_pages, v_pages, s, k, v, P)
+            qs.append(q[cached:].reshape(n, nq * D))
+            row0.append(row0[-1] + n)
+            starts.append(cached)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+        q_all, out = torch.cat(qs).to(DEV), None
+        fixed = (k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0), i32(list(range(len(segs)))), i32(starts))
+        kw = dict(max_qlen=200, min_qlen=1, max_kv_len=max(lengths), num_q_heads=nq, num_kv_heads=nkv, head_dim=D,
+                  page_size=P, scale=1.0 / math.sqrt(D), splits=splits)
+        eager = torch.empty_like(q_all)
+        ops.attn_paged_mfma(q_all, eager, *fixed, **kw)          # also makes the side stream, outside the capture
+        torch.cuda.synchronize()
+        assert torch.equal(eager.cpu(), results[1])
+        captured = torch.empty_like(q_all)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            ops.attn_paged_mfma(q_all, captured, *fixed, **kw)
+        for rep in range(4):
+            captured.fill_(float("nan"))
+            graph.replay()
+            again = torch.empty_like(q_all)
+            ops.attn_paged_mfma(q_all, again, *fixed, **kw)      # eager work between the replays
+            torch.cuda.synchronize()
+            assert torch.equal(captured, eager) and torch.equal(again, eager), rep
+    finally:
+        lib.function("arle_attn_side_branch")(1)
