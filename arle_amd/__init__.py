@@ -15,9 +15,12 @@ def __getattr__(name):
     if name in ("LLM", "generate", "CompletionOutput"):
         from .engine import api
         return getattr(api, name)
-    if name in ("Engine", "StepEntry"):
+    if name in ("Engine", "StepEntry", "DeviceToken"):
         from . import engine
         return getattr(engine, name)
+    if name in ("PRIORITY_LOW", "PRIORITY_NORMAL", "PRIORITY_HIGH"):
+        from .engine import scheduler
+        return getattr(scheduler, name)
     if name == "SamplingParams":
         from .sampling import SamplingParams
         return SamplingParams

@@ -104,17 +104,21 @@ class LLM:
         return self.tokenizer.encode(text).ids
 
     def generate(self, prompts, max_tokens: int = 16, temperature: float = 0.0, seed: int | None = None,
-                 ignore_eos: bool = False, sampling: SamplingParams | None = None, logprobs: bool = False) -> list:
+                 ignore_eos: bool = False, sampling: SamplingParams | None = None, logprobs: bool = False,
+                 priorities=None) -> list:
         """prompts: a list of token-id lists (or strings, with a tokenizer).  One CompletionOutput each,
-        in order.  `sampling` overrides temperature / seed / ignore_eos / logprobs when given."""
+        in order.  `sampling` overrides temperature / seed / ignore_eos / logprobs when given.
+        priorities: one of PRIORITY_LOW / NORMAL / HIGH (0, 1, 2) a prompt; the higher is served first."""
         sched = Scheduler(self.engine, self.sampler, self.sched_config, seed=self.seed,
                           stop_token_ids=self.engine.spec.stop_token_ids)
         ids = []
-        for p in prompts:
+        if priorities is not None and len(priorities) != len(prompts):
+            raise ValueError("one priority a prompt")
+        for i, p in enumerate(prompts):
             toks = self.tokenize(p) if isinstance(p, str) else list(p)
             params = sampling or SamplingParams(temperature=temperature, seed=seed, ignore_eos=ignore_eos,
                                                 logprobs=logprobs)
-            ids.append(sched.submit(toks, params, max_tokens))
+            ids.append(sched.submit(toks, params, max_tokens, **({} if priorities is None else {"priority": priorities[i]})))
         sched.run_until_done()
         self.last_stats = sched.stats
         outs = []

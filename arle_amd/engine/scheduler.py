@@ -4,6 +4,9 @@ token budget, decode, finish and free -- and what happens when pages run out.
 One `iteration()` does, in the reference's order (infer/src/scheduler/cuda/runtime/scheduler_loop.rs:116-199,
 infer/src/scheduler/cuda/execution.rs:385-425,669-800):
 
+0. intake: a request joins the waiting queue behind every request of its own or a higher priority and before
+   those of a lower one (infer/src/scheduler/cuda/runtime/helpers.rs:200-266); a preempted request goes back in
+   front of its equals.
 1. admission: a waiting request enters when a slot is free and the pool has pages for its
    prompt + 1 token after the same target of every running request is set aside; decode
    growth is not reserved (scheduler_loop.rs:202-315, budget.rs:17-33).  A request that does
@@ -45,6 +48,7 @@ from ..sampling.params import SamplingParams
 from .batch import StepEntry
 
 LENGTH, STOP, ABORT = "length", "stop", "abort"
+PRIORITY_LOW, PRIORITY_NORMAL, PRIORITY_HIGH = 0, 1, 2   # infer/src/scheduler/types.rs:553-564
 REQUEST_INPUT_SLACK_TOKENS = 5      # infer/src/scheduler/types.rs:499
 DECODE_RESERVATION_CLIP = 4096      # infer/src/scheduler/cuda/budget.rs:3
 
@@ -99,6 +103,7 @@ class Request:
     t_finish: float | None = None
     t_tokens: list = field(default_factory=list)   # when each generated token arrived (for the time per output token)
     pending: int = 0                               # tokens that a launched step has chosen and the host has not read yet
+    priority: int = PRIORITY_NORMAL                # a higher one is served first among the waiting
 
     @property
     def remaining_prompt(self) -> int:
@@ -128,6 +133,19 @@ class _ChosenNow:
 
     def logprobs(self):
         return self._logprobs
+
+
+def insert_waiting(waiting: deque, req, before_equal: bool) -> None:
+    """Put `req` into the waiting queue: before the first request of a lower priority; among its equals behind
+    them (a new request: first come, first served) or in front of them (`before_equal`: a request that was
+    running already and gave its pages back).  infer/src/scheduler/cuda/runtime/helpers.rs:200-266; its tests
+    runtime/tests.rs:172-215."""
+    at = len(waiting)
+    for i, queued in enumerate(waiting):
+        if req.priority > queued.priority or (before_equal and req.priority == queued.priority):
+            at = i
+            break
+    waiting.insert(at, req)
 
 
 def retract_victim(decoding: list):
@@ -214,7 +232,7 @@ class Scheduler:
 
     # -- intake ---------------------------------------------------------------------------
     def submit(self, prompt_tokens, sampling: SamplingParams | None = None,
-               max_tokens: int | None = None) -> int:
+               max_tokens: int | None = None, priority: int = PRIORITY_NORMAL) -> int:
         """Queue a request; returns its id.  Rejections finish at once with `length` and no tokens
         (infer/src/scheduler/cuda/runtime/admission.rs:71-120)."""
         sampling = sampling or SamplingParams()
@@ -226,14 +244,17 @@ class Scheduler:
         if max_tokens is None:
             max_tokens = sampling.max_new_tokens if sampling.max_new_tokens is not None else self.max_request_len
         seed = sampling.seed if sampling.seed is not None else (self.seed * 0x9E3779B1 + rid) & ((1 << 63) - 1)
-        req = Request(rid, prompt, sampling, int(max_tokens), seed, feed=list(prompt), t_submit=time.perf_counter())
+        if priority not in (PRIORITY_LOW, PRIORITY_NORMAL, PRIORITY_HIGH):
+            raise ValueError("priority is PRIORITY_LOW, PRIORITY_NORMAL or PRIORITY_HIGH")
+        req = Request(rid, prompt, sampling, int(max_tokens), seed, feed=list(prompt), t_submit=time.perf_counter(),
+                      priority=int(priority))
         if not prompt or len(prompt) >= self.max_request_input_len or req.max_tokens <= 0:
             self.stats["rejected"] += 1
             self._finish(req, LENGTH)
             self.finished[rid] = req
             return rid
         req.max_tokens = min(req.max_tokens, max(self.max_request_len - len(prompt) - 1, 0))
-        self.waiting.append(req)
+        insert_waiting(self.waiting, req, before_equal=False)
         return rid
 
     def abort(self, rid: int) -> bool:
@@ -465,7 +486,7 @@ class Scheduler:
         r.fed = 0
         r.preemptions += 1
         self.stats["preemptions"] += 1
-        self.waiting.appendleft(r)
+        insert_waiting(self.waiting, r, before_equal=True)
 
     def _cleanup(self) -> None:
         for group in (self.prefilling, self.decoding):

@@ -511,3 +511,36 @@ def test_random_traffic_gives_the_same_tokens_with_and_without_steps_launched_ah
         else:
             assert results[0][j] == results[1][j], j
     assert ahead > 0
+
+
+def test_waiting_requests_are_ordered_by_priority_then_first_come():
+    """infer/src/scheduler/cuda/runtime/tests.rs:172-215: a new request goes behind its equals, a requeued one in
+    front of them, both behind every higher priority; here also: the scheduler serves them in that order."""
+    from collections import deque
+    from arle_amd.engine.scheduler import PRIORITY_HIGH, PRIORITY_LOW, PRIORITY_NORMAL, insert_waiting
+
+    def req(label, priority):
+        r = Request(0, [1], SamplingParams(), 1, 0, priority=priority)
+        r.label = label
+        return r
+
+    waiting = deque([req("high", PRIORITY_HIGH), req("first-normal", PRIORITY_NORMAL)])
+    insert_waiting(waiting, req("second-normal", PRIORITY_NORMAL), before_equal=False)
+    assert [r.label for r in waiting] == ["high", "first-normal", "second-normal"]
+    waiting = deque([req("high", PRIORITY_HIGH), req("queued-normal", PRIORITY_NORMAL)])
+    insert_waiting(waiting, req("requeued-normal", PRIORITY_NORMAL), before_equal=True)
+    assert [r.label for r in waiting] == ["high", "requeued-normal", "queued-normal"]
+    insert_waiting(waiting, req("low", PRIORITY_LOW), before_equal=True)
+    insert_waiting(waiting, req("late-high", PRIORITY_HIGH), before_equal=False)
+    assert [r.label for r in waiting] == ["high", "late-high", "requeued-normal", "queued-normal", "low"]
+
+    eng, s = make(slots=1)
+    low = s.submit(prompt(5, 1), max_tokens=2, priority=PRIORITY_LOW)
+    normal = s.submit(prompt(5, 2), max_tokens=2)
+    high = s.submit(prompt(5, 3), max_tokens=2, priority=PRIORITY_HIGH)
+    s.run_until_done()
+    first_steps = [step[0][0] for step in eng.steps if step[0][1] == 5]      # the prompts, in the order they ran
+    assert first_steps == [high, normal, low]
+    assert all(s.finished[r].generated == expected_output(prompt(5, k), 2) for r, k in ((low, 1), (normal, 2), (high, 3)))
+    with pytest.raises(ValueError):
+        s.submit(prompt(3), priority=7)
