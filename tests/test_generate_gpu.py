@@ -325,3 +325,49 @@ def test_steps_launched_ahead_give_the_tokens_of_steps_that_wait(folders, dtype)
     assert results[False] == results[True]
     if free_run is not None:
         assert results[True][0][0] == free_run
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_random_traffic_on_the_real_engine_with_and_without_steps_launched_ahead(folders, seed):
+    """Requests of random lengths, budgets, priorities and sampling arriving while others run, through few slots
+    and a pool so small that requests give pages back, some meeting stop tokens: with steps launched ahead and
+    with steps that wait for their tokens every request ends with the same tokens and reason, and the cache is
+    empty and consistent at the end."""
+    import random
+
+    from arle_amd.engine import Engine
+    from arle_amd.engine.scheduler import Scheduler, SchedulerConfig
+    from arle_amd.sampling import Sampler
+
+    cfg, _ = read_folder(folders["B"])
+    rng = random.Random(seed)
+    arrivals = []
+    for i in range(10):
+        params = SamplingParams(temperature=rng.choice([0.0, 0.0, 0.9]), top_p=rng.choice([1.0, 0.8]), seed=i,
+                                logprobs=rng.random() < 0.3, repetition_penalty=rng.choice([1.0, 1.0, 1.0, 1.2]))
+        arrivals.append((rng.randint(0, 18), random_tokens(rng.randint(1, 40), cfg["vocab_size"], 900 + 10 * seed + i),
+                         params, rng.randint(1, 14), rng.choice([0, 1, 1, 2])))
+    stops = tuple(rng.randrange(cfg["vocab_size"]) for _ in range(12))
+    pages = rng.choice([14, 40])
+    results = []
+    for overlap in (True, False):
+        eng = Engine.from_folder(folders["B"], dtype="float32", page_size=TINY["B"][1], num_pages=pages, max_slots=3,
+                                 max_request_tokens=96)
+        s = Scheduler(eng, Sampler(eng.device), SchedulerConfig(num_slots=3, chunked_prefill_size=16, max_num_batched_tokens=40,
+                                                                max_seq_len=96, async_overlap=overlap), stop_token_ids=stops)
+        ids, it = {}, 0
+        while it < 600 and (s.has_work() or len(ids) < len(arrivals)):
+            for j, (when, toks, params, budget, priority) in enumerate(arrivals):
+                if when == it:
+                    ids[j] = s.submit(toks, params, max_tokens=budget, priority=priority)
+            s.iteration()
+            it += 1
+        assert not s.has_work() and len(ids) == len(arrivals)
+        assert not eng.cache.slot_of
+        for g in eng.cache.groups:
+            g.check()
+            assert g.pool.free_count == g.pool.num_pages
+        results.append({j: (s.finished[i].generated, s.finished[i].finish_reason) for j, i in ids.items()})
+        if overlap:
+            assert s.stats.get("steps_ahead", 0) > 5
+    assert results[0] == results[1]
