@@ -43,9 +43,12 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--num-slots", type=int, default=4)
     ap.add_argument("--max-seq-len", type=int, default=None)
-    ap.add_argument("--chunked-prefill-size", type=int, default=512)
+    ap.add_argument("--chunked-prefill-size", type=int, default=None,
+                    help="longest prompt portion of one request in a step; default: by the GPU's memory "
+                         "(<35 GiB 2048, <60 4096, <90 8192, else 16384)")
     ap.add_argument("--max-num-batched-tokens", type=int, default=16384)
-    ap.add_argument("--max-prefill-tokens", type=int, default=16384)
+    ap.add_argument("--max-prefill-tokens", type=int, default=None,
+                    help="prompt tokens of all requests in a step; default: --max-num-batched-tokens")
     ap.add_argument("--prefill-max-requests", type=int, default=None)
     ap.add_argument("--kv-cache-tokens", type=int, default=None,
                     help="tokens the paged cache holds (default: sized from free GPU memory, see --mem-fraction-static)")

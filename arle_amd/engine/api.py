@@ -43,11 +43,18 @@ class CompletionOutput:
     token_logprobs: list = field(default_factory=list)   # log-probability of every generated token, if asked for
 
 
+def _gpu_total_bytes(device) -> int:
+    import torch
+
+    device = torch.device(device)
+    return torch.cuda.get_device_properties(device).total_memory if device.type == "cuda" else 0
+
+
 class LLM:
     def __init__(self, model, *, dtype="bfloat16", device=None, page_size: int | None = None,
                  kv_cache_tokens: int | None = None, num_slots: int = 4, max_seq_len: int | None = None,
-                 chunked_prefill_size: int = 512, max_num_batched_tokens: int = 16384,
-                 max_prefill_tokens: int = 16384, prefill_max_requests: int | None = None, seed: int = 42,
+                 chunked_prefill_size: int | None = None, max_num_batched_tokens: int = 16384,
+                 max_prefill_tokens: int | None = None, prefill_max_requests: int | None = None, seed: int = 42,
                  cuda_graph: bool = True, weight_tiles: bool | None = None, mem_fraction_static: float = 0.85,
                  async_overlap: bool = True):
         """model: a model folder, or an Engine that is already built.
@@ -56,6 +63,11 @@ class LLM:
         free memory after the weights are loaded, less a headroom of (1 - mem_fraction_static) of its whole
         memory (the reference's --mem-fraction-static, default 0.85), and never more than num_slots requests
         of max_seq_len tokens (default: the model's positions) can fill.
+        chunked_prefill_size: the longest prompt portion of one request in a step.  Default: by the GPU's
+        whole memory, as the reference's server picks it (2,048 below 35 GiB up to 16,384 from 90 GiB on, so
+        16,384 on an MI355X), and at most max_num_batched_tokens.  max_prefill_tokens: the prompt tokens of
+        all requests in a step; default max_num_batched_tokens.  While requests are decoding a portion is at
+        most 4,096 tokens (long_prefill_token_threshold).
         cuda_graph, weight_tiles: as for Engine (captured steps; the decode-friendly second copy of the weights).
         async_overlap: decode steps are launched from the last step's tokens on the GPU, and those are read back
         while the new step runs (SchedulerConfig.async_overlap); the tokens are the same either way.
@@ -77,10 +89,12 @@ class LLM:
                                              weight_tiles=weight_tiles, mem_fraction_static=mem_fraction_static)
         self.model_dir = model if isinstance(model, str) else None
         self.seed = seed
-        self.sched_config = SchedulerConfig(
-            num_slots=self.engine.cache.max_slots, chunked_prefill_size=chunked_prefill_size,
-            max_num_batched_tokens=max_num_batched_tokens, max_prefill_tokens=max_prefill_tokens,
-            prefill_max_requests=prefill_max_requests, max_seq_len=max_seq_len, async_overlap=async_overlap)
+        cfg = SchedulerConfig.runtime_defaults(self.engine.cache.max_slots)
+        cfg.max_num_batched_tokens = max_num_batched_tokens
+        cfg.prefill_max_requests, cfg.max_seq_len, cfg.async_overlap = prefill_max_requests, max_seq_len, async_overlap
+        self.sched_config = cfg.resolve_runtime_envelope(_gpu_total_bytes(self.engine.device), chunked_prefill_size,
+                                                         max_prefill_tokens)
+        self.sched_config.validate()
         self.sampler = Sampler(self.engine.device)
         self.tokenizer = self._load_tokenizer()
         self.last_stats: dict = {}

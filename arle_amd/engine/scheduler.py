@@ -53,6 +53,21 @@ REQUEST_INPUT_SLACK_TOKENS = 5      # infer/src/scheduler/types.rs:499
 DECODE_RESERVATION_CLIP = 4096      # infer/src/scheduler/cuda/budget.rs:3
 
 
+GIB = 1 << 30
+
+
+def pick_chunked_prefill_size_for_hbm(gpu_total_bytes: int) -> int:
+    """The longest prompt portion of one request by the GPU's whole memory: the larger the GPU, the larger
+    the portion (infer/src/scheduler/types.rs:251-260).  An MI355X (288 GB) takes 16,384 tokens."""
+    if gpu_total_bytes < 35 * GIB:
+        return 2048
+    if gpu_total_bytes < 60 * GIB:
+        return 4096
+    if gpu_total_bytes < 90 * GIB:
+        return 8192
+    return 16384
+
+
 class SchedulerFull(RuntimeError):
     pass
 
@@ -72,6 +87,28 @@ class SchedulerConfig:
     async_overlap: bool = True   # launch a decode step from the last one's tokens on the GPU, read those back after
     step_row_alignment: int = 128  # a portion that does not end its prompt stops where the step's rows are a multiple
                                    # of this (aligned_portion; 0: portions as the reference cuts them)
+
+    @classmethod
+    def runtime_defaults(cls, num_slots: int) -> "SchedulerConfig":
+        """What a serving scheduler starts from, before the GPU's memory is known
+        (infer/src/scheduler/types.rs:270-278); the plain defaults above are those of the reference's
+        accounting layer without a GPU."""
+        return cls(num_slots=num_slots, chunked_prefill_size=4096, max_num_batched_tokens=16384,
+                   long_prefill_token_threshold=4096)
+
+    def resolve_runtime_envelope(self, gpu_total_bytes: int, chunked_prefill_size: int | None = None,
+                                 max_prefill_tokens: int | None = None) -> "SchedulerConfig":
+        """Settle the sizes of a step on a given GPU (infer/src/scheduler/types.rs:315-334).  A value that
+        the caller gives stands; chunked_prefill_size otherwise follows the GPU's memory and never exceeds
+        max_num_batched_tokens, max_prefill_tokens otherwise is the whole step's budget, and
+        long_prefill_token_threshold is no longer than a portion."""
+        self.chunked_prefill_size = (chunked_prefill_size if chunked_prefill_size is not None
+                                     else pick_chunked_prefill_size_for_hbm(gpu_total_bytes))
+        if self.max_num_batched_tokens > 0:
+            self.chunked_prefill_size = min(self.chunked_prefill_size, self.max_num_batched_tokens)
+        self.max_prefill_tokens = max_prefill_tokens if max_prefill_tokens is not None else self.max_num_batched_tokens
+        self.long_prefill_token_threshold = min(self.long_prefill_token_threshold, self.chunked_prefill_size)
+        return self
 
     def validate(self) -> None:
         for name in ("num_slots", "chunked_prefill_size", "max_num_batched_tokens",

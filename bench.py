@@ -657,11 +657,12 @@ def main() -> int:
     config = Qwen3Config.from_dict(raw)
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
     elt = 2 if dkey == "bf16" else 4
-    max_batch = args.batch if (args.no_points or args.parts_only) else max(args.batch, 64)
+    max_batch = args.batch if (args.no_points or args.parts_only or args.prefill_only) else max(args.batch, 64)
+    longest = max(CONTEXT, PROMPT + 64)    # --prompt-len may ask for a longer prefill than the default run's context
     t0 = time.time()
     engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype=args.dtype,
-                                page_size=PAGE, max_tokens=(max_batch + 1) * CONTEXT, max_slots=max_batch + 1,
-                                max_request_tokens=CONTEXT, weight_tiles=False if args.no_weight_tiles else None)
+                                page_size=PAGE, max_tokens=(max_batch + 1) * longest, max_slots=max_batch + 1,
+                                max_request_tokens=longest, weight_tiles=False if args.no_weight_tiles else None)
     print(f"[bench] engine ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
     gen = torch.Generator().manual_seed(1234)
     sampler = Sampler(engine.device)       # the product's sampler: greedy rows are one argmax kernel, read back on its own stream

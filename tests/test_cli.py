@@ -16,8 +16,9 @@ def test_global_options_and_run():
 
 def test_defaults_are_the_reference_library_defaults():
     args = build_parser().parse_args(["--model-path", "/m", "run", "--prompt", "hi"])
-    # infer/src/scheduler/types.rs:192-238: slots 4, chunk 512, 16384 tokens a step; greedy (crates/cli/src/args.rs)
-    assert (args.num_slots, args.chunked_prefill_size, args.max_num_batched_tokens, args.max_prefill_tokens) == (4, 512, 16384, 16384)
+    # infer/src/main.rs:90-105: slots 4, 16384 tokens a step, the portion and the prompt tokens of a step left to be
+    # settled by the GPU's memory (infer/src/scheduler/types.rs:315-334); greedy (crates/cli/src/args.rs)
+    assert (args.num_slots, args.chunked_prefill_size, args.max_num_batched_tokens, args.max_prefill_tokens) == (4, None, 16384, None)
     assert args.temperature == 0.0 and args.top_k == -1 and args.top_p == 1.0 and args.min_p == 0.0 and args.seed == 42
     assert not args.no_cuda_graph and not args.no_weight_tiles and args.dtype == "bfloat16"
 

@@ -237,6 +237,39 @@ def test_config_is_validated():
         SchedulerConfig(num_slots=8, max_num_batched_tokens=4).validate()
 
 
+def test_a_serving_scheduler_takes_its_portion_size_from_the_gpus_memory():
+    """The vectors of the reference's own tests (infer/src/scheduler/types.rs:788-797,950-1000)."""
+    from arle_amd.engine.scheduler import GIB, pick_chunked_prefill_size_for_hbm
+
+    assert [pick_chunked_prefill_size_for_hbm(n * GIB) for n in (0, 22, 48, 80, 140)] == [2048, 2048, 4096, 8192, 16384]
+    assert pick_chunked_prefill_size_for_hbm(35 * GIB) == 4096 and pick_chunked_prefill_size_for_hbm(90 * GIB) == 16384
+    cfg = SchedulerConfig.runtime_defaults(8)
+    assert (cfg.num_slots, cfg.chunked_prefill_size, cfg.max_num_batched_tokens, cfg.max_prefill_tokens,
+            cfg.long_prefill_token_threshold, cfg.prefill_max_requests) == (8, 4096, 16384, 16384, 4096, None)
+    cfg.validate()
+    # nothing given: the portion follows the memory, the prompt tokens of a step the step's budget, and the cap on
+    # portions beside decoding requests is no longer than a portion
+    cfg = SchedulerConfig.runtime_defaults(8).resolve_runtime_envelope(22 * GIB)
+    assert (cfg.chunked_prefill_size, cfg.max_prefill_tokens, cfg.long_prefill_token_threshold) == (2048, 16384, 2048)
+    cfg = SchedulerConfig.runtime_defaults(4).resolve_runtime_envelope(288 * GIB)
+    assert (cfg.chunked_prefill_size, cfg.max_prefill_tokens, cfg.long_prefill_token_threshold) == (16384, 16384, 4096)
+    # what the caller gives stands
+    cfg = SchedulerConfig.runtime_defaults(4).resolve_runtime_envelope(22 * GIB, 6144, 12288)
+    assert (cfg.chunked_prefill_size, cfg.max_prefill_tokens) == (6144, 12288)
+    # a tighter step never starves a long prompt: the portion is at most the step
+    cfg = SchedulerConfig.runtime_defaults(4)
+    cfg.max_num_batched_tokens = 1024
+    cfg.resolve_runtime_envelope(288 * GIB)
+    assert (cfg.chunked_prefill_size, cfg.max_prefill_tokens, cfg.long_prefill_token_threshold) == (1024, 1024, 1024)
+    cfg.validate()
+    cfg = SchedulerConfig.runtime_defaults(8)
+    cfg.max_num_batched_tokens = 4096
+    cfg.resolve_runtime_envelope(80 * GIB)
+    assert (cfg.chunked_prefill_size, cfg.max_prefill_tokens) == (4096, 4096)
+    cfg = SchedulerConfig.runtime_defaults(4).resolve_runtime_envelope(22 * GIB, 3072)
+    assert (cfg.chunked_prefill_size, cfg.max_prefill_tokens) == (3072, 16384)
+
+
 def test_sampling_params_greedy_rule():
     # infer/src/sampler.rs:82-84,178-
     assert SamplingParams().is_greedy()
