@@ -31,6 +31,7 @@ SIGNATURES = {
     "arle_gemm_stream": ("gemm_rows", [_p, _ll, _p, _ll, _i, _p, _ll, _ll, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "arle_gemm_rows_lds": ("gemm_rows", [_i, _i, _i]),
     "arle_gemm_tiles": ("gemm_tiles", [_p, _ll, _p, _p, _ll, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _ll, _p]),
+    "arle_gemm_tiles_patch": ("gemm_tiles", [_i, _i]),
     "arle_gemm_rows_lds_max": ("gemm_rows", []),
     "arle_gemm_f32": ("gemm_f32", [_p, _ll, _p, _ll, _p, _ll, _i, _i, _i, _p]),
     "arle_qk_prep": ("rope_kv", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _p, _i, _p, _p, _i, _p, _p, _p,

@@ -891,7 +891,8 @@ def test_gemm_rows_fused_activation_from_operand_tiles():
 
 
 @pytest.mark.parametrize("variant", ops.TILES_VARIANTS)
-@pytest.mark.parametrize("M,N,K", [(300, 200, 72), (129, 520, 264), (257, 256, 32), (1, 40, 8), (640, 1000, 1096)])
+@pytest.mark.parametrize("M,N,K", [(300, 200, 72), (129, 520, 264), (257, 256, 32), (1, 40, 8), (640, 1000, 1096),
+                                   (2300, 4900, 64)])
 def test_gemm_tiles_many_rows_from_operand_tiles(variant, M, N, K):
     """Rows, columns and K that end inside a workgroup's block, inside a tile and inside a step of 32; fewer steps
     than a ring holds; every workgroup shape and ring depth."""
@@ -942,6 +943,33 @@ def test_gemm_tiles_parts_of_k_as_a_stack(variant, M, N, K, splits):
     assert _rel(got.double().sum(0), x.double() @ w.double().T) < 1e-5
     with pytest.raises(ops.ShapeError, match="float32 stack"):
         ops.gemm_tiles(x.to(DEV), tiles, N, torch.bfloat16, variant=variant, splits=splits)
+
+
+def test_gemm_tiles_patches_of_workgroups_cover_every_tile():
+    """However the workgroups that run side by side on an XCD are laid out over the row and column blocks (patches
+    that end beyond the last row block, the last column block, or both; one workgroup a patch), every tile is
+    computed once, with the same bits."""
+    from arle_amd.kernels import lib
+
+    M, N, K = 1100, 2100, 64
+    x = torch.randn(M, K, generator=_g(136)).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=_g(137)) * 0.1).bfloat16().to(DEV)
+    tiles = ops.pack_weight_tiles(w)
+    want = x.double().cpu() @ w.double().cpu().T
+    patch = lib.function("arle_gemm_tiles_patch")
+    try:
+        results = []
+        for rows, cols in ((8, 8), (3, 2), (1, 1), (5, 1), (2, 7), (4096, 1)):
+            patch(rows, cols)
+            for variant in ((4, 44), (8, 144), (4, 44, 1)):
+                junk = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+                del junk        # the result takes this memory: a tile left out would show
+                out = ops.gemm_tiles(x, tiles, N, torch.float32, variant=variant)
+                assert _rel(out.cpu(), want) < 1e-5, (rows, cols, variant)
+                results.append(out)
+        assert all(torch.equal(results[0], r) for r in results[1:])
+    finally:
+        patch(8, 8)
 
 
 def test_gemm_tiles_refuses_what_it_cannot_take():
