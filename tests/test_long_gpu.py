@@ -183,3 +183,46 @@ def test_a_portion_of_two_thousand_rows_takes_the_many_rows_kernel(tmp_path):
     for i, got in enumerate(again):
         for (_, pos), logits in got.items():
             assert torch.equal(logits, whole[("w", pos)]), (i, pos)
+
+
+def test_a_step_of_six_thousand_rows_agrees_with_portions_and_the_plain_implementation(tmp_path):
+    """The longest portion of one request follows the GPU's memory (16,384 tokens on an MI355X), so a long prompt is
+    one step: 6,200 rows (the library's products; 194 row blocks of the portions' attention) against the plain
+    implementation at every position, whole and in portions of 4,200 and 2,000 (the first takes the many-rows
+    product with its activation: 17 row blocks of 256 and 17 column blocks, so that its workgroups run in patches
+    of row and column blocks that end beyond the last block both ways)."""
+    import os
+    from arle_amd.config import Qwen3Config
+    from arle_amd.kernels import ops
+    from arle_amd.weights import write_random_model
+
+    raw = dict(num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+               intermediate_size=2048 + 80, vocab_size=300, rope_theta=10000.0, rms_norm_eps=1e-6,
+               tie_word_embeddings=True, max_position_embeddings=8192)
+    d = os.path.join(str(tmp_path), "wide_ffn_long")
+    write_random_model(d, "Qwen3ForCausalLM", Qwen3Config.from_dict(raw), seed=6, std=0.03, norm_std=0.02)
+    cfg, weights = read_folder(d)
+    n = 6200
+    assert not ops.gemm_tiles_preferred(n, 2 * raw["intermediate_size"], raw["hidden_size"], raw["hidden_size"], fused=True)
+    assert ops.gemm_tiles_preferred(4200, 2 * raw["intermediate_size"], raw["hidden_size"], raw["hidden_size"], fused=True)
+    toks = random_tokens(n, raw["vocab_size"], 13)
+    want_at = list(range(n))
+    ref = replay.plain_logits(cfg, weights, toks).double()
+    scale = float(ref.abs().max())
+
+    def check(got, what):
+        assert len(got) == n
+        err = torch.stack([(got[(rid, p)].double() - ref[p]).abs().max() for (rid, p) in got])
+        worst = int(err.argmax())
+        assert float(err[worst]) / scale <= TOL["bfloat16"], f"{what}: worst at {list(got)[worst]}: {float(err[worst]) / scale:.3e}"
+
+    eng = Engine.from_folder(d, dtype="bfloat16", page_size=16, max_tokens=2 * 6208, max_slots=2, max_request_tokens=6208)
+    whole = replay.run_steps(eng, [{"entries": [("w", toks, want_at)], "end": ["w"]}])
+    check(whole, "6,200 rows in one step")
+    steps, at = [], 0
+    for size in (4200, 2000):       # the first portion takes the many-rows product with its activation
+        wanted = [p - at for p in want_at if at <= p < at + size]
+        steps.append({"entries": [("p", toks[at:at + size], wanted)], "end": []})
+        at += size
+    cut = replay.run_steps(eng, steps)
+    check(cut, "6,200 rows in portions of 4,200 and 2,000")
