@@ -478,6 +478,39 @@ def step_gaps(args) -> int:
     return 0
 
 
+def first_token(args) -> int:
+    """Time to the first token through `LLM.generate` (scheduler, sampler, engine) for one prompt of 2,048, 8,192 and
+    16,000 tokens and for four prompts of 2,048 at once, with the portion size that the GPU's memory gives (the
+    default) and with portions of 512: one JSON line each."""
+    import torch
+
+    from arle_amd.config import Qwen3Config
+    from arle_amd.engine import Engine
+    from arle_amd.engine.api import LLM
+
+    raw = dict(QWEN3_4B, num_hidden_layers=args.layers)
+    config = Qwen3Config.from_dict(raw)
+    longest = 16384 + 64
+    engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype="bfloat16", page_size=PAGE,
+                                max_tokens=4 * longest, max_slots=4, max_request_tokens=longest)
+    gen = torch.Generator().manual_seed(1234)
+    rand = lambda n: torch.randint(0, config.vocab_size, (n,), generator=gen).tolist()
+    for chunk in (None, 512):
+        llm = LLM(engine, num_slots=4, chunked_prefill_size=chunk, max_seq_len=longest)
+        for prompts in ([2048], [8192], [16000], [2048] * 4):
+            batch = [rand(n) for n in prompts]
+            for _ in range(3):      # the third run replays what the first two captured
+                outs = llm.generate(batch, max_tokens=4, ignore_eos=True)
+            ttft = max(o.ttft_s for o in outs)
+            print(json.dumps({"metric": f"time to the first token of {len(prompts)} prompt(s) of {prompts[0]:,} tokens "
+                                        f"through LLM.generate (Qwen3-4B shape)", "value": round(ttft * 1e3, 2), "unit": "ms",
+                              "higher_is_better": False, "n_gpus": 1, "dtype": "bf16", "layers": args.layers,
+                              "chunked_prefill_size": llm.sched_config.chunked_prefill_size,
+                              "prefill_steps": llm.last_stats["steps"]["prefill"],
+                              "prompt_tok_s": round(sum(prompts) / ttft, 1)}), flush=True)
+    return 0
+
+
 def sweep(args) -> int:
     """Further sizes of the Qwen3-4B shape, one JSON line each with its fraction of the roofline: decode at batch 16
     and 32 (2,048-token prompts), at batch 128 (1,024 tokens of context), at batch 8 with 8,192 and 32,768 tokens of
@@ -621,6 +654,8 @@ def main() -> int:
                     help="measure the 2,048-token prefill alone (for profiles of its kernels) and print that")
     ap.add_argument("--gaps", action="store_true",
                     help="decode steps that wait for their tokens against steps launched ahead: time a step, GPU busy and idle")
+    ap.add_argument("--first-token", action="store_true",
+                    help="time to the first token through LLM.generate, portions by the GPU's memory against portions of 512")
     ap.add_argument("--sweep", action="store_true",
                     help="further sizes of the Qwen3-4B shape (batch 16/32, 8k/32k context, 8,192-token prefill, portions "
                          "beside decoding requests), one JSON line each")
@@ -637,6 +672,8 @@ def main() -> int:
         return ceilings()
     if args.sweep:
         return sweep(args)
+    if args.first_token:
+        return first_token(args)
     if args.gaps:
         return step_gaps(args)
     if args.workload == "qwen3-4b" and args.batch is None:
