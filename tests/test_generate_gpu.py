@@ -291,6 +291,29 @@ def test_the_pool_is_sized_from_free_memory_when_no_size_is_given(folders):
         Engine.from_folder(folders["A"], dtype="bfloat16", mem_fraction_static=1e-6)
 
 
+def test_the_sizes_of_a_step_follow_the_gpus_memory_unless_given(folders):
+    """Nothing given: the longest portion of one request is what the GPU's whole memory gives (16,384 tokens from
+    90 GiB on), so a 700-token prompt is one step; with chunked_prefill_size=256 it is three, and the tokens are the
+    same."""
+    from arle_amd.engine.scheduler import pick_chunked_prefill_size_for_hbm
+
+    cfg, _ = read_folder(folders["B"])
+    llm = LLM(folders["B"], dtype="float32", page_size=TINY["B"][1], kv_cache_tokens=2048, max_seq_len=1024)
+    total = torch.cuda.get_device_properties(llm.engine.device).total_memory
+    sc = llm.sched_config
+    assert sc.chunked_prefill_size == pick_chunked_prefill_size_for_hbm(total) == 16384
+    assert (sc.max_prefill_tokens, sc.long_prefill_token_threshold) == (16384, 4096)
+    prompt = random_tokens(700, cfg["vocab_size"], 21)
+    whole = llm.generate([prompt], max_tokens=6, ignore_eos=True)[0]
+    assert llm.last_stats["steps"]["prefill"] == 1
+    cut = LLM(llm.engine, chunked_prefill_size=256, max_prefill_tokens=512, max_seq_len=1024)
+    assert (cut.sched_config.chunked_prefill_size, cut.sched_config.max_prefill_tokens,
+            cut.sched_config.long_prefill_token_threshold) == (256, 512, 256)
+    pieces = cut.generate([prompt], max_tokens=6, ignore_eos=True)[0]
+    assert cut.last_stats["steps"]["prefill"] == 3
+    assert pieces.response_token_ids == whole.response_token_ids
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_steps_launched_ahead_give_the_tokens_of_steps_that_wait(folders, dtype):
     """Decode steps fed from the last step's tokens on the GPU, read back one step late, against steps that
