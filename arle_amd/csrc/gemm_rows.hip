@@ -20,6 +20,8 @@
 //     been multiplied, so every wave keeps PD kilobyte-sized loads in flight.  The X operand comes
 //     from LDS through a shorter ring of its own, so that no step waits for an LDS read;
 //   * the WK partial sums of a column tile are added through LDS in the fixed order wk = 0..WK-1.
+//   * ROUNDS (the fused activation for up to 64 rows): where the X rows of the whole k slice do not fit into LDS,
+//     the slice is walked in rounds, each staged, multiplied and left behind a barrier; the sums stay in registers.
 //
 // Operand layout (lane = 16 g + i):  A lane (i, g) = W[n0 + i][32 s + 8 g .. +7],
 // B lane (j, g) = X[m0 + j][32 s + 8 g .. +7], C lane (j, g) register r = C[m0 + j][n0 + 4 g + r].
@@ -52,6 +54,7 @@ struct RowsArgs {
   int steps_per_split;   // k steps of 32 that one k split covers
   int64_t split_stride;  // elements between the partial products of two k splits
   int tiled;             // w holds operand tiles (see below) instead of rows
+  int steps_per_round;   // ROUNDS: k steps of 32 whose X rows are in LDS at one time (the slice is walked in rounds)
 };
 
 // W as operand tiles: [ceil(N/16)][ceil(K/32)][64 lanes][8], tile (t, s) lane 16 g + i = W[16 t + i][32 s + 8 g .. +7],
@@ -63,7 +66,10 @@ __device__ __forceinline__ const uint16_t* tile_base(const RowsArgs& a, int n0, 
   return a.w + static_cast<int64_t>(tile) * ((a.K + 31) / 32) * 512 + lane * 8;
 }
 
-template <int MT, int WN, int WK, int PD, int XD, int EPI, typename TOut>
+// ROUNDS: the k slice of a workgroup is too long for its X rows to fit into LDS at once (more than 27 rows of
+// 2,560 columns); it is walked in rounds of steps_per_round steps, each staged, multiplied and left behind a
+// barrier, with the sums staying in registers, so that whole sums meet the fused activation for up to 64 rows.
+template <int MT, int WN, int WK, int PD, int XD, int EPI, typename TOut, bool ROUNDS = false>
 __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a) {
   constexpr int kThreads = WN * WK * 64;
   static_assert(PD % XD == 0, "the X ring must divide the W ring");
@@ -78,11 +84,18 @@ __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a
   const int M = a.M, N = a.N, K = a.K;
 
   const int steps_total = (K + 31) / 32;
-  const int s_begin = blockIdx.y * a.steps_per_split;
-  const int s_end = min(s_begin + a.steps_per_split, steps_total);
-  const int pitch = a.steps_per_split * 32 + kPad;
+  const int slice_begin = blockIdx.y * a.steps_per_split;
+  const int slice_end = min(slice_begin + a.steps_per_split, steps_total);
+  const int staged_steps = ROUNDS ? a.steps_per_round : a.steps_per_split;   // steps whose X rows LDS holds at a time
+  const int pitch = staged_steps * 32 + kPad;
 
-  // this wave's steps: the wk-th part of the slice
+  f32x4 acc[MT];
+#pragma unroll
+  for (int b = 0; b < MT; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // one round: the steps [s_begin, s_end) of the slice, staged and multiplied (without ROUNDS: the whole slice)
+  auto round = [&](const int s_begin, const int s_end) {
+  // this wave's steps: the wk-th part of the round
   const int per = (s_end - s_begin + WK - 1) / WK;
   const int w_begin = s_begin + wk * per;
   const int n_steps = max(0, min(w_begin + per, s_end) - w_begin);
@@ -107,7 +120,7 @@ __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a
   // row in LDS is its 16-byte pieces and one piece of padding; padding lanes and lanes past K fetch a piece
   // that exists, and the pieces past K are put to zero afterwards (W is clamped there, X must not count).
   {
-    const int cpr = a.steps_per_split * 4;  // pieces of 8 elements per row
+    const int cpr = staged_steps * 4;       // pieces of 8 elements per row
     const int cpp = cpr + kPad / 8;         // ... with the padding
     const int total = M * cpp;
     const int k0 = s_begin * 32, k1 = min(s_end * 32, K);
@@ -128,10 +141,6 @@ __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a
     }
   }
   __syncthreads();
-
-  f32x4 acc[MT];
-#pragma unroll
-  for (int b = 0; b < MT; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const uint16_t* xrow[MT];  // lanes past the last row read the last row; their results are not stored
 #pragma unroll
@@ -183,6 +192,16 @@ __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a
         acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
       if (s + XD < n_steps) load_x(s + XD, xring[u % XD]);
     }
+  }
+
+  };  // round
+  if constexpr (ROUNDS) {
+    for (int r = slice_begin; r < slice_end; r += staged_steps) {
+      if (r > slice_begin) __syncthreads();   // every wave has read the rows of the round before
+      round(r, min(r + staged_steps, slice_end));
+    }
+  } else {
+    round(slice_begin, slice_end);
   }
 
   // add the WK partial sums of every column tile in the order wk = 0, 1, ...: waves wk > 0 park
@@ -405,6 +424,27 @@ int launch_rows(const RowsArgs& a, int splits, hipStream_t s) {
   return launch_status();
 }
 
+// The fused activation for more rows than LDS holds of all of K at once: one k slice, walked in rounds.
+template <int MT, int WN, int WK, int PD, int XD, typename TOut>
+int launch_rows_rounds(const RowsArgs& a, hipStream_t s) {
+  const size_t lds = rows_lds_bytes(a.M, a.steps_per_round, MT, WN, WK);
+  if (lds > kRowsLdsMax) return static_cast<int>(hipErrorInvalidValue);
+  auto kernel = gemm_rows_kernel<MT, WN, WK, PD, XD, kEpiSiluMul, TOut, true>;
+  static size_t allowed = 64 * 1024;
+  if (lds > allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       static_cast<int>(kRowsLdsMax));
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return static_cast<int>(e);
+    }
+    allowed = kRowsLdsMax;
+  }
+  const int col_groups = (a.N + WN * 16 - 1) / (WN * 16);
+  kernel<<<dim3(col_groups, 1), WN * WK * 64, lds, s>>>(a);
+  return launch_status();
+}
+
 template <int MT, int WN, int WK, int PD, int XD, int EPI>
 int launch_rows_out(const RowsArgs& a, int splits, int out_dtype, hipStream_t s) {
   if (out_dtype == kF32) return launch_rows<MT, WN, WK, PD, XD, EPI, float>(a, splits, s);
@@ -484,7 +524,7 @@ extern "C" int arle_gemm_rows(const void* x, long long ldx, const void* w, long 
   if (epilogue != kEpiNone && epilogue != kEpiSiluMul) return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const RowsArgs a{static_cast<const uint16_t*>(x), ldx, static_cast<const uint16_t*>(w), ldw, out, ldo, M, N, K,
-                   steps_per_split, split_stride, w_tiled ? 1 : 0};
+                   steps_per_split, split_stride, w_tiled ? 1 : 0, 0};
   switch (variant) {
 #define X(ID, WN, WK, PD)                                                                       \
   case ID:                                                                                      \
@@ -495,6 +535,24 @@ extern "C" int arle_gemm_rows(const void* x, long long ldx, const void* w, long 
 #undef X
   }
   return static_cast<int>(hipErrorInvalidValue);
+}
+
+// gate|up with the fused activation for up to 64 rows: as arle_gemm_rows with epilogue 1, variant 3 (eight waves,
+// one column tile each) and one k split, but the X rows of only steps_per_round steps of 32 are in LDS at a time
+// (arle_gemm_rows_lds(3, M, steps_per_round) <= arle_gemm_rows_lds_max()); all of K is walked in such rounds.
+extern "C" int arle_gemm_rows_rounds(const void* x, long long ldx, const void* w, long long ldw, int w_tiled, void* out,
+                                     long long ldo, int out_dtype, int M, int N, int K, int steps_per_round, void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K % 8 != 0 || K <= 0 || ldx % 8 != 0 || ldw % 8 != 0 || N % 32 != 0 || steps_per_round < 1)
+    return static_cast<int>(hipErrorInvalidValue);
+  const int steps_total = (K + 31) / 32;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const RowsArgs a{static_cast<const uint16_t*>(x), ldx, static_cast<const uint16_t*>(w), ldw, out, ldo, M, N, K,
+                   steps_total, 0, w_tiled ? 1 : 0, steps_per_round < steps_total ? steps_per_round : steps_total};
+  const bool f32 = out_dtype == kF32;
+  if (M <= 16) return f32 ? launch_rows_rounds<1, 8, 1, 4, 4, float>(a, s) : launch_rows_rounds<1, 8, 1, 4, 4, bf16>(a, s);
+  if (M <= 32) return f32 ? launch_rows_rounds<2, 8, 1, 4, 2, float>(a, s) : launch_rows_rounds<2, 8, 1, 4, 2, bf16>(a, s);
+  return f32 ? launch_rows_rounds<4, 8, 1, 4, 2, float>(a, s) : launch_rows_rounds<4, 8, 1, 4, 2, bf16>(a, s);
 }
 
 // Shapes of a staying workgroup, by `variant`: (WN, PD).
@@ -568,7 +626,7 @@ extern "C" int arle_gemm_stream(const void* x, long long ldx, const void* w, lon
   if (splits > 1 && out_dtype != kF32) return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const RowsArgs a{static_cast<const uint16_t*>(x), ldx, static_cast<const uint16_t*>(w), ldw, out, ldo, M, N, K,
-                   steps_per_split, split_stride, w_tiled ? 1 : 0};
+                   steps_per_split, split_stride, w_tiled ? 1 : 0, 0};
   switch (variant) {
 #define X(ID, WN, PD) \
   case ID:            \

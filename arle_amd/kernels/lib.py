@@ -24,6 +24,7 @@ SIGNATURES = {
     "arle_rmsnorm": ("norm", [_p, _i, _ll, _p, _i, _p, _i, _p, _i, _i, _f, _p]),
     "arle_add_rmsnorm": ("norm", [_p, _p, _i, _ll, _i, _p, _i, _p, _i, _p, _i, _i, _f, _p]),
     "arle_sum_partials": ("elementwise", [_p, _i, _ll, _p, _i, _ll, _p]),
+    "arle_gemm_rows_rounds": ("gemm_rows", [_p, _ll, _p, _ll, _i, _p, _ll, _i, _i, _i, _i, _i, _p]),
     "arle_gemm_rows": ("gemm_rows", [_p, _ll, _p, _ll, _i, _p, _ll, _ll, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "arle_gemm_rows_geometry": ("gemm_rows", [_i]),
     "arle_gemm_stream_geometry": ("gemm_rows", [_i]),

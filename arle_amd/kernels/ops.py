@@ -577,7 +577,7 @@ _ROWS_MAX_SPLITS = 4             # ... the consumer pays for every part of the s
 _ROWS_PARTIAL_BYTES = 3 << 20    # ... and the float32 partial products stay below this
 _ROWS_WIDE_N = 32768             # from here on (an output head) N alone gives enough workgroups
 _ROWS_NARROW_N = 4096            # up to here N gives so few that one column tile a workgroup is best
-_ROWS_FUSED_MAX = 32             # gate|up with the activation: as many rows as fit into LDS with all of K (27 at K = 2560): 4.20 against 4.41 ms a step at batch 20
+_ROWS_FUSED_MAX = 32             # gate|up with the activation in one go: as many rows as fit into LDS with all of K (27 at K = 2560): 4.20 against 4.41 ms a step at batch 20; more rows: gemm_rows_rounds
 _ROWS_PREFERRED = 16             # with more rows the library is at least as fast on MI355X
 _V_GENERAL, _V_FUSED_FEW, _V_NARROW, _V_SHARED = 0, 1, 2, 3
 ROWS_VARIANTS = 5
@@ -707,6 +707,65 @@ def gemm_rows(x, w, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, varia
     lib.call("arle_gemm_rows", x.data_ptr(), x.stride(0), (w if tiles is None else tiles).data_ptr(), w.stride(0),
              int(tiles is not None), out.data_ptr(), ldo, stride,
              code, M, N, K, int(epilogue), variant, splits, per_split, _stream())
+    return out
+
+
+def gemm_rows_rounds_preferred(rows: int, n: int, k: int, x_stride: int) -> bool:
+    """Whether gate|up with its activation should run in the few-rows kernel that walks K in rounds: up to 64
+    rows.  Measured on MI355X at the Qwen3-4B shape against the library's product and the activation kernel, in
+    us: 23.7 against 27.5 at 28 rows, 25.7 against 29.2 at 40, 26.5 against 30.4 at 48, 29.4 against 31.0 at 64."""
+    return gemm_rows_supported(rows, k, x_stride) and n % 32 == 0
+
+
+@functools.lru_cache(maxsize=None)
+def _rows_round_steps(rows: int, k: int) -> int:
+    """Steps of 32 k whose x rows the fused few-rows kernel can hold in LDS at a time, cut so that the rounds
+    that cover K are of one length."""
+    steps = -(-k // 32)
+    need = lib.function("arle_gemm_rows_lds")
+    need.restype = ctypes.c_longlong
+    cap_fn = lib.function("arle_gemm_rows_lds_max")
+    cap_fn.restype = ctypes.c_longlong
+    most, fit = cap_fn(), steps
+    while fit > 1 and need(_V_SHARED, rows, fit) > most:
+        fit -= 1
+    _need(need(_V_SHARED, rows, fit) <= most, f"gemm_rows_rounds: {rows} rows of 32 columns do not fit into LDS")
+    rounds = -(-steps // fit)
+    return -(-steps // rounds)
+
+
+def gemm_rows_rounds(x, w, out_dtype=torch.bfloat16, *, tiles: torch.Tensor | None = None, round_steps: int | None = None):
+    """silu(x . gate^T) * (x . up^T) for 1..64 rows of x, w holding gate and up rows interleaved in blocks of 16:
+    gemm_rows with the fused activation where the x rows of all of K do not fit into LDS at once (more than 27
+    rows at K = 2,560).  K is walked in rounds of `round_steps` steps of 32, the sums stay in registers.
+    Returns [M, N/2]."""
+    _gpu(x, w)
+    _rows(x, "x")
+    _need(w.dim() == 2 and w.is_contiguous(), "w must be contiguous [N, K]")
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_rows_rounds takes bfloat16 operands")
+    M, K = x.shape
+    N = w.shape[0]
+    _need(w.shape[1] == K, f"gemm_rows_rounds: inner sizes differ ({K} vs {w.shape[1]})")
+    _need(gemm_rows_supported(M, K, x.stride(0)),
+          f"gemm_rows_rounds takes 1..{ROWS_KERNEL_MAX} rows and K % 8 == 0 (got {M} rows, K = {K})")
+    _need(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
+    _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_rows_rounds writes bfloat16 or float32")
+    _need(N % 32 == 0, "the fused activation needs gate/up interleaved in blocks of 16")
+    if round_steps is None:
+        round_steps = _rows_round_steps(M, K)
+    _need(round_steps >= 1, "a round is at least one step of 32")
+    round_steps = min(int(round_steps), -(-K // 32))
+    need = lib.function("arle_gemm_rows_lds")
+    need.restype = ctypes.c_longlong
+    cap_fn = lib.function("arle_gemm_rows_lds_max")
+    cap_fn.restype = ctypes.c_longlong
+    _need(need(_V_SHARED, M, round_steps) <= cap_fn(),
+          f"gemm_rows_rounds: {M} rows of {round_steps * 32} columns do not fit into LDS; take shorter rounds")
+    if tiles is not None:
+        _check_tiles(tiles, N, K)
+    out = torch.empty((M, N // 2), dtype=out_dtype, device=x.device)
+    lib.call("arle_gemm_rows_rounds", x.data_ptr(), x.stride(0), (w if tiles is None else tiles).data_ptr(), w.stride(0),
+             int(tiles is not None), out.data_ptr(), out.stride(0), _CODES[out_dtype], M, N, K, int(round_steps), _stream())
     return out
 
 

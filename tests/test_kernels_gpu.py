@@ -890,6 +890,28 @@ def test_gemm_rows_fused_activation_from_operand_tiles():
     assert torch.equal(rows, ops.gemm_rows(x, fused, torch.bfloat16, ops.EPI_SILU_MUL, tiles=ops.pack_weight_tiles(fused)))
 
 
+@pytest.mark.parametrize("M,inter,K,round_steps", [(64, 224, 2560, None), (40, 48, 200, 3), (28, 160, 1096, 7), (33, 64, 96, 1),
+                                                   (5, 32, 72, 2), (17, 96, 2560, 80), (64, 32, 264, 4)])
+def test_gemm_rows_fused_activation_with_k_walked_in_rounds(M, inter, K, round_steps):
+    """gate|up with the activation for more rows than LDS holds of all of K: rounds of every length (one step, one
+    round for all of K, a last round that is shorter, K that ends inside a step), every row-tile count, from rows
+    and from operand tiles; where one round holds everything the bits are those of the kernel without rounds."""
+    x = torch.randn(M, K, generator=_g(140)).bfloat16()
+    gate = (torch.randn(inter, K, generator=_g(141)) * 0.1).bfloat16()
+    up = (torch.randn(inter, K, generator=_g(142)) * 0.1).bfloat16()
+    fused = torch.stack([gate.view(-1, 16, K), up.view(-1, 16, K)], dim=1).reshape(2 * inter, K).contiguous().to(DEV)
+    want = plain.silu(x.double() @ gate.double().T) * (x.double() @ up.double().T)
+    xd, tiles = x.to(DEV), ops.pack_weight_tiles(fused)
+    got = ops.gemm_rows_rounds(xd, fused, torch.float32, round_steps=round_steps)
+    assert got.shape == (M, inter) and _rel(got.cpu(), want) < 1e-5
+    assert torch.equal(got, ops.gemm_rows_rounds(xd, fused, torch.float32, tiles=tiles, round_steps=round_steps))
+    assert _rel(ops.gemm_rows_rounds(xd, fused, torch.bfloat16, tiles=tiles, round_steps=round_steps).cpu(), want) < 5e-3
+    if M <= 16 and K <= 2560:      # fits in one go: the same sums in the same order
+        assert torch.equal(got, ops.gemm_rows(xd, fused, torch.float32, ops.EPI_SILU_MUL, variant=3, splits=1))
+    with pytest.raises(ops.ShapeError):
+        ops.gemm_rows_rounds(xd, fused, round_steps=10 ** 6 if M * K > 60000 else 0)
+
+
 @pytest.mark.parametrize("variant", ops.TILES_VARIANTS)
 @pytest.mark.parametrize("M,N,K", [(300, 200, 72), (129, 520, 264), (257, 256, 32), (1, 40, 8), (640, 1000, 1096),
                                    (2300, 4900, 64)])
