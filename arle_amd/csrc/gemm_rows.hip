@@ -95,104 +95,104 @@ __global__ __launch_bounds__(WN* WK * 64) void gemm_rows_kernel(const RowsArgs a
 
   // one round: the steps [s_begin, s_end) of the slice, staged and multiplied (without ROUNDS: the whole slice)
   auto round = [&](const int s_begin, const int s_end) {
-  // this wave's steps: the wk-th part of the round
-  const int per = (s_end - s_begin + WK - 1) / WK;
-  const int w_begin = s_begin + wk * per;
-  const int n_steps = max(0, min(w_begin + per, s_end) - w_begin);
+    // this wave's steps: the wk-th part of the round
+    const int per = (s_end - s_begin + WK - 1) / WK;
+    const int w_begin = s_begin + wk * per;
+    const int n_steps = max(0, min(w_begin + per, s_end) - w_begin);
 
-  // rows: lane (i, g) reads 16 bytes of row n0 + i; tiles: the wave reads tile s of its column tile, lane by lane
-  const uint16_t* wrow = a.tiled ? tile_base(a, n0, lane) : a.w + static_cast<int64_t>(min(n0 + li, N - 1)) * a.ldw;
-  const int w_step = a.tiled ? 512 : 32, w_first = a.tiled ? 0 : 8 * g, w_last = a.tiled ? (steps_total - 1) * 512 : K - 8;
-  auto load_w = [&](int s) {
-    const int e = min(w_step * s + w_first, w_last);  // clamped: always inside the row (the column tile)
-    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(wrow + e));
-  };
+    // rows: lane (i, g) reads 16 bytes of row n0 + i; tiles: the wave reads tile s of its column tile, lane by lane
+    const uint16_t* wrow = a.tiled ? tile_base(a, n0, lane) : a.w + static_cast<int64_t>(min(n0 + li, N - 1)) * a.ldw;
+    const int w_step = a.tiled ? 512 : 32, w_first = a.tiled ? 0 : 8 * g, w_last = a.tiled ? (steps_total - 1) * 512 : K - 8;
+    auto load_w = [&](int s) {
+      const int e = min(w_step * s + w_first, w_last);  // clamped: always inside the row (the column tile)
+      return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(wrow + e));
+    };
 
-  // the first PD steps of W are on their way before anything else happens; without a condition (a step past
-  // the wave's last one is clamped into the row and never used), because a load under a condition is waited
-  // for at the end of its branch
-  bf16x8 ring[PD];
-#pragma unroll
-  for (int u = 0; u < PD; ++u) ring[u] = load_w(w_begin + u);
+    // the first PD steps of W are on their way before anything else happens; without a condition (a step past
+    // the wave's last one is clamped into the row and never used), because a load under a condition is waited
+    // for at the end of its branch
+    bf16x8 ring[PD];
+  #pragma unroll
+    for (int u = 0; u < PD; ++u) ring[u] = load_w(w_begin + u);
 
-  // X rows of the slice -> LDS, straight from memory (no registers in between, so every piece of the slice is
-  // on its way at once): a wave's 64 lanes fill 1 KB of LDS in lane order from 64 addresses of their own.  A
-  // row in LDS is its 16-byte pieces and one piece of padding; padding lanes and lanes past K fetch a piece
-  // that exists, and the pieces past K are put to zero afterwards (W is clamped there, X must not count).
-  {
-    const int cpr = staged_steps * 4;       // pieces of 8 elements per row
-    const int cpp = cpr + kPad / 8;         // ... with the padding
-    const int total = M * cpp;
-    const int k0 = s_begin * 32, k1 = min(s_end * 32, K);
-    for (int q0 = wave * 64; q0 < total; q0 += kThreads) {
-      const int q = min(q0 + lane, total - 1);
-      const int row = q / cpp, cc = q % cpp;
-      const int col = k0 + cc * 8;
-      const uint16_t* src = a.x + static_cast<int64_t>(row) * a.ldx + ((cc < cpr && col < k1) ? col : k0);
-      __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)(lds + q0 * 8),
-                                       16, 0, 0);
+    // X rows of the slice -> LDS, straight from memory (no registers in between, so every piece of the slice is
+    // on its way at once): a wave's 64 lanes fill 1 KB of LDS in lane order from 64 addresses of their own.  A
+    // row in LDS is its 16-byte pieces and one piece of padding; padding lanes and lanes past K fetch a piece
+    // that exists, and the pieces past K are put to zero afterwards (W is clamped there, X must not count).
+    {
+      const int cpr = staged_steps * 4;       // pieces of 8 elements per row
+      const int cpp = cpr + kPad / 8;         // ... with the padding
+      const int total = M * cpp;
+      const int k0 = s_begin * 32, k1 = min(s_end * 32, K);
+      for (int q0 = wave * 64; q0 < total; q0 += kThreads) {
+        const int q = min(q0 + lane, total - 1);
+        const int row = q / cpp, cc = q % cpp;
+        const int col = k0 + cc * 8;
+        const uint16_t* src = a.x + static_cast<int64_t>(row) * a.ldx + ((cc < cpr && col < k1) ? col : k0);
+        __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)(lds + q0 * 8),
+                                         16, 0, 0);
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (k1 < s_end * 32) {
+        __syncthreads();  // the pieces put to zero were fetched by other waves: all of them have to be in first
+        const int z0 = (k1 - k0) / 8, nz = (s_end * 32 - k1) / 8;
+        for (int i = tid; i < M * nz; i += kThreads)
+          *reinterpret_cast<uint4*>(lds + (i / nz) * pitch + (z0 + i % nz) * 8) = uint4{0u, 0u, 0u, 0u};
+      }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (k1 < s_end * 32) {
-      __syncthreads();  // the pieces put to zero were fetched by other waves: all of them have to be in first
-      const int z0 = (k1 - k0) / 8, nz = (s_end * 32 - k1) / 8;
-      for (int i = tid; i < M * nz; i += kThreads)
-        *reinterpret_cast<uint4*>(lds + (i / nz) * pitch + (z0 + i % nz) * 8) = uint4{0u, 0u, 0u, 0u};
-    }
-  }
-  __syncthreads();
+    __syncthreads();
 
-  const uint16_t* xrow[MT];  // lanes past the last row read the last row; their results are not stored
-#pragma unroll
-  for (int b = 0; b < MT; ++b) xrow[b] = lds + min(16 * b + li, M - 1) * pitch + (w_begin - s_begin) * 32 + 8 * g;
-  auto load_x = [&](int s, bf16x8 (&dst)[MT]) {
-#pragma unroll
-    for (int b = 0; b < MT; ++b) dst[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(xrow[b] + 32 * s));
-  };
-  bf16x8 xring[XD][MT];
-#pragma unroll
-  for (int u = 0; u < XD; ++u)
-    if (u < n_steps) load_x(u, xring[u]);
+    const uint16_t* xrow[MT];  // lanes past the last row read the last row; their results are not stored
+  #pragma unroll
+    for (int b = 0; b < MT; ++b) xrow[b] = lds + min(16 * b + li, M - 1) * pitch + (w_begin - s_begin) * 32 + 8 * g;
+    auto load_x = [&](int s, bf16x8 (&dst)[MT]) {
+  #pragma unroll
+      for (int b = 0; b < MT; ++b) dst[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(xrow[b] + 32 * s));
+    };
+    bf16x8 xring[XD][MT];
+  #pragma unroll
+    for (int u = 0; u < XD; ++u)
+      if (u < n_steps) load_x(u, xring[u]);
 
-  // While a whole round of PD steps and of PD loads ahead is left, the round runs without a condition: only
-  // then does each product wait for its own load alone (a load under a condition in a loop makes the next wait
-  // a wait for every load).  The last two rounds are written out, not looped over.
-  int base = 0;
-  for (; base + 2 * PD <= n_steps; base += PD) {
-#pragma unroll
-    for (int u = 0; u < PD; ++u) {
-      const int s = base + u;  // relative to w_begin
-#pragma unroll
-      for (int b = 0; b < MT; ++b)
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
-      load_x(s + XD, xring[u % XD]);
-      ring[u] = load_w(w_begin + s + PD);
-      __builtin_amdgcn_sched_barrier(0);  // keep each load right behind its product: PD - 1 stay in flight
+    // While a whole round of PD steps and of PD loads ahead is left, the round runs without a condition: only
+    // then does each product wait for its own load alone (a load under a condition in a loop makes the next wait
+    // a wait for every load).  The last two rounds are written out, not looped over.
+    int base = 0;
+    for (; base + 2 * PD <= n_steps; base += PD) {
+  #pragma unroll
+      for (int u = 0; u < PD; ++u) {
+        const int s = base + u;  // relative to w_begin
+  #pragma unroll
+        for (int b = 0; b < MT; ++b)
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
+        load_x(s + XD, xring[u % XD]);
+        ring[u] = load_w(w_begin + s + PD);
+        __builtin_amdgcn_sched_barrier(0);  // keep each load right behind its product: PD - 1 stay in flight
+      }
     }
-  }
-  if (base + PD <= n_steps) {  // a whole round of products, fewer than PD loads ahead
-#pragma unroll
+    if (base + PD <= n_steps) {  // a whole round of products, fewer than PD loads ahead
+  #pragma unroll
+      for (int u = 0; u < PD; ++u) {
+        const int s = base + u;
+  #pragma unroll
+        for (int b = 0; b < MT; ++b)
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
+        if (s + XD < n_steps) load_x(s + XD, xring[u % XD]);
+        if (s + PD < n_steps) ring[u] = load_w(w_begin + s + PD);
+      }
+      base += PD;
+    }
+    // the last steps, fewer than PD: W is in the ring or on its way, only X is left to fetch
+  #pragma unroll
     for (int u = 0; u < PD; ++u) {
       const int s = base + u;
-#pragma unroll
-      for (int b = 0; b < MT; ++b)
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
-      if (s + XD < n_steps) load_x(s + XD, xring[u % XD]);
-      if (s + PD < n_steps) ring[u] = load_w(w_begin + s + PD);
+      if (s < n_steps) {
+  #pragma unroll
+        for (int b = 0; b < MT; ++b)
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
+        if (s + XD < n_steps) load_x(s + XD, xring[u % XD]);
+      }
     }
-    base += PD;
-  }
-  // the last steps, fewer than PD: W is in the ring or on its way, only X is left to fetch
-#pragma unroll
-  for (int u = 0; u < PD; ++u) {
-    const int s = base + u;
-    if (s < n_steps) {
-#pragma unroll
-      for (int b = 0; b < MT; ++b)
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[u], xring[u % XD][b], acc[b], 0, 0, 0);
-      if (s + XD < n_steps) load_x(s + XD, xring[u % XD]);
-    }
-  }
 
   };  // round
   if constexpr (ROUNDS) {
