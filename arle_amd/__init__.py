@@ -12,7 +12,7 @@ __version__ = "0.1.0"
 
 def __getattr__(name):
     # heavy imports (torch) happen only when the entry points are asked for
-    if name in ("LLM", "generate", "CompletionOutput"):
+    if name in ("LLM", "generate", "CompletionOutput", "CompletionStreamDelta"):
         from .engine import api
         return getattr(api, name)
     if name in ("Engine", "StepEntry", "DeviceToken"):

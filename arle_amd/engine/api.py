@@ -50,6 +50,21 @@ def _gpu_total_bytes(device) -> int:
     return torch.cuda.get_device_properties(device).total_memory if device.type == "cuda" else 0
 
 
+@dataclass
+class CompletionStreamDelta:
+    """What one request has newly produced (the reference's CompletionStreamDelta,
+    infer/src/server_engine/types.rs:68-81): the tokens that the host has read since the last delta, their text
+    if there is a tokenizer, their log-probabilities if asked for; the request's last delta carries its finish
+    reason and usage (and may carry no token: a stop token is not emitted)."""
+
+    index: int                      # which prompt of the call
+    token_ids: list
+    text_delta: str | None = None
+    logprobs: list = field(default_factory=list)
+    finish_reason: str | None = None
+    usage: TokenUsage | None = None
+
+
 class LLM:
     def __init__(self, model, *, dtype="bfloat16", device=None, page_size: int | None = None,
                  kv_cache_tokens: int | None = None, num_slots: int = 4, max_seq_len: int | None = None,
@@ -123,16 +138,7 @@ class LLM:
         """prompts: a list of token-id lists (or strings, with a tokenizer).  One CompletionOutput each,
         in order.  `sampling` overrides temperature / seed / ignore_eos / logprobs when given.
         priorities: one of PRIORITY_LOW / NORMAL / HIGH (0, 1, 2) a prompt; the higher is served first."""
-        sched = Scheduler(self.engine, self.sampler, self.sched_config, seed=self.seed,
-                          stop_token_ids=self.engine.spec.stop_token_ids)
-        ids = []
-        if priorities is not None and len(priorities) != len(prompts):
-            raise ValueError("one priority a prompt")
-        for i, p in enumerate(prompts):
-            toks = self.tokenize(p) if isinstance(p, str) else list(p)
-            params = sampling or SamplingParams(temperature=temperature, seed=seed, ignore_eos=ignore_eos,
-                                                logprobs=logprobs)
-            ids.append(sched.submit(toks, params, max_tokens, **({} if priorities is None else {"priority": priorities[i]})))
+        sched, ids = self._submit(prompts, max_tokens, temperature, seed, ignore_eos, sampling, logprobs, priorities)
         sched.run_until_done()
         self.last_stats = sched.stats
         outs = []
@@ -147,6 +153,63 @@ class LLM:
                                          response_token_ids=list(r.generated), ttft_s=ttft, tpot_s=tpot,
                                          token_logprobs=list(r.logprobs)))
         return outs
+
+
+    def _submit(self, prompts, max_tokens, temperature, seed, ignore_eos, sampling, logprobs, priorities):
+        sched = Scheduler(self.engine, self.sampler, self.sched_config, seed=self.seed,
+                          stop_token_ids=self.engine.spec.stop_token_ids)
+        ids = []
+        if priorities is not None and len(priorities) != len(prompts):
+            raise ValueError("one priority a prompt")
+        for i, p in enumerate(prompts):
+            toks = self.tokenize(p) if isinstance(p, str) else list(p)
+            params = sampling or SamplingParams(temperature=temperature, seed=seed, ignore_eos=ignore_eos,
+                                                logprobs=logprobs)
+            ids.append(sched.submit(toks, params, max_tokens, **({} if priorities is None else {"priority": priorities[i]})))
+        return sched, ids
+
+    def generate_stream(self, prompts, max_tokens: int = 16, temperature: float = 0.0, seed: int | None = None,
+                        ignore_eos: bool = False, sampling: SamplingParams | None = None, logprobs: bool = False,
+                        priorities=None):
+        """`generate` as a generator of CompletionStreamDelta: after every iteration of the scheduler, what each
+        request has newly produced, in the order of the prompts; a request's last delta has its finish reason and
+        usage.  The tokens of all deltas of a request are `generate`'s response_token_ids.  (With steps launched
+        ahead a token is read, and so handed on, one iteration after the step that chose it.)"""
+        sched, ids = self._submit(prompts, max_tokens, temperature, seed, ignore_eos, sampling, logprobs, priorities)
+        index = {rid: i for i, rid in enumerate(ids)}
+        sent, text_sent, open_ids = {rid: 0 for rid in ids}, {rid: "" for rid in ids}, set(ids)
+        idle = 0
+        while open_ids:
+            if sched.has_work():
+                plan = sched.iteration()
+                idle = idle + 1 if plan.kind == "idle" else 0
+                if idle > 2:
+                    raise RuntimeError("scheduler makes no progress: a waiting request can never be admitted")
+            live = {r.id: r for r in list(sched.waiting) + sched.prefilling + sched.decoding}
+            for rid in ids:
+                if rid not in open_ids:
+                    continue
+                r = sched.finished.get(rid) or live.get(rid)
+                if r is None:
+                    continue
+                done = rid in sched.finished
+                new = r.generated[sent[rid]:]
+                if not new and not done:
+                    continue
+                delta = CompletionStreamDelta(index[rid], list(new), logprobs=list(r.logprobs[sent[rid]:sent[rid] + len(new)]))
+                sent[rid] += len(new)
+                if self.tokenizer is not None:
+                    text = self.tokenizer.decode(r.generated[:sent[rid]])
+                    if done or not text.endswith("\ufffd"):     # a character whose bytes are not all there yet waits
+                        delta.text_delta, text_sent[rid] = text[len(text_sent[rid]):], text
+                    else:
+                        delta.text_delta = ""
+                if done:
+                    delta.finish_reason = r.finish_reason
+                    delta.usage = TokenUsage(len(r.prompt), len(r.generated))
+                    open_ids.discard(rid)
+                yield delta
+        self.last_stats = sched.stats
 
 
 def generate(model, prompts, max_tokens: int = 16, temperature: float = 0.0, seed: int | None = None,

@@ -291,6 +291,39 @@ def test_the_pool_is_sized_from_free_memory_when_no_size_is_given(folders):
         Engine.from_folder(folders["A"], dtype="bfloat16", mem_fraction_static=1e-6)
 
 
+@pytest.mark.parametrize("overlap", [True, False])
+def test_streamed_deltas_add_up_to_what_generate_returns(folders, overlap):
+    """generate_stream hands on what every request has newly produced after each iteration: the tokens and
+    log-probabilities of a request's deltas are those of `generate`, a request's last delta alone carries its finish
+    reason and usage (without a token when a stop token ended it), requests that wait for a slot start later, and an
+    empty prompt ends at once."""
+    cfg, _ = read_folder(folders["A"])
+    llm = LLM(folders["A"], dtype="float32", page_size=4, kv_cache_tokens=256, max_seq_len=64, num_slots=2,
+              async_overlap=overlap)
+    prompts = [random_tokens(n, cfg["vocab_size"], 30 + n) for n in (5, 9, 3)] + [[]]
+    params = SamplingParams(temperature=0.7, seed=11, logprobs=True, ignore_eos=True)
+    whole = llm.generate(prompts, max_tokens=7, sampling=params)
+    deltas = list(llm.generate_stream(prompts, max_tokens=7, sampling=params))
+    for i, want in enumerate(whole):
+        mine = [d for d in deltas if d.index == i]
+        assert [t for d in mine for t in d.token_ids] == want.response_token_ids
+        assert np.allclose([x for d in mine for x in d.logprobs], want.token_logprobs)
+        assert [d.finish_reason for d in mine[:-1]] == [None] * (len(mine) - 1) and mine[-1].finish_reason == want.finish_reason
+        assert mine[-1].usage.completion_tokens == len(want.response_token_ids) and all(d.usage is None for d in mine[:-1])
+        assert all(d.text_delta is None for d in mine)            # a folder without a tokenizer
+    assert len([d for d in deltas if d.index == 3]) == 1          # the empty prompt: one delta, its end
+    first_of = {i: next(k for k, d in enumerate(deltas) if d.index == i and d.token_ids) for i in range(3)}
+    assert first_of[2] > first_of[0] and first_of[2] > first_of[1]   # two slots: the third request starts when one is free
+    assert len([d for d in deltas if d.index == 0]) >= 6           # token by token, not all at the end
+    # a request that a stop token ends: its last delta has no token
+    stop = whole[0].response_token_ids[3]
+    if stop not in whole[0].response_token_ids[:3]:
+        cut = SamplingParams(temperature=0.7, seed=11, stop_token_ids=[stop])
+        mine = list(llm.generate_stream([prompts[0]], max_tokens=7, sampling=cut))
+        assert [t for d in mine for t in d.token_ids] == whole[0].response_token_ids[:3]
+        assert mine[-1].finish_reason == "stop" and mine[-1].token_ids == []
+
+
 def test_the_sizes_of_a_step_follow_the_gpus_memory_unless_given(folders):
     """Nothing given: the longest portion of one request is what the GPU's whole memory gives (16,384 tokens from
     90 GiB on), so a 700-token prompt is one step; with chunked_prefill_size=256 it is three, and the tokens are the
