@@ -18,7 +18,7 @@ from dataclasses import dataclass, field
 
 from ..sampling import Sampler, SamplingParams
 from .engine import Engine
-from .scheduler import Scheduler, SchedulerConfig
+from .scheduler import STOP, Scheduler, SchedulerConfig
 
 
 @dataclass
@@ -50,6 +50,20 @@ def _gpu_total_bytes(device) -> int:
     return torch.cuda.get_device_properties(device).total_memory if device.type == "cuda" else 0
 
 
+def check_stop_sequences(text: str, stops) -> tuple:
+    """(True, where the stop string begins) for the first of `stops`, in their order, that `text` holds; else
+    (False, how much of `text` may be handed on): all but as many bytes at its end as the longest stop string
+    has, in case one straddles the end of what is decoded so far (infer/src/scheduler/cuda/request.rs:396-413).
+    Positions are in characters; empty stop strings do not count."""
+    for stop in stops:
+        if stop and stop in text:
+            return True, text.index(stop)
+    hold = max((len(stop.encode("utf-8")) for stop in stops), default=0)
+    raw = text.encode("utf-8")
+    safe = raw[:max(0, len(raw) - hold)].decode("utf-8", errors="ignore")   # back to the boundary of a character
+    return False, len(safe)
+
+
 @dataclass
 class CompletionStreamDelta:
     """What one request has newly produced (the reference's CompletionStreamDelta,
@@ -63,6 +77,7 @@ class CompletionStreamDelta:
     logprobs: list = field(default_factory=list)
     finish_reason: str | None = None
     usage: TokenUsage | None = None
+    prompt_token_ids: list = field(default_factory=list)   # with the finish reason: the prompt as the engine saw it
 
 
 class LLM:
@@ -134,10 +149,15 @@ class LLM:
 
     def generate(self, prompts, max_tokens: int = 16, temperature: float = 0.0, seed: int | None = None,
                  ignore_eos: bool = False, sampling: SamplingParams | None = None, logprobs: bool = False,
-                 priorities=None) -> list:
+                 priorities=None, stop=None) -> list:
         """prompts: a list of token-id lists (or strings, with a tokenizer).  One CompletionOutput each,
         in order.  `sampling` overrides temperature / seed / ignore_eos / logprobs when given.
-        priorities: one of PRIORITY_LOW / NORMAL / HIGH (0, 1, 2) a prompt; the higher is served first."""
+        priorities: one of PRIORITY_LOW / NORMAL / HIGH (0, 1, 2) a prompt; the higher is served first.
+        stop: strings that end a request where its text first holds one of them (the text stops in front of it,
+        the finish reason is `stop`); needs a tokenizer."""
+        if stop:
+            return self._collect(prompts, self.generate_stream(prompts, max_tokens, temperature, seed, ignore_eos,
+                                                               sampling, logprobs, priorities, stop))
         sched, ids = self._submit(prompts, max_tokens, temperature, seed, ignore_eos, sampling, logprobs, priorities)
         sched.run_until_done()
         self.last_stats = sched.stats
@@ -155,6 +175,20 @@ class LLM:
         return outs
 
 
+    def _collect(self, prompts, deltas) -> list:
+        """The deltas of a streamed call put together as `generate` returns them."""
+        n = len(prompts)
+        toks, lps, text, end = [[] for _ in range(n)], [[] for _ in range(n)], [""] * n, [None] * n
+        for d in deltas:
+            toks[d.index] += d.token_ids
+            lps[d.index] += d.logprobs
+            text[d.index] += d.text_delta or ""
+            if d.finish_reason is not None:
+                end[d.index] = d
+        return [CompletionOutput(text=text[i] if self.tokenizer is not None else None, finish_reason=end[i].finish_reason,
+                                 usage=end[i].usage, prompt_token_ids=list(end[i].prompt_token_ids),
+                                 response_token_ids=toks[i], token_logprobs=lps[i]) for i in range(n)]
+
     def _submit(self, prompts, max_tokens, temperature, seed, ignore_eos, sampling, logprobs, priorities):
         sched = Scheduler(self.engine, self.sampler, self.sched_config, seed=self.seed,
                           stop_token_ids=self.engine.spec.stop_token_ids)
@@ -170,11 +204,16 @@ class LLM:
 
     def generate_stream(self, prompts, max_tokens: int = 16, temperature: float = 0.0, seed: int | None = None,
                         ignore_eos: bool = False, sampling: SamplingParams | None = None, logprobs: bool = False,
-                        priorities=None):
+                        priorities=None, stop=None):
         """`generate` as a generator of CompletionStreamDelta: after every iteration of the scheduler, what each
         request has newly produced, in the order of the prompts; a request's last delta has its finish reason and
         usage.  The tokens of all deltas of a request are `generate`'s response_token_ids.  (With steps launched
-        ahead a token is read, and so handed on, one iteration after the step that chose it.)"""
+        ahead a token is read, and so handed on, one iteration after the step that chose it.)
+        stop: as for `generate`; text that may still turn out to be the beginning of a stop string is held back
+        (infer/src/scheduler/cuda/request.rs:72-117), and the request ends where one is found."""
+        stops = [s for s in (stop or []) if s]
+        if stops and self.tokenizer is None:
+            raise RuntimeError("stop strings are looked for in the text: this model folder has no tokenizer.json")
         sched, ids = self._submit(prompts, max_tokens, temperature, seed, ignore_eos, sampling, logprobs, priorities)
         index = {rid: i for i, rid in enumerate(ids)}
         sent, text_sent, open_ids = {rid: 0 for rid in ids}, {rid: "" for rid in ids}, set(ids)
@@ -200,13 +239,22 @@ class LLM:
                 sent[rid] += len(new)
                 if self.tokenizer is not None:
                     text = self.tokenizer.decode(r.generated[:sent[rid]])
-                    if done or not text.endswith("\ufffd"):     # a character whose bytes are not all there yet waits
-                        delta.text_delta, text_sent[rid] = text[len(text_sent[rid]):], text
-                    else:
-                        delta.text_delta = ""
+                    upto = len(text)
+                    if stops:
+                        found, upto = check_stop_sequences(text, stops)
+                        if found and not done:      # the scheduler does not see the text: the request ends here
+                            sched.abort(rid, STOP)
+                            done = True
+                        elif done and not found:
+                            upto = len(text)        # nothing more can come: what was held back goes out
+                    elif not done and text.endswith("\ufffd"):
+                        upto = len(text_sent[rid])  # a character whose bytes are not all there yet waits
+                    upto = max(upto, len(text_sent[rid]))
+                    delta.text_delta, text_sent[rid] = text[len(text_sent[rid]):upto], text[:upto]
                 if done:
                     delta.finish_reason = r.finish_reason
                     delta.usage = TokenUsage(len(r.prompt), len(r.generated))
+                    delta.prompt_token_ids = list(r.prompt)
                     open_ids.discard(rid)
                 yield delta
         self.last_stats = sched.stats

@@ -294,22 +294,23 @@ class Scheduler:
         insert_waiting(self.waiting, req, before_equal=False)
         return rid
 
-    def abort(self, rid: int) -> bool:
+    def abort(self, rid: int, reason: str = ABORT) -> bool:
         """End request `rid` now, whatever its phase: out of the queue, or its pages and slot given back.
         True if it was still running or waiting; False if it had finished already or was never submitted.
-        The tokens it has generated so far stay on its record (finish reason `abort`)."""
+        The tokens it has generated so far stay on its record (finish reason `abort`; `stop` when the caller
+        has found a stop string in its text, which the scheduler does not see)."""
         for req in self.waiting:
             if req.id == rid:
                 self.waiting.remove(req)
-                self._finish(req, ABORT)
+                self._finish(req, reason)
                 self.finished[rid] = req
-                self.stats["aborted"] += 1
+                self.stats["aborted"] += reason == ABORT
                 return True
         for group in (self.prefilling, self.decoding):
             for req in group:
                 if req.id == rid and req.phase != "finished":
-                    self._finish(req, ABORT)
-                    self.stats["aborted"] += 1
+                    self._finish(req, reason)
+                    self.stats["aborted"] += reason == ABORT
                     self._cleanup()
                     return True
         return False

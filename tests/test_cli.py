@@ -32,3 +32,18 @@ def test_bad_values_are_refused(capsys):
         build_parser().parse_args(["run", "--prompt", "x", "--stdin"])
     assert main(["run", "--prompt", "x"]) == 2          # no model folder
     assert "--model-path" in capsys.readouterr().err
+
+
+def test_stop_strings_are_found_in_list_order_and_their_length_is_held_back():
+    """The reading of infer/src/scheduler/cuda/request.rs:396-413 (the reference holds no vectors for it): the first
+    stop string of the list that the text holds decides, not the one that comes first in the text; empty ones do
+    not count; without a hit all but the longest stop string's bytes may go out, cut back to a whole character."""
+    from arle_amd.engine.api import check_stop_sequences
+
+    assert check_stop_sequences("one two three", ["three", "two"]) == (True, 8)
+    assert check_stop_sequences("one two three", ["", "two"]) == (True, 4)
+    assert check_stop_sequences("one two", ["three"]) == (False, 2)          # 7 - 5
+    assert check_stop_sequences("on", ["three"]) == (False, 0)
+    assert check_stop_sequences("one two", []) == (False, 7) and check_stop_sequences("one two", [""]) == (False, 7)
+    assert check_stop_sequences("aé", ["xy"]) == (False, 1)                 # 3 bytes - 2 falls inside the é: back to "a"
+    assert check_stop_sequences("ab\u00e9\u00e9", ["\u00e9x"]) == (False, 2)    # 6 bytes - 3: inside the first é

@@ -324,6 +324,48 @@ def test_streamed_deltas_add_up_to_what_generate_returns(folders, overlap):
         assert mine[-1].finish_reason == "stop" and mine[-1].token_ids == []
 
 
+@pytest.mark.parametrize("overlap", [True, False])
+def test_a_stop_string_ends_a_request_in_front_of_it(folders, tmp_path, overlap):
+    """With a tokenizer (one word a token, made here) a stop string that begins in one token and ends in the next
+    ends the request: the text stops in front of it, streamed or not, nothing of it was handed on early, the tokens
+    are those read up to the one that completed it, and the finish reason is `stop`."""
+    import shutil
+    from tokenizers import Tokenizer, models, pre_tokenizers
+
+    cfg, _ = read_folder(folders["A"])
+    d = str(tmp_path / "with_tokenizer")
+    shutil.copytree(folders["A"], d)
+    tok = Tokenizer(models.WordLevel({f"w{i}": i for i in range(cfg["vocab_size"])}, unk_token="w0"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    tok.save(os.path.join(d, "tokenizer.json"))
+    llm = LLM(d, dtype="float32", page_size=4, kv_cache_tokens=256, max_seq_len=64, async_overlap=overlap)
+    prompt = random_tokens(6, cfg["vocab_size"], 77)
+    params = SamplingParams(temperature=0.9, seed=5, ignore_eos=True)
+    whole = llm.generate([prompt, "w3 w4 w5"], max_tokens=10, sampling=params)
+    words = [f"w{t}" for t in whole[0].response_token_ids]
+    assert whole[0].text == " ".join(words) and whole[1].prompt_token_ids == [3, 4, 5]
+    full = " ".join(words)
+    # the end of word k, a blank, the head of word k + 1, where that does not occur earlier in the text
+    k = next(i for i in range(2, 9)
+             if full.find(f"{words[i][1:]} w") == len(" ".join(words[:i + 1])) - len(words[i][1:]))
+    stop = f"{words[k][1:]} w"
+    want_text = full[:full.find(stop)]
+    cut = llm.generate([prompt, "w3 w4 w5"], max_tokens=10, sampling=params, stop=["never", "", stop])
+    assert cut[0].text == want_text and cut[0].finish_reason == "stop"
+    assert cut[0].response_token_ids == whole[0].response_token_ids[:k + 2]
+    assert cut[1].response_token_ids == whole[1].response_token_ids and cut[1].finish_reason == "length"
+    deltas = [x for x in llm.generate_stream([prompt], max_tokens=10, sampling=params, stop=[stop]) if x.index == 0]
+    assert "".join(x.text_delta for x in deltas) == want_text and deltas[-1].finish_reason == "stop"
+    sent = ""
+    for x in deltas:        # what has gone out never reaches into the stop string
+        sent += x.text_delta
+        assert want_text.startswith(sent)
+    assert any(x.text_delta for x in deltas[:-1])      # and text does go out before the end
+    assert llm.engine.cache.free_pages() == [64] and not llm.engine.cache.slot_of
+    with pytest.raises(RuntimeError, match="tokenizer"):
+        LLM(llm.engine).generate([prompt], stop=["x"])
+
+
 def test_the_sizes_of_a_step_follow_the_gpus_memory_unless_given(folders):
     """Nothing given: the longest portion of one request is what the GPU's whole memory gives (16,384 tokens from
     90 GiB on), so a 700-token prompt is one step; with chunked_prefill_size=256 it is three, and the tokens are the
