@@ -117,7 +117,24 @@ def main(argv=None) -> int:
     params = SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p,
                             min_p=args.min_p, ignore_eos=args.ignore_eos)
     t0 = time.perf_counter()
-    out = llm.generate([prompt], max_tokens=max_tokens, sampling=params)[0]
+    if args.json or llm.tokenizer is None:
+        out = llm.generate([prompt], max_tokens=max_tokens, sampling=params)[0]
+    else:       # text goes out as it is generated, as the reference's prompt loop prints it (crates/cli/src/repl.rs:760-800)
+        first = None
+
+        def shown(deltas):
+            nonlocal first
+            for d in deltas:
+                if first is None and d.token_ids:
+                    first = time.perf_counter() - t0
+                if d.text_delta:
+                    sys.stdout.write(d.text_delta)
+                    sys.stdout.flush()
+                yield d
+
+        out = llm._collect([prompt], shown(llm.generate_stream([prompt], max_tokens=max_tokens, sampling=params)))[0]
+        out.ttft_s = first
+        print()
     elapsed = time.perf_counter() - t0
     if args.json:
         print(json.dumps({"model": args.model_path, "backend": "hip-gfx950", "text": out.text,
@@ -125,8 +142,8 @@ def main(argv=None) -> int:
                           "usage": {"prompt_tokens": out.usage.prompt_tokens,
                                     "completion_tokens": out.usage.completion_tokens,
                                     "total_tokens": out.usage.total_tokens}}))
-    else:
-        print(out.text if out.text is not None else " ".join(str(t) for t in out.response_token_ids))
+    elif llm.tokenizer is None:
+        print(" ".join(str(t) for t in out.response_token_ids))
     ttft = out.ttft_s or elapsed
     decode_time = max(elapsed - ttft, 1e-9)
     print(f"prompt {out.usage.prompt_tokens / max(ttft, 1e-9):.1f} tok/s | TTFT {ttft * 1e3:.1f} ms | "
