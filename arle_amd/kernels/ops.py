@@ -710,11 +710,20 @@ def gemm_rows(x, w, out_dtype=torch.bfloat16, epilogue: int = EPI_NONE, *, varia
     return out
 
 
+_ROUNDS_MAX_WORKGROUPS = 256     # one workgroup a compute unit (its x rows take most of a CU's LDS): more would run in two turns
+_ROUNDS_TALL_MIN_N = 16384       # 33 to 64 rows (four row tiles a wave): only outputs this wide gain
+
+
 def gemm_rows_rounds_preferred(rows: int, n: int, k: int, x_stride: int) -> bool:
-    """Whether gate|up with its activation should run in the few-rows kernel that walks K in rounds: up to 64
-    rows.  Measured on MI355X at the Qwen3-4B shape against the library's product and the activation kernel, in
-    us: 23.7 against 27.5 at 28 rows, 25.7 against 29.2 at 40, 26.5 against 30.4 at 48, 29.4 against 31.0 at 64."""
-    return gemm_rows_supported(rows, k, x_stride) and n % 32 == 0
+    """Whether gate|up with its activation should run in the few-rows kernel that walks K in rounds (up to 64
+    rows), not as the library's product and the activation kernel.  Measured on MI355X, in us, rounds against
+    library, at 28 / 48 / 64 rows: 19,456 x 2,560 (Qwen3-4B) 24.4 / 27.1 / 31.0 against 27.7 / 30.4 / 31.8;
+    24,576 x 4,096 (8B) 45.7 / 49.7 / 52.7 against 53.1 / 53.6 / 54.1; 6,144 x 1,024 (0.6B) 8.6 / 11.0 / 12.9
+    against 12.1 / 12.8 / 12.6; 12,288 x 2,048 (1.7B, 96 workgroups) 19.9 / 22.6 / 24.9 against 20.5 / 21.4 / 21.8;
+    51,200 x 5,120 (32B: 400 workgroups for 256 compute units, two turns) 105.7 / 113.8 / 123.6 against
+    100.5 / 104.2 / 110.4.  So: no more workgroups than compute units, and beyond 32 rows a wide output."""
+    return (gemm_rows_supported(rows, k, x_stride) and n % 32 == 0 and -(-n // 128) <= _ROUNDS_MAX_WORKGROUPS
+            and (rows <= 32 or n >= _ROUNDS_TALL_MIN_N))
 
 
 @functools.lru_cache(maxsize=None)
