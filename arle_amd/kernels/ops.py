@@ -721,9 +721,14 @@ def gemm_rows_rounds_preferred(rows: int, n: int, k: int, x_stride: int) -> bool
     24,576 x 4,096 (8B) 45.7 / 49.7 / 52.7 against 53.1 / 53.6 / 54.1; 6,144 x 1,024 (0.6B) 8.6 / 11.0 / 12.9
     against 12.1 / 12.8 / 12.6; 12,288 x 2,048 (1.7B, 96 workgroups) 19.9 / 22.6 / 24.9 against 20.5 / 21.4 / 21.8;
     51,200 x 5,120 (32B: 400 workgroups for 256 compute units, two turns) 105.7 / 113.8 / 123.6 against
-    100.5 / 104.2 / 110.4.  So: no more workgroups than compute units, and beyond 32 rows a wide output."""
-    return (gemm_rows_supported(rows, k, x_stride) and n % 32 == 0 and -(-n // 128) <= _ROUNDS_MAX_WORKGROUPS
-            and (rows <= 32 or n >= _ROUNDS_TALL_MIN_N))
+    100.5 / 104.2 / 110.4.  So: no more workgroups than compute units, and beyond 32 rows a wide output.  Up to 16
+    rows the x rows of a round are small enough for several workgroups a compute unit and the kernel is level with
+    the library at every width (32B shape, 16 rows: 94 against 94 us), where the product alone without the
+    activation, as a stack of parts of K, takes 123 + 5 + 5 us: so rows that the kernel without rounds cannot
+    hold (14 to 16 rows at K = 5,120) come here."""
+    if not (gemm_rows_supported(rows, k, x_stride) and n % 32 == 0):
+        return False
+    return rows <= _ROWS_PREFERRED or (-(-n // 128) <= _ROUNDS_MAX_WORKGROUPS and (rows <= 32 or n >= _ROUNDS_TALL_MIN_N))
 
 
 @functools.lru_cache(maxsize=None)

@@ -912,6 +912,20 @@ def test_gemm_rows_fused_activation_with_k_walked_in_rounds(M, inter, K, round_s
         ops.gemm_rows_rounds(xd, fused, round_steps=10 ** 6 if M * K > 60000 else 0)
 
 
+def test_which_kernel_takes_gate_up_with_its_activation_by_rows_and_shape():
+    """The few-rows kernel in one go while the x rows of all of K fit into LDS, then the kernel that walks K in
+    rounds where it was measured ahead of the library: up to 16 rows at every width, up to 32 rows where the output
+    gives no more workgroups than the chip has compute units, up to 64 rows for a wide output."""
+    def taken(rows, n, k):
+        if ops.gemm_rows_preferred(rows, n, k, k, fused=True):
+            return "one go"
+        return "rounds" if ops.gemm_rows_rounds_preferred(rows, n, k, k) else "library"
+    assert [taken(r, 19456, 2560) for r in (8, 27, 28, 48, 64, 65)] == ["one go"] * 2 + ["rounds"] * 3 + ["library"]
+    assert [taken(r, 51200, 5120) for r in (8, 13, 14, 16, 17, 32)] == ["one go"] * 2 + ["rounds"] * 2 + ["library"] * 2
+    assert [taken(r, 12288, 2048) for r in (16, 32, 33, 64)] == ["one go", "one go", "library", "library"]
+    assert [taken(r, 24576, 4096) for r in (16, 17, 32, 64)] == ["one go", "rounds", "rounds", "rounds"]
+
+
 @pytest.mark.parametrize("variant", ops.TILES_VARIANTS)
 @pytest.mark.parametrize("M,N,K", [(300, 200, 72), (129, 520, 264), (257, 256, 32), (1, 40, 8), (640, 1000, 1096),
                                    (2300, 4900, 64)])
