@@ -979,8 +979,10 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
 # product of the parts, it fills the chip: 33 us at 512 rows, 29 at 128.  The parts come back as a float32 stack
 # for the consumer to add in order, like the stacks of the few-rows kernels (added in float32, where the single
 # product rounds its sum to bfloat16).  More parts make a larger stack to write and read, so wide outputs and
-# rows beyond 1,024 stay whole.
-_LIB_SPLIT_MAX_N = 4096
+# rows beyond 1,024 stay whole.  Outputs of 5,120 columns (the 14B and 32B shapes) gain most: down (5,120 x 25,600)
+# whole takes 172 / 182 / 261 / 272 / 349 us at 65 / 128 / 256 / 512 / 1,024 rows and 60 / 63 / 79 / 120 / 247 in
+# parts; o (5,120 x 8,192) 31 / 46 / 74 / 70 / 94 whole and 31 / 32 / 37 / 48 / 89 in parts.
+_LIB_SPLIT_MAX_N = 5120
 _LIB_SPLIT_MIN_K = 2048
 _LIB_SPLIT_MAX_ROWS = 1024
 _BMM_OUT_DTYPE_OK = None
