@@ -985,6 +985,8 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
 _LIB_SPLIT_MAX_N = 5120
 _LIB_SPLIT_MIN_K = 2048
 _LIB_SPLIT_MAX_ROWS = 1024
+_LIB_SPLIT_LONG_K = 8192
+_LIB_SPLIT_LONG_K_MAX_ROWS = 3072
 _BMM_OUT_DTYPE_OK = None
 
 
@@ -1016,9 +1018,15 @@ def narrow_tiles_splits(rows: int, n: int, k: int, x_stride: int) -> int:
 
 def library_k_splits(rows: int, n: int, k: int) -> int:
     """Into how many parts along K the library's product is cut (1: not at all)."""
-    if not (ROWS_KERNEL_MAX < rows <= _LIB_SPLIT_MAX_ROWS and n <= _LIB_SPLIT_MAX_N and k >= _LIB_SPLIT_MIN_K):
+    if not (ROWS_KERNEL_MAX < rows and n <= _LIB_SPLIT_MAX_N and k >= _LIB_SPLIT_MIN_K):
         return 1
-    if k >= 8192:
+    if rows > _LIB_SPLIT_MAX_ROWS:
+        # a very long K still gains from two parts: down of the Qwen3-4B shape 76 / 91 / 126 us at 1,536 / 2,048 /
+        # 3,072 rows against 92 / 111 / 146 whole (the consumer pays 6 to 10 us for the stack); at 4,096 whole is ahead
+        if not (k >= _LIB_SPLIT_LONG_K and rows <= _LIB_SPLIT_LONG_K_MAX_ROWS):
+            return 1
+        splits = 2
+    elif k >= 8192:
         splits = 8 if rows <= 256 else 4
     else:
         splits = 4 if rows <= 512 else 2

@@ -801,15 +801,22 @@ def test_gemm_rows_with_fused_activation(M, inter, K):
     assert _rel(got, want) < 1e-2
 
 
-@pytest.mark.parametrize("M,N,K", [(65, 2560, 4096), (200, 333, 2048), (512, 2560, 9728), (1024, 96, 8192), (300, 2560, 2080)])
+@pytest.mark.parametrize("M,N,K", [(65, 2560, 4096), (200, 333, 2048), (512, 2560, 9728), (1024, 96, 8192), (300, 2560, 2080),
+                                   (1500, 160, 8256), (3100, 96, 8192), (1100, 96, 4096), (700, 5120, 8192), (700, 5152, 8192)])
 def test_library_product_cut_along_k_for_narrow_outputs(M, N, K):
-    """65 to 1,024 rows, a narrow output and a long K: the library's product is run as a batched product of parts
-    of K, and the parts come back as a float32 stack whose sum, in order, is the product."""
+    """65 to 1,024 rows, a narrow output (up to 5,120 columns) and a long K: the library's product is run as a
+    batched product of parts of K, and the parts come back as a float32 stack whose sum, in order, is the product;
+    with K of 8,192 and more, two parts up to 3,072 rows."""
     x = torch.randn(M, K, generator=_g(150)).bfloat16()
     w = (torch.randn(N, K, generator=_g(151)) * 0.05).bfloat16()
     want = x.double() @ w.double().T
     splits = ops.library_k_splits(M, N, K)
-    assert splits == {4096: 4 if M <= 512 else 2, 2048: 4, 9728: 4, 8192: 4, 2080: 1}[K] or (K == 4096 and M == 65 and splits == 4)
+    if M > 1024:
+        assert splits == {(1500, 8256): 2, (3100, 8192): 1, (1100, 4096): 1}[(M, K)]
+    elif N > 4096:
+        assert splits == (4 if N == 5120 else 1)
+    else:
+        assert splits == {4096: 4 if M <= 512 else 2, 2048: 4, 9728: 4, 8192: 4, 2080: 1}[K] or (K == 4096 and M == 65 and splits == 4)
     got = ops.gemm_bf16(x.to(DEV), w.to(DEV), torch.bfloat16, partials_ok=True)
     if splits > 1:
         assert got.dtype == torch.float32 and got.shape == (splits, M, N)
