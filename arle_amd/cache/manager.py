@@ -115,6 +115,15 @@ def pages_for_memory(free_bytes: int, total_bytes: int, mem_fraction_static: flo
     return int(min(pages, most_pages) if most_pages is not None else pages)
 
 
+AUTO_SLOTS_MIN, AUTO_SLOTS_MAX = 4, 128       # infer/src/main.rs:807-808
+
+
+def slots_for_tokens(cache_tokens: int, longest_request: int) -> int:
+    """How many requests run at a time when the caller does not say: as many of the longest length as the cache
+    holds, no fewer than 4 and no more than 128 (the reference's server: infer/src/main.rs:782-855)."""
+    return max(AUTO_SLOTS_MIN, min(AUTO_SLOTS_MAX, int(cache_tokens) // max(1, int(longest_request))))
+
+
 @dataclass
 class PagedView:
     """What a mixer sees of its paged cache during a step."""

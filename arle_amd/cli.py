@@ -29,6 +29,15 @@ def _max_tokens(value: str) -> int:
     return n
 
 
+def _num_slots(value: str):
+    if value.strip().lower() == "auto":
+        return None
+    n = int(value)
+    if n < 1:
+        raise argparse.ArgumentTypeError("--num-slots must be at least 1 (or auto)")
+    return n
+
+
 def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="arle-amd", description="Qwen3 inference on one MI355X")
     ap.add_argument("--model-path", required=False, help="model folder (config.json + safetensors)")
@@ -41,7 +50,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--ignore-eos", action="store_true")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
-    ap.add_argument("--num-slots", type=int, default=4)
+    ap.add_argument("--num-slots", type=_num_slots, default=4,
+                    help="requests that run at a time; auto: as many of --max-seq-len as the cache holds, 4 to 128")
     ap.add_argument("--max-seq-len", type=int, default=None)
     ap.add_argument("--chunked-prefill-size", type=int, default=None,
                     help="longest prompt portion of one request in a step; default: by the GPU's memory "

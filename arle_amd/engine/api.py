@@ -82,7 +82,7 @@ class CompletionStreamDelta:
 
 class LLM:
     def __init__(self, model, *, dtype="bfloat16", device=None, page_size: int | None = None,
-                 kv_cache_tokens: int | None = None, num_slots: int = 4, max_seq_len: int | None = None,
+                 kv_cache_tokens: int | None = None, num_slots: int | None = 4, max_seq_len: int | None = None,
                  chunked_prefill_size: int | None = None, max_num_batched_tokens: int = 16384,
                  max_prefill_tokens: int | None = None, prefill_max_requests: int | None = None, seed: int = 42,
                  cuda_graph: bool = True, weight_tiles: bool | None = None, mem_fraction_static: float = 0.85,
@@ -98,6 +98,8 @@ class LLM:
         16,384 on an MI355X), and at most max_num_batched_tokens.  max_prefill_tokens: the prompt tokens of
         all requests in a step; default max_num_batched_tokens.  While requests are decoding a portion is at
         most 4,096 tokens (long_prefill_token_threshold).
+        num_slots: requests that run at a time; None: as many requests of max_seq_len tokens as the cache holds, from 4
+        to 128 (the reference's --num-slots left unset).
         cuda_graph, weight_tiles: as for Engine (captured steps; the decode-friendly second copy of the weights).
         async_overlap: decode steps are launched from the last step's tokens on the GPU, and those are read back
         while the new step runs (SchedulerConfig.async_overlap); the tokens are the same either way.

@@ -15,7 +15,7 @@ import os
 import torch
 
 from .. import models  # noqa: F401  (registers the architectures)
-from ..cache.manager import (CacheManager, PagedNeed, cache_bytes_per_token, pages_for_memory,
+from ..cache.manager import (CacheManager, PagedNeed, cache_bytes_per_token, pages_for_memory, slots_for_tokens,
                              state_bytes_per_slot)
 from ..config.registry import detect_architecture, load_model_config
 from ..models.decoder import DEBUG_DUMP_ENV, build_model, expected_checkpoint_tensors
@@ -54,7 +54,7 @@ def parse_dtype(name) -> torch.dtype:
 class Engine:
     def __init__(self, spec, tensors: dict, *, dtype=torch.bfloat16, device=None,
                  page_size: int = DEFAULT_PAGE_SIZE, max_tokens: int | None = None,
-                 num_pages: int | None = None, max_slots: int = 4,
+                 num_pages: int | None = None, max_slots: int | None = 4,
                  max_request_tokens: int | None = None, cuda_graph: bool = True,
                  weight_tiles: bool | None = None, mem_fraction_static: float = DEFAULT_MEM_FRACTION_STATIC):
         """
@@ -64,6 +64,9 @@ class Engine:
             weights are loaded, less a headroom of (1 - mem_fraction_static) of the whole memory, divided by
             the bytes of a page over all layers; never more than max_slots requests of max_request_tokens
             (default: the model's positions) can hold, since pages are not shared.
+        max_slots: requests that run at a time.  None: as many requests of max_request_tokens (default: the model's
+            positions) as the cache's tokens, given or sized from memory, hold; at least 4 and at most 128, as the
+            reference's server picks them (infer/src/main.rs:782-855).
         max_request_tokens: longest single request (default: min(model's positions, cache capacity)).
         cuda_graph: replay steps of single decoded tokens from captured HIP graphs (the reference captures
             its decode path per batch size: infer/src/model/qwen3/batch_decode.rs:1691-1730).
@@ -82,6 +85,14 @@ class Engine:
         self.model = build_model(spec, tensors, self.rt)
         needs, readers = self.model.cache_needs()
         self.kv_bytes_per_token = cache_bytes_per_token(needs, self.dtype)
+        if max_slots is None:
+            longest = min(max_request_tokens or spec.max_positions, spec.max_positions)
+            if num_pages is not None or max_tokens is not None:
+                holds = num_pages * page_size if num_pages is not None else int(max_tokens)
+            else:
+                free, total = torch.cuda.mem_get_info(self.device)
+                holds = page_size * pages_for_memory(free, total, mem_fraction_static, self.kv_bytes_per_token * page_size)
+            max_slots = slots_for_tokens(holds, longest)
         if num_pages is None and max_tokens is None:
             longest = min(max_request_tokens or spec.max_positions, spec.max_positions)
             free, total = torch.cuda.mem_get_info(self.device)

@@ -47,3 +47,15 @@ def test_stop_strings_are_found_in_list_order_and_their_length_is_held_back():
     assert check_stop_sequences("one two", []) == (False, 7) and check_stop_sequences("one two", [""]) == (False, 7)
     assert check_stop_sequences("aé", ["xy"]) == (False, 1)                 # 3 bytes - 2 falls inside the é: back to "a"
     assert check_stop_sequences("ab\u00e9\u00e9", ["\u00e9x"]) == (False, 2)    # 6 bytes - 3: inside the first é
+
+
+def test_slots_left_to_the_engine_follow_what_the_cache_holds():
+    """--num-slots auto (the reference's flag left unset, infer/src/main.rs:782-855): as many requests of the longest
+    length as the cache holds, from 4 to 128."""
+    from arle_amd.cache.manager import slots_for_tokens
+
+    assert build_parser().parse_args(["--num-slots", "auto", "run", "--prompt", "x"]).num_slots is None
+    assert build_parser().parse_args(["--num-slots", "7", "run", "--prompt", "x"]).num_slots == 7
+    with pytest.raises(SystemExit):
+        build_parser().parse_args(["--num-slots", "0", "run", "--prompt", "x"])
+    assert [slots_for_tokens(t, 64) for t in (0, 128, 256, 2048, 64 * 128, 10 ** 9)] == [4, 4, 4, 32, 128, 128]

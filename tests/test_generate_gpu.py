@@ -366,6 +366,21 @@ def test_a_stop_string_ends_a_request_in_front_of_it(folders, tmp_path, overlap)
         LLM(llm.engine).generate([prompt], stop=["x"])
 
 
+def test_slots_left_unset_follow_the_cache(folders):
+    """num_slots=None: as many requests of max_seq_len as the cache holds (4 to 128), with a given cache and with one
+    sized from the GPU's memory; more prompts than slots still all finish."""
+    cfg, _ = read_folder(folders["A"])
+    llm = LLM(folders["A"], dtype="float32", page_size=4, kv_cache_tokens=640, max_seq_len=64, num_slots=None)
+    assert llm.engine.cache.max_slots == 10 and llm.sched_config.num_slots == 10
+    prompts = [random_tokens(3 + i % 5, cfg["vocab_size"], 60 + i) for i in range(14)]
+    outs = llm.generate(prompts, max_tokens=4, ignore_eos=True)
+    assert [len(o.response_token_ids) for o in outs] == [4] * 14
+    assert LLM(folders["A"], dtype="float32", page_size=4, kv_cache_tokens=100, max_seq_len=64,
+               num_slots=None).engine.cache.max_slots == 4
+    big = LLM(folders["A"], dtype="bfloat16", page_size=16, max_seq_len=200, num_slots=None)    # a tiny model on a large GPU
+    assert big.engine.cache.max_slots == 128 and big.engine.cache.groups[0].pool.num_pages == 128 * 13
+
+
 def test_the_sizes_of_a_step_follow_the_gpus_memory_unless_given(folders):
     """Nothing given: the longest portion of one request is what the GPU's whole memory gives (16,384 tokens from
     90 GiB on), so a 700-token prompt is one step; with chunked_prefill_size=256 it is three, and the tokens are the
