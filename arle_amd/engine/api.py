@@ -161,7 +161,10 @@ class LLM:
             return self._collect(prompts, self.generate_stream(prompts, max_tokens, temperature, seed, ignore_eos,
                                                                sampling, logprobs, priorities, stop))
         sched, ids = self._submit(prompts, max_tokens, temperature, seed, ignore_eos, sampling, logprobs, priorities)
-        sched.run_until_done()
+        try:
+            sched.run_until_done()
+        finally:
+            sched.close()   # after an error no request of this call keeps a slot or pages
         self.last_stats = sched.stats
         outs = []
         for rid in ids:
@@ -220,45 +223,49 @@ class LLM:
         index = {rid: i for i, rid in enumerate(ids)}
         sent, text_sent, open_ids = {rid: 0 for rid in ids}, {rid: "" for rid in ids}, set(ids)
         idle = 0
-        while open_ids:
-            if sched.has_work():
-                plan = sched.iteration()
-                idle = idle + 1 if plan.kind == "idle" else 0
-                if idle > 2:
-                    raise RuntimeError("scheduler makes no progress: a waiting request can never be admitted")
-            live = {r.id: r for r in list(sched.waiting) + sched.prefilling + sched.decoding}
-            for rid in ids:
-                if rid not in open_ids:
-                    continue
-                r = sched.finished.get(rid) or live.get(rid)
-                if r is None:
-                    continue
-                done = rid in sched.finished
-                new = r.generated[sent[rid]:]
-                if not new and not done:
-                    continue
-                delta = CompletionStreamDelta(index[rid], list(new), logprobs=list(r.logprobs[sent[rid]:sent[rid] + len(new)]))
-                sent[rid] += len(new)
-                if self.tokenizer is not None:
-                    text = self.tokenizer.decode(r.generated[:sent[rid]])
-                    upto = len(text)
-                    if stops:
-                        found, upto = check_stop_sequences(text, stops)
-                        if found and not done:      # the scheduler does not see the text: the request ends here
-                            sched.abort(rid, STOP)
-                            done = True
-                        elif done and not found:
-                            upto = len(text)        # nothing more can come: what was held back goes out
-                    elif not done and text.endswith("\ufffd"):
-                        upto = len(text_sent[rid])  # a character whose bytes are not all there yet waits
-                    upto = max(upto, len(text_sent[rid]))
-                    delta.text_delta, text_sent[rid] = text[len(text_sent[rid]):upto], text[:upto]
-                if done:
-                    delta.finish_reason = r.finish_reason
-                    delta.usage = TokenUsage(len(r.prompt), len(r.generated))
-                    delta.prompt_token_ids = list(r.prompt)
-                    open_ids.discard(rid)
-                yield delta
+        try:
+            while open_ids:
+                if sched.has_work():
+                    plan = sched.iteration()
+                    idle = idle + 1 if plan.kind == "idle" else 0
+                    if idle > 2:
+                        raise RuntimeError("scheduler makes no progress: a waiting request can never be admitted")
+                live = {r.id: r for r in list(sched.waiting) + sched.prefilling + sched.decoding}
+                for rid in ids:
+                    if rid not in open_ids:
+                        continue
+                    r = sched.finished.get(rid) or live.get(rid)
+                    if r is None:
+                        continue
+                    done = rid in sched.finished
+                    new = r.generated[sent[rid]:]
+                    if not new and not done:
+                        continue
+                    delta = CompletionStreamDelta(index[rid], list(new), logprobs=list(r.logprobs[sent[rid]:sent[rid] + len(new)]))
+                    sent[rid] += len(new)
+                    if self.tokenizer is not None:
+                        text = self.tokenizer.decode(r.generated[:sent[rid]])
+                        upto = len(text)
+                        if stops:
+                            found, upto = check_stop_sequences(text, stops)
+                            if found and not done:      # the scheduler does not see the text: the request ends here
+                                sched.abort(rid, STOP)
+                                done = True
+                            elif done and not found:
+                                upto = len(text)        # nothing more can come: what was held back goes out
+                        elif not done and text.endswith("\ufffd"):
+                            upto = len(text_sent[rid])  # a character whose bytes are not all there yet waits
+                        upto = max(upto, len(text_sent[rid]))
+                        delta.text_delta, text_sent[rid] = text[len(text_sent[rid]):upto], text[:upto]
+                    if done:
+                        delta.finish_reason = r.finish_reason
+                        delta.usage = TokenUsage(len(r.prompt), len(r.generated))
+                        delta.prompt_token_ids = list(r.prompt)
+                        open_ids.discard(rid)
+                    yield delta
+        finally:
+            # a consumer that stops reading, or an error in an iteration or in the tokenizer: nothing stays held
+            sched.close()
         self.last_stats = sched.stats
 
 

@@ -315,6 +315,18 @@ class Scheduler:
                     return True
         return False
 
+    def close(self) -> None:
+        """End every request that has not finished (finish reason `abort`) and read what is still pending, so that
+        no slot or page stays held: what a caller does that walks away from a scheduler in mid-run (a consumer that
+        stops reading a stream, an error between two iterations).  Harmless when nothing is left."""
+        for req in list(self.waiting) + list(self.prefilling) + list(self.decoding):
+            if req.phase != "finished":
+                self.abort(req.id)
+        try:
+            self._settle()
+        finally:
+            self._cleanup()
+
     # -- one iteration ------------------------------------------------------------------------
     def has_work(self) -> bool:
         return bool(self.waiting or self.prefilling or self.decoding or self._pending is not None)

@@ -577,3 +577,68 @@ def test_waiting_requests_are_ordered_by_priority_then_first_come():
     assert all(s.finished[r].generated == expected_output(prompt(5, k), 2) for r, k in ((low, 1), (normal, 2), (high, 3)))
     with pytest.raises(ValueError):
         s.submit(prompt(3), priority=7)
+
+
+def test_a_full_waiting_queue_refuses_the_next_request():
+    """Back-pressure at intake (infer/src/scheduler/types.rs:132-133,598: `max_waiting_requests`, SchedulerFull):
+    the request over the limit is refused and takes no id, and room comes back as the queue drains."""
+    from arle_amd.engine.scheduler import SchedulerFull
+
+    eng, s = make(slots=2, max_waiting_requests=3)
+    ids = [s.submit(prompt(5, k), max_tokens=2) for k in range(3)]
+    with pytest.raises(SchedulerFull):
+        s.submit(prompt(5, 9), max_tokens=2)
+    assert len(s.waiting) == 3 and s._next_id == 3
+    s.iteration()                      # two are admitted: one place in the queue is free again
+    ids.append(s.submit(prompt(5, 4), max_tokens=2))
+    s.run_until_done()
+    for k, rid in zip((0, 1, 2, 4), ids):
+        assert s.finished[rid].generated == expected_output(prompt(5, k), 2)
+    assert not eng.cache.slot_of
+
+
+def fake_llm(eng, **cfg):
+    """An LLM around the fake engine: what `LLM.__init__` sets, without a GPU."""
+    from arle_amd.engine.api import LLM
+
+    llm = LLM.__new__(LLM)
+    llm.engine, llm.model_dir, llm.seed, llm.tokenizer, llm.last_stats = eng, None, 42, None, {}
+    llm.sampler = FakeSampler()
+    llm.sched_config = SchedulerConfig(num_slots=eng.cache.max_slots, **cfg)
+    return llm
+
+
+def test_a_stream_that_is_left_early_gives_everything_back():
+    """A consumer that stops reading `generate_stream`, or an error inside an iteration, must not leave requests
+    live in the engine's cache: the next call's requests start at id 0 again."""
+    eng = FakeEngine(slots=2)
+    llm = fake_llm(eng, chunked_prefill_size=4)
+    stream = llm.generate_stream([prompt(9, 1), prompt(6, 2), prompt(7, 3)], max_tokens=8)
+    first = next(stream)
+    assert first.token_ids
+    assert eng.cache.slot_of                    # requests are live in mid-stream
+    stream.close()                              # what `break` in a for loop does
+    assert not eng.cache.slot_of and eng.cache.free_pages() == [64]
+    eng.cache.check()
+    outs = llm.generate([prompt(9, 1), prompt(6, 2)], max_tokens=4)
+    assert [o.response_token_ids for o in outs] == [expected_output(prompt(9, 1), 4), expected_output(prompt(6, 2), 4)]
+
+    class Boom(RuntimeError):
+        pass
+
+    steps = {"n": 0}
+    real_step = eng.step
+
+    def failing_step(entries):
+        steps["n"] += 1
+        if steps["n"] == 3:
+            raise Boom("the engine fails in mid-run")
+        return real_step(entries)
+
+    eng.step = failing_step
+    with pytest.raises(Boom):
+        llm.generate([prompt(9, 1), prompt(6, 2)], max_tokens=6)
+    assert not eng.cache.slot_of and eng.cache.free_pages() == [64]
+    eng.step = real_step
+    outs = llm.generate([prompt(5, 5)], max_tokens=3)
+    assert outs[0].response_token_ids == expected_output(prompt(5, 5), 3)
