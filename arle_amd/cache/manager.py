@@ -58,6 +58,7 @@ class PagedNeed:
     head_dim: int = 0
     window: int | None = None  # None: every earlier token is kept
     tensors: tuple = ()        # of PageTensor; empty: "k" [kv_heads, PAGE, head_dim] and "v" [kv_heads, head_dim, PAGE]
+    page_size: int | None = None   # tokens a page of this need holds; None: the manager's own page length
 
     def page_tensors(self) -> tuple:
         if self.tensors:
@@ -159,14 +160,16 @@ class CacheManager:
         """
         needs: one entry per schedule entry: PagedNeed, StateNeed or None.
         readers: {entry index -> entry index whose cache it reads} for entries that own none.
-        num_pages: pages of every paged group (each group has its own ids and buffers).
+        page_size, num_pages: page length and pages of every paged group (each group has its own ids and
+            buffers).  A need that names a page length of its own gets pages of that length, as many as hold
+            the same number of tokens (num_pages * page_size), and block tables of its own width.
         max_request_tokens: longest request; fixes the width of the block tables.
         """
         self.page_size = page_size
         self.max_slots = max_slots
         self.device = device
         self.dtype = dtype
-        self.max_pages_per_request = max(1, -(-max_request_tokens // page_size))
+        self.max_pages_per_request = max(1, -(-max_request_tokens // page_size))   # of a group with the default page length
         self.needs = list(needs)
         self.readers = dict(readers or {})
 
@@ -177,9 +180,13 @@ class CacheManager:
         for entry, need in enumerate(self.needs):
             if isinstance(need, PagedNeed):
                 if need not in self._group_needs:
+                    own = int(need.page_size or page_size)
+                    if own <= 0:
+                        raise ValueError("a paged need's page_size must be positive")
                     self._group_needs.append(need)
                     self._group_entries.append([])
-                    self.groups.append(PageGroup(num_pages, page_size, need.window))
+                    self.groups.append(PageGroup(num_pages if own == page_size else (num_pages * page_size) // own,
+                                                 own, need.window))
                 g = self._group_needs.index(need)
                 self._entry_place[entry] = (g, len(self._group_entries[g]))
                 self._group_entries[g].append(entry)
@@ -189,9 +196,12 @@ class CacheManager:
         self.slot_of: dict = {}         # request key -> slot
         self._lengths: dict = {}        # request key -> tokens appended so far
 
+        # the longest request that every group's block table can map
+        self._table_widths = [max(1, -(-max_request_tokens // g.page_size)) for g in self.groups]
+        self.request_capacity = min((w * g.page_size for w, g in zip(self._table_widths, self.groups)),
+                                    default=self.max_pages_per_request * page_size)
         # host mirrors of the block tables, one per group
-        self._tables_host = [np.full((max_slots, self.max_pages_per_request), 0, dtype=np.int32)
-                             for _ in self.groups]
+        self._tables_host = [np.full((max_slots, w), 0, dtype=np.int32) for w in self._table_widths]
         self._dirty = [set() for _ in self.groups]
 
         # device buffers
@@ -201,11 +211,12 @@ class CacheManager:
         if device is not None:
             for g, need in enumerate(self._group_needs):
                 n = len(self._group_entries[g])
+                group = self.groups[g]
                 self.page_buffers.append({
-                    t.name: torch.zeros((n, num_pages, *t.page_shape(page_size)), dtype=t.dtype or dtype, device=device)
+                    t.name: torch.zeros((n, group.pool.num_pages, *t.page_shape(group.page_size)),
+                                        dtype=t.dtype or dtype, device=device)
                     for t in need.page_tensors()})
-                self.tables_dev.append(torch.zeros((max_slots, self.max_pages_per_request),
-                                                   dtype=torch.int32, device=device))
+                self.tables_dev.append(torch.zeros((max_slots, self._table_widths[g]), dtype=torch.int32, device=device))
             for entry, need in enumerate(self.needs):
                 if isinstance(need, StateNeed):
                     self.state_buffers[entry] = torch.zeros((max_slots, *need.shape),
@@ -261,6 +272,14 @@ class CacheManager:
     def free_tokens(self) -> int:
         return min((g.free_tokens() for g in self.groups), default=0)
 
+    def pool_tokens(self) -> int:
+        """Tokens that the smallest group's pages hold in all."""
+        return min((g.pool.num_pages * g.page_size for g in self.groups), default=1 << 30)
+
+    def pages_for_length(self, tokens: int) -> list:
+        """Per group, the pages that a request of `tokens` tokens maps (before any window gives some back)."""
+        return [-(-int(tokens) // g.page_size) for g in self.groups]
+
     def append(self, appends) -> None:
         """Room for n more tokens of each request, in every group; all or nothing."""
         for key, n in appends:
@@ -268,9 +287,9 @@ class CacheManager:
                 raise KeyError(f"request {key!r} is not live")
             if n <= 0:
                 raise ValueError("append: token count must be positive")
-            if self.groups and self.length(key) + n > self.max_pages_per_request * self.page_size:
+            if self.groups and self.length(key) + n > self.request_capacity:
                 raise OutOfPages(f"request {key!r} would exceed the longest request the block "
-                                 f"tables were sized for ({self.max_pages_per_request * self.page_size} tokens)")
+                                 f"tables were sized for ({self.request_capacity} tokens)")
         needs = self.pages_needed(appends)
         for g, (need, group) in enumerate(zip(needs, self.groups)):
             if need > group.pool.free_count:
@@ -338,7 +357,7 @@ class CacheManager:
             has = self.device is not None
             pages = {t.name: (self.page_buffers[g][t.name][idx] if has else None) for t in need.page_tensors()}
             return PagedView(pages=pages, block_table=self.tables_dev[g] if has else None,
-                             page_size=self.page_size, window=need.window, writes=owner == entry)
+                             page_size=self.groups[g].page_size, window=need.window, writes=owner == entry)
         if isinstance(need, StateNeed):
             return StateView(state=self.state_buffers.get(owner))
         return None

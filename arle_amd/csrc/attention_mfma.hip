@@ -1428,15 +1428,23 @@ struct PlanMade {
   unsigned blocks = 0, segments = 0;
   int group = 0, min_rows = 0, listed = 0;
   void* stream = nullptr;
+  int device = -1;
 };
 static PlanMade g_plan_made;
 
-inline bool plan_is_current(const AttnArgs& a, dim3 grid, int min_rows, int listed) {
-  const PlanMade now{a.plan_token, a.seg_row0, a.seg_start, a.seg_slot, grid.x, grid.z, a.nq / a.nkv, min_rows, listed, nullptr};
-  const bool same = a.plan_token != 0 && now.token == g_plan_made.token && now.seg_row0 == g_plan_made.seg_row0 &&
+// The list and its counters are one set of device variables a GPU: a list is current only for the stream and the
+// device it was made on (another stream's launches are not ordered behind the planning kernel, another device has
+// a list of its own), and for the same step, segments and launch shape.
+inline bool plan_is_current(const AttnArgs& a, dim3 grid, int min_rows, int listed, hipStream_t s) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) dev = -1;
+  const PlanMade now{a.plan_token, a.seg_row0, a.seg_start, a.seg_slot, grid.x, grid.z, a.nq / a.nkv, min_rows, listed,
+                     static_cast<void*>(s), dev};
+  const bool same = a.plan_token != 0 && dev >= 0 && now.token == g_plan_made.token && now.seg_row0 == g_plan_made.seg_row0 &&
                     now.seg_start == g_plan_made.seg_start && now.seg_slot == g_plan_made.seg_slot &&
                     now.blocks == g_plan_made.blocks && now.segments == g_plan_made.segments &&
-                    now.group == g_plan_made.group && now.min_rows == g_plan_made.min_rows && now.listed == g_plan_made.listed;
+                    now.group == g_plan_made.group && now.min_rows == g_plan_made.min_rows && now.listed == g_plan_made.listed &&
+                    now.stream == g_plan_made.stream && now.device == g_plan_made.device;
   g_plan_made = now;
   return same;
 }
@@ -1462,7 +1470,7 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
   const int per_cu = 1;  // eight waves: two on every SIMD, with all the registers they want
   const unsigned workgroups = static_cast<unsigned>(items < static_cast<long long>(per_cu) * cus ? items : per_cu * cus);
   const int listed = static_cast<long long>(grid.x) * grid.z <= kPfPlanMax && grid.x <= 65535 && grid.z <= 65535;
-  if (!plan_is_current(a, grid, min_rows, listed))
+  if (!plan_is_current(a, grid, min_rows, listed, s))
     attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, a.seg_start, a.seg_slot, static_cast<int>(grid.z),
                                                static_cast<int>(grid.x), a.nq / a.nkv, min_rows, listed);
   if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);  // the merge walks the list
@@ -1499,7 +1507,7 @@ int launch_prefill_dma_groups(const AttnArgs& a, dim3 grid, int min_rows, int cu
   const unsigned workgroups = static_cast<unsigned>(items < places ? items : places);
   const int listed = static_cast<long long>(grid.x) * grid.z <= kPfPlanMax && grid.x <= 65535 && grid.z <= 65535;
   if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);
-  if (!plan_is_current(a, grid, min_rows, listed))
+  if (!plan_is_current(a, grid, min_rows, listed, s))
     attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, a.seg_start, a.seg_slot, static_cast<int>(grid.z),
                                                static_cast<int>(grid.x), a.nq / a.nkv, min_rows, listed);
   const int pair_up = GROUPS == 1 && g_prefill_pair_up ? static_cast<int>(cus / (static_cast<long long>(a.nkv) * a.portion_splits)) : 0;
@@ -1690,17 +1698,29 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
     dim3 grid((max_rows + kPfRows - 1) / kPfRows, nkv, segments);
     SideBranch* side = (min_rows <= 16 && g_side_branch) ? side_branch(s) : nullptr;
     if (side != nullptr) {   // fork: what follows on the side stream waits for what the caller queued so far
-      if (hipEventRecord(side->fork, s) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
-        return static_cast<int>(hipGetLastError());
+      if (hipEventRecord(side->fork, s) != hipSuccess) return static_cast<int>(hipGetLastError());
+      if (hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess) {
+        side = nullptr;      // nothing was queued on the side stream: go on without the branch
+        (void)hipGetLastError();
+      }
+    }
+    int side_rc = 0;
+    if (side != nullptr) {
       AttnArgs b = a;
       b.rows_max = 16;
-      rc = launch_attn<1>(b, dim3(1, nkv, static_cast<unsigned>(z)), side->stream);
-      if (rc == 0 && splits > 1) {
+      side_rc = launch_attn<1>(b, dim3(1, nkv, static_cast<unsigned>(z)), side->stream);
+      if (side_rc == 0 && splits > 1) {
         attn_merge_kernel<<<dim3(segments * b.ws_rows, nq), kMergeWaves * kWave, 0, side->stream>>>(
             ws_o, ws_ml, b.out, o_stride, seg_row0, b.ws_rows, b.rows_max, nq, nkv, D, splits);
-        rc = launch_status();
+        side_rc = launch_status();
       }
-      if (rc != 0) return rc;
+    }
+    if (side != nullptr && side_rc != 0) {
+      // the branch is forked off already: it is joined before the error goes back, so that a capture of `s` does not
+      // end with a stream that never came home, and nothing is still writing when the caller goes on
+      if (hipEventRecord(side->join, side->stream) == hipSuccess) (void)hipStreamWaitEvent(s, side->join, 0);
+      (void)hipGetLastError();
+      return side_rc;
     }
     if (D == 64)
       rc = launch_prefill_lds<64, true>(a, grid, 17, s);
@@ -1715,9 +1735,12 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
       rc = launch_prefill_lds<128, false>(a, grid, 17, s);
     else
       rc = launch_prefill_lds<256, false>(a, grid, 17, s);
-    if (side != nullptr) {   // join: the caller's stream goes on when the side branch is done
-      if (hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(s, side->join, 0) != hipSuccess)
-        return static_cast<int>(hipGetLastError());
+    if (side != nullptr) {   // join: the caller's stream goes on when the side branch is done, also after an error
+      const bool joined = hipEventRecord(side->join, side->stream) == hipSuccess && hipStreamWaitEvent(s, side->join, 0) == hipSuccess;
+      if (!joined) {
+        const int e = static_cast<int>(hipGetLastError());
+        return rc != 0 ? rc : e;
+      }
       return rc;
     }
     if (rc != 0 || min_rows > 16) return rc;

@@ -114,6 +114,8 @@ class Engine:
                                   device=self.device, dtype=self.dtype, readers=readers)
         self.page_size = page_size
         self.max_request_tokens = max_request_tokens
+        # whatever a part keeps per position is made for the longest request now: no step, eager or captured, grows it
+        self.model.prepare(max_request_tokens)
         self.steps_run = 0
         # the debugging dump of hidden states reads them on the host after every layer: such steps are not captured
         self.use_graphs = bool(cuda_graph) and self.model.graph_safe and os.environ.get(DEBUG_DUMP_ENV) is None
@@ -232,7 +234,6 @@ class Engine:
             batch = build_step_batch(all_rows, self.cache.slot_of.__getitem__, length_before,
                                      self.spec.vocab_size, self.device, into=static)
             batch.kv_splits = None
-            self._prepare_for_positions(self.max_request_tokens)
             logits = self.model.forward(batch, self.cache)   # this step's result, and the warm-up
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
@@ -295,7 +296,6 @@ class Engine:
             tokens, wanted = sum(key[0]), key[1]
             static = torch.empty(packed_size(tokens, len(entries), wanted), dtype=torch.int32, device=self.device)
             batch = build_step_batch(entries, slot_of, length_before, self.spec.vocab_size, self.device, into=static)
-            self._prepare_for_positions(self.max_request_tokens)
             logits = self.model.forward(batch, self.cache)   # this step's result, and the warm-up
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
@@ -314,10 +314,3 @@ class Engine:
             logits = static_logits.clone()
         self._graphs[key] = rec    # most recently used last
         return logits
-
-    def _prepare_for_positions(self, n: int) -> None:
-        """Grow every position table to n positions now, so that no captured step has to."""
-        for block in self.model.blocks:
-            position = getattr(block.mixer, "position", None)
-            if position is not None:
-                position.ensure_positions(n)

@@ -258,9 +258,9 @@ class Scheduler:
         self.finished: dict = {}
         self._next_id = 0
         self._pending = None    # (requests, Chosen) of the step whose tokens have not been read back
-        pool_tokens = min((g.pool.num_pages for g in self.cache.groups), default=1 << 30) * self.cache.page_size
+        pool_tokens = self.cache.pool_tokens()
         context = self.cfg.max_seq_len or pool_tokens
-        context = min(context, self.cache.max_pages_per_request * self.cache.page_size)
+        context = min(context, self.cache.request_capacity)
         # infer/src/scheduler/types.rs:511-553
         self.max_request_len = min(max(context - 1, 0), max(pool_tokens - 1, 0))
         self.max_request_input_len = max(self.max_request_len - REQUEST_INPUT_SLACK_TOKENS, 0)
@@ -364,25 +364,23 @@ class Scheduler:
                 raise RuntimeError("scheduler makes no progress: a waiting request can never be admitted")
 
     # -- admission ------------------------------------------------------------------------------
-    def _pages(self, tokens: int) -> int:
-        return -(-tokens // self.cache.page_size)
-
     def _admit(self) -> None:
         if not self.waiting:
             return
-        free = min(self.cache.free_pages(), default=1 << 30)
+        pages = self.cache.pages_for_length     # per group of layers: each has pages of its own, of its own length
+        free = list(self.cache.free_pages())
         # pages that running requests still need to reach prompt + 1
         for r in self.prefilling + self.decoding:
-            target = len(r.feed) + 1
-            free -= max(0, self._pages(target) - self._pages(self.cache.length(r.id)))
+            have, target = pages(self.cache.length(r.id)), pages(len(r.feed) + 1)
+            free = [f - max(0, t - h) for f, t, h in zip(free, target, have)]
         deferred = deque()
         while self.waiting:
             req = self.waiting.popleft()
-            need = self._pages(len(req.feed) + 1)
-            if self.cache.free_slot_count == 0 or need > free:
+            need = pages(len(req.feed) + 1)
+            if self.cache.free_slot_count == 0 or any(n > f for n, f in zip(need, free)):
                 deferred.append(req)
                 continue
-            free -= need
+            free = [f - n for f, n in zip(free, need)]
             self.engine.add_request(req.id)
             req.phase = "prefilling"
             req.fed = 0

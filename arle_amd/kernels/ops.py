@@ -1035,25 +1035,30 @@ def library_k_splits(rows: int, n: int, k: int) -> int:
     return splits
 
 
+def _bmm_takes_out_dtype(device) -> bool:
+    """Whether this torch's batched product hands back float32 sums of bfloat16 operands; asked once, on a tiny
+    product, so that no failure of a real call (out of memory, say) is taken for the answer."""
+    global _BMM_OUT_DTYPE_OK
+    if _BMM_OUT_DTYPE_OK is None:
+        probe = torch.zeros((2, 16, 32), dtype=torch.bfloat16, device=device)
+        try:
+            torch.bmm(probe, probe.transpose(1, 2), out_dtype=torch.float32)
+            _BMM_OUT_DTYPE_OK = True
+        except (TypeError, RuntimeError):
+            _BMM_OUT_DTYPE_OK = False
+    return _BMM_OUT_DTYPE_OK
+
+
 def _library_mm_split_k(x, w, splits: int):
     """float32 [splits, M, N]: part s is x[:, s-th part of K] . w[:, s-th part of K]^T; None if this torch cannot
     give a batched product float32 results."""
-    global _BMM_OUT_DTYPE_OK
-    if _BMM_OUT_DTYPE_OK is False:
+    if not _bmm_takes_out_dtype(x.device):
         return None
     m, k = x.shape
     n, part = w.shape[0], k // splits
     xs = x.as_strided((splits, m, part), (part, x.stride(0), 1))
-    ws = w.as_strided((splits, part, n), (part, 1, k))
-    try:
-        out = torch.bmm(xs, ws, out_dtype=torch.float32)
-        _BMM_OUT_DTYPE_OK = True
-        return out
-    except (TypeError, RuntimeError):
-        if _BMM_OUT_DTYPE_OK:
-            raise
-        _BMM_OUT_DTYPE_OK = False
-        return None
+    ws = w.as_strided((splits, part, n), (part, 1, w.stride(0)))
+    return torch.bmm(xs, ws, out_dtype=torch.float32)
 
 
 # 17..64 rows: the kernel whose workgroups stay beats the library where the output is narrow and K long (the
@@ -1108,13 +1113,13 @@ _MM_OUT_DTYPE_OK = None
 def _library_mm_f32out(x, w):
     """bfloat16 x bfloat16 -> float32 through the library.  With a torch that takes `out_dtype` the 32-bit
     accumulators are returned as they are; an older one hands back bfloat16, which is then only widened (the
-    result has been rounded once)."""
+    result has been rounded once).  Which torch this is, is asked once on a tiny product."""
     global _MM_OUT_DTYPE_OK
     if _MM_OUT_DTYPE_OK is None:
+        probe = torch.zeros((16, 32), dtype=torch.bfloat16, device=x.device)
         try:
-            y = torch.mm(x, w.t(), out_dtype=torch.float32)
+            torch.mm(probe, probe.t(), out_dtype=torch.float32)
             _MM_OUT_DTYPE_OK = True
-            return y
         except (TypeError, RuntimeError):
             _MM_OUT_DTYPE_OK = False
     if _MM_OUT_DTYPE_OK:

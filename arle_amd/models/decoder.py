@@ -105,7 +105,15 @@ class DecoderModel:
         parts = [self.embedding, self.final_norm, self.head, *self._extra_parts]
         for b in self.blocks:
             parts += [p for p in (b.mixer, b.feed_forward) if p is not None] + list(getattr(b, "norms", {}).values())
+        self.parts = parts
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in parts)
+
+    def prepare(self, max_positions: int) -> None:
+        """Every part gets to size what it keeps per position for the longest request, before the first step."""
+        for part in self.parts:
+            prepare = getattr(part, "prepare", None)
+            if prepare is not None:
+                prepare(max_positions)
 
     def cache_needs(self):
         """(need of every schedule entry that owns a cache, {reader entry -> owner entry})."""

@@ -27,7 +27,7 @@ from dataclasses import dataclass
 
 import torch
 
-from .spec import PartSpec, WeightDecl
+from .spec import PartSpec, Rows, WeightDecl, tensor_name
 
 ROLES = ("embedding", "norm", "position", "mixer", "feed_forward", "block", "head")
 _REGISTRY: dict = {role: {} for role in ROLES}
@@ -100,6 +100,17 @@ class Part:
     def __init__(self, params: dict, tensors: dict, rt: Runtime, children: dict | None = None):
         self.params = params
         self.rt = rt
+        self.child_parts = dict(children or {})
+
+    def prepare(self, max_positions: int) -> None:
+        """Called by the engine once the longest request is known, before any step runs or is captured: whatever
+        a part keeps that grows with the position (a table of angles, slopes, a window of taps) is made for
+        `max_positions` positions here, so that no step has to allocate.  The default hands the call on to the
+        parts nested in this one."""
+        for child in getattr(self, "child_parts", {}).values():
+            prepare = getattr(child, "prepare", None)
+            if prepare is not None:
+                prepare(max_positions)
 
 
 def expected_tensors(role: str, spec: PartSpec) -> dict:
@@ -109,7 +120,17 @@ def expected_tensors(role: str, spec: PartSpec) -> dict:
     for pname, decl in cls.declare_weights(spec.params).items():
         if pname not in spec.weights:
             raise ValueError(f"{role} part {spec.kind!r}: no tensor name given for parameter {pname!r}")
-        out[spec.weights[pname]] = decl
+        source = spec.weights[pname]
+        if isinstance(source, Rows):
+            # the parameter is some rows of a larger checkpoint tensor: that tensor is what the folder must hold
+            if not decl.shape or decl.shape[0] != source.stop - source.start:
+                raise ValueError(f"{role} part {spec.kind!r}: parameter {pname!r} has {decl.shape[0] if decl.shape else 0} "
+                                 f"rows, the recipe gives it rows {source.start}:{source.stop} of '{source.tensor}'")
+            decl = WeightDecl((source.of, *decl.shape[1:]), decl.init)
+        name = tensor_name(source)
+        if name in out and tuple(out[name].shape) != tuple(decl.shape):
+            raise ValueError(f"tensor '{name}' is used with two shapes: {out[name].shape} and {decl.shape}")
+        out[name] = decl
     for _, (child_role, child_spec) in cls.children(spec.params).items():
         out.update(expected_tensors(child_role, child_spec))
     return out
@@ -118,10 +139,14 @@ def expected_tensors(role: str, spec: PartSpec) -> dict:
 def build_part(role: str, spec: PartSpec, fetch, rt: Runtime):
     """Construct a part; `fetch(tensor_name)` returns the loaded tensor."""
     cls = lookup(role, spec.kind)
-    tensors = {pname: fetch(spec.weights[pname]) for pname in cls.declare_weights(spec.params)}
+    tensors = {}
+    for pname in cls.declare_weights(spec.params):
+        source = spec.weights[pname]
+        whole = fetch(tensor_name(source))
+        tensors[pname] = whole[source.start:source.stop] if isinstance(source, Rows) else whole
     kids = {name: build_part(r, s, fetch, rt) for name, (r, s) in cls.children(spec.params).items()}
     return cls(spec.params, tensors, rt, kids)
 
 
 __all__ = ["register", "lookup", "Runtime", "Part", "expected_tensors", "build_part", "WeightDecl",
-           "PartSpec", "UnknownPart", "ROLES"]
+           "PartSpec", "Rows", "UnknownPart", "ROLES"]

@@ -61,6 +61,9 @@ class RopeNeox(Part):
         if n > self.cos.shape[0]:
             self.cos, self.sin = self._table(max(n, 2 * self.cos.shape[0]))
 
+    def prepare(self, max_positions: int) -> None:
+        self.ensure_positions(max_positions)
+
     def fused_rotary(self):
         return self.cos, self.sin, self.rotary_dim
 

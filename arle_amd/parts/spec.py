@@ -6,7 +6,7 @@ writer, the cache manager and the step function -- reads only the spec, never th
 architecture's name.
 
 * `PartSpec`  one part: its kind (a name in the registry of its role), its sizes and
-  constants, and the checkpoint tensor behind each of its parameters.
+  constants, and the checkpoint tensor (or the rows of one: `Rows`) behind each of its parameters.
 * `LayerSpec` one block: the arrangement and the mixer, feed-forward and norms in it.
   Layers need not be alike.
 * `ModelSpec.schedule` the order in which layers run, as a list.  An entry may name a
@@ -26,11 +26,31 @@ class WeightDecl:
     init: str = "normal"  # a name known to weights.random_init: "normal" N(0, std), "ones" 1 + N(0, norm_std), "zeros", ...
 
 
+@dataclass(frozen=True)
+class Rows:
+    """A parameter that is rows [start, stop) of a checkpoint tensor of `of` rows: what a recipe names in
+    `PartSpec.weights` where the checkpoint stores several projections as one matrix (q|k|v, gate|up)."""
+
+    tensor: str
+    start: int
+    stop: int
+    of: int     # rows of the whole checkpoint tensor, so that its shape is known from the recipe alone
+
+    def __post_init__(self):
+        if not 0 <= self.start < self.stop <= self.of:
+            raise ValueError(f"rows {self.start}:{self.stop} do not lie in a tensor of {self.of} rows")
+
+
+def tensor_name(source) -> str:
+    """The checkpoint tensor behind a `PartSpec.weights` value (a name, or `Rows` of a named tensor)."""
+    return source.tensor if isinstance(source, Rows) else source
+
+
 @dataclass
 class PartSpec:
     kind: str
     params: dict = field(default_factory=dict)
-    weights: dict = field(default_factory=dict)  # parameter name -> tensor name in the checkpoint
+    weights: dict = field(default_factory=dict)  # parameter name -> tensor name in the checkpoint, or Rows of one
 
 
 @dataclass

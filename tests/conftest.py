@@ -20,3 +20,18 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """With ARLE_TEST_STATS=<file>: the worst maximum and rms errors that the comparisons with the plain
+    implementation saw, one line a comparison (what the tolerances are set against)."""
+    path = os.environ.get("ARLE_TEST_STATS")
+    if not path:
+        return
+    try:
+        import replay
+    except ImportError:
+        return
+    with open(path, "w") as fh:
+        for what, (worst, rms, spread) in sorted(replay.last_stats.items()):
+            fh.write(f"{worst:.3e} {rms:.3e} {spread:5.2f} {what}\n")

@@ -65,7 +65,9 @@ def test_sharp_attention_shows_a_wrong_key_in_float32(model_b, tmp_path):
     toks = random_tokens(200, cfg["vocab_size"], 12)
     eng = Engine.from_folder(str(tmp_path / "sharp"), dtype="float32", page_size=TINY["B"][1], max_tokens=256, max_slots=2)
     got = replay.run_steps(eng, replay.portions("x", toks, sizes=(8, 9, 7, 16, 1, 24, 3)))
-    replay.compare(got, cfg2, weights2, {"x": toks}, TOL["float32"], "sharp/float32")
+    # scores sixteen times as large amplify rounding unevenly (a row with two near-equal top keys more than one
+    # with a clear winner): rows differ by up to five times the median here, where other comparisons stay under three
+    replay.compare(got, cfg2, weights2, {"x": toks}, TOL["float32"], "sharp/float32", outlier_tol=10.0)
     # the test has teeth: reading one wrong key at a page's edge moves the last logits far beyond the tolerance
     other = list(toks)
     other[TINY["B"][1] - 1] = (other[TINY["B"][1] - 1] + 1) % cfg["vocab_size"]
