@@ -67,6 +67,9 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--page-size", type=int, default=None)
     ap.add_argument("--no-cuda-graph", action="store_true",
                     help="launch every step kernel by kernel instead of replaying captured HIP graphs")
+    ap.add_argument("--warm-up", action="store_true",
+                    help="capture the decode graphs of every batch size before the first request (the reference's "
+                         "server does so when it starts; a single prompt gains nothing from it)")
     ap.add_argument("--no-weight-tiles", action="store_true",
                     help="do not keep the second, decode-friendly copy of the projection weights")
     sub = ap.add_subparsers(dest="command")
@@ -115,7 +118,7 @@ def main(argv=None) -> int:
               prefill_max_requests=args.prefill_max_requests, kv_cache_tokens=args.kv_cache_tokens,
               page_size=args.page_size, seed=args.seed, cuda_graph=not args.no_cuda_graph,
               mem_fraction_static=args.mem_fraction_static,
-              weight_tiles=False if args.no_weight_tiles else None)
+              weight_tiles=False if args.no_weight_tiles else None, warm_up=args.warm_up)
     if args.prompt_ids:
         prompt = [int(t) for t in args.prompt_ids.replace(" ", "").split(",") if t]
     else:

@@ -15,7 +15,7 @@ import os
 import torch
 
 from .. import models  # noqa: F401  (registers the architectures)
-from ..cache.manager import (CacheManager, PagedNeed, cache_bytes_per_token, pages_for_memory, slots_for_tokens,
+from ..cache.manager import (CacheManager, OutOfPages, PagedNeed, cache_bytes_per_token, pages_for_memory, slots_for_tokens,
                              state_bytes_per_slot)
 from ..config.registry import detect_architecture, load_model_config
 from ..models.decoder import DEBUG_DUMP_ENV, build_model, expected_checkpoint_tensors
@@ -33,6 +33,16 @@ DEFAULT_MEM_FRACTION_STATIC = 0.85   # infer/src/scheduler/types.rs:215
 
 class EngineError(RuntimeError):
     pass
+
+
+def decode_warmup_sizes(max_batch: int) -> list:
+    """The batch sizes whose decode graphs are captured ahead: every size up to 64, then every sixteenth from 80 on,
+    and the largest itself (infer/src/scheduler/cuda/core/warmup.rs:267-285)."""
+    sizes = list(range(1, min(64, max_batch) + 1))
+    sizes += list(range(80, max_batch + 1, 16))
+    if sizes and sizes[-1] != max_batch and max_batch > 8:
+        sizes.append(max_batch)
+    return sizes
 
 
 def _device(device=None) -> torch.device:
@@ -219,13 +229,14 @@ class Engine:
 
         The graph computes the logits of every row; the wanted ones are picked afterwards.  What
         varies from step to step (token ids, positions, slots) is copied into the graph's fixed
-        input buffer; block tables are device tensors at fixed addresses already.  The launch
-        shape of the split-KV attention is part of the graph, so a graph is keyed by the number
-        of rows and by the cap that the longest context puts on the number of splits.
+        input buffer; block tables are device tensors at fixed addresses already.  Launch shapes
+        are part of the graph, so a graph is keyed by the number of rows and by what the parts say
+        their launches depend on beside it (`Part.decode_launch_class`: the split-KV factor of the
+        attention, which follows the longest context).
         """
         rows = len(entries)
         max_kv = max(before[e.request] for e in entries) + 1
-        key = (rows, ops.decode_split_cap(max_kv))
+        key = (rows, self.model.decode_launch_class(rows, max_kv))
         all_rows = [StepEntry(e.request, e.tokens, [0]) for e in entries]
         length_before = before.__getitem__
         rec = self._graphs.pop(key, None)
@@ -256,6 +267,44 @@ class Engine:
         if wanted == list(range(rows)):
             return logits
         return logits[torch.tensor(wanted, dtype=torch.long, device=self.device)]
+
+    def warm_up(self, batch_sizes=None, max_context: int | None = None) -> int:
+        """Capture the graphs of decode steps before the first request, so that no step of serving pays for an
+        eager pass and a capture: for every batch size asked for (default: `decode_warmup_sizes` of the slots, the
+        reference's schedule) and every class of context length up to `max_context` (default: the longest request)
+        that changes a launch.  The reference does this when its scheduler starts
+        (infer/src/scheduler/cuda/core/warmup.rs:11-160).  Runs dummy requests of token 0 through `step`, which
+        leaves nothing behind but the graphs and pages that were written and given back.  Returns how many graphs
+        were captured; batch sizes and contexts that the slots or the pool cannot hold are left out."""
+        if not self.use_graphs:
+            return 0
+        sizes = sorted({int(b) for b in (batch_sizes or decode_warmup_sizes(self.cache.max_slots))
+                        if 0 < int(b) <= self.cache.free_slot_count})
+        longest = max(1, min(int(max_context or self.max_request_tokens), self.max_request_tokens))
+        contexts = sorted({1, longest} | {1 << k for k in range(1, longest.bit_length()) if (1 << k) <= longest})
+        wanted = {}
+        for rows in sizes:
+            for context in contexts:
+                wanted.setdefault((rows, self.model.decode_launch_class(rows, context)), context)
+        todo = [(key, context) for key, context in wanted.items() if key not in self._graphs]
+        self.max_graphs = max(self.max_graphs, len(self._graphs) + len(todo) + 16)
+        captured = 0
+        for (rows, _), context in todo:
+            names = [("__warm_up__", i) for i in range(rows)]
+            try:
+                for name in names:
+                    self.add_request(name)
+                if context > 1:
+                    self.cache.append([(names[0], context - 1)])    # bookkeeping only: the keys are whatever the pages hold
+                self.step([StepEntry(name, [0], [0]) for name in names])
+                captured += 1
+            except OutOfPages:
+                pass        # the pool does not hold this context beside the other rows: serving will not see it either
+            finally:
+                for name in names:
+                    if self.cache.is_live(name):
+                        self.end_request(name)
+        return captured
 
     # -- captured steps of any shape ---------------------------------------------------------------
     def _repeated_shape(self, entries, before):

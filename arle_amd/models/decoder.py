@@ -115,6 +115,17 @@ class DecoderModel:
             if prepare is not None:
                 prepare(max_positions)
 
+    def decode_launch_class(self, rows: int, max_context: int) -> tuple:
+        """What the launches of a step of `rows` single decoded tokens depend on beyond `rows`, over all parts (the
+        distinct answers of `Part.decode_launch_class`, in a fixed order)."""
+        found = set()
+        for part in self.parts:
+            ask = getattr(part, "decode_launch_class", None)
+            answer = ask(rows, max_context) if ask is not None else None
+            if answer is not None:
+                found.add(answer)
+        return tuple(sorted(found, key=repr))
+
     def cache_needs(self):
         """(need of every schedule entry that owns a cache, {reader entry -> owner entry})."""
         needs, readers = [], {}

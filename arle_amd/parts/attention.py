@@ -86,6 +86,12 @@ class PagedAttention(Part):
     def cache_need(self):
         return self.declare_cache(self.params)
 
+    def decode_launch_class(self, rows, max_context):
+        # the split-KV factor of the matrix-core kernel is the one launch dimension that follows the context
+        if self.rt.is_f32 or self.D % 16 or self.D > ops.MFMA_MAX_HEAD_DIM:
+            return None
+        return ops.decode_splits(rows, self.nkv, max_context)
+
     def forward(self, x, batch, cache):
         """x [T, H] -> [T, H], or a float32 stack [S, T, H] to be added in order (see Linear)."""
         Q, KV = self.q_width, self.kv_width

@@ -102,6 +102,13 @@ class Part:
         self.rt = rt
         self.child_parts = dict(children or {})
 
+    def decode_launch_class(self, rows: int, max_context: int):
+        """What of a step of `rows` single decoded tokens, the longest of whose contexts is `max_context` tokens,
+        the launches of this part depend on beyond `rows` (a hashable value; None: nothing).  Two such steps with
+        equal answers from every part launch the same kernels with the same arguments, so one captured graph
+        serves both."""
+        return None
+
     def prepare(self, max_positions: int) -> None:
         """Called by the engine once the longest request is known, before any step runs or is captured: whatever
         a part keeps that grows with the position (a table of angles, slopes, a window of taps) is made for

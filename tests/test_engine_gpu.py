@@ -243,3 +243,35 @@ def test_tokens_fed_from_gpu_memory_give_the_bits_of_tokens_fed_from_the_host(mo
     with pytest.raises(ValueError, match="outside its tensor"):
         eng.step([StepEntry(0, [DeviceToken(source, 2)], [0])])
     assert eng.length(0) == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_warm_up_captures_every_decode_graph_before_the_first_request(model, dtype):
+    """After `warm_up` no decode step is run eagerly or captured in mid-serving: every one is a replay, the number of
+    graphs does not change, nothing is left in the cache, and the logits are those of an engine that was not warmed
+    (infer/src/scheduler/cuda/core/warmup.rs:11-160)."""
+    from arle_amd.engine.engine import decode_warmup_sizes
+
+    assert decode_warmup_sizes(4) == [1, 2, 3, 4] and decode_warmup_sizes(100)[-4:] == [64, 80, 96, 100]
+    assert decode_warmup_sizes(9) == list(range(1, 10)) and decode_warmup_sizes(70)[-2:] == [64, 70]
+    name, d, cfg, _ = model
+    make = lambda: Engine.from_folder(d, dtype=dtype, page_size=TINY[name][1], max_tokens=3 * 320, max_slots=3,
+                                      max_request_tokens=320)
+    cold, warm = make(), make()
+    captured = warm.warm_up()
+    assert captured == len(warm._graphs) >= 3               # at least one graph a batch size
+    assert {rows for rows, _ in warm._graphs} == {1, 2, 3}
+    assert not warm.cache.slot_of and warm.cache.free_pages() == cold.cache.free_pages()
+    warm.cache.check()
+    assert warm.warm_up() == 0                              # all there already
+    reqs = {f"w{i}": random_tokens(n, cfg["vocab_size"], 300 + i) for i, n in enumerate([150, 40, 20])}
+    steps = [{"entries": [(rid, t[:-12], [len(t) - 13]) for rid, t in reqs.items()], "end": []}]
+    for i in range(12, 0, -1):    # three decoding requests, then two, then one, with contexts in several classes
+        live = [rid for k, rid in enumerate(reqs) if i > 4 * k]
+        steps.append({"entries": [(rid, reqs[rid][-i:len(reqs[rid]) - i + 1], [0]) for rid in live], "end": []})
+    graphs_before = len(warm._graphs)
+    a = replay.run_steps(cold, steps)
+    b = replay.run_steps(warm, steps)
+    assert warm.graph_replays == 12 and len(warm._graphs) == graphs_before
+    for key in a:
+        assert torch.equal(a[key], b[key]), key
