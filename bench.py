@@ -788,11 +788,19 @@ def main() -> int:
             calls = [lambda: prefill_once(("parts", 0))] * 3 + [one_step] * 5
             traced = profiled_steps(torch, calls)
             out = {"ceilings": {"hbm_read_gbs": round(read_ceiling / 1e9, 1), "mfma_tflops": round(mfma_ceiling / 1e12, 1)}}
-            us, of_peak, of_ceiling = part_report(part_times(traced[:3], args.layers), part_flops_prefill(raw, PROMPT),
-                                                  PEAK_FLOPS[dkey], mfma_ceiling)
+            times = part_times(traced[:3], args.layers)
+            flops = part_flops_prefill(raw, PROMPT)
+            head_flops = flops.pop("head")      # one row against the whole table: a stream of weights, judged by its bytes
+            us, of_peak, of_ceiling = part_report(times, flops, PEAK_FLOPS[dkey], mfma_ceiling)
+            head_bytes = raw["vocab_size"] * raw["hidden_size"] * elt
+            of_peak["head_hbm"] = round(head_bytes / (times["head"] * 1e-6) / (PEAK_HBM_GBS * 1e9), 4)
+            of_ceiling["head_hbm"] = round(head_bytes / (times["head"] * 1e-6) / read_ceiling, 4)
+            # the profiled pass is longer than the timed one (the profiler's own cost a kernel): both are given
+            us["sum"] = round(sum(v for k, v in us.items() if k != "kernels"), 1)
             out.update(prefill_parts_us=us, prefill_parts_frac_peak=of_peak, prefill_parts_frac_ceiling=of_ceiling)
             us, of_peak, of_ceiling = part_report(part_times(traced[3:], args.layers),
                                                   part_bytes_decode(raw, batch, ctx_now, elt), PEAK_HBM_GBS * 1e9, read_ceiling)
+            us["sum"] = round(sum(v for k, v in us.items() if k != "kernels"), 1)
             out.update(decode_parts_us=us, decode_parts_frac_peak=of_peak, decode_parts_frac_ceiling=of_ceiling)
             for k in keys:
                 engine.end_request(k)
@@ -837,6 +845,10 @@ def main() -> int:
     }
     if not args.no_parts and dkey == "bf16":
         line.update(parts_in_a_child_process(args))
+        # the parts come from a second, profiled run: their sums stand beside the timed steps they are read against
+        if isinstance(line.get("prefill_parts_us"), dict):
+            line["prefill_parts_us"]["timed_step"] = round(prefill["ms"] * 1e3, 1)
+            line["decode_parts_us"]["timed_step"] = round(ms_per_step * 1e3, 1)
     if args.batch != 8:
         line["metric"] = line["metric"].replace("batch 8", f"batch {args.batch}")
     print(json.dumps(line))
