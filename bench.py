@@ -513,8 +513,9 @@ def first_token(args) -> int:
 
 def sweep(args) -> int:
     """Further sizes of the Qwen3-4B shape, one JSON line each with its fraction of the roofline: decode at batch 16
-    and 32 (2,048-token prompts), at batch 128 (1,024 tokens of context), at batch 8 with 8,192 and 32,768 tokens of
-    context, prefills of 8,192, 512 and 128 tokens, and a 504-token prompt portion beside 8 decoding requests."""
+    and 32 (2,048-token prompts), at batch 128 and 256 (1,024 tokens of context), at batch 8 with 8,192, 16,384 and
+    32,768 tokens of context, at batch 64 with 16,384, prefills of 32,768, 16,384, 8,192, 512 and 128 tokens, and a
+    504-token prompt portion beside 8 decoding requests."""
     import torch
 
     from arle_amd.config import Qwen3Config
@@ -524,12 +525,13 @@ def sweep(args) -> int:
     raw = dict(QWEN3_4B, num_hidden_layers=args.layers)
     config = Qwen3Config.from_dict(raw)
     longest = 32768 + args.steps + 16     # the longest context, its warm-up and timed steps
+    most_tokens = max(8 * longest + 40 * 4096, 64 * (16384 + args.steps + 16), 256 * (1024 + args.steps + 16))
     engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype="bfloat16", page_size=PAGE,
-                                max_tokens=8 * longest + 40 * 4096, max_slots=129, max_request_tokens=longest)
+                                max_tokens=most_tokens, max_slots=257, max_request_tokens=longest)
     gen = torch.Generator().manual_seed(1234)
     rand = lambda n: torch.randint(0, config.vocab_size, (n,), generator=gen).tolist()
     from arle_amd.sampling import Sampler, SamplingParams
-    sampler, greedy_rows = Sampler(engine.device), [(SamplingParams(), 0, 0, [])] * 129
+    sampler, greedy_rows = Sampler(engine.device), [(SamplingParams(), 0, 0, [])] * 257
     base = {"n_gpus": 1, "dtype": "bf16", "higher_is_better": True, "data": "synthetic", "layers": args.layers}
 
     def fill(keys, context, portion=8192):
@@ -616,8 +618,12 @@ def sweep(args) -> int:
     for batch in (16, 32):
         decode_point(batch, 2048, args.steps)
     decode_point(128, 1024, args.steps)
-    for context in (8192, 32768):
+    decode_point(256, 1024, args.steps)
+    for context in (8192, 16384, 32768):
         decode_point(8, context, args.steps)
+    decode_point(64, 16384, min(args.steps, 16))
+    prefill_point(32768)
+    prefill_point(16384)
     prefill_point(8192)
     prefill_point(512)
     prefill_point(128)

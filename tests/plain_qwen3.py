@@ -99,7 +99,7 @@ def prepare_heads(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, cos, s
     return apply_rope(qk_norm(x, norm_weight, eps), cos, sin)
 
 
-def causal_attention(q, k, v, num_kv_heads: int, window: int | None = None) -> torch.Tensor:
+def causal_attention(q, k, v, num_kv_heads: int, window: int | None = None, rows=None) -> torch.Tensor:
     """softmax(q k^T / sqrt(D) + causal mask) v with grouped heads.
 
     q [T, nq, D], k/v [T, nkv, D]; q head j uses kv head j // (nq/nkv)
@@ -108,20 +108,23 @@ def causal_attention(q, k, v, num_kv_heads: int, window: int | None = None) -> t
     row r sees columns c <= r (crates/autograd/src/ops/attention.rs:52-92).
     `window` (keys c > r - window) is not part of Qwen3; it exists to pin the
     engine's generic attention part in tests.
+    `rows`: only these query rows are worked out (the others stay zero), against all
+    keys as before: for tests of very long sequences that look at a few rows.
     """
     T, nq, D = q.shape
     group = nq // num_kv_heads
     scale = 1.0 / math.sqrt(D)
     out = torch.zeros_like(q)
+    which = list(range(T)) if rows is None else [int(r) for r in rows]
     for h in range(nq):
         kh = h // group
-        scores = (q[:, h, :] @ k[:, kh, :].T) * scale
-        for r in range(T):
-            scores[r, r + 1:] = float("-inf")
+        scores = (q[which, h, :] @ k[:, kh, :].T) * scale
+        for i, r in enumerate(which):
+            scores[i, r + 1:] = float("-inf")
             if window is not None and r - window >= 0:
-                scores[r, : r - window + 1] = float("-inf")
+                scores[i, : r - window + 1] = float("-inf")
         probs = torch.softmax(scores, dim=-1)
-        out[:, h, :] = probs @ v[:, kh, :]
+        out[which, h, :] = probs @ v[:, kh, :]
     return out
 
 

@@ -114,3 +114,68 @@ def test_a_portion_of_9000_tokens_beside_60_decoded_tokens(tmp_path):
     reference = {"long": replay.plain_logits(cfg, weights, long_toks)}
     replay.check_rows(got, reference, TOL["bfloat16"], "a portion of 9,000 beside 60 decoded tokens", need_all=False)
     assert sum(1 for key in got if key[0] == "long") == 13
+
+
+# ---- contexts of 16 k and 32 k tokens: one layer, so that its keys and values follow from the tokens alone ----------
+
+ONE_LAYER_128 = dict(HEADS128, num_hidden_layers=1, max_position_embeddings=40960)
+
+
+def _one_layer_plain_rows(cfg, w, toks, rows):
+    """float64 logits of the chosen rows of a one-layer model: keys and values of every token (no attention is
+    needed for those in the first layer), attention and everything after it for the chosen rows only."""
+    import plain_qwen3 as plain
+
+    w = {k: t.double() for k, t in w.items()}
+    T, nq, nkv, D, eps = len(toks), cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["rms_norm_eps"]
+    p = "model.layers.0."
+    h = plain.embedding(w["model.embed_tokens.weight"], toks)
+    a = plain.rms_norm(h, w[p + "input_layernorm.weight"], eps)
+    cos, sin = plain.rope_cos_sin(list(range(T)), D, cfg["rope_theta"], dtype=torch.float64)
+    q = plain.prepare_heads(plain.linear(a, w[p + "self_attn.q_proj.weight"]).reshape(T, nq, D),
+                            w[p + "self_attn.q_norm.weight"], eps, cos, sin)
+    k = plain.prepare_heads(plain.linear(a, w[p + "self_attn.k_proj.weight"]).reshape(T, nkv, D),
+                            w[p + "self_attn.k_norm.weight"], eps, cos, sin)
+    v = plain.linear(a, w[p + "self_attn.v_proj.weight"]).reshape(T, nkv, D)
+    att = plain.causal_attention(q, k, v, nkv, rows=rows)[rows].reshape(len(rows), nq * D)
+    h = h[rows] + plain.linear(att, w[p + "self_attn.o_proj.weight"])
+    b = plain.rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)
+    h = h + plain.swiglu_mlp(b, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
+    return plain.linear(plain.rms_norm(h, w["model.norm.weight"], eps), head)
+
+
+def test_decoding_at_32k_and_16k_tokens_of_context_in_one_batch(tmp_path):
+    """Four requests that decode side by side 32,760, 16,390, 9,001 and 31 tokens into their contexts (the split-KV
+    attention at its most splits, block tables of 2,048 pages, a short request beside long ones), after prompts fed in
+    portions of 16,384.  The last rows of the long prompts' second portions (16,376 keys behind them) are looked at too."""
+    d, cfg, weights = _folder(tmp_path, "one_layer", ONE_LAYER_128, 24, 0.04)
+    lengths = {"a": 32760, "b": 16390, "c": 9001, "d": 31}
+    decoded = 6
+    reqs = {rid: random_tokens(n + decoded, ONE_LAYER_128["vocab_size"], 60 + i) for i, (rid, n) in enumerate(lengths.items())}
+    eng = Engine.from_folder(d, dtype="bfloat16", page_size=16, max_tokens=sum(lengths.values()) + 4 * 64, max_slots=4,
+                             max_request_tokens=32768 + 64)
+    looked, steps = {rid: [] for rid in reqs}, []
+    for rid, n in lengths.items():      # the prompts, one request a step, 16,384 tokens at most a portion
+        for at in range(0, n, PORTION):
+            size = min(PORTION, n - at)
+            want = list(range(max(0, size - 40), size)) if at + size == n else []
+            looked[rid] += [at + w for w in want]
+            steps.append({"entries": [(rid, reqs[rid][at:at + size], want)], "end": []})
+    for i in range(decoded):            # then all four decode together
+        steps.append({"entries": [(rid, [reqs[rid][lengths[rid] + i]], [0]) for rid in reqs], "end": []})
+        for rid in reqs:
+            looked[rid].append(lengths[rid] + i)
+    steps[-1]["end"] = list(reqs)
+    got = replay.run_steps(eng, steps)
+    for rid, toks in reqs.items():
+        rows = sorted(looked[rid])
+        ref = _one_layer_plain_rows(cfg, weights, toks, rows)
+        scale = float(ref.abs().max())
+        every = []
+        for i, pos in enumerate(rows):
+            err, rms = replay.row_errors(got[(rid, pos)], ref[i], scale)
+            every.append(rms)
+            assert err <= TOL["bfloat16"], f"request {rid} ({lengths[rid]} tokens) position {pos}: {err:.3e}"
+        assert max(every) <= 4.0 * sorted(every)[len(every) // 2], (rid, max(every), sorted(every)[len(every) // 2])
+    assert eng.cache.free_pages() == [eng.cache.groups[0].pool.num_pages]

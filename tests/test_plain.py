@@ -287,3 +287,13 @@ def test_penalties_of_the_reference():
     l = torch.tensor([2.0, -2.0, 1.0])
     out = plain.apply_penalties(l, {0: 2, 1: 1}, repetition=2.0, frequency=0.5, presence=0.25)
     assert torch.allclose(out, torch.tensor([1.0 - 1.0 - 0.25, -4.0 - 0.5 - 0.25, 1.0]))
+
+
+def test_attention_of_chosen_rows_equals_those_rows_of_the_whole():
+    torch.manual_seed(3)
+    q, k, v = torch.randn(11, 4, 8, dtype=torch.float64), torch.randn(11, 2, 8, dtype=torch.float64), torch.randn(11, 2, 8, dtype=torch.float64)
+    whole = plain.causal_attention(q, k, v, 2)
+    some = plain.causal_attention(q, k, v, 2, rows=[0, 4, 10])
+    assert torch.allclose(some[[0, 4, 10]], whole[[0, 4, 10]], rtol=0, atol=1e-14) and float(some[[1, 2, 3, 5]].abs().max()) == 0.0
+    windowed = plain.causal_attention(q, k, v, 2, window=3)
+    assert torch.allclose(plain.causal_attention(q, k, v, 2, window=3, rows=[7])[7], windowed[7], rtol=0, atol=1e-14)
