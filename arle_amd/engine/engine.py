@@ -66,7 +66,8 @@ class Engine:
                  page_size: int = DEFAULT_PAGE_SIZE, max_tokens: int | None = None,
                  num_pages: int | None = None, max_slots: int | None = 4,
                  max_request_tokens: int | None = None, cuda_graph: bool = True,
-                 weight_tiles: bool | None = None, mem_fraction_static: float = DEFAULT_MEM_FRACTION_STATIC):
+                 weight_tiles: bool | None = None, mem_fraction_static: float = DEFAULT_MEM_FRACTION_STATIC,
+                 product_table=None):
         """
         max_tokens: tokens the cache holds over all live requests (num_pages = ceil(max_tokens / page_size)
             unless num_pages is given).  With neither, the pool is sized from the GPU's memory as the
@@ -80,6 +81,9 @@ class Engine:
         max_request_tokens: longest single request (default: min(model's positions, cache capacity)).
         cuda_graph: replay steps of single decoded tokens from captured HIP graphs (the reference captures
             its decode path per batch size: infer/src/model/qwen3/batch_decode.rs:1691-1730).
+        product_table: a table (or the path of its file) that says which kernel runs each matrix product at each
+            row count, measured for this model's widths (`bench.py --tune-products`); without one, the rules that
+            were measured at the Qwen3-4B, 8B and 32B widths decide.  The table is the process's, not this engine's.
         weight_tiles: hold every bfloat16 projection weight a second time in the layout that the few-rows
             kernels stream fastest (decode steps about a tenth faster, twice the weight memory).  Default:
             yes if both copies together stay under a third of the GPU's memory.
@@ -87,6 +91,8 @@ class Engine:
         self.device = _device(device)
         self.dtype = parse_dtype(dtype)
         self.spec = spec
+        if product_table is not None:
+            ops.load_product_table(product_table)
         if weight_tiles is None:
             held = sum(t.numel() * t.element_size() for t in tensors.values() if t.dim() == 2)
             weight_tiles = 2 * held * 3 <= torch.cuda.get_device_properties(self.device).total_memory

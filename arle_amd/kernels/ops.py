@@ -8,9 +8,11 @@ live on the GPU.
 from __future__ import annotations
 
 import ctypes
+import dataclasses
 import functools
 import itertools
 import math
+import os
 
 import torch
 
@@ -930,9 +932,10 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
               tiles: torch.Tensor | None = None):
     """out[M, N] = x[M, K] . w[N, K]^T, bfloat16 operands, float32 accumulation.
 
-    Few rows (decode steps, short portions) run the hand-written weight-streaming kernel.  More rows go
+    Few rows (decode steps, short portions) run the hand-written weight-streaming kernels.  More rows go
     to the vendor library (hipBLASLt through torch.matmul), the matrix product the reference also leaves
-    to a library (crates/cuda-kernels/csrc/gemm/gemv.cu:240-330).
+    to a library (crates/cuda-kernels/csrc/gemm/gemv.cu:240-330).  Which kernel it is for a shape is decided in
+    one place, `choose_product`: by a measured table where one is loaded for these widths, else by the rules.
     partials_ok: the caller adds a float32 stack [S, M, N] itself (in the order of S) if that is what the
     kernel leaves behind; otherwise the stack is added here by one more small kernel.
     tiles: pack_weight_tiles(w), for the hand-written kernels to stream instead of w.
@@ -944,33 +947,9 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
     _need(x.shape[1] == w.shape[1], f"gemm_bf16: inner sizes differ ({x.shape[1]} vs {w.shape[1]})")
     _need(out_dtype in (torch.bfloat16, torch.float32), "gemm_bf16 writes bfloat16 or float32")
     rows, n, k = x.shape[0], w.shape[0], x.shape[1]
-    aligned = x.data_ptr() % 16 == 0
-    staying = aligned and gemm_stream_preferred(rows, n, k, x.stride(0), tiled=tiles is not None)
-    if not staying and aligned and gemm_rows_preferred(rows, n, k, x.stride(0)):
-        out = gemm_rows(x, w, out_dtype, tiles=tiles)
-        if out.dim() == 3 and not partials_ok:
-            out = sum_partials(out, out_dtype)
-        return out
-    if staying:
-        variant, splits = _stream_plan(rows, n, k, tiles is not None)
-        out = gemm_stream(x, w, out_dtype, variant=variant, splits=splits, tiles=tiles)
-        # a large stack is added here by many workgroups; the consumer would add it with one workgroup a row
-        if out.dim() == 3 and (not partials_ok or out.numel() * 4 > _STREAM_PARTIAL_BYTES):
-            out = sum_partials(out, out_dtype)
-        return out
-    if partials_ok and tiles is not None and aligned:
-        splits = narrow_tiles_splits(rows, n, k, x.stride(0))
-        if splits:
-            return gemm_tiles(x, tiles, n, torch.float32, variant=_NARROW_TILES_VARIANT, splits=splits)
-    if partials_ok:
-        splits = library_k_splits(rows, n, k)
-        if splits > 1:
-            stack = _library_mm_split_k(x, w, splits)
-            if stack is not None:
-                return stack
-    if out_dtype == torch.float32:
-        return _library_mm_f32out(x, w)
-    return torch.matmul(x, w.t())
+    choice = choose_product(rows, n, k, x.stride(0), tiled=tiles is not None, fused=False, partials_ok=partials_ok,
+                            aligned=x.data_ptr() % 16 == 0)
+    return run_product(choice, x, w, tiles, out_dtype, partials_ok)
 
 
 # The library runs a product with a narrow output and a long K (o and down: 2,560 columns) as a few dozen
@@ -1125,3 +1104,200 @@ def _library_mm_f32out(x, w):
     if _MM_OUT_DTYPE_OK:
         return torch.mm(x, w.t(), out_dtype=torch.float32)
     return torch.matmul(x, w.t()).float()
+
+
+# ------------------------------------------------------ which kernel runs a product
+#
+# One place decides.  A choice names a kernel and what it needs to be launched; `product_by_rules` holds the
+# thresholds that were measured at the Qwen3-4B, 8B and 32B widths (the constants above, each beside the numbers that
+# set it); a table measured for a model's own widths (`arle_amd.kernels.tune`, `bench.py --tune-products`) takes
+# their place where one is loaded: {(N, K, fused, tiled): [(most rows, choice), ...]}.  Another width then costs a
+# run of the tuner, not a reading of these rules.
+
+
+@dataclasses.dataclass(frozen=True)
+class ProductChoice:
+    kernel: str            # "rows", "stream", "rounds", "tiles", "tiles_parts", "library", "library_parts"
+    variant: tuple = ()    # the kernel's own variant, where it has several
+    splits: int = 0        # parts of K; 0: the kernel's own plan
+
+
+PRODUCT_KERNELS = ("rows", "stream", "rounds", "tiles", "tiles_parts", "library", "library_parts")
+_PRODUCT_TABLE: dict = {}
+
+
+def product_by_rules(rows: int, n: int, k: int, x_stride: int, *, tiled: bool, fused: bool, partials_ok: bool,
+                     aligned: bool = True) -> ProductChoice:
+    """The kernel for x[rows, k] . w[n, k]^T by the measured thresholds.  fused: gate|up with SiLU·mul (w holds
+    gate and up rows interleaved in blocks of 16), whose result is the activation [rows, n/2]."""
+    if fused:
+        if rows and aligned and gemm_rows_preferred(rows, n, k, x_stride, fused=True):
+            return ProductChoice("rows", (_fused_variant(rows),), 1)
+        if rows and aligned and tiled and gemm_rows_rounds_preferred(rows, n, k, x_stride):
+            return ProductChoice("rounds")
+        if aligned and tiled and gemm_tiles_preferred(rows, n, k, x_stride, fused=True):
+            return ProductChoice("tiles", (8, 144) if rows >= _TILES_BIG_ROWS else (4, 44))
+        return ProductChoice("library")
+    staying = aligned and gemm_stream_preferred(rows, n, k, x_stride, tiled=tiled)
+    if not staying and aligned and gemm_rows_preferred(rows, n, k, x_stride):
+        return ProductChoice("rows")
+    if staying:
+        variant, splits = _stream_plan(rows, n, k, tiled)
+        return ProductChoice("stream", (variant,), splits)
+    if partials_ok and tiled and aligned:
+        splits = narrow_tiles_splits(rows, n, k, x_stride)
+        if splits:
+            return ProductChoice("tiles_parts", _NARROW_TILES_VARIANT, splits)
+    if partials_ok:
+        splits = library_k_splits(rows, n, k)
+        if splits > 1:
+            return ProductChoice("library_parts", (), splits)
+    return ProductChoice("library")
+
+
+_CANDIDATE_STACK_BYTES = 32 << 20     # a candidate may leave a stack of partial products of at most this size
+
+
+def product_candidates(rows: int, n: int, k: int, x_stride: int, *, tiled: bool, fused: bool) -> list:
+    """Every choice that can run this shape (what a tuner times against each other): the library whole and in parts
+    of K, and the hand-written kernels in their variants with several numbers of parts."""
+    found = [ProductChoice("library")]
+    eight = k % 8 == 0 and x_stride % 8 == 0
+    few = gemm_rows_supported(rows, k, x_stride)
+    steps = -(-k // 32)
+    small = lambda parts: parts * rows * n * 4 <= _CANDIDATE_STACK_BYTES
+    if fused:
+        if few and n % 32 == 0:
+            for variant in (_V_GENERAL, _V_FUSED_FEW, _V_SHARED, 4):
+                if _rows_geometry(variant)[2] == 1 and _rows_min_splits(variant, rows, k) == 1:
+                    found.append(ProductChoice("rows", (variant,), 1))
+            if tiled:
+                found.append(ProductChoice("rounds"))
+        if tiled and eight and n % 32 == 0 and rows > ROWS_KERNEL_MAX:
+            found += [ProductChoice("tiles", v) for v in ((4, 44), (8, 144))]
+        return found
+    if few:
+        for variant in range(ROWS_VARIANTS):
+            least = _rows_min_splits(variant, rows, k)
+            for parts in (1, 2, 3, 4, 6, 8):
+                if least <= parts <= steps and small(parts):
+                    found.append(ProductChoice("rows", (variant,), parts))
+        for variant in range(STREAM_VARIANTS):
+            least = _stream_min_splits(variant, rows, k)
+            for parts in (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16):
+                if least <= parts <= steps and small(parts):
+                    found.append(ProductChoice("stream", (variant,), parts))
+    if rows > ROWS_KERNEL_MAX // 2:
+        for parts in (2, 4, 8):
+            if k % (32 * parts) == 0 and small(parts):
+                found.append(ProductChoice("library_parts", (), parts))
+            if tiled and eight and rows <= 1024 and k >= 320 * parts and small(parts):
+                found.append(ProductChoice("tiles_parts", _NARROW_TILES_VARIANT, parts))
+    return list(dict.fromkeys(found))
+
+
+def load_product_table(table) -> None:
+    """Take a measured table in: {"N,K,fused,tiled": [[most rows, kernel, variant, splits], ...]} (what the tuner
+    writes, or the path of its JSON file).  Entries are looked up by the exact widths; other widths keep the rules."""
+    import json
+
+    if isinstance(table, (str, bytes)) or hasattr(table, "__fspath__"):
+        with open(table, encoding="utf-8") as fh:
+            table = json.load(fh)
+    for key, entries in table.items():
+        if isinstance(key, str):
+            n, k, fused, tiled = key.split(",")
+            key = (int(n), int(k), fused.strip() in ("1", "True", "true"), tiled.strip() in ("1", "True", "true"))
+        parsed = []
+        for most_rows, kernel, variant, splits in entries:
+            _need(kernel in PRODUCT_KERNELS, f"a product table names the kernel {kernel!r}; known: {', '.join(PRODUCT_KERNELS)}")
+            parsed.append((int(most_rows), ProductChoice(kernel, tuple(variant), int(splits))))
+        _PRODUCT_TABLE[key] = sorted(parsed, key=lambda e: e[0])
+
+
+def clear_product_table() -> None:
+    _PRODUCT_TABLE.clear()
+
+
+def choose_product(rows: int, n: int, k: int, x_stride: int, *, tiled: bool, fused: bool, partials_ok: bool,
+                   aligned: bool = True) -> ProductChoice:
+    """The table's entry for these widths and this many rows if there is one (the tables were measured with operands
+    on the 16-byte grid: others go by the rules), else `product_by_rules`."""
+    on_grid = aligned and k % 8 == 0 and x_stride % 8 == 0
+    entries = _PRODUCT_TABLE.get((n, k, fused, tiled)) if on_grid and _PRODUCT_TABLE else None
+    if entries:
+        for most_rows, choice in entries:
+            if rows <= most_rows:
+                return choice
+    return product_by_rules(rows, n, k, x_stride, tiled=tiled, fused=fused, partials_ok=partials_ok, aligned=aligned)
+
+
+def run_product(choice: ProductChoice, x, w, tiles, out_dtype, partials_ok: bool, fused: bool = False):
+    """Launch what `choice` names.  Plain products come back as [M, N] in out_dtype, or, where the caller said
+    partials_ok, possibly as a float32 stack [S, M, N]; fused ones as the activation [M, N/2]."""
+    kernel = choice.kernel
+    if fused:
+        if kernel == "rows":
+            return gemm_rows(x, w, x.dtype, EPI_SILU_MUL, variant=choice.variant[0] if choice.variant else None,
+                             splits=1 if choice.variant else None, tiles=tiles)
+        if kernel == "rounds":
+            return gemm_rows_rounds(x, w, x.dtype, tiles=tiles)
+        if kernel == "tiles":
+            return gemm_tiles(x, tiles, w.shape[0], x.dtype, EPI_SILU_MUL, variant=choice.variant or None)
+        return silu_mul_interleaved(gemm_bf16(x, w, x.dtype, tiles=tiles), 16)
+    if kernel == "rows":
+        out = gemm_rows(x, w, out_dtype, variant=choice.variant[0] if choice.variant else None,
+                        splits=choice.splits or None, tiles=tiles)
+    elif kernel == "stream":
+        out = gemm_stream(x, w, out_dtype, variant=choice.variant[0] if choice.variant else _STREAM_VARIANT,
+                          splits=choice.splits or None, tiles=tiles)
+    elif kernel == "tiles_parts":
+        out = gemm_tiles(x, tiles, w.shape[0], torch.float32, variant=choice.variant or _NARROW_TILES_VARIANT,
+                         splits=choice.splits)
+    elif kernel == "tiles":
+        out = gemm_tiles(x, tiles, w.shape[0], out_dtype, variant=choice.variant or None)
+    elif kernel == "library_parts":
+        out = _library_mm_split_k(x, w, choice.splits)
+        if out is None:
+            out = _library_mm_f32out(x, w) if out_dtype == torch.float32 else torch.matmul(x, w.t())
+    else:
+        out = _library_mm_f32out(x, w) if out_dtype == torch.float32 else torch.matmul(x, w.t())
+    # a large stack is added here by many workgroups; the consumer would add it with one workgroup a row
+    if out.dim() == 3 and (not partials_ok or (kernel in ("rows", "stream") and out.numel() * 4 > _STREAM_PARTIAL_BYTES)):
+        out = sum_partials(out, out_dtype)
+    elif out.dim() == 2 and out.dtype != out_dtype:
+        out = out.to(out_dtype)
+    return out
+
+
+def gate_up_act(x: torch.Tensor, w: torch.Tensor, tiles: torch.Tensor | None = None) -> torch.Tensor:
+    """silu(x . gate^T) * (x . up^T) for w [2I, K] holding gate and up rows interleaved in blocks of 16: [M, I]."""
+    _gpu(x, w)
+    _rows(x, "x")
+    rows, n, k = x.shape[0], w.shape[0], x.shape[1]
+    if rows == 0:
+        return torch.empty((0, n // 2), dtype=x.dtype, device=x.device)
+    choice = choose_product(rows, n, k, x.stride(0), tiled=tiles is not None, fused=True, partials_ok=False,
+                            aligned=x.data_ptr() % 16 == 0)
+    return run_product(choice, x, w, tiles, x.dtype, False, fused=True)
+
+
+PRODUCT_TABLE_ENV = "ARLE_AMD_PRODUCT_TABLE"   # the path of a table that is taken in when this module is loaded ("none": no table at all)
+PRODUCT_TABLE_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tables")
+
+
+def load_shipped_product_tables() -> int:
+    """The tables that come with the package (measured on an MI355X for the widths of Qwen3-4B, 8B and 32B)."""
+    count = 0
+    if os.path.isdir(PRODUCT_TABLE_DIR):
+        for name in sorted(os.listdir(PRODUCT_TABLE_DIR)):
+            if name.endswith(".json"):
+                load_product_table(os.path.join(PRODUCT_TABLE_DIR, name))
+                count += 1
+    return count
+
+
+if os.environ.get(PRODUCT_TABLE_ENV, "") != "none":
+    load_shipped_product_tables()
+    if os.environ.get(PRODUCT_TABLE_ENV):
+        load_product_table(os.environ[PRODUCT_TABLE_ENV])

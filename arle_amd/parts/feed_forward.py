@@ -45,16 +45,7 @@ class SwiGLU(Part):
     def forward(self, x):
         """x [T, H] -> [T, H], or a float32 stack [S, T, H] to be added in order (see Linear)."""
         if self.block:
-            w = self.gate_up.weight
-            if x.shape[0] and ops.gemm_rows_preferred(x.shape[0], w.shape[0], x.shape[1], x.stride(0), fused=True):
-                act = ops.gemm_rows(x, w, x.dtype, ops.EPI_SILU_MUL, tiles=self.gate_up.tiles)
-            elif (x.shape[0] and self.gate_up.tiles is not None
-                  and ops.gemm_rows_rounds_preferred(x.shape[0], w.shape[0], x.shape[1], x.stride(0))):
-                act = ops.gemm_rows_rounds(x, w, x.dtype, tiles=self.gate_up.tiles)
-            elif self.gate_up.tiles is not None and ops.gemm_tiles_preferred(x.shape[0], w.shape[0], x.shape[1], x.stride(0), fused=True):
-                act = ops.gemm_tiles(x, self.gate_up.tiles, w.shape[0], x.dtype, ops.EPI_SILU_MUL)
-            else:
-                act = ops.silu_mul_interleaved(self.gate_up(x), self.block)
+            act = ops.gate_up_act(x, self.gate_up.weight, self.gate_up.tiles)   # one product with the activation, or two kernels
         else:
             gu = self.gate_up(x)
             act = ops.silu_mul(gu[:, : self.inter], gu[:, self.inter:])

@@ -511,6 +511,31 @@ def first_token(args) -> int:
     return 0
 
 
+def tune_products(args) -> int:
+    """Measure the table of `arle_amd.kernels.tune` for one model's widths and write it; one line a (product, row
+    count) to stderr, and at the end what the table gains over the rules at every row count where they differ."""
+    from arle_amd.kernels import tune
+
+    named = {"4b": (2560, 4096, 1024, 9728, 151936), "8b": (4096, 4096, 1024, 12288, 151936),
+             "32b": (5120, 8192, 1024, 25600, 151936)}
+    widths = named.get(args.tune_products) or tuple(int(v) for v in args.tune_products.split(","))
+    if len(widths) not in (4, 5):
+        print("--tune-products takes 4b, 8b, 32b or hidden,q_width,kv_width,intermediate[,vocabulary]", file=sys.stderr)
+        return 2
+
+    def say(rec):
+        print(f"[tune] {rec['product']:8s} rows {rec['rows']:5d}: rule {rec['rule'][0]:13s} {rec['rule_us']:8.1f} us   "
+              f"best {rec['best'][0]:13s} {rec['best_us']:8.1f} us", file=sys.stderr, flush=True)
+
+    table, report = tune.tune_products(tune.model_products(*widths), say=say)
+    path = args.out or f"product_table_{args.tune_products.replace(',', '_')}.json"
+    tune.write_table(path, table)
+    changed = [r for r in report if r["best"] != r["rule"]]
+    print(json.dumps({"table": path, "points": len(report), "points_where_the_table_differs": len(changed),
+                      "gain_us": {f"{r['product']}@{r['rows']}": round(r["rule_us"] - r["best_us"], 1) for r in changed}}))
+    return 0
+
+
 def sweep(args) -> int:
     """Further sizes of the Qwen3-4B shape, one JSON line each with its fraction of the roofline: decode at batch 16
     and 32 (2,048-token prompts), at batch 128 and 256 (1,024 tokens of context), at batch 8 with 8,192, 16,384 and
@@ -665,6 +690,11 @@ def main() -> int:
     ap.add_argument("--sweep", action="store_true",
                     help="further sizes of the Qwen3-4B shape (batch 16/32, 8k/32k context, 8,192-token prefill, portions "
                          "beside decoding requests), one JSON line each")
+    ap.add_argument("--tune-products", metavar="WIDTHS", default=None,
+                    help="time every kernel that can run each of a layer's four matrix products, row count by row count, "
+                         "and write the table that ARLE_AMD_PRODUCT_TABLE / ops.load_product_table reads; WIDTHS: 4b, 8b, "
+                         "32b or hidden,q_width,kv_width,intermediate[,vocabulary]")
+    ap.add_argument("--out", default=None, help="--tune-products: the table's file (default: product_table_<widths>.json)")
     ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode"],
                     help="qwen3-4b is the default run; the other two are further workloads at larger shapes")
     args = ap.parse_args()
@@ -676,6 +706,8 @@ def main() -> int:
         PROMPT = args.prompt_len
     if args.ceilings:
         return ceilings()
+    if args.tune_products:
+        return tune_products(args)
     if args.sweep:
         return sweep(args)
     if args.first_token:

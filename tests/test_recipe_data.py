@@ -86,3 +86,33 @@ def test_admission_counts_pages_group_by_group():
     for k, rid in enumerate(ids):
         assert s.finished[rid].generated == expected_output(prompt(17, k), 3)
     assert eng.cache.free_pages() == [16, 4] and not eng.cache.slot_of
+
+
+def test_a_product_table_is_parsed_and_looked_up_by_widths_and_rows():
+    """The table that says which kernel runs a matrix product (what `bench.py --tune-products` writes): keys are the
+    widths, entries are looked up by the first row count that is not smaller; the tables that come with the package
+    parse, name known kernels only and are sorted by row count."""
+    import json
+    import os
+
+    from arle_amd.kernels import ops
+
+    saved = dict(ops._PRODUCT_TABLE)
+    try:
+        ops.clear_product_table()
+        ops.load_product_table({"640,320,0,1": [[64, "stream", [1], 4], [16, "rows", [], 0]], "640,320,1,1": [[8, "rounds", [], 0]]})
+        entries = ops._PRODUCT_TABLE[(640, 320, False, True)]
+        assert [m for m, _ in entries] == [16, 64] and entries[1][1] == ops.ProductChoice("stream", (1,), 4)
+        assert (640, 320, True, True) in ops._PRODUCT_TABLE
+        with pytest.raises(ops.ShapeError):
+            ops.load_product_table({"8,8,0,0": [[4, "magic", [], 0]]})
+        ops.clear_product_table()
+        assert ops.load_shipped_product_tables() >= 1
+        for name in os.listdir(ops.PRODUCT_TABLE_DIR):
+            table = json.load(open(os.path.join(ops.PRODUCT_TABLE_DIR, name)))
+            for key, rows in table.items():
+                assert len(key.split(",")) == 4 and [r[0] for r in rows] == sorted(r[0] for r in rows)
+                assert all(r[1] in ops.PRODUCT_KERNELS for r in rows)
+    finally:
+        ops.clear_product_table()
+        ops._PRODUCT_TABLE.update(saved)
