@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import os
 import sys
 import time
 
@@ -527,8 +528,11 @@ def tune_products(args) -> int:
         print(f"[tune] {rec['product']:8s} rows {rec['rows']:5d}: rule {rec['rule'][0]:13s} {rec['rule_us']:8.1f} us   "
               f"best {rec['best'][0]:13s} {rec['best_us']:8.1f} us", file=sys.stderr, flush=True)
 
-    table, report = tune.tune_products(tune.model_products(*widths), say=say)
+    table, report = tune.tune_products(tune.model_products(*widths), tiled=not args.no_weight_tiles, say=say)
     path = args.out or f"product_table_{args.tune_products.replace(',', '_')}.json"
+    if os.path.exists(path):       # a file may hold the tables of several runs (with and without operand tiles)
+        with open(path, encoding="utf-8") as fh:
+            table = {**json.load(fh), **table}
     tune.write_table(path, table)
     changed = [r for r in report if r["best"] != r["rule"]]
     print(json.dumps({"table": path, "points": len(report), "points_where_the_table_differs": len(changed),
