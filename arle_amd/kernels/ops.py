@@ -1173,6 +1173,10 @@ def product_candidates(rows: int, n: int, k: int, x_stride: int, *, tiled: bool,
                     found.append(ProductChoice("rows", (variant,), 1))
             if tiled:
                 found.append(ProductChoice("rounds"))
+                longest = _rows_round_steps(rows, k)
+                for round_steps in (8, 13, 20, 27, 40):       # shorter rounds than the longest that fits
+                    if round_steps < longest:
+                        found.append(ProductChoice("rounds", (round_steps,)))
         if tiled and eight and n % 32 == 0 and rows > ROWS_KERNEL_MAX:
             found += [ProductChoice("tiles", v) for v in ((4, 44), (8, 144))]
         return found
@@ -1187,6 +1191,8 @@ def product_candidates(rows: int, n: int, k: int, x_stride: int, *, tiled: bool,
             for parts in (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16):
                 if least <= parts <= steps and small(parts):
                     found.append(ProductChoice("stream", (variant,), parts))
+                    if parts in (2, 4, 8):      # and with two workgroups for every compute unit
+                        found.append(ProductChoice("stream", (variant, 2 * _STREAM_TARGET_WORKGROUPS // parts), parts))
     if rows > ROWS_KERNEL_MAX // 2:
         for parts in (2, 4, 8):
             if k % (32 * parts) == 0 and small(parts):
@@ -1241,7 +1247,7 @@ def run_product(choice: ProductChoice, x, w, tiles, out_dtype, partials_ok: bool
             return gemm_rows(x, w, x.dtype, EPI_SILU_MUL, variant=choice.variant[0] if choice.variant else None,
                              splits=1 if choice.variant else None, tiles=tiles)
         if kernel == "rounds":
-            return gemm_rows_rounds(x, w, x.dtype, tiles=tiles)
+            return gemm_rows_rounds(x, w, x.dtype, tiles=tiles, round_steps=choice.variant[0] if choice.variant else None)
         if kernel == "tiles":
             return gemm_tiles(x, tiles, w.shape[0], x.dtype, EPI_SILU_MUL, variant=choice.variant or None)
         return silu_mul_interleaved(gemm_bf16(x, w, x.dtype, tiles=tiles), 16)
@@ -1250,7 +1256,8 @@ def run_product(choice: ProductChoice, x, w, tiles, out_dtype, partials_ok: bool
                         splits=choice.splits or None, tiles=tiles)
     elif kernel == "stream":
         out = gemm_stream(x, w, out_dtype, variant=choice.variant[0] if choice.variant else _STREAM_VARIANT,
-                          splits=choice.splits or None, tiles=tiles)
+                          splits=choice.splits or None, workgroups=choice.variant[1] if len(choice.variant) > 1 else None,
+                          tiles=tiles)
     elif kernel == "tiles_parts":
         out = gemm_tiles(x, tiles, w.shape[0], torch.float32, variant=choice.variant or _NARROW_TILES_VARIANT,
                          splits=choice.splits)
