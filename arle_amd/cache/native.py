@@ -32,6 +32,9 @@ _SIGNATURES = {
     "arle_group_check": (_i, [_p, ctypes.c_char_p, _i]),
     "arle_pack_step": (_i, [_i, _p, _p, _p, _p, _p, _p, _i, _p, _ll, _ip, _ip]),
     "arle_retract_victim": (_i, [_i, _ip, _ip]),
+    "arle_plan_prefill": (_i, [_i, _p, _i, _p, _ip, _i, _p, _ip, _ip, _i, _i, _i, _i, _i, _i, _i, _ip, _ip]),
+    "arle_aligned_portion": (_i, [_i, _i, _i, _i]),
+    "arle_admit": (_i, [_i, _ip, _ip, _i, _i, _ip, _ip, _i, _ip, _ip]),
 }
 
 UNKNOWN_KEY, OUT_OF_PAGES, BUFFER_TOO_SMALL, OUT_OF_RANGE, NOT_HELD, KEY_EXISTS = -1, -2, -3, -4, -5, -6

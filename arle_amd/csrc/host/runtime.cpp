@@ -322,4 +322,104 @@ int arle_retract_victim(int n, const int* generated, const int* prompt_len) {
   return best;
 }
 
+// How many of the n tokens that a prompt with `remaining` tokens could bring to a step of rows_before rows it brings:
+// a portion that is cut anyway gives up the tokens that stand over a multiple of `align` rows, if at least `align`
+// tokens stay and the prompt needs no further step for it (the products of a step run in tiles of 128 and 256 rows).
+static int aligned_portion(int n, int remaining, int rows_before, int align) {
+  if (align <= 0 || n >= remaining) return n;
+  const int over = (rows_before + n) % align;
+  const int m = n - over;
+  if (over == 0 || m < align) return n;
+  if ((remaining + m - 1) / m != (remaining + n - 1) / n) return n;
+  return m;
+}
+
+int arle_aligned_portion(int n, int remaining, int rows_before, int align) {
+  return aligned_portion(n, remaining, rows_before, align);
+}
+
+// The prompt portions of one step (infer/src/scheduler/cuda/execution.rs:265-317, budget.rs:229-264): the queue is
+// walked in order; a request brings min(remaining, chunked_prefill_size) tokens (at most the long-prefill threshold
+// beside decoding requests); one that does not fit the tokens left, the requests left or the pages is skipped whole,
+// never shrunk, and a later one may still fit.  Pages: on top of what the decoding requests are reserved
+// (decode_growth tokens each) and what the portions picked so far take, in every group.
+//   groups[n_groups]; decode_keys[n_groups][n_decode], queue_keys[n_groups][n_queue]: a request's key in each group;
+//   first_decode[j]: 1 if the request's first decoded token needs a slot when its prompt completes.
+// picked[j]: tokens of request j in this step (0: none); page_tokens[j]: tokens its pages were asked for.
+// Returns how many were picked, or kUnknownKey.
+int arle_plan_prefill(int n_groups, void* const* groups, int n_decode, const long long* decode_keys, const int* decode_growth,
+                      int n_queue, const long long* queue_keys, const int* remaining, const int* first_decode,
+                      int decode_rows, int max_num_batched_tokens, int max_prefill_tokens, int prefill_max_requests,
+                      int chunked_prefill_size, int long_prefill_token_threshold, int step_row_alignment, int* picked,
+                      int* page_tokens) {
+  std::vector<long long> reserved(n_groups > 0 ? n_groups : 0, 0);
+  for (int g = 0; g < n_groups; ++g) {
+    Group* grp = G(groups[g]);
+    for (int i = 0; i < n_decode; ++i) {
+      auto it = grp->tables.find(decode_keys[static_cast<size_t>(g) * n_decode + i]);
+      if (it == grp->tables.end()) return kUnknownKey;
+      reserved[g] += grp->pages_needed(it->second, decode_growth[i]);
+    }
+  }
+  int tokens_left = std::min(std::max(max_num_batched_tokens - decode_rows, 0), max_prefill_tokens);
+  int requests_left = prefill_max_requests >= 0 ? prefill_max_requests : n_queue;
+  int cap = chunked_prefill_size;
+  if (decode_rows > 0) cap = std::min(cap, long_prefill_token_threshold);
+  cap = std::max(cap, 1);
+  int count = 0, rows = decode_rows;
+  std::vector<int> need(n_groups > 0 ? n_groups : 0, 0);
+  for (int j = 0; j < n_queue; ++j) {
+    picked[j] = 0;
+    page_tokens[j] = 0;
+    if (remaining[j] <= 0) continue;
+    int n = std::min(remaining[j], cap);
+    if (n > tokens_left || requests_left <= 0) continue;  // skipped whole; a later, smaller one may still fit
+    n = aligned_portion(n, remaining[j], rows, step_row_alignment);
+    const int asked = n + ((n == remaining[j] && first_decode[j]) ? 1 : 0);
+    bool fits = true;
+    for (int g = 0; g < n_groups && fits; ++g) {
+      Group* grp = G(groups[g]);
+      auto it = grp->tables.find(queue_keys[static_cast<size_t>(g) * n_queue + j]);
+      if (it == grp->tables.end()) return kUnknownKey;
+      need[g] = grp->pages_needed(it->second, asked);
+      fits = reserved[g] + need[g] <= static_cast<long long>(grp->pool.free_.size());
+    }
+    if (!fits) continue;
+    for (int g = 0; g < n_groups; ++g) reserved[g] += need[g];
+    picked[j] = n;
+    page_tokens[j] = asked;
+    tokens_left -= n;
+    requests_left -= 1;
+    rows += n;
+    count += 1;
+  }
+  return count;
+}
+
+// Which waiting requests are admitted (infer/src/scheduler/cuda/runtime/scheduler_loop.rs:202-315, budget.rs:17-33):
+// a request needs a free slot and, in every group, pages for its prompt and one token more, after the pages that the
+// running requests still need to reach theirs are set aside; one that does not fit waits, later ones may still go in.
+//   page_size[g], free_pages[g]; running_length[i] (tokens cached), running_target[i], waiting_target[j] (tokens).
+// admit[j]: 1 or 0.  Returns how many are admitted.
+int arle_admit(int n_groups, const int* page_size, const int* free_pages, int free_slots, int n_running,
+               const int* running_length, const int* running_target, int n_waiting, const int* waiting_target, int* admit) {
+  std::vector<long long> left(n_groups > 0 ? n_groups : 0, 0);
+  auto pages = [&](int g, int tokens) { return (static_cast<long long>(tokens) + page_size[g] - 1) / page_size[g]; };
+  for (int g = 0; g < n_groups; ++g) {
+    left[g] = free_pages[g];
+    for (int i = 0; i < n_running; ++i) left[g] -= std::max(0LL, pages(g, running_target[i]) - pages(g, running_length[i]));
+  }
+  int count = 0;
+  for (int j = 0; j < n_waiting; ++j) {
+    bool fits = free_slots > 0;
+    for (int g = 0; g < n_groups && fits; ++g) fits = pages(g, waiting_target[j]) <= left[g];
+    admit[j] = fits ? 1 : 0;
+    if (!fits) continue;
+    for (int g = 0; g < n_groups; ++g) left[g] -= pages(g, waiting_target[j]);
+    free_slots -= 1;
+    count += 1;
+  }
+  return count;
+}
+
 }  // extern "C"

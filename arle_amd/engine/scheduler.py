@@ -200,46 +200,60 @@ def aligned_portion(n: int, remaining: int, rows_before: int, align: int) -> int
     are 520 rows and cost a tenth more than 512 (measured on MI355X, Qwen3-4B shape: 9.8 against 8.7 ms).  So a
     portion that is cut anyway gives up the few tokens that stand over a multiple of `align` rows, if at least
     `align` tokens stay and the prompt does not need one more step for it (a 2,048-token prompt in portions of 512
-    stays at four steps)."""
-    if align <= 0 or n >= remaining:
-        return n
-    over = (rows_before + n) % align
-    m = n - over
-    if over == 0 or m < align or -(-remaining // m) != -(-remaining // n):
-        return n
-    return m
+    stays at four steps).  Worked out by the native runtime core."""
+    return int(native.lib().arle_aligned_portion(int(n), int(remaining), int(rows_before), int(align)))
 
 
-def plan_prefill(queue, decode_rows: int, cfg: SchedulerConfig, fits) -> list:
-    """Pick portions of queued prompts for this step: [(request, tokens)].
+def plan_prefill(queue, decode_rows: int, cfg: SchedulerConfig, cache=None, growth=(), asked: list | None = None) -> list:
+    """Pick portions of queued prompts for this step: [(request, tokens)], by the native runtime core
+    (`arle_plan_prefill` in csrc/host/runtime.cpp, which also counts the pages in every group of the cache).
 
-    queue: prefilling requests in queue order.  fits(reserved, request, page_tokens) says whether
-    the pool can take `page_tokens` more tokens of `request` on top of `reserved`, the
-    [(request, page_tokens)] of the portions picked before it.
+    queue: prefilling requests in queue order.  cache: the CacheManager whose pools have to take the portions
+    (None: pages are not looked at); growth: [(request id, tokens)] that the decoding requests are reserved before
+    any portion.  asked: a list that receives (request, tokens its pages were asked for) of the picked ones: a
+    portion that completes its prompt asks for one token more, the first decoded one.
     """
-    tokens_left = min(max(cfg.max_num_batched_tokens - decode_rows, 0), cfg.max_prefill_tokens)
-    requests_left = cfg.prefill_max_requests if cfg.prefill_max_requests is not None else len(queue)
-    cap = cfg.chunked_prefill_size
-    if decode_rows > 0:
-        cap = min(cap, cfg.long_prefill_token_threshold)
-    picked, reserved = [], []
-    for req in queue:
-        remaining = req.remaining_prompt
-        if remaining <= 0:
-            continue
-        n = min(remaining, max(cap, 1))
-        if n > tokens_left or requests_left <= 0:
-            continue  # skipped whole, never shrunk; a later, smaller one may still fit
-        n = aligned_portion(n, remaining, decode_rows + sum(m for _, m in picked), cfg.step_row_alignment)
-        completes = n == remaining
-        first_decode = 1 if completes and req.max_tokens - len(req.generated) > 0 else 0
-        if not fits(reserved, req, n + first_decode):
-            continue
-        picked.append((req, n))
-        reserved.append((req, n + first_decode))
-        tokens_left -= n
-        requests_left -= 1
-    return picked
+    n_queue = len(queue)
+    if n_queue == 0:
+        return []
+    groups = list(cache.groups) if cache is not None else []
+    n_groups, n_decode = len(groups), len(growth)
+    handles = (ctypes.c_void_p * max(n_groups, 1))(*[g._h for g in groups])
+    decode_keys = (ctypes.c_longlong * max(n_groups * n_decode, 1))(*[g._ids[key] for g in groups for key, _ in growth])
+    decode_growth = (ctypes.c_int * max(n_decode, 1))(*[int(n) for _, n in growth])
+    queue_keys = (ctypes.c_longlong * max(n_groups * n_queue, 1))(*[g._ids[r.id] for g in groups for r in queue])
+    remaining = (ctypes.c_int * n_queue)(*[int(r.remaining_prompt) for r in queue])
+    first = (ctypes.c_int * n_queue)(*[1 if r.max_tokens - len(r.generated) > 0 else 0 for r in queue])
+    picked, page_tokens = (ctypes.c_int * n_queue)(), (ctypes.c_int * n_queue)()
+    count = native.lib().arle_plan_prefill(
+        n_groups, handles, n_decode, decode_keys, decode_growth, n_queue, queue_keys, remaining, first, int(decode_rows),
+        int(cfg.max_num_batched_tokens), int(cfg.max_prefill_tokens),
+        -1 if cfg.prefill_max_requests is None else int(cfg.prefill_max_requests), int(cfg.chunked_prefill_size),
+        int(cfg.long_prefill_token_threshold), int(cfg.step_row_alignment), picked, page_tokens)
+    if count < 0:
+        raise KeyError("a request of the plan has no block table in the cache")
+    out = [(r, picked[j]) for j, r in enumerate(queue) if picked[j] > 0]
+    if asked is not None:
+        asked.extend((r, page_tokens[j]) for j, r in enumerate(queue) if picked[j] > 0)
+    return out
+
+
+def admit_waiting(cache, free_slots: int, running, waiting) -> list:
+    """Which of the waiting requests enter now (a list of booleans, in queue order), by the native runtime core
+    (`arle_admit`): a free slot and, in every group, pages for prompt + 1 after the same target of every running
+    request is set aside.  running: [(tokens cached, target tokens)]; waiting: [target tokens]."""
+    if not waiting:
+        return []
+    groups = list(cache.groups)
+    n_groups = len(groups)
+    sizes = (ctypes.c_int * max(n_groups, 1))(*[g.page_size for g in groups])
+    free = (ctypes.c_int * max(n_groups, 1))(*cache.free_pages())
+    lengths = (ctypes.c_int * max(len(running), 1))(*[int(have) for have, _ in running])
+    targets = (ctypes.c_int * max(len(running), 1))(*[int(target) for _, target in running])
+    wanted = (ctypes.c_int * len(waiting))(*[int(t) for t in waiting])
+    admit = (ctypes.c_int * len(waiting))()
+    native.lib().arle_admit(n_groups, sizes, free, int(free_slots), len(running), lengths, targets, len(waiting), wanted, admit)
+    return [bool(a) for a in admit]
 
 
 class Scheduler:
@@ -367,20 +381,14 @@ class Scheduler:
     def _admit(self) -> None:
         if not self.waiting:
             return
-        pages = self.cache.pages_for_length     # per group of layers: each has pages of its own, of its own length
-        free = list(self.cache.free_pages())
-        # pages that running requests still need to reach prompt + 1
-        for r in self.prefilling + self.decoding:
-            have, target = pages(self.cache.length(r.id)), pages(len(r.feed) + 1)
-            free = [f - max(0, t - h) for f, t, h in zip(free, target, have)]
+        running = [(self.cache.length(r.id), len(r.feed) + 1) for r in self.prefilling + self.decoding]
+        waiting = list(self.waiting)
+        enters = admit_waiting(self.cache, self.cache.free_slot_count, running, [len(r.feed) + 1 for r in waiting])
         deferred = deque()
-        while self.waiting:
-            req = self.waiting.popleft()
-            need = pages(len(req.feed) + 1)
-            if self.cache.free_slot_count == 0 or any(n > f for n, f in zip(need, free)):
+        for req, goes_in in zip(waiting, enters):
+            if not goes_in:
                 deferred.append(req)
                 continue
-            free = [f - n for f, n in zip(free, need)]
             self.engine.add_request(req.id)
             req.phase = "prefilling"
             req.fed = 0
@@ -402,10 +410,7 @@ class Scheduler:
                   for r in decode]
         growth = [(k, n) for k, n in growth if n > 0]
 
-        def fits(reserved, req, page_tokens):
-            return self.cache.can_append(growth + [(r.id, n) for r, n in reserved] + [(req.id, page_tokens)])
-
-        prefill = plan_prefill(self.prefilling, len(decode), self.cfg, fits)
+        prefill = plan_prefill(self.prefilling, len(decode), self.cfg, self.cache, growth)
         if not decode and not prefill and self.prefilling:
             # nothing is decoding and no portion fits beside the reservations: the pool is
             # simply too small for the queue's head portion; try it alone against the free pages

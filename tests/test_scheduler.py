@@ -132,24 +132,24 @@ def _req(i, remaining, generated=0, max_tokens=16, prompt_len=None):
 def test_a_portion_that_does_not_fit_is_skipped_whole_not_shrunk():
     cfg = SchedulerConfig(max_num_batched_tokens=100, max_prefill_tokens=10, chunked_prefill_size=8)
     queue = [_req(0, 8), _req(1, 5), _req(2, 2), _req(3, 1)]
-    picked = plan_prefill(queue, 0, cfg, lambda reserved, r, n: True)
+    picked = plan_prefill(queue, 0, cfg)
     # 8 fits (2 left); 5 does not and is skipped; 2 fits exactly; nothing left for the last
     assert [(r.id, n) for r, n in picked] == [(0, 8), (2, 2)]
     # FCFS among equals: queue order is the only priority
-    picked = plan_prefill([_req(5, 4), _req(4, 4), _req(6, 4)], 0, cfg, lambda reserved, r, n: True)
+    picked = plan_prefill([_req(5, 4), _req(4, 4), _req(6, 4)], 0, cfg)
     assert [r.id for r, _ in picked] == [5, 4]
     # decode rows shrink the budget first, and cap portions by the long-prefill threshold
     cfg = SchedulerConfig(max_num_batched_tokens=10, max_prefill_tokens=10, chunked_prefill_size=8,
                           long_prefill_token_threshold=3)
-    picked = plan_prefill([_req(0, 8), _req(1, 8)], 4, cfg, lambda reserved, r, n: True)
+    picked = plan_prefill([_req(0, 8), _req(1, 8)], 4, cfg)
     assert [(r.id, n) for r, n in picked] == [(0, 3), (1, 3)]
     # prefill_max_requests
     cfg = SchedulerConfig(prefill_max_requests=1)
-    assert len(plan_prefill([_req(0, 8), _req(1, 8)], 0, cfg, lambda reserved, r, n: True)) == 1
+    assert len(plan_prefill([_req(0, 8), _req(1, 8)], 0, cfg)) == 1
     # pages: the finishing portion asks for one token more (the first decoded token)
     asked = []
-    plan_prefill([_req(0, 8), _req(1, 600)], 0, SchedulerConfig(), lambda res, r, n: asked.append((r.id, n)) or True)
-    assert asked == [(0, 9), (1, 504)]     # the cut portion stops where the step has 8 + 504 = 512 rows
+    plan_prefill([_req(0, 8), _req(1, 600)], 0, SchedulerConfig(), asked=asked)
+    assert [(r.id, n) for r, n in asked] == [(0, 9), (1, 504)]     # the cut portion stops where the step has 8 + 504 = 512 rows
 
 
 def test_retract_victim_is_least_progress_then_longest_prompt():
@@ -477,22 +477,21 @@ def test_abort_while_a_step_is_pending():
 def test_a_cut_portion_gives_up_the_tokens_that_stand_over_a_multiple_of_128_rows():
     cfg = SchedulerConfig(num_slots=16, chunked_prefill_size=512, long_prefill_token_threshold=512)
     long_one = Request(0, prompt(2000), SamplingParams(), 8, 0, feed=prompt(2000))
-    fits = lambda reserved, req, n: True
-    assert plan_prefill([long_one], 8, cfg, fits) == [(long_one, 504)]          # 8 + 504 = 512 rows
-    assert plan_prefill([long_one], 0, cfg, fits) == [(long_one, 512)]
-    assert plan_prefill([long_one], 130, cfg, fits) == [(long_one, 510)]        # 130 + 510 = 640
+    assert plan_prefill([long_one], 8, cfg) == [(long_one, 504)]          # 8 + 504 = 512 rows
+    assert plan_prefill([long_one], 0, cfg) == [(long_one, 512)]
+    assert plan_prefill([long_one], 130, cfg) == [(long_one, 510)]        # 130 + 510 = 640
     short = Request(1, prompt(300), SamplingParams(), 8, 0, feed=prompt(300))
-    assert plan_prefill([short], 8, cfg, fits) == [(short, 300)]                # the end of a prompt is never cut
+    assert plan_prefill([short], 8, cfg) == [(short, 300)]                # the end of a prompt is never cut
     # 460 tokens would make 768 rows, but the prompt would then need five steps instead of four
-    assert plan_prefill([short, long_one], 8, cfg, fits) == [(short, 300), (long_one, 512)]
+    assert plan_prefill([short, long_one], 8, cfg) == [(short, 300), (long_one, 512)]
     even = Request(2, prompt(2048), SamplingParams(), 8, 0, feed=prompt(2048))
-    assert plan_prefill([even], 32, cfg, fits) == [(even, 512)]                # 480 would add a fifth step
+    assert plan_prefill([even], 32, cfg) == [(even, 512)]                # 480 would add a fifth step
     longer = Request(3, prompt(3600), SamplingParams(), 8, 0, feed=prompt(3600))
-    assert plan_prefill([short, longer], 8, cfg, fits) == [(short, 300), (longer, 460)]     # 768 rows; eight steps either way
+    assert plan_prefill([short, longer], 8, cfg) == [(short, 300), (longer, 460)]     # 768 rows; eight steps either way
     small = SchedulerConfig(num_slots=16, chunked_prefill_size=200, long_prefill_token_threshold=200)
-    assert plan_prefill([long_one], 8, small, fits) == [(long_one, 200)]        # fewer than 128 tokens would stay
+    assert plan_prefill([long_one], 8, small) == [(long_one, 200)]        # fewer than 128 tokens would stay
     off = SchedulerConfig(num_slots=16, chunked_prefill_size=512, long_prefill_token_threshold=512, step_row_alignment=0)
-    assert plan_prefill([long_one], 8, off, fits) == [(long_one, 512)]
+    assert plan_prefill([long_one], 8, off) == [(long_one, 512)]
 
 
 @pytest.mark.parametrize("seed", range(12))
@@ -642,3 +641,29 @@ def test_a_stream_that_is_left_early_gives_everything_back():
     eng.step = real_step
     outs = llm.generate([prompt(5, 5)], max_tokens=3)
     assert outs[0].response_token_ids == expected_output(prompt(5, 5), 3)
+
+
+def test_the_native_planner_counts_pages_in_every_group_beside_the_decoders_reservations():
+    """`plan_prefill` with a cache: a portion is skipped whole when one group cannot take its pages on top of what the
+    decoding requests are reserved and what the portions before it took; a later, smaller one still goes in."""
+    cache = CacheManager([PagedNeed(1, 16), PagedNeed(1, 16, page_size=8)], page_size=4, num_pages=16, max_slots=5,
+                         max_request_tokens=64)       # 64 tokens in either group: 16 pages of 4, 8 pages of 8
+    reqs = [Request(i, prompt(n), SamplingParams(), 8, 0, feed=prompt(n)) for i, n in enumerate([20, 30, 6, 3])]
+    for r in reqs:
+        cache.admit(r.id)
+    decoder = Request(9, prompt(5), SamplingParams(), 40, 0, feed=prompt(5), generated=[1])
+    cache.admit(decoder.id)
+    cache.append([(decoder.id, 5)])                    # holds 2 pages of 4 and 1 page of 8
+    cfg = SchedulerConfig(num_slots=5, step_row_alignment=0)
+    asked = []
+    picked = plan_prefill(reqs, 1, cfg, cache, growth=[(decoder.id, 11)], asked=asked)
+    # the decoder's 11 more tokens: 2 pages of 4, 1 page of 8.  Left: 12 and 6.  20 + 1 tokens take 6 and 3 (left 6 and
+    # 3); 30 + 1 would take 8 and 4: skipped whole; 6 + 1 take 2 and 1; 3 + 1 take 1 and 1
+    assert [(r.id, n) for r, n in picked] == [(0, 20), (2, 6), (3, 3)]
+    assert [(r.id, n) for r, n in asked] == [(0, 21), (2, 7), (3, 4)]
+    assert cache.can_append([(decoder.id, 11), (0, 21), (2, 7), (3, 4)]) and not cache.can_append([(decoder.id, 11), (0, 21), (1, 31)])
+    # without the reservation the long one fits too (14 and 7 pages free: 6 + 8 and 3 + 4), and nothing is left for the short ones
+    picked = plan_prefill(reqs, 1, cfg, cache)
+    assert [(r.id, n) for r, n in picked] == [(0, 20), (1, 30)]
+    with pytest.raises(KeyError):
+        plan_prefill([Request(77, prompt(4), SamplingParams(), 8, 0, feed=prompt(4))], 0, cfg, cache)
