@@ -70,6 +70,9 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--warm-up", action="store_true",
                     help="capture the decode graphs of every batch size before the first request (the reference's "
                          "server does so when it starts; a single prompt gains nothing from it)")
+    ap.add_argument("--tune-products", metavar="FILE", default=None,
+                    help="measure which kernel runs each matrix product of this model fastest, go by that and write the "
+                         "table to FILE (read again with ARLE_AMD_PRODUCT_TABLE=FILE); about a minute")
     ap.add_argument("--no-weight-tiles", action="store_true",
                     help="do not keep the second, decode-friendly copy of the projection weights")
     sub = ap.add_subparsers(dest="command")
@@ -118,7 +121,8 @@ def main(argv=None) -> int:
               prefill_max_requests=args.prefill_max_requests, kv_cache_tokens=args.kv_cache_tokens,
               page_size=args.page_size, seed=args.seed, cuda_graph=not args.no_cuda_graph,
               mem_fraction_static=args.mem_fraction_static,
-              weight_tiles=False if args.no_weight_tiles else None, warm_up=args.warm_up)
+              weight_tiles=False if args.no_weight_tiles else None, warm_up=args.warm_up,
+              tune_products=args.tune_products or False)
     if args.prompt_ids:
         prompt = [int(t) for t in args.prompt_ids.replace(" ", "").split(",") if t]
     else:

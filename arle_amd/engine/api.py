@@ -86,7 +86,7 @@ class LLM:
                  chunked_prefill_size: int | None = None, max_num_batched_tokens: int = 16384,
                  max_prefill_tokens: int | None = None, prefill_max_requests: int | None = None, seed: int = 42,
                  cuda_graph: bool = True, weight_tiles: bool | None = None, mem_fraction_static: float = 0.85,
-                 async_overlap: bool = True, warm_up: bool = False):
+                 async_overlap: bool = True, warm_up: bool = False, tune_products: bool | str = False):
         """model: a model folder, or an Engine that is already built.
 
         kv_cache_tokens: tokens the paged cache holds over all live requests.  Default: sized from the GPU's
@@ -103,6 +103,10 @@ class LLM:
         cuda_graph, weight_tiles: as for Engine (captured steps; the decode-friendly second copy of the weights).
         async_overlap: decode steps are launched from the last step's tokens on the GPU, and those are read back
         while the new step runs (SchedulerConfig.async_overlap); the tokens are the same either way.
+        tune_products: measure which kernel runs each of this model's matrix products fastest at each row count and
+        go by that (Engine.tune_products; up to a minute and a half); a string: also write the table there, for
+        `Engine(product_table=...)` or ARLE_AMD_PRODUCT_TABLE next time.  The widths of Qwen3-4B, 8B and 32B have
+        tables that come with the package.
         warm_up: capture the decode graphs of every batch size up to num_slots now (Engine.warm_up), as the
         reference's scheduler does when it starts; otherwise each is captured at its first step.
         """
@@ -130,6 +134,8 @@ class LLM:
                                                          max_prefill_tokens)
         self.sched_config.validate()
         self.sampler = Sampler(self.engine.device)
+        if tune_products:
+            self.engine.tune_products(path=tune_products if isinstance(tune_products, str) else None)
         if warm_up:
             self.engine.warm_up()
         self.tokenizer = self._load_tokenizer()

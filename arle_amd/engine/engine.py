@@ -312,6 +312,28 @@ class Engine:
                         self.end_request(name)
         return captured
 
+    def tune_products(self, rows=None, path: str | None = None, say=None) -> dict:
+        """Measure, for the widths of this model, which kernel runs each of its matrix products fastest at each row
+        count (`arle_amd.kernels.tune`), take the table in and, with `path`, write it there for the next start
+        (`product_table=path`).  The reference tunes its library products when its scheduler starts
+        (infer/src/scheduler/cuda/core/warmup.rs:100-131).  Half a minute to a minute and a half for a model of a
+        few billion parameters; captured steps are dropped, since they hold the old choices."""
+        from ..kernels import tune
+
+        found = {}
+        for part in self.model.parts:
+            for name, n, k, fused, consumer in (part.products() if hasattr(part, "products") else []):
+                found.setdefault((n, k, fused), (name, n, k, fused, consumer))
+        products = [p + ((tune.HEAD_ROWS,) if p[0] == "head" else ()) for p in found.values()]
+        table, _ = tune.tune_products(products, device=self.device, tiled=self.rt.weight_tiles, say=say, rows=rows)
+        ops.load_product_table(table)
+        if path:
+            tune.write_table(path, table)
+        self._graphs.clear()
+        self._shapes_seen.clear()
+        self._graph_pool = None
+        return table
+
     # -- captured steps of any shape ---------------------------------------------------------------
     def _repeated_shape(self, entries, before):
         """Key of this step's launch shape if a step of the same shape has been seen before, else None.

@@ -60,11 +60,15 @@ MIN_GAIN = 0.08     # a choice other than the rules' has to win by this much of 
 MIN_GAIN_US = 1.5   # (products timed alone gain a microsecond here and there that whole steps do not show)
 
 
-def tune_products(products, device="cuda:0", tiled: bool = True, iters: int = 20, say=None) -> tuple:
+def tune_products(products, device="cuda:0", tiled: bool = True, iters: int = 20, say=None, rows=None) -> tuple:
     """(table, report): table as `ops.load_product_table` reads it; report: one record a (product, row count) with
-    the microseconds of every candidate, of the rules' choice and of the best."""
+    the microseconds of every candidate, of the rules' choice and of the best.  products: (name, N, K, with the
+    activation, consumer[, row counts]); rows: the row counts for all of them (default: each product's own, else
+    ROWS)."""
     table, report = {}, []
-    for name, n, k, fused, consumer, rows in products:
+    only = rows
+    for name, n, k, fused, consumer, *own_rows in products:
+        rows = only if only is not None else (own_rows[0] if own_rows else ROWS)
         copies = max(2, -(-COLD_BYTES // (n * k * 2)))
         weights = [torch.randn(n, k, device=device).mul_(0.02).to(torch.bfloat16) for _ in range(copies)]
         tiles = [ops.pack_weight_tiles(w) for w in weights] if tiled else [None] * copies

@@ -86,6 +86,12 @@ class PagedAttention(Part):
     def cache_need(self):
         return self.declare_cache(self.params)
 
+    def products(self):
+        if self.qkv.weight.dtype != torch.bfloat16:
+            return []
+        return [("qkv", self.qkv.out_features, self.qkv.in_features, False, "norm"),
+                ("o", self.o.out_features, self.o.in_features, False, "norm")]
+
     def decode_launch_class(self, rows, max_context):
         # the split-KV factor of the matrix-core kernel is the one launch dimension that follows the context
         if self.rt.is_f32 or self.D % 16 or self.D > ops.MFMA_MAX_HEAD_DIM:

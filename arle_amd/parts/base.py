@@ -102,6 +102,12 @@ class Part:
         self.rt = rt
         self.child_parts = dict(children or {})
 
+    def products(self) -> list:
+        """The bfloat16 matrix products this part runs, for a tuner that measures which kernel runs each fastest:
+        [(name, N, K, with the gate|up activation, "norm" if the result goes into a residual add and norm or a
+        kernel that adds a stack of partial products itself, else None)]."""
+        return []
+
     def decode_launch_class(self, rows: int, max_context: int):
         """What of a step of `rows` single decoded tokens, the longest of whose contexts is `max_context` tokens,
         the launches of this part depend on beyond `rows` (a hashable value; None: nothing).  Two such steps with

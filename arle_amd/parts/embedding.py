@@ -44,5 +44,10 @@ class LinearHead(Part):
         super().__init__(params, tensors, rt, children)
         self.proj = Linear(tensors["weight"], rt.weight_tiles)
 
+    def products(self):
+        if self.proj.weight.dtype != torch.bfloat16:
+            return []
+        return [("head", self.proj.out_features, self.proj.in_features, False, None)]
+
     def forward(self, x):
         return self.proj(x, out_dtype=torch.float32)

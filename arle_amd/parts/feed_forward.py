@@ -42,6 +42,12 @@ class SwiGLU(Part):
         self.gate_up = Linear(fused.contiguous(), rt.weight_tiles)
         self.down = Linear(tensors["down"], rt.weight_tiles)
 
+    def products(self):
+        if self.gate_up.weight.dtype != torch.bfloat16:
+            return []
+        return [("gate_up", self.gate_up.out_features, self.gate_up.in_features, bool(self.block), None),
+                ("down", self.down.out_features, self.down.in_features, False, "norm")]
+
     def forward(self, x):
         """x [T, H] -> [T, H], or a float32 stack [S, T, H] to be added in order (see Linear)."""
         if self.block:

@@ -89,3 +89,36 @@ def test_a_loaded_table_decides_for_its_widths_and_the_rules_for_all_others(tmp_
     finally:
         ops.clear_product_table()
         ops._PRODUCT_TABLE.update(saved)
+
+
+def test_an_engine_tunes_the_products_of_its_own_widths(tmp_path):
+    """`Engine.tune_products` asks the model's parts for their products, measures them at the row counts given and
+    takes the table in; the engine stays right with whatever the table chose, and a second engine reads the file."""
+    import replay
+    from arle_amd.engine import Engine
+    from tiny import TINY, make_model_dir, random_tokens, read_folder
+
+    saved = dict(ops._PRODUCT_TABLE)
+    try:
+        d = make_model_dir(tmp_path, "D")
+        cfg, weights = read_folder(d)
+        eng = Engine.from_folder(d, dtype="bfloat16", page_size=TINY["D"][1], max_tokens=4 * 128, max_slots=4)
+        path = str(tmp_path / "table.json")
+        table = eng.tune_products(rows=(1, 20, 100), path=path)
+        h, q, kv, inter, vocab = cfg["hidden_size"], 8 * 64, 2 * 64, cfg["intermediate_size"], cfg["vocab_size"]
+        tiled = int(eng.rt.weight_tiles)
+        assert set(table) == {f"{q + 2 * kv},{h},0,{tiled}", f"{h},{q},0,{tiled}", f"{2 * inter},{h},{int(inter % 16 == 0)},{tiled}",
+                              f"{h},{inter},0,{tiled}", f"{vocab},{h},0,{tiled}"}
+        assert all(rows[-1][0] == 100 for rows in table.values())
+        assert (h, inter, False, bool(tiled)) in ops._PRODUCT_TABLE
+        reqs = {f"r{i}": random_tokens(n, cfg["vocab_size"], 70 + i) for i, n in enumerate([40, 90, 23])}
+        got = replay.run_steps(eng, replay.mixed(reqs, max_live=3, seed=5))
+        replay.compare(got, cfg, weights, reqs, 2e-2, "tuned engine/bfloat16")
+        ops.clear_product_table()
+        other = Engine.from_folder(d, dtype="bfloat16", page_size=TINY["D"][1], max_tokens=4 * 128, max_slots=4, product_table=path)
+        assert (h, inter, False, bool(tiled)) in ops._PRODUCT_TABLE
+        got = replay.run_steps(other, replay.whole("w", reqs["r1"]))
+        replay.compare(got, cfg, weights, {"w": reqs["r1"]}, 2e-2, "engine with a table from a file/bfloat16")
+    finally:
+        ops.clear_product_table()
+        ops._PRODUCT_TABLE.update(saved)
