@@ -667,3 +667,125 @@ def test_the_native_planner_counts_pages_in_every_group_beside_the_decoders_rese
     assert [(r.id, n) for r, n in picked] == [(0, 20), (1, 30)]
     with pytest.raises(KeyError):
         plan_prefill([Request(77, prompt(4), SamplingParams(), 8, 0, feed=prompt(4))], 0, cfg, cache)
+
+
+def _oracle_aligned(n, remaining, rows_before, align):
+    """The rule of `aligned_portion` stated once more: a cut portion stops at the last multiple of `align` rows if at
+    least `align` of its tokens stay and the prompt, in portions that short, needs no step more than in portions of n."""
+    if align <= 0 or n >= remaining:
+        return n
+    over = (rows_before + n) % align
+    shorter = n - over
+    if over == 0 or shorter < align:
+        return n
+    steps = lambda portion: -(-remaining // portion)
+    return shorter if steps(shorter) <= steps(n) else n
+
+
+def _oracle_plan(queue, decode_rows, cfg, page_sizes, free, held, growth):
+    """The planner's rule written out in Python for lists of numbers: held[g][id] pages that a request holds in group
+    g with length[id] tokens; returns [(id, tokens, tokens its pages are asked for)]."""
+    pages = lambda g, tokens: -(-tokens // page_sizes[g])
+    reserved = [sum(max(0, pages(g, length + n) - held[g][rid]) for rid, length, n in growth) for g in range(len(page_sizes))]
+    tokens_left = min(max(cfg.max_num_batched_tokens - decode_rows, 0), cfg.max_prefill_tokens)
+    requests_left = len(queue) if cfg.prefill_max_requests is None else cfg.prefill_max_requests
+    cap = max(1, min(cfg.chunked_prefill_size, cfg.long_prefill_token_threshold) if decode_rows > 0 else cfg.chunked_prefill_size)
+    rows, out = decode_rows, []
+    for rid, length, remaining, first in queue:
+        n = min(remaining, cap)
+        if remaining <= 0 or n > tokens_left or requests_left <= 0:
+            continue
+        n = _oracle_aligned(n, remaining, rows, cfg.step_row_alignment)
+        asked = n + (1 if n == remaining and first else 0)
+        need = [max(0, pages(g, length + asked) - held[g][rid]) for g in range(len(page_sizes))]
+        if any(reserved[g] + need[g] > free[g] for g in range(len(page_sizes))):
+            continue
+        reserved = [a + b for a, b in zip(reserved, need)]
+        out.append((rid, n, asked))
+        tokens_left, requests_left, rows = tokens_left - n, requests_left - 1, rows + n
+    return out
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_the_native_planner_and_admission_against_the_rules_written_out(seed):
+    """Random queues, budgets, page lengths and pools: what `arle_plan_prefill`, `arle_aligned_portion` and
+    `arle_admit` decide is what the rules say (scheduler/cuda/execution.rs:200-330, budget.rs:17-33 of the reference
+    for the budget and the pages; the alignment is this engine's own), and a plan never asks for more than the step's
+    budget or the pools hold."""
+    import random
+
+    from arle_amd.engine.scheduler import admit_waiting, aligned_portion
+
+    rng = random.Random(1000 + seed)
+    for _ in range(40):
+        n, remaining = rng.randint(1, 700), rng.randint(1, 3000)
+        n = min(n, remaining)
+        rows, align = rng.randint(0, 300), rng.choice([0, 16, 64, 128])
+        assert aligned_portion(n, remaining, rows, align) == _oracle_aligned(n, remaining, rows, align), (n, remaining, rows, align)
+    for _ in range(25):
+        page_sizes = [rng.choice([4, 8, 16]) for _ in range(rng.randint(1, 2))]
+        base = min(page_sizes)
+        num_pages = rng.randint(6, 40)
+        needs = [PagedNeed(1, 16, page_size=p) for p in page_sizes]
+        cache = CacheManager(needs, page_size=base, num_pages=num_pages, max_slots=12, max_request_tokens=base * num_pages)
+        page_sizes = [g.page_size for g in cache.groups]   # needs of one kind share a group
+        # requests in the middle of their prompts, and decoders
+        held = [dict() for _ in page_sizes]
+        reqs = []
+        for rid in range(rng.randint(1, 6)):
+            total = rng.randint(1, 60)
+            done = rng.randint(0, total - 1) if rng.random() < 0.5 else 0
+            r = Request(rid, prompt(total), SamplingParams(), rng.choice([0, 1, 8]), 0, feed=prompt(total))
+            cache.admit(rid)
+            try:
+                if done:
+                    cache.append([(rid, done)])
+            except OutOfPages:
+                done = 0
+            r.fed = done
+            reqs.append(r)
+        decoders = []
+        for rid in range(100, 100 + rng.randint(0, 3)):
+            have = rng.randint(1, 20)
+            cache.admit(rid)
+            try:
+                cache.append([(rid, have)])
+            except OutOfPages:
+                cache.release(rid)
+                continue
+            decoders.append((rid, have, rng.randint(1, 4)))
+        free = cache.free_pages()
+        for g, p in enumerate(page_sizes):
+            for r in reqs:
+                held[g][r.id] = -(-r.fed // p)
+            for rid, have, _ in decoders:
+                held[g][rid] = -(-have // p)
+        cfg = SchedulerConfig(num_slots=12, max_num_batched_tokens=rng.choice([16, 40, 100]), max_prefill_tokens=rng.choice([16, 64, 100]),
+                              chunked_prefill_size=rng.choice([8, 16, 48]), long_prefill_token_threshold=rng.choice([8, 16, 48]),
+                              prefill_max_requests=rng.choice([None, 1, 2, 5]), step_row_alignment=rng.choice([0, 8, 16]))
+        decode_rows = len(decoders)
+        asked = []
+        picked = plan_prefill(reqs, decode_rows, cfg, cache, growth=[(rid, n) for rid, _, n in decoders], asked=asked)
+        want = _oracle_plan([(r.id, r.fed, r.remaining_prompt, r.max_tokens - len(r.generated) > 0) for r in reqs], decode_rows, cfg,
+                            page_sizes, free, held, decoders)
+        assert [(r.id, n) for r, n in picked] == [(rid, n) for rid, n, _ in want], (seed, cfg)
+        assert [(r.id, n) for r, n in asked] == [(rid, a) for rid, _, a in want]
+        assert sum(n for _, n in picked) + decode_rows <= max(cfg.max_num_batched_tokens, decode_rows)
+        # what the plan asks for is what the cache can take in one go (the decoders' growth with it)
+        grow = [(rid, n) for rid, _, n in decoders]
+        if cache.can_append(grow):
+            assert cache.can_append(grow + [(r.id, a) for r, a in asked])
+        # admission: slots and pages for every target after the running requests' own
+        running = [(r.fed, len(r.prompt) + 1) for r in reqs] + [(have, have + 6) for _, have, _ in decoders]
+        waiting = [rng.randint(2, 80) for _ in range(rng.randint(1, 5))]
+        slots = rng.randint(0, 3)
+        got = admit_waiting(cache, slots, running, waiting)
+        left = [free[g] - sum(max(0, -(-t // p) - -(-h // p)) for h, t in running) for g, p in enumerate(page_sizes)]
+        expect = []
+        for t in waiting:
+            ok = slots > 0 and all(-(-t // p) <= left[g] for g, p in enumerate(page_sizes))
+            expect.append(ok)
+            if ok:
+                slots -= 1
+                left = [left[g] - -(-t // p) for g, p in enumerate(page_sizes)]
+        assert got == expect, (seed, waiting, running)
