@@ -419,14 +419,16 @@ constexpr int kPfKeys = 64;             // keys of a tile
 constexpr int kPfVPad = 4;              // padding of a value row in LDS: 34 dwords a row, so that the 16 rows which
                                         // 16 lanes read or write together (8 bytes each) fall into 16 different bank pairs
 
-// Work is handed out at run time.  A causal prompt is a triangle: the last 128 rows of a segment see 32 times
-// the keys of the first 128, and a fixed assignment of row blocks to workgroups leaves most of the chip idle
-// while the heaviest ones finish.  So the launch has one workgroup per CU and every workgroup takes the next
-// item (row block, kv head, segment), heaviest row blocks first, from a counter until none is left.  The counter
-// is a device variable of this module, put to zero by the planning kernel and again by the last workgroup that
-// leaves a launch: launches of this kernel on one device must not overlap (they never do on one stream).
+// Work is handed out by the item (row block, kv head, segment, part of the keys).  A causal prompt is a triangle:
+// the last 128 rows of a segment see 32 times the keys of the first 128, and row blocks assigned to workgroups by
+// their number alone leave most of the chip idle while the heaviest ones finish.  So the launch has one or two
+// workgroups per CU and the items are listed from the heaviest to the lightest.  Either every workgroup takes the
+// next item from a counter until none is left (the counter is a device variable of this module, put to zero by the
+// planning kernel and again by the last workgroup that leaves a launch), or, in the kernel that loads tiles straight
+// into LDS, the list is dealt out to and fro over the workgroups before the launch (its launcher says when).
+// Launches of these kernels on one device must not overlap (they never do on one stream).
 //
-// The planning kernel (one workgroup) also lists the live (row block, segment) pairs in that order: a step
+// The planning kernel (one workgroup) lists the live (row block, segment) pairs in that order: a step
 // that mixes a few portions with many decoded tokens has far more pairs that are dead (segments left to the
 // other kernel, row blocks past a short segment's end) than live ones, and asking for an item only to drop it
 // costs a round trip to the counter each time.  Steps with more pairs than the list holds go without it.
@@ -441,46 +443,75 @@ __global__ __launch_bounds__(256) void attn_prefill_plan_kernel(const int* __res
                                                                  const int* __restrict__ seg_start,
                                                                  const int* __restrict__ seg_slot, int segments,
                                                                  int blocks_x, int G, int min_rows, int listed) {
-  __shared__ unsigned int wave_count[4];
-  __shared__ unsigned int base;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // The list is ordered by what an entry costs, the tiles of 64 keys that its rows see, heaviest first (a counting
+  // sort over that number; entries of one cost in the order their atomics land, which no result depends on):
+  // whether the entries are taken from a counter or dealt out to and fro, the heavy ones start first and the
+  // light ones fill up.
+  constexpr int kBuckets = 2048;  // tiles of 64 keys; longer contexts share the last one
+  __shared__ unsigned int bucket[kBuckets];
+  __shared__ unsigned int sums[256];
+  const int tid = threadIdx.x;
   if (tid == 0) {
-    base = 0u;
     g_prefill_next_item = 0u;
     g_prefill_left = 0u;
   }
   if (!listed) return;  // the whole workgroup
+  for (int b = tid; b < kBuckets; b += 256) bucket[b] = 0u;
   __syncthreads();
   const int total = blocks_x * segments;
-  for (int i0 = 0; i0 < total; i0 += 256) {
-    const int i = i0 + tid;
-    bool live = false;
-    unsigned int entry = 0u;
-    int4 of_seg = {0, 0, 0, 0};
-    if (i < total) {
-      const int seg = i % segments, rb = blocks_x - 1 - i / segments;  // the last rows see the most keys: first
-      const int row0 = seg_row0[seg], qlen = seg_row0[seg + 1] - row0;
-      const int rows = qlen * G;
-      live = rows >= min_rows && rb * kPfRows < rows;
-      entry = (static_cast<unsigned int>(rb) << 16) | static_cast<unsigned int>(seg);
-      // what a workgroup needs to know of the segment, beside the entry: one load instead of a chain of them
-      if (live) of_seg = int4{row0, qlen, seg_start[seg], seg_slot[seg]};
-    }
-    const unsigned long long votes = __ballot(live);
-    const unsigned int before = __popcll(votes & ((1ull << lane) - 1ull));
-    if (lane == 0) wave_count[wave] = __popcll(votes);
-    __syncthreads();
-    unsigned int offset = base;
-    for (int w = 0; w < wave; ++w) offset += wave_count[w];
-    if (live) {
-      g_prefill_plan[offset + before] = entry;
-      g_prefill_seg[offset + before] = of_seg;
-    }
-    __syncthreads();
-    if (tid == 0) base += wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
-    __syncthreads();
+  auto look = [&](int i, unsigned int& entry, int4& of_seg, int& cost) {
+    const int seg = i % segments, rb = blocks_x - 1 - i / segments;
+    const int row0 = seg_row0[seg], qlen = seg_row0[seg + 1] - row0;
+    const int rows = qlen * G;
+    if (rows < min_rows || rb * kPfRows >= rows) return false;
+    entry = (static_cast<unsigned int>(rb) << 16) | static_cast<unsigned int>(seg);
+    // what a workgroup needs to know of the segment, beside the entry: one load instead of a chain of them
+    const int start = seg_start[seg];
+    of_seg = int4{row0, qlen, start, seg_slot[seg]};
+    const int tok_max = (min((rb + 1) * kPfRows, rows) - 1) / G;
+    cost = min((start + tok_max + 1 + 63) / 64, kBuckets - 1);
+    return true;
+  };
+  for (int i = tid; i < total; i += 256) {
+    unsigned int entry;
+    int4 of_seg;
+    int cost;
+    if (look(i, entry, of_seg, cost)) atomicAdd(&bucket[kBuckets - 1 - cost], 1u);   // heaviest first
   }
-  if (tid == 0) g_prefill_pairs = base;
+  __syncthreads();
+  // where each bucket begins: a thread adds up its eight buckets, thread 0 the 256 sums
+  constexpr int kMine = kBuckets / 256;
+  unsigned int mine = 0u;
+  for (int e = 0; e < kMine; ++e) mine += bucket[tid * kMine + e];
+  sums[tid] = mine;
+  __syncthreads();
+  if (tid == 0) {
+    unsigned int run = 0u;
+    for (int t = 0; t < 256; ++t) {
+      const unsigned int n = sums[t];
+      sums[t] = run;
+      run += n;
+    }
+    g_prefill_pairs = run;
+  }
+  __syncthreads();
+  unsigned int at = sums[tid];
+  for (int e = 0; e < kMine; ++e) {
+    const unsigned int n = bucket[tid * kMine + e];
+    bucket[tid * kMine + e] = at;
+    at += n;
+  }
+  __syncthreads();
+  for (int i = tid; i < total; i += 256) {
+    unsigned int entry;
+    int4 of_seg;
+    int cost;
+    if (look(i, entry, of_seg, cost)) {
+      const unsigned int place = atomicAdd(&bucket[kBuckets - 1 - cost], 1u);
+      g_prefill_plan[place] = entry;
+      g_prefill_seg[place] = of_seg;
+    }
+  }
 }
 
 // One workgroup a CU: two waves on every SIMD, each with the registers it wants (16 rows a wave keep the
@@ -938,7 +969,7 @@ __device__ __forceinline__ void load_to_lds_16(const void* base_uniform, uint32_
 // tiles of keys, and the launch lasts as long as the heaviest).
 template <bool WHOLE, int GROUPS>
 __global__ __launch_bounds__(GROUPS* kDmWaves* kWave, GROUPS == 1 ? 2 : 1) void attn_prefill_dma_kernel(
-    const AttnArgs a, int min_rows, int blocks_x, int segments, int listed, int pair_up) {
+    const AttnArgs a, int min_rows, int blocks_x, int segments, int listed, int pair_up, int fixed_rounds) {
   constexpr int D = kDmD;
   extern __shared__ __align__(16) unsigned char lds_all[];
   __shared__ unsigned int item_of_workgroup;
@@ -953,19 +984,43 @@ __global__ __launch_bounds__(GROUPS* kDmWaves* kWave, GROUPS == 1 ? 2 : 1) void 
   const unsigned int items = pairs * nkv * parts;
   const int P = a.P, ps = a.p_shift, pm = P - 1;
   const uint32_t page_elems32 = static_cast<uint32_t>(a.nkv) * P * D;  // the launcher refuses pages of 2^31 elements
+ // With few items a workgroup (up to fixed_rounds) the items are dealt out before the launch instead of taken from
+ // the counter: workgroup b takes item b of the first round of gridDim.x items, item gridDim.x - 1 - b of the
+ // second, and so on to and fro, so that on a list that runs from heavy to light every workgroup gets about the
+ // same, and an item begins without the counter's round trip to memory; its list entry was asked for while the
+ // item before it ran.
+ const bool dealt = fixed_rounds > 0 && listed && items <= static_cast<unsigned long long>(fixed_rounds) * gridDim.x;
+ unsigned int round = 0u;
+ unsigned int ahead_entry = 0u;
+ int4 ahead_seg = {0, 0, 0, 0};
+ auto dealt_item = [&](unsigned int r) {
+   return r * gridDim.x + ((r & 1u) ? gridDim.x - 1u - blockIdx.x : blockIdx.x);
+ };
+ if (dealt && blockIdx.x < items) {
+   ahead_entry = g_prefill_plan[blockIdx.x / (nkv * parts)];
+   ahead_seg = g_prefill_seg[blockIdx.x / (nkv * parts)];
+ }
  for (;;) {
-  if (tid == 0) item_of_workgroup = atomicAdd(&g_prefill_next_item, 1u);
-  __syncthreads();
-  const unsigned int item = item_of_workgroup;
-  __syncthreads();
-  if (item >= items) {
-    // The last workgroup to leave puts the counters back to zero: the layers of a step hand out the same list one
-    // after the other, and only the first of them runs the planning kernel.
-    if (tid == 0 && atomicAdd(&g_prefill_left, 1u) == gridDim.x - 1) {
-      g_prefill_next_item = 0u;
-      g_prefill_left = 0u;
+  unsigned int item;
+  if (dealt) {
+    // two groups: group 0 reads the other's sums from LDS at the end of an item, where its next tiles will land
+    if (GROUPS == 2 && round > 0u) __syncthreads();
+    item = dealt_item(round);
+    if (item >= items) return;  // every later round lies behind this one
+  } else {
+    if (tid == 0) item_of_workgroup = atomicAdd(&g_prefill_next_item, 1u);
+    __syncthreads();
+    item = item_of_workgroup;
+    __syncthreads();
+    if (item >= items) {
+      // The last workgroup to leave puts the counters back to zero: the layers of a step hand out the same list one
+      // after the other, and only the first of them runs the planning kernel.
+      if (tid == 0 && atomicAdd(&g_prefill_left, 1u) == gridDim.x - 1) {
+        g_prefill_next_item = 0u;
+        g_prefill_left = 0u;
+      }
+      return;
     }
-    return;
   }
   unsigned int pair = item / (nkv * parts);
   const int kvh = static_cast<int>((item / parts) % nkv);
@@ -974,13 +1029,23 @@ __global__ __launch_bounds__(GROUPS* kDmWaves* kWave, GROUPS == 1 ? 2 : 1) void 
   // half of the first round of workgroups lands beside the first half: so the first pair_up pairs are handed
   // out as they are, the next pair_up from the light end, and then the middle, which gives every CU a heavy
   // and a light item to start with instead of two heavy ones here and two light ones there.
-  if (pair_up > 0 && pairs >= 2u * pair_up) {
+  if (!dealt && pair_up > 0 && pairs >= 2u * pair_up) {
     const unsigned int h = static_cast<unsigned int>(pair_up);
     if (pair >= h) pair = pair < 2u * h ? pairs - 1u - (pair - h) : pair - h;
   }
   int seg = static_cast<int>(pair % segments), wg_row = (blocks_x - 1 - static_cast<int>(pair / segments)) * kPfRows;
   int row0, qlen, start, slot;
-  if (listed) {  // the entry and what the list holds of its segment: two loads side by side
+  if (dealt) {
+    seg = static_cast<int>(ahead_entry & 0xffffu);
+    wg_row = static_cast<int>(ahead_entry >> 16) * kPfRows;
+    row0 = ahead_seg.x, qlen = ahead_seg.y, start = ahead_seg.z, slot = ahead_seg.w;
+    ++round;
+    const unsigned int next = dealt_item(round);
+    if (next < items) {
+      ahead_entry = g_prefill_plan[next / (nkv * parts)];
+      ahead_seg = g_prefill_seg[next / (nkv * parts)];
+    }
+  } else if (listed) {  // the entry and what the list holds of its segment: two loads side by side
     const unsigned int entry = g_prefill_plan[pair];
     const int4 of_seg = g_prefill_seg[pair];
     seg = static_cast<int>(entry & 0xffffu);
@@ -1484,11 +1549,13 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
 }
 
 static int g_prefill_pair_up = 1;
+static int g_prefill_fixed_rounds = -1;  // items a workgroup up to which they are dealt out before the launch (0: never; -1: by the rule below)
+constexpr int kDealtMaxKeys = 4096;      // contexts up to which every launch deals its items out
 
 static int g_prefill_groups = -1;  // -1: the launcher decides; 1, 2: forced (measurements and tests)
 
 template <int GROUPS>
-int launch_prefill_dma_groups(const AttnArgs& a, dim3 grid, int min_rows, int cus, hipStream_t s) {
+int launch_prefill_dma_groups(const AttnArgs& a, dim3 grid, int min_rows, int cus, int max_kv_len, hipStream_t s) {
   const size_t lds = GROUPS * 2 * kDmStageBytes;
   static bool asked = false;  // dynamic LDS of 64 KiB and more has to be asked for, once
   if (!asked) {
@@ -1511,12 +1578,19 @@ int launch_prefill_dma_groups(const AttnArgs& a, dim3 grid, int min_rows, int cu
     attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, a.seg_start, a.seg_slot, static_cast<int>(grid.z),
                                                static_cast<int>(grid.x), a.nq / a.nkv, min_rows, listed);
   const int pair_up = GROUPS == 1 && g_prefill_pair_up ? static_cast<int>(cus / (static_cast<long long>(a.nkv) * a.portion_splits)) : 0;
+  // Items are dealt out before the launch (see the kernel) when none is long, or when a workgroup gets two at most;
+  // with long items, several a workgroup, taking them from the counter follows the compute units' differing speeds
+  // and the counter's round trip is little beside an item.  Measured on MI355X, dealt against taken, us: a fresh
+  // prompt of 2,048 tokens 56.5 against 65.0, of 1,024 30.7 against 34.9, 504 tokens beside 8 decoded ones 32.9
+  // against 42.4, four prompts of 2,048 179 against 190, 512 tokens behind 3,584 cached 62.9 against 71.9, segments
+  // of 64 to 800 tokens behind 0 to 2,300 372 against 387; a fresh prompt of 8,192 tokens 615 against 598.
+  const int fixed_rounds = g_prefill_fixed_rounds >= 0 ? g_prefill_fixed_rounds : (max_kv_len <= kDealtMaxKeys ? 1 << 20 : 2);
   if (a.P % kDmKeys == 0)
     attn_prefill_dma_kernel<true, GROUPS><<<workgroups, GROUPS * kDmWaves * kWave, lds, s>>>(
-        a, min_rows, static_cast<int>(grid.x), static_cast<int>(grid.z), listed, pair_up);
+        a, min_rows, static_cast<int>(grid.x), static_cast<int>(grid.z), listed, pair_up, fixed_rounds);
   else
     attn_prefill_dma_kernel<false, GROUPS><<<workgroups, GROUPS * kDmWaves * kWave, lds, s>>>(
-        a, min_rows, static_cast<int>(grid.x), static_cast<int>(grid.z), listed, pair_up);
+        a, min_rows, static_cast<int>(grid.x), static_cast<int>(grid.z), listed, pair_up, fixed_rounds);
   if (a.portion_splits > 1) {
     const long long most = static_cast<long long>(grid.x) * grid.y * grid.z * (kPfRows / kPfWaves);
     attn_merge_portions_kernel<<<static_cast<unsigned>(most < 4LL * cus ? most : 4LL * cus), kPfWaves * kWave, 0, s>>>(a);
@@ -1545,7 +1619,8 @@ int launch_prefill_dma(const AttnArgs& a, dim3 grid, int min_rows, int max_qlen,
   const bool unequal = 2LL * max_qlen > max_kv_len;  // the first rows see less than half of what the last see
   const bool two = g_prefill_groups >= 0 ? g_prefill_groups == 2
                                          : (4 * items > cus && (2 * items <= 3LL * cus || (unequal && items <= 2LL * cus)));
-  return two ? launch_prefill_dma_groups<2>(a, grid, min_rows, cus, s) : launch_prefill_dma_groups<1>(a, grid, min_rows, cus, s);
+  return two ? launch_prefill_dma_groups<2>(a, grid, min_rows, cus, max_kv_len, s)
+             : launch_prefill_dma_groups<1>(a, grid, min_rows, cus, max_kv_len, s);
 }
 
 // -1: the launcher decides (below); 1: head_dim 128 portions always run attn_prefill_dma_kernel; 0: always
@@ -1609,6 +1684,7 @@ SideBranch* side_branch(hipStream_t s) {
 
 extern "C" void arle_attn_prefill_variant(int dma) { g_prefill_dma = dma; }
 extern "C" void arle_attn_prefill_pair_up(int on) { g_prefill_pair_up = on; }
+extern "C" void arle_attn_prefill_fixed_rounds(int rounds) { g_prefill_fixed_rounds = rounds; }
 extern "C" void arle_attn_prefill_groups(int groups) { g_prefill_groups = groups; }
 
 // Token rows that the split-KV workspace holds for every segment: the most tokens of a segment whose rows

@@ -41,6 +41,7 @@ SIGNATURES = {
                                                 _i, _i, _i, _i, _f, _i, _p]),
     "arle_attn_prefill_variant": ("attention_mfma", [_i]),
     "arle_attn_prefill_pair_up": ("attention_mfma", [_i]),
+    "arle_attn_prefill_fixed_rounds": ("attention_mfma", [_i]),
     "arle_attn_prefill_groups": ("attention_mfma", [_i]),
     "arle_attn_side_branch": ("attention_mfma", [_i]),
     "arle_attn_paged_mfma": ("attention_mfma", [_p, _ll, _p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i,

@@ -649,6 +649,56 @@ def test_attention_portions_list_their_work_once_for_calls_that_name_the_same_st
         lib.function("arle_attn_prefill_variant")(-1)
 
 
+@pytest.mark.parametrize("groups,heads", [(1, 24), (2, 12)])
+@pytest.mark.parametrize("parts", [None, 2])
+def test_attention_portions_dealt_out_before_the_launch_or_taken_from_the_counter(groups, heads, parts):
+    """The kernel that loads tiles straight into LDS gets its (row block, kv head, part) items either from a counter
+    at run time or dealt out to and fro over the workgroups before the launch; the list of both is ordered by the
+    keys an entry sees.  Segments of very different lengths and contexts, more items than workgroups (so that a
+    workgroup gets a second and third item), one or two groups of waves: the same bits either way, and the plain
+    result at rows of every segment."""
+    from arle_amd.kernels import lib
+    nq = nkv = heads
+    D, P, dt = 128, 16, torch.bfloat16
+    segs = [(100, 512), (0, 2048), (40, 1), (1500, 256), (700, 128)]
+    lengths = [a + b for a, b in segs]
+    table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, 410)
+    qs, row0, starts, checks = [], [0], [], []
+    for s_, (cached, n) in enumerate(segs):
+        g = _g(411 + s_)
+        q, k, v = (torch.randn(cached + n, h, D, generator=g).to(dt) for h in (nq, nkv, nkv))
+        _fill_cache(table, k_pages, v_pages, s_, k, v, P)
+        rows = sorted({cached, cached + n // 2, cached + n - 1})
+        want = plain.causal_attention(q.double(), k.double(), v.double(), nkv, rows=rows)
+        checks += [(row0[-1] + r - cached, want[r].reshape(-1)) for r in rows]
+        qs.append(q[cached:].reshape(n, -1))
+        row0.append(row0[-1] + n)
+        starts.append(cached)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    q_all = torch.cat(qs).to(DEV)
+    args = (k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0), i32(list(range(len(segs)))), i32(starts))
+    kw = dict(max_qlen=2048, min_qlen=1, max_kv_len=max(lengths), num_q_heads=nq, num_kv_heads=nkv, head_dim=D,
+              page_size=P, scale=1.0 / math.sqrt(D), portion_splits=parts)
+    lib.function("arle_attn_prefill_variant")(1)
+    lib.function("arle_attn_prefill_groups")(groups)
+    outs = {}
+    try:
+        for rounds in (0, 64, -1, 2):   # never dealt; always; by the launcher's rule; up to two items a workgroup
+            lib.function("arle_attn_prefill_fixed_rounds")(rounds)
+            out = torch.full_like(q_all, float("nan"))
+            ops.attn_paged_mfma(q_all, out, *args, **kw)
+            outs[rounds] = out.cpu()
+    finally:
+        lib.function("arle_attn_prefill_variant")(-1)
+        lib.function("arle_attn_prefill_groups")(-1)
+        lib.function("arle_attn_prefill_fixed_rounds")(-1)
+    for rounds, out in outs.items():
+        assert torch.isfinite(out.float()).all()
+        assert torch.equal(out, outs[0]), rounds
+    for row, want in checks:
+        assert _rel(outs[0][row].float(), want) < 8e-3
+
+
 @pytest.mark.parametrize("P", [16, 64, 128])
 def test_attention_mfma_dma_kernel_masks_stale_slots(P):
     """The kernel that loads tiles straight into LDS: pages hold NaN bits in every slot that was never written
