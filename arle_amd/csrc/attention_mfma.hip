@@ -66,6 +66,20 @@ struct AttnArgs {
   float* pws_ml;       // [token row][q head][part][2]
   int rows_max;  // the streaming kernel skips segments with more rows than this (0: takes all)
   long long plan_token;  // names the step for the portions kernels' list of work (0: no name, plan every time)
+  // The kernel that prepares q, k and v itself (PREP; steps of single decoded tokens): the fused q|k|v projection
+  // comes as a stack of float32 partial products [prep_n][token rows][(nq + 2 nkv) D], q is unused.
+  const float* prep_parts;
+  int prep_n;
+  int64_t prep_part_stride, prep_row_stride;  // elements between the parts, and between the rows of a part
+  const void* prep_qw;   // per-head norm weights [D] of q and k (null: no norm), float32 if prep_w_f32 else bfloat16
+  const void* prep_kw;
+  int prep_w_f32;
+  const float* prep_cos;  // [positions][prep_rot / 2]
+  const float* prep_sin;
+  int prep_rot;           // rotated width: 0, or a multiple of 64 up to D
+  float prep_eps;
+  uint16_t* prep_k_pages;  // the pages again, to write the new token's key and value into
+  uint16_t* prep_v_pages;
 };
 
 __device__ __forceinline__ bf16x8 load_bf16x8(const uint16_t* p) {
@@ -88,8 +102,17 @@ __device__ __forceinline__ float group_sum4(float v) {
 
 // EXACT: head_dim == DMAX, known at compile time, so every "is this chunk inside the head" test and
 // every multiplication by head_dim folds away; otherwise head_dim is any multiple of 16 up to DMAX.
-template <int NT, int DMAX, bool EXACT>
+//
+// PREP (steps of single decoded tokens, NT == 1, EXACT): the kernel that prepared q, k and v for this one is folded
+// into it.  Every wave adds up its q heads from the stack of partial products of the q|k|v projection, norms and
+// rotates them (a lane holds d = 32 c + 8 g .. + 7 of its row, c = 0 .. D / 32 - 1: the rotation partner, rot / 2
+// away, is in the same lane when rot is a multiple of 64, and the four lanes of a row add their squares together).
+// The one wave of a (segment, kv head) whose keys end with the new token's does the same for its k head, takes the
+// v head as it is, writes both into the cache and puts them where the loads of the last block would have brought
+// them (the slot in the page still holds what was there before).  A layer of a decode step is one kernel shorter.
+template <int NT, int DMAX, bool EXACT, bool PREP = false>
 __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
+  static_assert(!PREP || (NT == 1 && EXACT), "the folded preparation is written for one row tile and a head_dim known here");
   constexpr int DCH = DMAX / 32;  // contraction chunks of the first product
   constexpr int DTL = DMAX / 16;  // d tiles of the output
   const int lane = threadIdx.x, li = lane & 15, g = lane >> 4;
@@ -130,6 +153,7 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
     my_tok[n] = min(row / G, qlen - 1);
     my_head[n] = kvh * G + row % G;
     my_pos[n] = start + my_tok[n];
+    if constexpr (PREP) continue;  // q is made below
     const uint16_t* qp = a.q + static_cast<int64_t>(row0 + my_tok[n]) * a.q_stride + my_head[n] * D;
 #pragma unroll
     for (int c = 0; c < DCH; ++c) {
@@ -207,8 +231,210 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
 
   bf16x8 kcur[2][DCH];
   u32x4 vraw[DTL];  // the second product's operand for each d tile: keys 4g..4g+3 of both 16-key tiles
-  if (b0 < b1) {
-    refill_pages(clamp_key(b0 * 32) >> ps);
+  if (b0 < b1) refill_pages(clamp_key(b0 * 32) >> ps);
+
+  // PREP: q of this lane's row, and in the wave whose keys end with the new token's (`owner`) that token's key as
+  // the lanes (any i, g) of a key operand hold it and its value at d = 16 dt + i.  Loads of one kind go out together
+  // (a missing part of the stack is fetched from the last one and not added: a load under a condition would be
+  // waited for on the spot); the arithmetic of q runs while the first keys and values of
+  // the cache and the stack's k and v are on their way.
+  [[maybe_unused]] bf16x8 knew[DCH];
+  [[maybe_unused]] uint32_t vnew[DTL];
+  [[maybe_unused]] const int last_blk = (kv_hi + 31) / 32 - 1;
+  [[maybe_unused]] const bool owner = PREP && b0 <= last_blk && last_blk < b1;  // the same in all lanes
+  if constexpr (PREP) {
+    constexpr int HC = DCH / 2;                 // chunks of 32 columns that half of a head holds
+    const int hc = a.prep_rot / 64;             // and that half of the rotated width holds
+    const float* prow = a.prep_parts + static_cast<int64_t>(row0) * a.prep_row_stride;  // the segment's one token
+    const int n_parts = a.prep_n;
+    // Every load of this prologue is issued without a condition around it (a load under a condition is waited for at
+    // the end of its branch, and the loads behind it wait with it): what is not needed is fetched from a place
+    // that exists and dropped.
+    //
+    // The parts of the stack are spread over lanes that would otherwise fetch the same thing, so that a head's parts
+    // are all on their way at once: lane i of a q head's row takes the parts i / gp, i / gp + 16 / gp, ... (gp: the
+    // group's heads rounded up to a power of two; rows past the group are copies), the lanes i of the k head the
+    // parts i % kp, i % kp + kp, ..., the four lanes g of a value the parts g % vp, g % vp + vp, ...  A lane adds
+    // its parts in ascending order; the lanes' sums then meet pairwise, the lanes 8, 4, 2, 1 apart in turn (rotations
+    // of the 16 lanes i), which leaves every lane that holds the head with the same total: one fixed order, whatever
+    // else the step holds.
+    auto fetch_part = [&](int col0, int u, float4 (&got)[DCH][2]) {
+      const float* pu = prow + col0 + 8 * g + static_cast<int64_t>(min(u, n_parts - 1)) * a.prep_part_stride;
+#pragma unroll
+      for (int c = 0; c < DCH; ++c) {
+        got[c][0] = *reinterpret_cast<const float4*>(pu + 32 * c);
+        got[c][1] = *reinterpret_cast<const float4*>(pu + 32 * c + 4);
+      }
+    };
+    // x = the lane's parts added up (the first round's loads are `got`); mine, apart: the lane's first part and the
+    // distance to its next
+    auto add_parts = [&](int col0, int mine, int apart, float4 (&got)[DCH][2], float (&x)[DCH][8]) {
+#pragma unroll
+      for (int c = 0; c < DCH; ++c)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[c][e] = 0.f;
+      for (int base = 0; base < n_parts; base += apart) {   // the same number of rounds in all lanes
+        const int u = base + mine;
+        if (base > 0) fetch_part(col0, u, got);
+        const bool there = u < n_parts;
+#pragma unroll
+        for (int c = 0; c < DCH; ++c) {
+          const float4 lo = got[c][0], hi = got[c][1];
+          x[c][0] += there ? lo.x : 0.f, x[c][1] += there ? lo.y : 0.f, x[c][2] += there ? lo.z : 0.f, x[c][3] += there ? lo.w : 0.f;
+          x[c][4] += there ? hi.x : 0.f, x[c][5] += there ? hi.y : 0.f, x[c][6] += there ? hi.z : 0.f, x[c][7] += there ? hi.w : 0.f;
+        }
+      }
+    };
+    // x += x of the lane `n` to the side in the row of 16 lanes i (a rotation: row_ror)
+#define ARLE_MEET(CTRL)                                                                                              \
+  _Pragma("unroll") for (int c = 0; c < DCH; ++c) _Pragma("unroll") for (int e = 0; e < 8; ++e)                         \
+      x[c][e] += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x[c][e]), CTRL, 0xf, 0xf, false))
+    auto meet = [&](float (&x)[DCH][8], int from, int to) {   // the lanes from, from / 2, ..., to apart
+      if (from >= 8 && to <= 8) { ARLE_MEET(0x128); }
+      if (from >= 4 && to <= 4) { ARLE_MEET(0x124); }
+      if (from >= 2 && to <= 2) { ARLE_MEET(0x122); }
+      if (from >= 1 && to <= 1) { ARLE_MEET(0x121); }
+    };
+#undef ARLE_MEET
+    // a head's norm weights as this lane holds the head, bfloat16 or float32 in memory: two loads of 16 bytes either
+    // way (the second one of bfloat16 weights is the first one again), sorted out afterwards
+    auto fetch_weights = [&](const void* w, uint4 (&raw)[DCH][2]) {
+      const unsigned char* base = static_cast<const unsigned char*>(w != nullptr ? w : a.prep_parts);
+      const int elem = a.prep_w_f32 ? 4 : 2;
+#pragma unroll
+      for (int c = 0; c < DCH; ++c) {
+        const unsigned char* at = base + static_cast<size_t>(32 * c + 8 * g) * elem;
+        raw[c][0] = *reinterpret_cast<const uint4*>(at);
+        raw[c][1] = *reinterpret_cast<const uint4*>(at + (a.prep_w_f32 ? 16 : 0));
+      }
+    };
+    auto weight_of = [&](const uint4 (&raw)[DCH][2], int c, int e) {   // e is a constant where this is called
+      const uint32_t lo[4] = {raw[c][0].x, raw[c][0].y, raw[c][0].z, raw[c][0].w};
+      const uint32_t hi[4] = {raw[c][1].x, raw[c][1].y, raw[c][1].z, raw[c][1].w};
+      const float wide = __uint_as_float(e < 4 ? lo[e & 3] : hi[e & 3]);
+      const uint32_t pair = lo[e >> 1];
+      const float narrow = __uint_as_float((e & 1) ? pair & 0xffff0000u : pair << 16);
+      return a.prep_w_f32 ? wide : narrow;
+    };
+    // the angles of the token's position, for the chunks of half of the rotated width
+    float cs[HC > 0 ? HC : 1][8], sn[HC > 0 ? HC : 1][8];
+    {
+      const bool turns = hc > 0;
+      const float* ct = turns ? a.prep_cos + static_cast<int64_t>(start) * (a.prep_rot / 2) : prow;
+      const float* st = turns ? a.prep_sin + static_cast<int64_t>(start) * (a.prep_rot / 2) : prow;
+#pragma unroll
+      for (int c = 0; c < HC; ++c) {
+        const int at = 32 * min(c, max(hc - 1, 0)) + 8 * g;
+        const float4 c0 = *reinterpret_cast<const float4*>(ct + at), c1 = *reinterpret_cast<const float4*>(ct + at + 4);
+        const float4 s0 = *reinterpret_cast<const float4*>(st + at), s1 = *reinterpret_cast<const float4*>(st + at + 4);
+        cs[c][0] = c0.x, cs[c][1] = c0.y, cs[c][2] = c0.z, cs[c][3] = c0.w, cs[c][4] = c1.x, cs[c][5] = c1.y, cs[c][6] = c1.z, cs[c][7] = c1.w;
+        sn[c][0] = s0.x, sn[c][1] = s0.y, sn[c][2] = s0.z, sn[c][3] = s0.w, sn[c][4] = s1.x, sn[c][5] = s1.y, sn[c][6] = s1.z, sn[c][7] = s1.w;
+      }
+    }
+    // one head as this lane's part of an operand: norm, rotation, bfloat16
+    auto finish_head = [&](float (&x)[DCH][8], bool normed, const uint4 (&wraw)[DCH][2], bf16x8 (&dst)[DCH]) {
+      if (normed) {
+        float ss = 0.f;
+#pragma unroll
+        for (int c = 0; c < DCH; ++c)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ss += x[c][e] * x[c][e];
+        ss = group_sum4(ss);
+        const float inv = 1.0f / sqrtf(ss / static_cast<float>(DMAX) + a.prep_eps);
+#pragma unroll
+        for (int c = 0; c < DCH; ++c)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[c][e] = x[c][e] * inv * weight_of(wraw, c, e);
+      }
+      // d < rot / 2 turns with d + rot / 2, hc chunks up in the same lane.  The chunk numbers are written out for
+      // each rotated width that there is (indexed by hc, the arrays would leave the registers).
+      auto turn = [&](float (&lo)[8], float (&hi)[8], const float (&c)[8], const float (&s_)[8]) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float l_ = lo[e], h_ = hi[e];
+          lo[e] = l_ * c[e] - h_ * s_[e];
+          hi[e] = l_ * s_[e] + h_ * c[e];
+        }
+      };
+      if (hc == HC) {
+#pragma unroll
+        for (int c = 0; c < HC; ++c) turn(x[c], x[c + HC], cs[c], sn[c]);
+      } else if (hc > 0) {
+        if constexpr (HC == 2) turn(x[0], x[1], cs[0], sn[0]);   // half of a head of 128 is rotated: hc == 1
+      }
+#pragma unroll
+      for (int c = 0; c < DCH; ++c) {
+        uint4 pk;
+        pk.x = pack_bf16x2(x[c][0], x[c][1]);
+        pk.y = pack_bf16x2(x[c][2], x[c][3]);
+        pk.z = pack_bf16x2(x[c][4], x[c][5]);
+        pk.w = pack_bf16x2(x[c][6], x[c][7]);
+        dst[c] = __builtin_bit_cast(bf16x8, pk);
+      }
+    };
+    int gp = 1;
+    while (gp < G) gp <<= 1;                                   // G <= 16
+    int kp = 1, vp = 1;                  // lanes i (lanes g) that share the key's (the value's) parts
+    while (kp < n_parts && kp < 16) kp <<= 1;
+    while (vp < n_parts && vp < 4) vp <<= 1;
+    const int q_col = (kvh * G + min(li & (gp - 1), G - 1)) * DMAX;    // live rows (i < G) take their own head
+    const int k_col = (a.nq + kvh) * DMAX;
+    const int v_mine = g & (vp - 1);
+    const float* pv = prow + (a.nq + a.nkv + kvh) * DMAX + li;
+    float xq[DCH][8];
+    float4 gq[DCH][2];
+    uint4 wq[DCH][2];
+    fetch_weights(a.prep_qw, wq);
+    fetch_part(q_col, li / gp, gq);
+    if (b0 < b1) {   // the first keys and values of the cache
+      load_k(b0, kcur);
+      load_v(b0, vraw);
+    }
+    // the owner's key and value: behind the cache's loads, and waited for behind the arithmetic of q
+    [[maybe_unused]] float4 gk[DCH][2];
+    [[maybe_unused]] uint4 wk[DCH][2];
+    [[maybe_unused]] float vgot[DTL];
+    if (owner) {
+      fetch_weights(a.prep_kw, wk);
+      fetch_part(k_col, li & (kp - 1), gk);
+#pragma unroll
+      for (int dt = 0; dt < DTL; ++dt) vgot[dt] = pv[static_cast<int64_t>(min(v_mine, n_parts - 1)) * a.prep_part_stride + 16 * dt];
+    }
+    add_parts(q_col, li / gp, 16 / gp, gq, xq);
+    if (n_parts > 1) meet(xq, 8, gp);
+    finish_head(xq, a.prep_qw != nullptr, wq, qreg[0]);
+    if (owner) {
+      float xk[DCH][8], vsum[DTL];
+      add_parts(k_col, li & (kp - 1), kp, gk, xk);
+      meet(xk, kp / 2, 1);
+#pragma unroll
+      for (int dt = 0; dt < DTL; ++dt) vsum[dt] = v_mine < n_parts ? vgot[dt] : 0.f;
+      for (int base = vp; base < n_parts; base += vp) {
+        const int u = base + v_mine;
+#pragma unroll
+        for (int dt = 0; dt < DTL; ++dt) vgot[dt] = pv[static_cast<int64_t>(min(u, n_parts - 1)) * a.prep_part_stride + 16 * dt];
+#pragma unroll
+        for (int dt = 0; dt < DTL; ++dt) vsum[dt] += u < n_parts ? vgot[dt] : 0.f;
+      }
+      if (vp > 1) {
+        float far[DTL];
+#pragma unroll
+        for (int dt = 0; dt < DTL; ++dt) far[dt] = __shfl_xor(vsum[dt], 16, kWave);
+#pragma unroll
+        for (int dt = 0; dt < DTL; ++dt) vsum[dt] += far[dt];
+      }
+      if (vp > 2) {
+        float far[DTL];
+#pragma unroll
+        for (int dt = 0; dt < DTL; ++dt) far[dt] = __shfl_xor(vsum[dt], 32, kWave);
+#pragma unroll
+        for (int dt = 0; dt < DTL; ++dt) vsum[dt] += far[dt];
+      }
+      finish_head(xk, a.prep_kw != nullptr, wk, knew);
+#pragma unroll
+      for (int dt = 0; dt < DTL; ++dt) vnew[dt] = f32_to_bf16_bits(vsum[dt]);
+    }
+  } else if (b0 < b1) {
     load_k(b0, kcur);
     load_v(b0, vraw);
   }
@@ -217,6 +443,16 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
     const int key_base = blk * 32;
     const bool more = blk + 1 < b1;
     if (more) cover(blk + 1);
+    if constexpr (PREP) {
+      if (owner && blk == last_blk && li == (start & 15)) {   // the new token's key, where the load brought the slot's old bits
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+          if (t == ((start >> 4) & 1)) {
+#pragma unroll
+            for (int c = 0; c < DCH; ++c) kcur[t][c] = knew[c];
+          }
+      }
+    }
 
     // scores S^T: s[n][t][r] belongs to key key_base + 16t + 4g + r and row (n, li)
     f32x4 s[NT][2];
@@ -246,6 +482,19 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
           if (key4 + 2 >= kv_total) vraw[dt][2 * t + 1] &= 0xffff0000u;
           if (key4 + 3 >= kv_total) vraw[dt][2 * t + 1] &= 0x0000ffffu;
         }
+      }
+    }
+
+    if constexpr (PREP) {
+      if (owner && blk == last_blk && g == ((start & 15) >> 2)) {   // and its value, one half of a register
+        const int word = 2 * ((start >> 4) & 1) + ((start & 3) >> 1);
+        const bool upper = (start & 1) != 0;
+#pragma unroll
+        for (int dt = 0; dt < DTL; ++dt)
+#pragma unroll
+          for (int w = 0; w < 4; ++w)
+            if (w == word)
+              vraw[dt][w] = upper ? (vraw[dt][w] & 0x0000ffffu) | (vnew[dt] << 16) : (vraw[dt][w] & 0xffff0000u) | vnew[dt];
       }
     }
 
@@ -303,6 +552,26 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
     }
     // and the value registers after the second product
     if (more) load_v(blk + 1, vraw);
+  }
+
+  if constexpr (PREP) {
+    // the new token's key and value go into the cache (their page is among those that the last block had in reach)
+    if (owner && a.prep_k_pages != nullptr) {
+      const int page = page_of(start);
+      const int64_t at = page * page_elems + k_head;
+      const int in_page = start & pm;
+      if (li == 0) {
+#pragma unroll
+        for (int c = 0; c < DCH; ++c)
+          *reinterpret_cast<uint4*>(a.prep_k_pages + at + static_cast<int64_t>(in_page) * DMAX + 32 * c + 8 * g) =
+              __builtin_bit_cast(uint4, knew[c]);
+      }
+      if (g == 0) {
+#pragma unroll
+        for (int dt = 0; dt < DTL; ++dt)
+          a.prep_v_pages[at + static_cast<int64_t>(16 * dt + li) * P + in_page] = static_cast<uint16_t>(vnew[dt]);
+      }
+    }
   }
 
   // acc[n][dt][r] is O^T[d = 16dt + 4g + r][row (n, li)]
@@ -1726,6 +1995,15 @@ static AttnArgs make_args(const void* q, long long q_stride, void* out, long lon
   a.pws_o = nullptr;
   a.pws_ml = nullptr;
   a.rows_max = 0;
+  a.prep_parts = nullptr;
+  a.prep_n = 0;
+  a.prep_part_stride = a.prep_row_stride = 0;
+  a.prep_qw = a.prep_kw = nullptr;
+  a.prep_w_f32 = 0;
+  a.prep_cos = a.prep_sin = nullptr;
+  a.prep_rot = 0;
+  a.prep_eps = 0.f;
+  a.prep_k_pages = a.prep_v_pages = nullptr;
   return a;
 }
 
@@ -1832,6 +2110,60 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
   const int nt = max_rows <= 16 ? 1 : 2;
   dim3 grid((max_rows + 16 * nt - 1) / (16 * nt), nkv, static_cast<unsigned>(z));
   rc = nt == 1 ? launch_attn<1>(a, grid, s) : launch_attn<2>(a, grid, s);
+  if (rc != 0 || splits == 1) return rc;
+  attn_merge_kernel<<<dim3(segments * a.ws_rows, nq), kMergeWaves * kWave, 0, s>>>(
+      ws_o, ws_ml, a.out, o_stride, seg_row0, a.ws_rows, 0, nq, nkv, D, splits);
+  return launch_status();
+}
+
+// A step of single decoded tokens with the preparation of q, k and v folded into the attention: segment s is the
+// one token row s.  parts: the fused q|k|v projection of the step as n_parts float32 partial products
+// [token rows][(nq + 2 nkv) D] (part_stride elements apart, rows row_stride apart; both multiples of 4, parts
+// 16-byte aligned), added in order.  q_w / k_w: per-head norm weights [D] (both or neither; float32 if w_f32, else
+// bfloat16; 16-byte aligned), eps inside the root.  cos / sin: float32 [positions][rot / 2], rot 0 (no rotation) or a
+// multiple of 64 up to D.  The new token's key and value are written to its slot of the pages (which the block table
+// must already hold) and take part in the attention from registers.  D 64 or 128, nq / nkv <= 16; everything else
+// as arle_attn_paged_mfma with max_qlen 1.  The same results as arle_qk_prep followed by arle_attn_paged_mfma but
+// for the order in which a head's squares are added for its norm.
+extern "C" int arle_attn_decode_prep(const float* parts, int n_parts, long long part_stride, long long row_stride,
+                                     const void* q_w, const void* k_w, int w_f32, const float* cos_t, const float* sin_t,
+                                     int rot, float eps, void* out, long long o_stride, void* k_pages, void* v_pages,
+                                     const int* block_table, int table_stride, const int* seg_row0, const int* seg_slot,
+                                     const int* seg_start, int segments, int nq, int nkv, int D, int page_size,
+                                     float scale, int window, int splits, float* ws_o, float* ws_ml, void* stream) {
+  if (segments == 0) return 0;
+  auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  if ((D != 64 && D != 128) || page_size < 4 || (page_size & (page_size - 1)) != 0 || nkv <= 0 || nq % nkv != 0 ||
+      nq / nkv > 16 || splits < 1 || splits > 64 || (splits > 1 && (ws_o == nullptr || ws_ml == nullptr)) ||
+      parts == nullptr || n_parts < 1 || part_stride % 4 != 0 || row_stride % 4 != 0 || !aligned(parts) ||
+      (q_w == nullptr) != (k_w == nullptr) || !aligned(q_w) || !aligned(k_w) || rot < 0 || rot > D || rot % 64 != 0 ||
+      (rot > 0 && (cos_t == nullptr || sin_t == nullptr || !aligned(cos_t) || !aligned(sin_t))) ||
+      k_pages == nullptr || v_pages == nullptr || !aligned(k_pages))
+    return static_cast<int>(hipErrorInvalidValue);
+  const long long z = static_cast<long long>(segments) * splits;
+  if (nkv > 65535 || z > 65535) return static_cast<int>(hipErrorInvalidValue);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  AttnArgs a = make_args(nullptr, 0, out, o_stride, k_pages, v_pages, block_table, table_stride, seg_row0, seg_slot,
+                         seg_start, 1, nq, nkv, D, page_size, scale, window, splits, ws_o, ws_ml);
+  a.prep_parts = parts;
+  a.prep_n = n_parts;
+  a.prep_part_stride = part_stride;
+  a.prep_row_stride = row_stride;
+  a.prep_qw = q_w;
+  a.prep_kw = k_w;
+  a.prep_w_f32 = w_f32;
+  a.prep_cos = cos_t;
+  a.prep_sin = sin_t;
+  a.prep_rot = rot;
+  a.prep_eps = eps;
+  a.prep_k_pages = static_cast<uint16_t*>(k_pages);
+  a.prep_v_pages = static_cast<uint16_t*>(v_pages);
+  const dim3 grid(1, nkv, static_cast<unsigned>(z));
+  if (D == 128)
+    attn_mfma_kernel<1, 128, true, true><<<grid, kWave, 0, s>>>(a);
+  else
+    attn_mfma_kernel<1, 64, true, true><<<grid, kWave, 0, s>>>(a);
+  const int rc = launch_status();
   if (rc != 0 || splits == 1) return rc;
   attn_merge_kernel<<<dim3(segments * a.ws_rows, nq), kMergeWaves * kWave, 0, s>>>(
       ws_o, ws_ml, a.out, o_stride, seg_row0, a.ws_rows, 0, nq, nkv, D, splits);

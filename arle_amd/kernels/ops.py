@@ -445,6 +445,74 @@ def attn_paged_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, s
     return out
 
 
+_PREP_HEAD_DIMS = (64, 128)
+
+
+def attn_decode_prep_supported(dtype, head_dim: int, page_size: int, group: int, rotary_dim: int) -> bool:
+    """Whether attn_decode_prep takes these sizes: bfloat16 pages, a head_dim whose kernel is made for it, up to 16
+    q heads a kv head, and a rotated width whose halves are whole chunks of 32 columns (or none)."""
+    return (attn_mfma_supported(dtype, head_dim, page_size) and head_dim in _PREP_HEAD_DIMS and 1 <= group <= _ATTN_ROW_TILE
+            and rotary_dim % 64 == 0 and 0 <= rotary_dim <= head_dim)
+
+
+def attn_decode_prep(parts, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *, max_kv_len: int,
+                     num_q_heads: int, num_kv_heads: int, head_dim: int, page_size: int, scale: float, eps: float,
+                     q_weight=None, k_weight=None, cos=None, sin=None, rotary_dim: int = 0, window: int = 0,
+                     splits: int | None = None):
+    """A step of single decoded tokens (segment s is token row s) from the float32 stack of partial products
+    [S, T, (nq + 2 nkv) D] of its fused q|k|v projection: what qk_prep and attn_paged_mfma do one after the other,
+    in the attention's own kernel.  Every wave sums, norms and rotates its q heads itself; the wave whose keys end
+    with the new token's does the same for the k head, writes key and value into the cache and uses them from its
+    registers.  out: bfloat16 [T, nq*D]."""
+    _gpu(parts, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, q_weight, k_weight, cos, sin)
+    group = num_q_heads // max(num_kv_heads, 1)
+    width = (num_q_heads + 2 * num_kv_heads) * head_dim
+    _need(parts.dtype == torch.float32 and parts.dim() == 3 and parts.shape[0] >= 1 and parts.shape[2] == width
+          and parts.is_contiguous(), f"parts must be contiguous float32 [S, T, {width}]")
+    tokens = parts.shape[1]
+    _need(out.dtype == torch.bfloat16 and out.shape == (tokens, num_q_heads * head_dim) and out.is_contiguous(),
+          "out must be contiguous bfloat16 [T, nq*D]")
+    _need(num_kv_heads > 0 and num_q_heads % num_kv_heads == 0, "q heads must be a multiple of kv heads")
+    _need(attn_decode_prep_supported(out.dtype, head_dim, page_size, group, rotary_dim),
+          f"attn_decode_prep takes head_dim {_PREP_HEAD_DIMS}, up to {_ATTN_ROW_TILE} q heads a kv head and a rotated width "
+          f"that is a multiple of 64 (got head_dim {head_dim}, {group} heads, rotary_dim {rotary_dim})")
+    _check_pages(k_pages, v_pages, num_kv_heads, page_size, head_dim, out.dtype)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "block_table must be contiguous int32 [slots, pages]")
+    segments = seg_slot.numel()
+    _need(segments == tokens, "attn_decode_prep takes one token a segment")
+    _i32(seg_row0, "seg_row0", segments + 1)
+    _i32(seg_slot, "seg_slot")
+    _i32(seg_start, "seg_start", segments)
+    _need((q_weight is None) == (k_weight is None), "give both q and k norm weights or neither")
+    w_f32 = 0
+    if q_weight is not None:
+        _need(q_weight.shape == (head_dim,) and k_weight.shape == (head_dim,) and q_weight.dtype == k_weight.dtype
+              and q_weight.dtype in (torch.float32, torch.bfloat16) and q_weight.is_contiguous() and k_weight.is_contiguous()
+              and q_weight.data_ptr() % 16 == 0 and k_weight.data_ptr() % 16 == 0,
+              "q/k norm weights must be 16-byte aligned [head_dim] of one type, float32 or bfloat16")
+        w_f32 = int(q_weight.dtype == torch.float32)
+    if rotary_dim:
+        _need(cos is not None and sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32
+              and cos.dim() == 2 and cos.shape == sin.shape and cos.shape[1] == rotary_dim // 2 and cos.is_contiguous()
+              and sin.is_contiguous() and cos.data_ptr() % 16 == 0 and sin.data_ptr() % 16 == 0,
+              "cos/sin must be contiguous 16-byte aligned float32 [positions, rotary_dim/2]")
+    if splits is None:
+        splits = decode_splits(segments, num_kv_heads, max_kv_len)
+    _need(1 <= splits <= 64, "splits must be 1..64")
+    _need(segments * splits <= _GRID_Y_MAX and num_kv_heads <= _GRID_Y_MAX, "too many segments for one launch")
+    ws_o = ws_ml = None
+    if splits > 1:
+        ws_o = torch.empty((segments, num_q_heads, splits, head_dim), dtype=torch.float32, device=out.device)
+        ws_ml = torch.empty((segments, num_q_heads, splits, 2), dtype=torch.float32, device=out.device)
+    lib.call("arle_attn_decode_prep", parts.data_ptr(), parts.shape[0], parts.stride(0), parts.stride(1), _ptr(q_weight),
+             _ptr(k_weight), w_f32, _ptr(cos), _ptr(sin), int(rotary_dim), float(eps), out.data_ptr(), out.stride(0),
+             k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], seg_row0.data_ptr(),
+             seg_slot.data_ptr(), seg_start.data_ptr(), segments, num_q_heads, num_kv_heads, head_dim, page_size,
+             float(scale), int(window), int(splits), _ptr(ws_o), _ptr(ws_ml), _stream())
+    return out
+
+
 _plan_tokens = itertools.count(1)
 
 

@@ -77,6 +77,9 @@ class PagedAttention(Part):
         # multiple of 16, so the q rows are whole operand tiles too)
         self.q_only = Linear(self.qkv.weight[: self.q_width], packed=self.qkv.tiles)
         self.o = Linear(tensors["o"], rt.weight_tiles)
+        # steps of single decoded tokens run norm, rotation and cache write inside the attention's kernel where it
+        # has that form (ops.attn_decode_prep_supported); params["fold_preparation"] = False keeps the two kernels
+        self.folds_preparation = bool(params.get("fold_preparation", True))
 
     @classmethod
     def declare_cache(cls, params):
@@ -113,6 +116,16 @@ class PagedAttention(Part):
                             k_pages=cache.k_pages, v_pages=cache.v_pages, page_size=cache.page_size)
         # the fused preparation kernel can add a stack of partial products itself
         projected = (self.qkv if cache.writes else self.q_only)(x, partials_ok=fused)
+        if (projected.dim() == 3 and cache.writes and batch.max_qlen == 1 and self.folds_preparation
+                and ops.attn_decode_prep_supported(x.dtype, self.D, cache.page_size, self.nq // self.nkv, rot)):
+            # single decoded tokens: the attention's kernel sums, norms, rotates and writes to the cache itself
+            out = torch.empty((x.shape[0], Q), dtype=x.dtype, device=x.device)
+            ops.attn_decode_prep(projected, out, cache.k_pages, cache.v_pages, cache.block_table, batch.seg_row0,
+                                 batch.seg_slot, batch.seg_start, max_kv_len=batch.max_position + 1,
+                                 num_q_heads=self.nq, num_kv_heads=self.nkv, head_dim=self.D, page_size=cache.page_size,
+                                 scale=self.scale, eps=self.eps, q_weight=self.q_norm, k_weight=self.k_norm, cos=cos,
+                                 sin=sin, rotary_dim=rot, window=self.window or 0, splits=getattr(batch, "kv_splits", None))
+            return self.o(out, partials_ok=True)
         if projected.dim() == 3:
             q = torch.empty((x.shape[0], Q), dtype=x.dtype, device=x.device)
             ops.qk_prep(q, None, None, q_weight=self.q_norm, k_weight=self.k_norm, cos=cos, sin=sin,

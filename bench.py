@@ -84,14 +84,17 @@ def _completes_gate_up(name: str) -> bool:
 
 def classify_step(names, layers: int) -> list:
     """The part of the model that each kernel of one step belongs to, from the order in which a layer launches
-    them: norm, q|k|v product, q/k preparation, attention (+ merges), o product, norm, gate|up (+ activation),
-    down product; after the last layer the final norm and the head."""
+    them: norm, q|k|v product, q/k preparation (a kernel of its own, or inside the attention's for single decoded
+    tokens), attention (+ merges), o product, norm, gate|up (+ activation), down product; after the last layer the
+    final norm and the head."""
     out, phase, layers_done = [], "qkv", 0
     for name in names:
         if "qk_prep" in name:
             part, phase = "qk_prep", "o"
         elif "attn_" in name:
             part = "attention"
+            if phase == "qkv":     # single decoded tokens: the attention's kernel prepares q, k and v itself
+                phase = "o"
         elif "rmsnorm" in name:
             part = "norm"
             if phase == "o":
@@ -145,7 +148,7 @@ def part_times(steps, layers: int) -> dict:
     most = max(len(k) for k in steps)
     steps = [k for k in steps if len(k) == most]
     for kernels in steps:
-        seen = sum(1 for n, _ in kernels if "qk_prep" in n)
+        seen = (sum(1 for n, _ in kernels if "rmsnorm" in n) - 1) // 2   # two norms a layer and the last one
         if seen != layers:
             raise RuntimeError(f"a profiled step shows {seen} of {layers} layers")
     total = {p: 0.0 for p in PARTS}

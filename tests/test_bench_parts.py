@@ -25,6 +25,13 @@ def test_kernels_of_a_step_are_sorted_into_the_parts_of_a_layer():
              "gemm_tiles_kernel<4, 2, 4, 4, false, 1, arle::bf16>", "Cijk_c", "rmsnorm", "Cijk_head"]
     assert bench.classify_step(tiles, layers=1) == ["norm", "qkv", "qk_prep", "attention", "o", "norm", "gate_up", "down",
                                                     "norm", "head"]
+    # single decoded tokens: no preparation kernel, the attention's kernel is the first behind the q|k|v product
+    folded = ["embed_gather_kernel", "rmsnorm", "gemm_rows_kernel<1, 2, 2, 4, 4, 0, float>", "attn_mfma_kernel<1, 128, true, true>",
+              "attn_merge_kernel", "gemm_rows_kernel<1, 1, 4, 4, 4, 0, float>", "add_stack_rmsnorm_kernel<bf16>",
+              "gemm_rows_kernel<1, 8, 1, 4, 4, 1, arle::bf16>", "gemm_rows_kernel<1, 1, 4, 4, 4, 0, float>", "rmsnorm", "Cijk_head"]
+    assert bench.classify_step(folded, layers=1) == ["other", "norm", "qkv", "attention", "attention", "o", "norm", "gate_up",
+                                                     "down", "norm", "head"]
+    assert bench.part_times([[(n, 1.0) for n in folded]], layers=1)["attention"] == 2.0
 
 
 def test_a_step_whose_kernels_are_not_all_sorted_is_refused():

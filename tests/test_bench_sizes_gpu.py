@@ -319,5 +319,7 @@ def test_bench_sorts_the_kernels_of_real_steps_into_every_part_of_a_layer():
     line = json.loads(lines[-1])
     for step in ("prefill_parts_us", "decode_parts_us"):
         for part in ("qkv", "o", "gate_up", "down", "head", "attention", "qk_prep", "norm"):
+            if (step, part) == ("decode_parts_us", "qk_prep"):
+                continue     # single decoded tokens are prepared inside the attention's kernel
             assert line[step][part] > 0, (step, part, line[step])
     assert line["prefill_parts_us"]["gate_up"] > line["prefill_parts_us"]["qkv"] > line["prefill_parts_us"]["head"] / 100

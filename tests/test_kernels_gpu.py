@@ -649,6 +649,93 @@ def test_attention_portions_list_their_work_once_for_calls_that_name_the_same_st
         lib.function("arle_attn_prefill_variant")(-1)
 
 
+@pytest.mark.parametrize("nq,nkv,D,rot,P", [(32, 8, 128, 128, 16), (8, 8, 64, 64, 8), (16, 1, 128, 64, 64), (6, 2, 64, 0, 4),
+                                            (4, 4, 128, 0, 32), (12, 2, 128, 128, 128)])
+@pytest.mark.parametrize("n_parts,splits,window,w_dtype", [(1, 1, 0, torch.bfloat16), (4, None, 0, torch.float32),
+                                                           (3, 5, 37, torch.bfloat16), (7, 64, 0, None)])
+def test_decode_attention_with_the_preparation_folded_in(nq, nkv, D, rot, P, n_parts, splits, window, w_dtype):
+    """A step of single decoded tokens from the float32 stack of its q|k|v projection: sum, per-head norm, rotation,
+    cache write and attention in one kernel.  Requests whose new token is the first of all, the first or last of
+    a page and of a 32-key block, deep in a long context; slots of the cache that hold NaN bits where nothing was
+    written yet (the new token's own slot among them).  Against the plain implementation, and against the two
+    kernels that it replaces: the same cache to the last bit but one, and nothing else touched."""
+    dt, eps, theta = torch.bfloat16, 1e-6, 1e4
+    cached = [0, 1, 31, 32, 63, P - 1, P, 700, 1029, 255]     # tokens a request holds before the step
+    lengths = [c + 1 for c in cached]
+    T = len(cached)
+    table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, 500)
+    k_pages.fill_(float("nan"))
+    v_pages.fill_(float("nan"))
+    Q, KV = nq * D, nkv * D
+    qw = kw = None
+    if w_dtype is not None:
+        qw = (1.0 + 0.2 * torch.randn(D, generator=_g(501))).to(w_dtype)
+        kw = (1.0 + 0.2 * torch.randn(D, generator=_g(502))).to(w_dtype)
+    cos = sin = None
+    if rot:
+        cos, sin = plain.rope_cos_sin(range(max(lengths) + 1), rot, theta)
+    def prepared(x, w, positions):   # [n, heads, D] float64 -> norm, rotation of the first rot columns
+        if w is not None:
+            x = plain.qk_norm(x, w.double(), eps)
+        if rot:
+            c, s_ = plain.rope_cos_sin(positions, rot, theta, dtype=torch.float64)
+            x = torch.cat([plain.apply_rope(x[..., :rot], c, s_), x[..., rot:]], -1)
+        return x
+    new_rows, wants = [], []
+    for s_, n in enumerate(cached):
+        g = _g(510 + s_)
+        raw = torch.randn(n + 1, (nq + 2 * nkv) * D, generator=g)
+        raw[:n] = raw[:n].to(dt).float()         # earlier tokens were projections in bfloat16
+        x = raw.double()
+        q = prepared(x[:, :Q].reshape(n + 1, nq, D), qw, list(range(n + 1)))
+        k = prepared(x[:, Q:Q + KV].reshape(n + 1, nkv, D), kw, list(range(n + 1))).to(dt)
+        v = x[:, Q + KV:].reshape(n + 1, nkv, D).to(dt)
+        _fill_cache(table, k_pages, v_pages, s_, k[:n], v[:n], P)
+        wants.append(plain.causal_attention(q.to(dt).double(), k.double(), v.double(), nkv, window=window or None,
+                                            rows=[n])[n].reshape(-1))
+        new_rows.append(raw[n])
+    row = torch.stack(new_rows)                                      # [T, width] float32
+    stack = torch.randn(n_parts, T, row.shape[1], generator=_g(503))
+    stack[-1] = row - (stack[:-1].double().sum(0)).float() if n_parts > 1 else row
+    exact = stack.double().sum(0)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    dev = lambda t: None if t is None else t.to(DEV)
+    seg = (i32(list(range(T + 1))), i32(list(range(T))), i32(cached))
+    kw_args = dict(num_q_heads=nq, num_kv_heads=nkv, head_dim=D, page_size=P, scale=1.0 / math.sqrt(D), window=window)
+    dk, dv = k_pages.to(DEV), v_pages.to(DEV)
+    out = torch.full((T, Q), float("nan"), dtype=dt, device=DEV)
+    ops.attn_decode_prep(stack.to(DEV), out, dk, dv, table.to(DEV), *seg, max_kv_len=max(lengths), eps=eps, q_weight=dev(qw),
+                         k_weight=dev(kw), cos=dev(cos), sin=dev(sin), rotary_dim=rot, splits=splits, **kw_args)
+    assert torch.isfinite(out.float()).all()
+    # the stack's own sum is what the kernel saw: compare with plain values made from it
+    for s_, n in enumerate(cached):
+        x = exact[s_]
+        k_want = prepared(x[Q:Q + KV].reshape(1, nkv, D), kw, [n])[0]
+        page, at = int(table[s_, n // P]), n % P
+        assert _rel(dk[page, :, at].cpu(), k_want) < 6e-3
+        assert _rel(dv[page, :, :, at].cpu(), x[Q + KV:].reshape(nkv, D)) < 6e-3
+    assert _rel(out.cpu(), torch.stack(wants)) < 1e-2
+    # the two kernels that it stands for
+    dk2, dv2 = k_pages.to(DEV), v_pages.to(DEV)
+    q2 = torch.empty((T, Q), dtype=dt, device=DEV)
+    ops.qk_prep(q2, None, None, num_q_heads=nq, num_kv_heads=nkv, head_dim=D, eps=eps, q_weight=dev(qw), k_weight=dev(kw),
+                cos=dev(cos), sin=dev(sin), rotary_dim=rot, positions=seg[2], slot_of_token=seg[1], block_table=table.to(DEV),
+                k_pages=dk2, v_pages=dv2, page_size=P, parts=stack.to(DEV))
+    out2 = torch.full((T, Q), float("nan"), dtype=dt, device=DEV)
+    ops.attn_paged_mfma(q2, out2, dk2, dv2, table.to(DEV), *seg, max_qlen=1, max_kv_len=max(lengths), splits=splits, **kw_args)
+    assert _rel(out.cpu(), out2.cpu()) < 4e-3
+    # the same cache: every slot but the new tokens' bit for bit as it was, theirs as the two kernels leave them but
+    # for the last bits (the parts of the stack and the squares of a head are added in another order)
+    ka, kb, va, vb = (t.cpu().view(torch.int16).clone() for t in (dk, dk2, dv, dv2))
+    for s_, n in enumerate(cached):
+        page, at = int(table[s_, n // P]), n % P
+        assert _rel(dk[page, :, at].cpu(), dk2[page, :, at].cpu()) < 8e-3
+        assert _rel(dv[page, :, :, at].cpu(), dv2[page, :, :, at].cpu()) < 8e-3
+        ka[page, :, at] = kb[page, :, at] = 0
+        va[page, :, :, at] = vb[page, :, :, at] = 0
+    assert torch.equal(ka, kb) and torch.equal(va, vb)
+
+
 @pytest.mark.parametrize("groups,heads", [(1, 24), (2, 12)])
 @pytest.mark.parametrize("parts", [None, 2])
 def test_attention_portions_dealt_out_before_the_launch_or_taken_from_the_counter(groups, heads, parts):
