@@ -110,13 +110,21 @@ __device__ __forceinline__ float group_sum4(float v) {
 // The one wave of a (segment, kv head) whose keys end with the new token's does the same for its k head, takes the
 // v head as it is, writes both into the cache and puts them where the loads of the last block would have brought
 // them (the slot in the page still holds what was there before).  A layer of a decode step is one kernel shorter.
-template <int NT, int DMAX, bool EXACT, bool PREP = false>
-__global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
+//
+// INWG (NT == 1, up to four splits): the waves of a (segment, kv head) that share its keys are one workgroup, wave s
+// takes split s, and at the end wave 0 takes the others' sums and statistics from LDS and writes the result: no
+// partial results in memory and no merge kernel.  For launches with a workgroup for every compute unit without it
+// (many requests, few splits); with fewer, one-wave workgroups spread the same waves over more compute units.
+constexpr int kInWgWavesMax = 4;
+template <int NT, int DMAX, bool EXACT, bool PREP = false, bool INWG = false>
+__global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfma_kernel(const AttnArgs a) {
   static_assert(!PREP || (NT == 1 && EXACT), "the folded preparation is written for one row tile and a head_dim known here");
+  static_assert(!INWG || NT == 1, "the merge inside the workgroup is written for one row tile");
   constexpr int DCH = DMAX / 32;  // contraction chunks of the first product
   constexpr int DTL = DMAX / 16;  // d tiles of the output
-  const int lane = threadIdx.x, li = lane & 15, g = lane >> 4;
-  const int seg = blockIdx.z / a.splits, split = blockIdx.z % a.splits;
+  const int lane = threadIdx.x & (kWave - 1), li = lane & 15, g = lane >> 4;
+  const int seg = INWG ? static_cast<int>(blockIdx.z) : static_cast<int>(blockIdx.z) / a.splits;
+  const int split = INWG ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6) : static_cast<int>(blockIdx.z) % a.splits;
   const int kvh = blockIdx.y;
   const int G = a.nq / a.nkv;
   const int row0 = a.seg_row0[seg];
@@ -574,12 +582,45 @@ __global__ __launch_bounds__(kWave) void attn_mfma_kernel(const AttnArgs a) {
     }
   }
 
+  if constexpr (INWG) {
+    // the waves 1 .. splits - 1 hand their sums to wave 0, lane to lane (a lane holds the same rows and columns in
+    // every wave): out = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m), added in the order of the splits
+    constexpr int kPitch = 4 * DTL + 4;   // floats a lane: its sums, m and l, and padding to 16 bytes
+    __shared__ __align__(16) float handed[kInWgWavesMax - 1][kWave][kPitch];
+    if (split > 0) {
+      float* mine = handed[split - 1][lane];
+#pragma unroll
+      for (int dt = 0; dt < DTL; ++dt)
+        *reinterpret_cast<float4*>(mine + 4 * dt) = float4{acc[0][dt][0], acc[0][dt][1], acc[0][dt][2], acc[0][dt][3]};
+      *reinterpret_cast<float2*>(mine + 4 * DTL) = float2{m[0], l[0]};
+    }
+    __syncthreads();
+    if (split > 0) return;
+    for (int w = 1; w < a.splits; ++w) {
+      const float* theirs = handed[w - 1][lane];
+      const float2 ml = *reinterpret_cast<const float2*>(theirs + 4 * DTL);
+      const float m_all = fmaxf(m[0], ml.x);
+      const float m_ref = m_all == -INFINITY ? 0.f : m_all;
+      const float f0 = exp2f(m[0] - m_ref), f1 = exp2f(ml.x - m_ref);
+      l[0] = l[0] * f0 + ml.y * f1;
+      m[0] = m_all;
+#pragma unroll
+      for (int dt = 0; dt < DTL; ++dt) {
+        const float4 v = *reinterpret_cast<const float4*>(theirs + 4 * dt);
+        acc[0][dt][0] = acc[0][dt][0] * f0 + v.x * f1;
+        acc[0][dt][1] = acc[0][dt][1] * f0 + v.y * f1;
+        acc[0][dt][2] = acc[0][dt][2] * f0 + v.z * f1;
+        acc[0][dt][3] = acc[0][dt][3] * f0 + v.w * f1;
+      }
+    }
+  }
+
   // acc[n][dt][r] is O^T[d = 16dt + 4g + r][row (n, li)]
 #pragma unroll
   for (int n = 0; n < NT; ++n) {
     if (!row_ok[n]) continue;
     const int64_t tok_row = row0 + my_tok[n];
-    if (a.splits == 1) {
+    if (INWG || a.splits == 1) {
       const float inv_l = l[n] > 0.f ? 1.0f / l[n] : 0.f;
       uint16_t* op = a.out + tok_row * a.o_stride + my_head[n] * D;
 #pragma unroll
@@ -2116,6 +2157,20 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
   return launch_status();
 }
 
+static int g_decode_inwg = -1;   // the splits of a decode step inside one workgroup: -1 by the rule, 0 never, 1 whenever they fit
+extern "C" void arle_attn_decode_inwg(int mode) { g_decode_inwg = mode; }
+
+static int compute_units() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cus = n;
+  }
+  return cus;
+}
+
 // A step of single decoded tokens with the preparation of q, k and v folded into the attention: segment s is the
 // one token row s.  parts: the fused q|k|v projection of the step as n_parts float32 partial products
 // [token rows][(nq + 2 nkv) D] (part_stride elements apart, rows row_stride apart; both multiples of 4, parts
@@ -2158,6 +2213,17 @@ extern "C" int arle_attn_decode_prep(const float* parts, int n_parts, long long 
   a.prep_eps = eps;
   a.prep_k_pages = static_cast<uint16_t*>(k_pages);
   a.prep_v_pages = static_cast<uint16_t*>(v_pages);
+  // two to four splits and a workgroup for every compute unit even so: the splits of a (segment, kv head) share a
+  // workgroup and merge in LDS (measured on MI355X at the Qwen3-4B widths, 64 requests at 2,048 tokens in two splits)
+  if (splits > 1 && splits <= kInWgWavesMax && g_decode_inwg != 0 &&
+      (g_decode_inwg > 0 || static_cast<long long>(segments) * nkv >= compute_units())) {
+    const dim3 grid(1, nkv, static_cast<unsigned>(segments));
+    if (D == 128)
+      attn_mfma_kernel<1, 128, true, true, true><<<grid, splits * kWave, 0, s>>>(a);
+    else
+      attn_mfma_kernel<1, 64, true, true, true><<<grid, splits * kWave, 0, s>>>(a);
+    return launch_status();
+  }
   const dim3 grid(1, nkv, static_cast<unsigned>(z));
   if (D == 128)
     attn_mfma_kernel<1, 128, true, true><<<grid, kWave, 0, s>>>(a);

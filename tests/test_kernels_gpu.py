@@ -652,7 +652,8 @@ def test_attention_portions_list_their_work_once_for_calls_that_name_the_same_st
 @pytest.mark.parametrize("nq,nkv,D,rot,P", [(32, 8, 128, 128, 16), (8, 8, 64, 64, 8), (16, 1, 128, 64, 64), (6, 2, 64, 0, 4),
                                             (4, 4, 128, 0, 32), (12, 2, 128, 128, 128)])
 @pytest.mark.parametrize("n_parts,splits,window,w_dtype", [(1, 1, 0, torch.bfloat16), (4, None, 0, torch.float32),
-                                                           (3, 5, 37, torch.bfloat16), (7, 64, 0, None)])
+                                                           (3, 5, 37, torch.bfloat16), (7, 64, 0, None),
+                                                           (2, 3, 0, torch.bfloat16), (5, 2, 37, torch.float32), (1, 4, 0, None)])
 def test_decode_attention_with_the_preparation_folded_in(nq, nkv, D, rot, P, n_parts, splits, window, w_dtype):
     """A step of single decoded tokens from the float32 stack of its q|k|v projection: sum, per-head norm, rotation,
     cache write and attention in one kernel.  Requests whose new token is the first of all, the first or last of
@@ -707,6 +708,24 @@ def test_decode_attention_with_the_preparation_folded_in(nq, nkv, D, rot, P, n_p
     ops.attn_decode_prep(stack.to(DEV), out, dk, dv, table.to(DEV), *seg, max_kv_len=max(lengths), eps=eps, q_weight=dev(qw),
                          k_weight=dev(kw), cos=dev(cos), sin=dev(sin), rotary_dim=rot, splits=splits, **kw_args)
     assert torch.isfinite(out.float()).all()
+    if splits in (2, 3, 4):
+        # the splits of a request's keys as the waves of one workgroup that merge in LDS, and as workgroups of their own
+        # whose parts a second kernel merges: here both are forced in turn
+        from arle_amd.kernels import lib
+        both = []
+        try:
+            for mode in (1, 0):
+                lib.function("arle_attn_decode_inwg")(mode)
+                o_ = torch.full((T, Q), float("nan"), dtype=dt, device=DEV)
+                ops.attn_decode_prep(stack.to(DEV), o_, k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), *seg,
+                                     max_kv_len=max(lengths), eps=eps, q_weight=dev(qw), k_weight=dev(kw), cos=dev(cos),
+                                     sin=dev(sin), rotary_dim=rot, splits=splits, **kw_args)
+                both.append(o_.cpu())
+        finally:
+            lib.function("arle_attn_decode_inwg")(-1)
+        for o_ in both:
+            assert torch.isfinite(o_.float()).all() and _rel(o_, torch.stack(wants)) < 1e-2
+        assert _rel(both[0], both[1]) < 4e-3 and torch.equal(out.cpu(), both[1] if T * nkv < 256 else both[0])
     # the stack's own sum is what the kernel saw: compare with plain values made from it
     for s_, n in enumerate(cached):
         x = exact[s_]
