@@ -687,14 +687,26 @@ __global__ __launch_bounds__(kMergeWaves* kWave) void attn_merge_kernel(
   float4 o = {0.f, 0.f, 0.f, 0.f};
   const bool mine = d0 < D;
   const float* src = ws_o + base * D + (mine ? d0 : 0);
-#pragma unroll 8
-  for (int s = wave; s < splits; s += kMergeWaves) {
-    const float w = __shfl(wgt, s, kWave);  // every lane takes part in the cross-lane read
-    const float4 v = *reinterpret_cast<const float4*>(src + static_cast<int64_t>(s) * D);
-    o.x += v.x * w;
-    o.y += v.y * w;
-    o.z += v.z * w;
-    o.w += v.w * w;
+  // rounds of four splits a wave, their loads without a condition (a split past the last one is fetched from the
+  // last and weighs nothing): in a loop of single splits every load was waited for before the next one went out
+  constexpr int kRound = 4;
+  for (int s0 = wave; s0 < splits; s0 += kRound * kMergeWaves) {
+    float4 v[kRound];
+    float w[kRound];
+#pragma unroll
+    for (int j = 0; j < kRound; ++j) {
+      const int sj = s0 + j * kMergeWaves, sc = min(sj, splits - 1);
+      v[j] = *reinterpret_cast<const float4*>(src + static_cast<int64_t>(sc) * D);
+      const float got = __shfl(wgt, sc, kWave);  // every lane takes part in the cross-lane read
+      w[j] = sj < splits ? got : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < kRound; ++j) {
+      o.x += v[j].x * w[j];
+      o.y += v[j].y * w[j];
+      o.z += v[j].z * w[j];
+      o.w += v[j].w * w[j];
+    }
   }
   if (mine) *reinterpret_cast<float4*>(&part[wave][d0]) = o;
   __syncthreads();
