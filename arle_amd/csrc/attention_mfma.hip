@@ -68,7 +68,8 @@ struct AttnArgs {
   long long plan_token;  // names the step for the portions kernels' list of work (0: no name, plan every time)
   // The kernel that prepares q, k and v itself (PREP; steps of single decoded tokens): the fused q|k|v projection
   // comes as a stack of float32 partial products [prep_n][token rows][(nq + 2 nkv) D], q is unused.
-  const float* prep_parts;
+  const void* prep_parts;   // float32, or with prep_bf16 the projection itself in bfloat16 (prep_n 1)
+  int prep_bf16;
   int prep_n;
   int64_t prep_part_stride, prep_row_stride;  // elements between the parts, and between the rows of a part
   const void* prep_qw;   // per-head norm weights [D] of q and k (null: no norm), float32 if prep_w_f32 else bfloat16
@@ -253,7 +254,11 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
   if constexpr (PREP) {
     constexpr int HC = DCH / 2;                 // chunks of 32 columns that half of a head holds
     const int hc = a.prep_rot / 64;             // and that half of the rotated width holds
-    const float* prow = a.prep_parts + static_cast<int64_t>(row0) * a.prep_row_stride;  // the segment's one token
+    // the segment's one token: element `index` of its row (float32 parts, or one bfloat16 row) at spot(index)
+    const int elem = a.prep_bf16 ? 2 : 4;
+    const unsigned char* prow = static_cast<const unsigned char*>(a.prep_parts) + static_cast<int64_t>(row0) * a.prep_row_stride * elem;
+    auto spot = [&](int64_t index) { return prow + index * elem; };
+    const unsigned char* somewhere = reinterpret_cast<const unsigned char*>(a.k_pages);   // a page: 512 bytes at least
     const int n_parts = a.prep_n;
     // Every load of this prologue is issued without a condition around it (a load under a condition is waited for at
     // the end of its branch, and the loads behind it wait with it): what is not needed is fetched from a place
@@ -266,13 +271,31 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
     // its parts in ascending order; the lanes' sums then meet pairwise, the lanes 8, 4, 2, 1 apart in turn (rotations
     // of the 16 lanes i), which leaves every lane that holds the head with the same total: one fixed order, whatever
     // else the step holds.
+    // (two loads of 16 bytes a chunk either way: the second one of a bfloat16 row is the first one again)
     auto fetch_part = [&](int col0, int u, float4 (&got)[DCH][2]) {
-      const float* pu = prow + col0 + 8 * g + static_cast<int64_t>(min(u, n_parts - 1)) * a.prep_part_stride;
+      const int64_t first = col0 + 8 * g + static_cast<int64_t>(min(u, n_parts - 1)) * a.prep_part_stride;
 #pragma unroll
       for (int c = 0; c < DCH; ++c) {
-        got[c][0] = *reinterpret_cast<const float4*>(pu + 32 * c);
-        got[c][1] = *reinterpret_cast<const float4*>(pu + 32 * c + 4);
+        const unsigned char* at = spot(first + 32 * c);
+        const uint4 lo = *reinterpret_cast<const uint4*>(at), hi = *reinterpret_cast<const uint4*>(at + (a.prep_bf16 ? 0 : 16));
+        const uint32_t wl[4] = {lo.x, lo.y, lo.z, lo.w}, wh[4] = {hi.x, hi.y, hi.z, hi.w};
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const uint32_t pair = wl[e >> 1];
+          const uint32_t narrow = (e & 1) ? pair & 0xffff0000u : pair << 16;
+          v[e] = __uint_as_float(a.prep_bf16 ? narrow : (e < 4 ? wl[e & 3] : wh[e & 3]));
+        }
+        got[c][0] = float4{v[0], v[1], v[2], v[3]};
+        got[c][1] = float4{v[4], v[5], v[6], v[7]};
       }
+    };
+    // one column of the token's row (a value): a load of four bytes either way
+    auto fetch_one = [&](int64_t index) {
+      const unsigned char* at = spot(index);
+      const uint32_t raw = *reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(at) & ~static_cast<uintptr_t>(3));
+      const uint32_t narrow = (reinterpret_cast<uintptr_t>(at) & 2) ? raw & 0xffff0000u : raw << 16;
+      return __uint_as_float(a.prep_bf16 ? narrow : raw);
     };
     // x = the lane's parts added up (the first round's loads are `got`); mine, apart: the lane's first part and the
     // distance to its next
@@ -307,11 +330,11 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
     // a head's norm weights as this lane holds the head, bfloat16 or float32 in memory: two loads of 16 bytes either
     // way (the second one of bfloat16 weights is the first one again), sorted out afterwards
     auto fetch_weights = [&](const void* w, uint4 (&raw)[DCH][2]) {
-      const unsigned char* base = static_cast<const unsigned char*>(w != nullptr ? w : a.prep_parts);
-      const int elem = a.prep_w_f32 ? 4 : 2;
+      const unsigned char* base = w != nullptr ? static_cast<const unsigned char*>(w) : somewhere;
+      const int w_elem = a.prep_w_f32 ? 4 : 2;
 #pragma unroll
       for (int c = 0; c < DCH; ++c) {
-        const unsigned char* at = base + static_cast<size_t>(32 * c + 8 * g) * elem;
+        const unsigned char* at = base + static_cast<size_t>(32 * c + 8 * g) * w_elem;
         raw[c][0] = *reinterpret_cast<const uint4*>(at);
         raw[c][1] = *reinterpret_cast<const uint4*>(at + (a.prep_w_f32 ? 16 : 0));
       }
@@ -328,8 +351,8 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
     float cs[HC > 0 ? HC : 1][8], sn[HC > 0 ? HC : 1][8];
     {
       const bool turns = hc > 0;
-      const float* ct = turns ? a.prep_cos + static_cast<int64_t>(start) * (a.prep_rot / 2) : prow;
-      const float* st = turns ? a.prep_sin + static_cast<int64_t>(start) * (a.prep_rot / 2) : prow;
+      const float* ct = turns ? a.prep_cos + static_cast<int64_t>(start) * (a.prep_rot / 2) : reinterpret_cast<const float*>(somewhere);
+      const float* st = turns ? a.prep_sin + static_cast<int64_t>(start) * (a.prep_rot / 2) : reinterpret_cast<const float*>(somewhere);
 #pragma unroll
       for (int c = 0; c < HC; ++c) {
         const int at = 32 * min(c, max(hc - 1, 0)) + 8 * g;
@@ -388,7 +411,7 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
     const int q_col = (kvh * G + min(li & (gp - 1), G - 1)) * DMAX;    // live rows (i < G) take their own head
     const int k_col = (a.nq + kvh) * DMAX;
     const int v_mine = g & (vp - 1);
-    const float* pv = prow + (a.nq + a.nkv + kvh) * DMAX + li;
+    const int64_t v_col = static_cast<int64_t>(a.nq + a.nkv + kvh) * DMAX + li;
     float xq[DCH][8];
     float4 gq[DCH][2];
     uint4 wq[DCH][2];
@@ -406,7 +429,7 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
       fetch_weights(a.prep_kw, wk);
       fetch_part(k_col, li & (kp - 1), gk);
 #pragma unroll
-      for (int dt = 0; dt < DTL; ++dt) vgot[dt] = pv[static_cast<int64_t>(min(v_mine, n_parts - 1)) * a.prep_part_stride + 16 * dt];
+      for (int dt = 0; dt < DTL; ++dt) vgot[dt] = fetch_one(v_col + static_cast<int64_t>(min(v_mine, n_parts - 1)) * a.prep_part_stride + 16 * dt);
     }
     add_parts(q_col, li / gp, 16 / gp, gq, xq);
     if (n_parts > 1) meet(xq, 8, gp);
@@ -420,7 +443,7 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
       for (int base = vp; base < n_parts; base += vp) {
         const int u = base + v_mine;
 #pragma unroll
-        for (int dt = 0; dt < DTL; ++dt) vgot[dt] = pv[static_cast<int64_t>(min(u, n_parts - 1)) * a.prep_part_stride + 16 * dt];
+        for (int dt = 0; dt < DTL; ++dt) vgot[dt] = fetch_one(v_col + static_cast<int64_t>(min(u, n_parts - 1)) * a.prep_part_stride + 16 * dt);
 #pragma unroll
         for (int dt = 0; dt < DTL; ++dt) vsum[dt] += u < n_parts ? vgot[dt] : 0.f;
       }
@@ -2049,6 +2072,7 @@ static AttnArgs make_args(const void* q, long long q_stride, void* out, long lon
   a.pws_ml = nullptr;
   a.rows_max = 0;
   a.prep_parts = nullptr;
+  a.prep_bf16 = 0;
   a.prep_n = 0;
   a.prep_part_stride = a.prep_row_stride = 0;
   a.prep_qw = a.prep_kw = nullptr;
@@ -2185,14 +2209,14 @@ static int compute_units() {
 
 // A step of single decoded tokens with the preparation of q, k and v folded into the attention: segment s is the
 // one token row s.  parts: the fused q|k|v projection of the step as n_parts float32 partial products
-// [token rows][(nq + 2 nkv) D] (part_stride elements apart, rows row_stride apart; both multiples of 4, parts
-// 16-byte aligned), added in order.  q_w / k_w: per-head norm weights [D] (both or neither; float32 if w_f32, else
+// [token rows][(nq + 2 nkv) D] (part_stride elements apart, rows row_stride apart; both multiples of 8, parts
+// 16-byte aligned), added in order; or, with parts_bf16, the projection itself in bfloat16 (n_parts 1).  q_w / k_w: per-head norm weights [D] (both or neither; float32 if w_f32, else
 // bfloat16; 16-byte aligned), eps inside the root.  cos / sin: float32 [positions][rot / 2], rot 0 (no rotation) or a
 // multiple of 64 up to D.  The new token's key and value are written to its slot of the pages (which the block table
 // must already hold) and take part in the attention from registers.  D 64 or 128, nq / nkv <= 16; everything else
 // as arle_attn_paged_mfma with max_qlen 1.  The same results as arle_qk_prep followed by arle_attn_paged_mfma but
 // for the order in which a head's squares are added for its norm.
-extern "C" int arle_attn_decode_prep(const float* parts, int n_parts, long long part_stride, long long row_stride,
+extern "C" int arle_attn_decode_prep(const void* parts, int parts_bf16, int n_parts, long long part_stride, long long row_stride,
                                      const void* q_w, const void* k_w, int w_f32, const float* cos_t, const float* sin_t,
                                      int rot, float eps, void* out, long long o_stride, void* k_pages, void* v_pages,
                                      const int* block_table, int table_stride, const int* seg_row0, const int* seg_slot,
@@ -2202,7 +2226,8 @@ extern "C" int arle_attn_decode_prep(const float* parts, int n_parts, long long 
   auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
   if ((D != 64 && D != 128) || page_size < 4 || (page_size & (page_size - 1)) != 0 || nkv <= 0 || nq % nkv != 0 ||
       nq / nkv > 16 || splits < 1 || splits > 64 || (splits > 1 && (ws_o == nullptr || ws_ml == nullptr)) ||
-      parts == nullptr || n_parts < 1 || part_stride % 4 != 0 || row_stride % 4 != 0 || !aligned(parts) ||
+      parts == nullptr || n_parts < 1 || (parts_bf16 && n_parts != 1) || part_stride % 8 != 0 || row_stride % 8 != 0 ||
+      !aligned(parts) ||
       (q_w == nullptr) != (k_w == nullptr) || !aligned(q_w) || !aligned(k_w) || rot < 0 || rot > D || rot % 64 != 0 ||
       (rot > 0 && (cos_t == nullptr || sin_t == nullptr || !aligned(cos_t) || !aligned(sin_t))) ||
       k_pages == nullptr || v_pages == nullptr || !aligned(k_pages))
@@ -2213,6 +2238,7 @@ extern "C" int arle_attn_decode_prep(const float* parts, int n_parts, long long 
   AttnArgs a = make_args(nullptr, 0, out, o_stride, k_pages, v_pages, block_table, table_stride, seg_row0, seg_slot,
                          seg_start, 1, nq, nkv, D, page_size, scale, window, splits, ws_o, ws_ml);
   a.prep_parts = parts;
+  a.prep_bf16 = parts_bf16;
   a.prep_n = n_parts;
   a.prep_part_stride = part_stride;
   a.prep_row_stride = row_stride;

@@ -39,7 +39,7 @@ SIGNATURES = {
                                  _i, _p, _p, _i, _i, _i, _i, _i, _f, _p, _i, _ll, _ll, _p]),
     "arle_attn_paged_simt": ("attention_simt", [_p, _ll, _p, _ll, _p, _p, _i, _p, _i, _p, _p, _p, _i,
                                                 _i, _i, _i, _i, _f, _i, _p]),
-    "arle_attn_decode_prep": ("attention_mfma", [_p, _i, _ll, _ll, _p, _p, _i, _p, _p, _i, _f, _p, _ll, _p, _p, _p, _i, _p,
+    "arle_attn_decode_prep": ("attention_mfma", [_p, _i, _i, _ll, _ll, _p, _p, _i, _p, _p, _i, _f, _p, _ll, _p, _p, _p, _i, _p,
                                                  _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p, _p, _p]),
     "arle_attn_decode_inwg": ("attention_mfma", [_i]),
     "arle_attn_prefill_variant": ("attention_mfma", [_i]),

@@ -460,16 +460,23 @@ def attn_decode_prep(parts, out, k_pages, v_pages, block_table, seg_row0, seg_sl
                      q_weight=None, k_weight=None, cos=None, sin=None, rotary_dim: int = 0, window: int = 0,
                      splits: int | None = None):
     """A step of single decoded tokens (segment s is token row s) from the float32 stack of partial products
-    [S, T, (nq + 2 nkv) D] of its fused q|k|v projection: what qk_prep and attn_paged_mfma do one after the other,
-    in the attention's own kernel.  Every wave sums, norms and rotates its q heads itself; the wave whose keys end
+    [S, T, (nq + 2 nkv) D] of its fused q|k|v projection, or from the projection itself in bfloat16 [T, (nq + 2 nkv) D]:
+    what qk_prep and attn_paged_mfma do one after the other, in the attention's own kernel.  Every wave sums, norms and rotates its q heads itself; the wave whose keys end
     with the new token's does the same for the k head, writes key and value into the cache and uses them from its
     registers.  out: bfloat16 [T, nq*D]."""
     _gpu(parts, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, q_weight, k_weight, cos, sin)
     group = num_q_heads // max(num_kv_heads, 1)
     width = (num_q_heads + 2 * num_kv_heads) * head_dim
-    _need(parts.dtype == torch.float32 and parts.dim() == 3 and parts.shape[0] >= 1 and parts.shape[2] == width
-          and parts.is_contiguous(), f"parts must be contiguous float32 [S, T, {width}]")
-    tokens = parts.shape[1]
+    whole = parts.dim() == 2     # the projection itself, not a stack of parts
+    if whole:
+        _rows(parts, "parts")
+        _need(parts.dtype == torch.bfloat16 and parts.shape[1] == width and parts.stride(0) % 8 == 0
+              and parts.data_ptr() % 16 == 0, f"a whole projection must be bfloat16 [T, {width}] with 16-byte aligned rows")
+        n_parts, part_stride, row_stride, tokens = 1, 0, parts.stride(0), parts.shape[0]
+    else:
+        _need(parts.dtype == torch.float32 and parts.dim() == 3 and parts.shape[0] >= 1 and parts.shape[2] == width
+              and parts.is_contiguous(), f"parts must be contiguous float32 [S, T, {width}]")
+        n_parts, part_stride, row_stride, tokens = parts.shape[0], parts.stride(0), parts.stride(1), parts.shape[1]
     _need(out.dtype == torch.bfloat16 and out.shape == (tokens, num_q_heads * head_dim) and out.is_contiguous(),
           "out must be contiguous bfloat16 [T, nq*D]")
     _need(num_kv_heads > 0 and num_q_heads % num_kv_heads == 0, "q heads must be a multiple of kv heads")
@@ -505,7 +512,7 @@ def attn_decode_prep(parts, out, k_pages, v_pages, block_table, seg_row0, seg_sl
     if splits > 1:
         ws_o = torch.empty((segments, num_q_heads, splits, head_dim), dtype=torch.float32, device=out.device)
         ws_ml = torch.empty((segments, num_q_heads, splits, 2), dtype=torch.float32, device=out.device)
-    lib.call("arle_attn_decode_prep", parts.data_ptr(), parts.shape[0], parts.stride(0), parts.stride(1), _ptr(q_weight),
+    lib.call("arle_attn_decode_prep", parts.data_ptr(), int(whole), n_parts, part_stride, row_stride, _ptr(q_weight),
              _ptr(k_weight), w_f32, _ptr(cos), _ptr(sin), int(rotary_dim), float(eps), out.data_ptr(), out.stride(0),
              k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], seg_row0.data_ptr(),
              seg_slot.data_ptr(), seg_start.data_ptr(), segments, num_q_heads, num_kv_heads, head_dim, page_size,

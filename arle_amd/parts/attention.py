@@ -116,7 +116,8 @@ class PagedAttention(Part):
                             k_pages=cache.k_pages, v_pages=cache.v_pages, page_size=cache.page_size)
         # the fused preparation kernel can add a stack of partial products itself
         projected = (self.qkv if cache.writes else self.q_only)(x, partials_ok=fused)
-        if (projected.dim() == 3 and cache.writes and batch.max_qlen == 1 and self.folds_preparation
+        if (fused and cache.writes and batch.max_qlen == 1 and self.folds_preparation
+                and (projected.dim() == 3 or projected.dtype == torch.bfloat16)
                 and ops.attn_decode_prep_supported(x.dtype, self.D, cache.page_size, self.nq // self.nkv, rot)):
             # single decoded tokens: the attention's kernel sums, norms, rotates and writes to the cache itself
             out = torch.empty((x.shape[0], Q), dtype=x.dtype, device=x.device)

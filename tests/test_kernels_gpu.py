@@ -653,7 +653,8 @@ def test_attention_portions_list_their_work_once_for_calls_that_name_the_same_st
                                             (4, 4, 128, 0, 32), (12, 2, 128, 128, 128)])
 @pytest.mark.parametrize("n_parts,splits,window,w_dtype", [(1, 1, 0, torch.bfloat16), (4, None, 0, torch.float32),
                                                            (3, 5, 37, torch.bfloat16), (7, 64, 0, None),
-                                                           (2, 3, 0, torch.bfloat16), (5, 2, 37, torch.float32), (1, 4, 0, None)])
+                                                           (2, 3, 0, torch.bfloat16), (5, 2, 37, torch.float32), (1, 4, 0, None),
+                                                           (0, None, 0, torch.bfloat16), (0, 3, 37, torch.float32)])
 def test_decode_attention_with_the_preparation_folded_in(nq, nkv, D, rot, P, n_parts, splits, window, w_dtype):
     """A step of single decoded tokens from the float32 stack of its q|k|v projection: sum, per-head norm, rotation,
     cache write and attention in one kernel.  Requests whose new token is the first of all, the first or last of
@@ -696,9 +697,13 @@ def test_decode_attention_with_the_preparation_folded_in(nq, nkv, D, rot, P, n_p
                                             rows=[n])[n].reshape(-1))
         new_rows.append(raw[n])
     row = torch.stack(new_rows)                                      # [T, width] float32
-    stack = torch.randn(n_parts, T, row.shape[1], generator=_g(503))
-    stack[-1] = row - (stack[:-1].double().sum(0)).float() if n_parts > 1 else row
-    exact = stack.double().sum(0)
+    if n_parts == 0:       # the projection itself in bfloat16 instead of a stack of its parts
+        stack = row.to(dt)
+        exact = stack.double()
+    else:
+        stack = torch.randn(n_parts, T, row.shape[1], generator=_g(503))
+        stack[-1] = row - (stack[:-1].double().sum(0)).float() if n_parts > 1 else row
+        exact = stack.double().sum(0)
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
     dev = lambda t: None if t is None else t.to(DEV)
     seg = (i32(list(range(T + 1))), i32(list(range(T))), i32(cached))
@@ -736,10 +741,16 @@ def test_decode_attention_with_the_preparation_folded_in(nq, nkv, D, rot, P, n_p
     assert _rel(out.cpu(), torch.stack(wants)) < 1e-2
     # the two kernels that it stands for
     dk2, dv2 = k_pages.to(DEV), v_pages.to(DEV)
-    q2 = torch.empty((T, Q), dtype=dt, device=DEV)
-    ops.qk_prep(q2, None, None, num_q_heads=nq, num_kv_heads=nkv, head_dim=D, eps=eps, q_weight=dev(qw), k_weight=dev(kw),
-                cos=dev(cos), sin=dev(sin), rotary_dim=rot, positions=seg[2], slot_of_token=seg[1], block_table=table.to(DEV),
-                k_pages=dk2, v_pages=dv2, page_size=P, parts=stack.to(DEV))
+    prep_args = dict(num_q_heads=nq, num_kv_heads=nkv, head_dim=D, eps=eps, q_weight=dev(qw), k_weight=dev(kw), cos=dev(cos),
+                     sin=dev(sin), rotary_dim=rot, positions=seg[2], slot_of_token=seg[1], block_table=table.to(DEV),
+                     k_pages=dk2, v_pages=dv2, page_size=P)
+    if n_parts == 0:
+        qkv2 = stack.to(DEV)
+        q2 = qkv2[:, :Q]
+        ops.qk_prep(q2, qkv2[:, Q:Q + KV], qkv2[:, Q + KV:], **prep_args)
+    else:
+        q2 = torch.empty((T, Q), dtype=dt, device=DEV)
+        ops.qk_prep(q2, None, None, parts=stack.to(DEV), **prep_args)
     out2 = torch.full((T, Q), float("nan"), dtype=dt, device=DEV)
     ops.attn_paged_mfma(q2, out2, dk2, dv2, table.to(DEV), *seg, max_qlen=1, max_kv_len=max(lengths), splits=splits, **kw_args)
     assert _rel(out.cpu(), out2.cpu()) < 4e-3
