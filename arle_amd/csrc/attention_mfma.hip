@@ -112,12 +112,14 @@ __device__ __forceinline__ float group_sum4(float v) {
 // v head as it is, writes both into the cache and puts them where the loads of the last block would have brought
 // them (the slot in the page still holds what was there before).  A layer of a decode step is one kernel shorter.
 //
+// WHOLE_IN: the projection comes whole, in bfloat16, instead of as a stack of float32 parts.
+//
 // INWG (NT == 1, up to four splits): the waves of a (segment, kv head) that share its keys are one workgroup, wave s
 // takes split s, and at the end wave 0 takes the others' sums and statistics from LDS and writes the result: no
 // partial results in memory and no merge kernel.  For launches with a workgroup for every compute unit without it
 // (many requests, few splits); with fewer, one-wave workgroups spread the same waves over more compute units.
 constexpr int kInWgWavesMax = 4;
-template <int NT, int DMAX, bool EXACT, bool PREP = false, bool INWG = false>
+template <int NT, int DMAX, bool EXACT, bool PREP = false, bool INWG = false, bool WHOLE_IN = false>
 __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfma_kernel(const AttnArgs a) {
   static_assert(!PREP || (NT == 1 && EXACT), "the folded preparation is written for one row tile and a head_dim known here");
   static_assert(!INWG || NT == 1, "the merge inside the workgroup is written for one row tile");
@@ -255,7 +257,7 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
     constexpr int HC = DCH / 2;                 // chunks of 32 columns that half of a head holds
     const int hc = a.prep_rot / 64;             // and that half of the rotated width holds
     // the segment's one token: element `index` of its row (float32 parts, or one bfloat16 row) at spot(index)
-    const int elem = a.prep_bf16 ? 2 : 4;
+    const int elem = WHOLE_IN ? 2 : 4;
     const unsigned char* prow = static_cast<const unsigned char*>(a.prep_parts) + static_cast<int64_t>(row0) * a.prep_row_stride * elem;
     auto spot = [&](int64_t index) { return prow + index * elem; };
     const unsigned char* somewhere = reinterpret_cast<const unsigned char*>(a.k_pages);   // a page: 512 bytes at least
@@ -271,35 +273,35 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
     // its parts in ascending order; the lanes' sums then meet pairwise, the lanes 8, 4, 2, 1 apart in turn (rotations
     // of the 16 lanes i), which leaves every lane that holds the head with the same total: one fixed order, whatever
     // else the step holds.
-    // (two loads of 16 bytes a chunk either way: the second one of a bfloat16 row is the first one again)
-    auto fetch_part = [&](int col0, int u, float4 (&got)[DCH][2]) {
+    // (two loads of 16 bytes a chunk either way: the second one of a bfloat16 row is the first one again; what
+    // they brought is only looked at where it is added, so that no load waits for the one before it)
+    auto fetch_part = [&](int col0, int u, uint4 (&got)[DCH][2]) {
       const int64_t first = col0 + 8 * g + static_cast<int64_t>(min(u, n_parts - 1)) * a.prep_part_stride;
 #pragma unroll
       for (int c = 0; c < DCH; ++c) {
         const unsigned char* at = spot(first + 32 * c);
-        const uint4 lo = *reinterpret_cast<const uint4*>(at), hi = *reinterpret_cast<const uint4*>(at + (a.prep_bf16 ? 0 : 16));
-        const uint32_t wl[4] = {lo.x, lo.y, lo.z, lo.w}, wh[4] = {hi.x, hi.y, hi.z, hi.w};
-        float v[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const uint32_t pair = wl[e >> 1];
-          const uint32_t narrow = (e & 1) ? pair & 0xffff0000u : pair << 16;
-          v[e] = __uint_as_float(a.prep_bf16 ? narrow : (e < 4 ? wl[e & 3] : wh[e & 3]));
-        }
-        got[c][0] = float4{v[0], v[1], v[2], v[3]};
-        got[c][1] = float4{v[4], v[5], v[6], v[7]};
+        got[c][0] = *reinterpret_cast<const uint4*>(at);
+        got[c][1] = *reinterpret_cast<const uint4*>(at + (WHOLE_IN ? 0 : 16));
       }
     };
-    // one column of the token's row (a value): a load of four bytes either way
+    auto value_of = [&](const uint4 (&got)[DCH][2], int c, int e) {   // c, e are constants where this is called
+      const uint32_t wl[4] = {got[c][0].x, got[c][0].y, got[c][0].z, got[c][0].w};
+      const uint32_t wh[4] = {got[c][1].x, got[c][1].y, got[c][1].z, got[c][1].w};
+      const uint32_t pair = wl[e >> 1];
+      const uint32_t narrow = (e & 1) ? pair & 0xffff0000u : pair << 16;
+      return __uint_as_float(WHOLE_IN ? narrow : (e < 4 ? wl[e & 3] : wh[e & 3]));
+    };
+    // one column of the token's row (a value): a load of four bytes either way, sorted out by one_of
     auto fetch_one = [&](int64_t index) {
-      const unsigned char* at = spot(index);
-      const uint32_t raw = *reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(at) & ~static_cast<uintptr_t>(3));
-      const uint32_t narrow = (reinterpret_cast<uintptr_t>(at) & 2) ? raw & 0xffff0000u : raw << 16;
-      return __uint_as_float(a.prep_bf16 ? narrow : raw);
+      return *reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(spot(index)) & ~static_cast<uintptr_t>(3));
+    };
+    auto one_of = [&](uint32_t raw, int64_t index) {
+      const uint32_t narrow = (index & 1) ? raw & 0xffff0000u : raw << 16;   // rows begin at multiples of eight elements
+      return __uint_as_float(WHOLE_IN ? narrow : raw);
     };
     // x = the lane's parts added up (the first round's loads are `got`); mine, apart: the lane's first part and the
     // distance to its next
-    auto add_parts = [&](int col0, int mine, int apart, float4 (&got)[DCH][2], float (&x)[DCH][8]) {
+    auto add_parts = [&](int col0, int mine, int apart, uint4 (&got)[DCH][2], float (&x)[DCH][8]) {
 #pragma unroll
       for (int c = 0; c < DCH; ++c)
 #pragma unroll
@@ -309,11 +311,9 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
         if (base > 0) fetch_part(col0, u, got);
         const bool there = u < n_parts;
 #pragma unroll
-        for (int c = 0; c < DCH; ++c) {
-          const float4 lo = got[c][0], hi = got[c][1];
-          x[c][0] += there ? lo.x : 0.f, x[c][1] += there ? lo.y : 0.f, x[c][2] += there ? lo.z : 0.f, x[c][3] += there ? lo.w : 0.f;
-          x[c][4] += there ? hi.x : 0.f, x[c][5] += there ? hi.y : 0.f, x[c][6] += there ? hi.z : 0.f, x[c][7] += there ? hi.w : 0.f;
-        }
+        for (int c = 0; c < DCH; ++c)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[c][e] += there ? value_of(got, c, e) : 0.f;
       }
     };
     // x += x of the lane `n` to the side in the row of 16 lanes i (a rotation: row_ror)
@@ -413,8 +413,7 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
     const int v_mine = g & (vp - 1);
     const int64_t v_col = static_cast<int64_t>(a.nq + a.nkv + kvh) * DMAX + li;
     float xq[DCH][8];
-    float4 gq[DCH][2];
-    uint4 wq[DCH][2];
+    uint4 gq[DCH][2], wq[DCH][2];
     fetch_weights(a.prep_qw, wq);
     fetch_part(q_col, li / gp, gq);
     if (b0 < b1) {   // the first keys and values of the cache
@@ -422,9 +421,8 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
       load_v(b0, vraw);
     }
     // the owner's key and value: behind the cache's loads, and waited for behind the arithmetic of q
-    [[maybe_unused]] float4 gk[DCH][2];
-    [[maybe_unused]] uint4 wk[DCH][2];
-    [[maybe_unused]] float vgot[DTL];
+    [[maybe_unused]] uint4 gk[DCH][2], wk[DCH][2];
+    [[maybe_unused]] uint32_t vgot[DTL];
     if (owner) {
       fetch_weights(a.prep_kw, wk);
       fetch_part(k_col, li & (kp - 1), gk);
@@ -439,13 +437,13 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
       add_parts(k_col, li & (kp - 1), kp, gk, xk);
       meet(xk, kp / 2, 1);
 #pragma unroll
-      for (int dt = 0; dt < DTL; ++dt) vsum[dt] = v_mine < n_parts ? vgot[dt] : 0.f;
+      for (int dt = 0; dt < DTL; ++dt) vsum[dt] = v_mine < n_parts ? one_of(vgot[dt], v_col + 16 * dt) : 0.f;
       for (int base = vp; base < n_parts; base += vp) {
         const int u = base + v_mine;
 #pragma unroll
         for (int dt = 0; dt < DTL; ++dt) vgot[dt] = fetch_one(v_col + static_cast<int64_t>(min(u, n_parts - 1)) * a.prep_part_stride + 16 * dt);
 #pragma unroll
-        for (int dt = 0; dt < DTL; ++dt) vsum[dt] += u < n_parts ? vgot[dt] : 0.f;
+        for (int dt = 0; dt < DTL; ++dt) vsum[dt] += u < n_parts ? one_of(vgot[dt], v_col + 16 * dt) : 0.f;
       }
       if (vp > 1) {
         float far[DTL];
@@ -2256,17 +2254,25 @@ extern "C" int arle_attn_decode_prep(const void* parts, int parts_bf16, int n_pa
   if (splits > 1 && splits <= kInWgWavesMax && g_decode_inwg != 0 &&
       (g_decode_inwg > 0 || static_cast<long long>(segments) * nkv >= compute_units())) {
     const dim3 grid(1, nkv, static_cast<unsigned>(segments));
-    if (D == 128)
-      attn_mfma_kernel<1, 128, true, true, true><<<grid, splits * kWave, 0, s>>>(a);
+    if (D == 128 && parts_bf16)
+      attn_mfma_kernel<1, 128, true, true, true, true><<<grid, splits * kWave, 0, s>>>(a);
+    else if (D == 128)
+      attn_mfma_kernel<1, 128, true, true, true, false><<<grid, splits * kWave, 0, s>>>(a);
+    else if (parts_bf16)
+      attn_mfma_kernel<1, 64, true, true, true, true><<<grid, splits * kWave, 0, s>>>(a);
     else
-      attn_mfma_kernel<1, 64, true, true, true><<<grid, splits * kWave, 0, s>>>(a);
+      attn_mfma_kernel<1, 64, true, true, true, false><<<grid, splits * kWave, 0, s>>>(a);
     return launch_status();
   }
   const dim3 grid(1, nkv, static_cast<unsigned>(z));
-  if (D == 128)
-    attn_mfma_kernel<1, 128, true, true><<<grid, kWave, 0, s>>>(a);
+  if (D == 128 && parts_bf16)
+    attn_mfma_kernel<1, 128, true, true, false, true><<<grid, kWave, 0, s>>>(a);
+  else if (D == 128)
+    attn_mfma_kernel<1, 128, true, true, false, false><<<grid, kWave, 0, s>>>(a);
+  else if (parts_bf16)
+    attn_mfma_kernel<1, 64, true, true, false, true><<<grid, kWave, 0, s>>>(a);
   else
-    attn_mfma_kernel<1, 64, true, true><<<grid, kWave, 0, s>>>(a);
+    attn_mfma_kernel<1, 64, true, true, false, false><<<grid, kWave, 0, s>>>(a);
   const int rc = launch_status();
   if (rc != 0 || splits == 1) return rc;
   attn_merge_kernel<<<dim3(segments * a.ws_rows, nq), kMergeWaves * kWave, 0, s>>>(

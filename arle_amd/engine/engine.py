@@ -287,7 +287,7 @@ class Engine:
         sizes = sorted({int(b) for b in (batch_sizes or decode_warmup_sizes(self.cache.max_slots))
                         if 0 < int(b) <= self.cache.free_slot_count})
         longest = max(1, min(int(max_context or self.max_request_tokens), self.max_request_tokens))
-        contexts = sorted({1, longest} | set(range(32, longest + 1, 32)))   # what a part's launches follow changes at some of these
+        contexts = sorted({1, longest} | {1 << k for k in range(1, longest.bit_length()) if (1 << k) <= longest})
         wanted = {}
         for rows in sizes:
             for context in contexts:

@@ -96,25 +96,10 @@ class PagedAttention(Part):
                 ("o", self.o.out_features, self.o.in_features, False, "norm")]
 
     def decode_launch_class(self, rows, max_context):
-        # the split-KV factor of the matrix-core kernel is the one launch dimension that follows the context, and
-        # with it whether the preparation of q, k and v is folded into that kernel
+        # the split-KV factor of the matrix-core kernel is the one launch dimension that follows the context
         if self.rt.is_f32 or self.D % 16 or self.D > ops.MFMA_MAX_HEAD_DIM:
             return None
-        splits = ops.decode_splits(rows, self.nkv, max_context)
-        return splits, self._folds(max_context, splits)
-
-    _FOLD_MIN_BLOCKS = 4    # blocks of 32 keys a wave from which the folded kernel is ahead
-
-    def _folds(self, max_context, splits) -> bool:
-        """Whether a step of single decoded tokens prepares q, k and v inside the attention's kernel.  The folded
-        kernel's longer head is paid by every wave; with fewer than four blocks of keys a wave (small batches at
-        short contexts, whose keys are cut into many parts) the preparation as a kernel of its own was level or ahead
-        (whole steps on MI355X, Qwen3-4B widths, 2,048 tokens: batch 1 to 4 0.7 to 1.4 % behind with it folded, batch 5
-        to 64 1.4 to 6 % ahead; 8,192 tokens: batch 1 to 4 1.5 to 2.8 % ahead)."""
-        if not self.folds_preparation:
-            return False
-        blocks = -(-int(max_context) // 32)
-        return -(-blocks // max(1, int(splits))) >= self._FOLD_MIN_BLOCKS
+        return ops.decode_splits(rows, self.nkv, max_context)
 
     def forward(self, x, batch, cache):
         """x [T, H] -> [T, H], or a float32 stack [S, T, H] to be added in order (see Linear)."""
@@ -131,20 +116,16 @@ class PagedAttention(Part):
                             k_pages=cache.k_pages, v_pages=cache.v_pages, page_size=cache.page_size)
         # the fused preparation kernel can add a stack of partial products itself
         projected = (self.qkv if cache.writes else self.q_only)(x, partials_ok=fused)
-        folded = False
         if (fused and cache.writes and batch.max_qlen == 1 and self.folds_preparation
                 and (projected.dim() == 3 or projected.dtype == torch.bfloat16)
                 and ops.attn_decode_prep_supported(x.dtype, self.D, cache.page_size, self.nq // self.nkv, rot)):
-            splits = getattr(batch, "kv_splits", None) or ops.decode_splits(x.shape[0], self.nkv, batch.max_position + 1)
-            folded = self._folds(batch.max_position + 1, splits)
-        if folded:
             # single decoded tokens: the attention's kernel sums, norms, rotates and writes to the cache itself
             out = torch.empty((x.shape[0], Q), dtype=x.dtype, device=x.device)
             ops.attn_decode_prep(projected, out, cache.k_pages, cache.v_pages, cache.block_table, batch.seg_row0,
                                  batch.seg_slot, batch.seg_start, max_kv_len=batch.max_position + 1,
                                  num_q_heads=self.nq, num_kv_heads=self.nkv, head_dim=self.D, page_size=cache.page_size,
                                  scale=self.scale, eps=self.eps, q_weight=self.q_norm, k_weight=self.k_norm, cos=cos,
-                                 sin=sin, rotary_dim=rot, window=self.window or 0, splits=splits)
+                                 sin=sin, rotary_dim=rot, window=self.window or 0, splits=getattr(batch, "kv_splits", None))
             return self.o(out, partials_ok=True)
         if projected.dim() == 3:
             q = torch.empty((x.shape[0], Q), dtype=x.dtype, device=x.device)
