@@ -863,7 +863,8 @@ __global__ __launch_bounds__(256) void attn_prefill_plan_kernel(const int* __res
 // uint4/uint2 structs went through scratch memory here.
 template <int DMAX, bool EXACT>
 __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_prefill_lds_kernel(const AttnArgs a, int min_rows,
-                                                                                         int blocks_x, int segments, int listed) {
+                                                                                         int blocks_x, int segments, int listed,
+                                                                                         int fixed_rounds) {
   constexpr int NT = kPfNT;
   constexpr int DCH = DMAX / 32, DTL = DMAX / 16;
   constexpr int kKPieces = (kPfKeys * (DMAX / 8) + kPfWaves * kWave - 1) / (kPfWaves * kWave);  // 16-byte pieces per thread
@@ -876,19 +877,40 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
   const unsigned int pairs = listed ? g_prefill_pairs : static_cast<unsigned int>(blocks_x) * segments;
   const unsigned int parts = static_cast<unsigned int>(a.portion_splits);
   const unsigned int items = pairs * nkv * parts;
+ // Items dealt out before the launch instead of taken from the counter, as in attn_prefill_dma_kernel (see there):
+ // workgroup b takes item b of the first round of gridDim.x items, item gridDim.x - 1 - b of the second, and so on
+ // to and fro; an item's list entry is asked for while the item before it runs.
+ const bool dealt = fixed_rounds > 0 && listed && items <= static_cast<unsigned long long>(fixed_rounds) * gridDim.x;
+ unsigned int round = 0u;
+ unsigned int ahead_entry = 0u;
+ int4 ahead_seg = {0, 0, 0, 0};
+ auto dealt_item = [&](unsigned int r) {
+   return r * gridDim.x + ((r & 1u) ? gridDim.x - 1u - blockIdx.x : blockIdx.x);
+ };
+ if (dealt && blockIdx.x < items) {
+   ahead_entry = g_prefill_plan[blockIdx.x / (nkv * parts)];
+   ahead_seg = g_prefill_seg[blockIdx.x / (nkv * parts)];
+ }
  for (;;) {  // one item per round; every wave of the workgroup leaves at the same round
-  if (tid == 0) item_of_workgroup = atomicAdd(&g_prefill_next_item, 1u);
-  __syncthreads();
-  const unsigned int item = item_of_workgroup;
-  __syncthreads();  // everyone has read it before thread 0 asks for the next
-  if (item >= items) {
-    // The last workgroup to leave puts the counters back to zero: the layers of a step hand out the same list one
-    // after the other, and only the first of them runs the planning kernel.
-    if (tid == 0 && atomicAdd(&g_prefill_left, 1u) == gridDim.x - 1) {
-      g_prefill_next_item = 0u;
-      g_prefill_left = 0u;
+  unsigned int item;
+  if (dealt) {
+    if (round > 0u) __syncthreads();  // the item's first tile goes where the last one's tiles were read
+    item = dealt_item(round);
+    if (item >= items) return;  // every later round lies behind this one
+  } else {
+    if (tid == 0) item_of_workgroup = atomicAdd(&g_prefill_next_item, 1u);
+    __syncthreads();
+    item = item_of_workgroup;
+    __syncthreads();  // everyone has read it before thread 0 asks for the next
+    if (item >= items) {
+      // The last workgroup to leave puts the counters back to zero: the layers of a step hand out the same list one
+      // after the other, and only the first of them runs the planning kernel.
+      if (tid == 0 && atomicAdd(&g_prefill_left, 1u) == gridDim.x - 1) {
+        g_prefill_next_item = 0u;
+        g_prefill_left = 0u;
+      }
+      return;
     }
-    return;
   }
   const unsigned int pair = item / (nkv * parts);
   const int kvh = static_cast<int>((item / parts) % nkv);
@@ -896,7 +918,17 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
   // the last rows of a segment see the most keys: they are handed out first
   int seg = static_cast<int>(pair % segments), wg_row = (blocks_x - 1 - static_cast<int>(pair / segments)) * kPfRows;
   int row0, qlen, start, slot;
-  if (listed) {  // the entry and what the list holds of its segment: two loads side by side
+  if (dealt) {
+    seg = static_cast<int>(ahead_entry & 0xffffu);
+    wg_row = static_cast<int>(ahead_entry >> 16) * kPfRows;
+    row0 = ahead_seg.x, qlen = ahead_seg.y, start = ahead_seg.z, slot = ahead_seg.w;
+    ++round;
+    const unsigned int next = dealt_item(round);
+    if (next < items) {
+      ahead_entry = g_prefill_plan[next / (nkv * parts)];
+      ahead_seg = g_prefill_seg[next / (nkv * parts)];
+    }
+  } else if (listed) {  // the entry and what the list holds of its segment: two loads side by side
     const unsigned int entry = g_prefill_plan[pair];
     const int4 of_seg = g_prefill_seg[pair];
     seg = static_cast<int>(entry & 0xffffu);
@@ -1857,8 +1889,12 @@ inline bool plan_is_current(const AttnArgs& a, dim3 grid, int min_rows, int list
   return same;
 }
 
+static int g_prefill_pair_up = 1;
+static int g_prefill_fixed_rounds = -1;  // items a workgroup up to which they are dealt out before the launch (0: never; -1: by the rule below)
+constexpr int kDealtMaxKeys = 4096;      // contexts up to which every launch deals its items out
+
 template <int DMAX, bool EXACT>
-int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s) {
+int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, int max_kv_len, hipStream_t s) {
   const size_t lds = prefill_lds_bytes(a.D);
   static size_t allowed = 64 * 1024;  // dynamic LDS above 64 KiB has to be asked for, once per kernel
   if (lds > allowed) {
@@ -1882,8 +1918,10 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
     attn_prefill_plan_kernel<<<1, 256, 0, s>>>(a.seg_row0, a.seg_start, a.seg_slot, static_cast<int>(grid.z),
                                                static_cast<int>(grid.x), a.nq / a.nkv, min_rows, listed);
   if (a.portion_splits > 1 && !listed) return static_cast<int>(hipErrorInvalidValue);  // the merge walks the list
+  // dealt out by the rule of launch_prefill_dma_groups (measured there)
+  const int fixed_rounds = g_prefill_fixed_rounds >= 0 ? g_prefill_fixed_rounds : (max_kv_len <= kDealtMaxKeys ? 1 << 20 : 2);
   attn_prefill_lds_kernel<DMAX, EXACT><<<workgroups, kPfWaves * kWave, lds, s>>>(a, min_rows, static_cast<int>(grid.x),
-                                                                                static_cast<int>(grid.z), listed);
+                                                                                static_cast<int>(grid.z), listed, fixed_rounds);
   if (a.portion_splits > 1) {
     const long long most = static_cast<long long>(grid.x) * grid.y * grid.z * (kPfRows / kPfWaves);
     attn_merge_portions_kernel<<<static_cast<unsigned>(most < 4LL * cus ? most : 4LL * cus), kPfWaves * kWave, 0, s>>>(a);
@@ -1891,9 +1929,6 @@ int launch_prefill_lds(const AttnArgs& a, dim3 grid, int min_rows, hipStream_t s
   return launch_status();
 }
 
-static int g_prefill_pair_up = 1;
-static int g_prefill_fixed_rounds = -1;  // items a workgroup up to which they are dealt out before the launch (0: never; -1: by the rule below)
-constexpr int kDealtMaxKeys = 4096;      // contexts up to which every launch deals its items out
 
 static int g_prefill_groups = -1;  // -1: the launcher decides; 1, 2: forced (measurements and tests)
 
@@ -2152,18 +2187,18 @@ extern "C" int arle_attn_paged_mfma(const void* q, long long q_stride, void* out
       return side_rc;
     }
     if (D == 64)
-      rc = launch_prefill_lds<64, true>(a, grid, 17, s);
+      rc = launch_prefill_lds<64, true>(a, grid, 17, max_kv_len, s);
     else if (D == 128 && page_size % 8 == 0 && static_cast<long long>(nkv) * page_size * D < (1LL << 31) &&
              prefill_dma_pays(grid, max_qlen, max_kv_len))
       rc = launch_prefill_dma(a, grid, 17, max_qlen, max_kv_len, s);
     else if (D == 128)
-      rc = launch_prefill_lds<128, true>(a, grid, 17, s);
+      rc = launch_prefill_lds<128, true>(a, grid, 17, max_kv_len, s);
     else if (D <= 64)
-      rc = launch_prefill_lds<64, false>(a, grid, 17, s);
+      rc = launch_prefill_lds<64, false>(a, grid, 17, max_kv_len, s);
     else if (D <= 128)
-      rc = launch_prefill_lds<128, false>(a, grid, 17, s);
+      rc = launch_prefill_lds<128, false>(a, grid, 17, max_kv_len, s);
     else
-      rc = launch_prefill_lds<256, false>(a, grid, 17, s);
+      rc = launch_prefill_lds<256, false>(a, grid, 17, max_kv_len, s);
     if (side != nullptr) {   // join: the caller's stream goes on when the side branch is done, also after an error
       const bool joined = hipEventRecord(side->join, side->stream) == hipSuccess && hipStreamWaitEvent(s, side->join, 0) == hipSuccess;
       if (!joined) {

@@ -766,14 +766,14 @@ def test_decode_attention_with_the_preparation_folded_in(nq, nkv, D, rot, P, n_p
     assert torch.equal(ka, kb) and torch.equal(va, vb)
 
 
-@pytest.mark.parametrize("groups,heads", [(1, 24), (2, 12)])
+@pytest.mark.parametrize("variant,groups,heads", [(1, 1, 24), (1, 2, 12), (0, -1, 12)])
 @pytest.mark.parametrize("parts", [None, 2])
-def test_attention_portions_dealt_out_before_the_launch_or_taken_from_the_counter(groups, heads, parts):
-    """The kernel that loads tiles straight into LDS gets its (row block, kv head, part) items either from a counter
-    at run time or dealt out to and fro over the workgroups before the launch; the list of both is ordered by the
-    keys an entry sees.  Segments of very different lengths and contexts, more items than workgroups (so that a
-    workgroup gets a second and third item), one or two groups of waves: the same bits either way, and the plain
-    result at rows of every segment."""
+def test_attention_portions_dealt_out_before_the_launch_or_taken_from_the_counter(variant, groups, heads, parts):
+    """Both portions kernels get their (row block, kv head, part) items either from a counter at run time or dealt
+    out to and fro over the workgroups before the launch; the list of both is ordered by the keys an entry sees.
+    Segments of very different lengths and contexts, more items than workgroups (so that a workgroup gets a second
+    and third item); the kernel that parks tiles in LDS, and the one that loads them straight there with one or two
+    groups of waves: the same bits either way, and the plain result at rows of every segment."""
     from arle_amd.kernels import lib
     nq = nkv = heads
     D, P, dt = 128, 16, torch.bfloat16
@@ -796,7 +796,7 @@ def test_attention_portions_dealt_out_before_the_launch_or_taken_from_the_counte
     args = (k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), i32(row0), i32(list(range(len(segs)))), i32(starts))
     kw = dict(max_qlen=2048, min_qlen=1, max_kv_len=max(lengths), num_q_heads=nq, num_kv_heads=nkv, head_dim=D,
               page_size=P, scale=1.0 / math.sqrt(D), portion_splits=parts)
-    lib.function("arle_attn_prefill_variant")(1)
+    lib.function("arle_attn_prefill_variant")(variant)
     lib.function("arle_attn_prefill_groups")(groups)
     outs = {}
     try:
