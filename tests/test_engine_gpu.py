@@ -275,3 +275,24 @@ def test_warm_up_captures_every_decode_graph_before_the_first_request(model, dty
     assert warm.graph_replays == 12 and len(warm._graphs) == graphs_before
     for key in a:
         assert torch.equal(a[key], b[key]), key
+
+
+def test_decode_steps_with_the_preparation_folded_into_the_attention_and_as_a_kernel_of_its_own(tmp_path):
+    """bfloat16 decode steps at a head_dim for which the attention's kernel can prepare q, k and v itself (config D:
+    64): with that and with `qk_prep` as a kernel of its own the logits are the plain ones, two requests decoded
+    token by token side by side after their prompts."""
+    d = make_model_dir(tmp_path, "D")
+    cfg, weights = read_folder(d)
+    reqs = _requests(cfg, [40, 57], 900)
+    for folded in (True, False):
+        eng = Engine.from_folder(d, dtype="bfloat16", page_size=TINY["D"][1], max_tokens=192, max_slots=4)
+        folds = [p for p in eng.model.parts if hasattr(p, "folds_preparation")]
+        assert folds and all(p.folds_preparation for p in folds)
+        for p in folds:
+            p.folds_preparation = folded
+        steps = [{"entries": [(rid, toks[:8], list(range(8))) for rid, toks in reqs.items()], "end": []}]
+        for t in range(8, 57):
+            steps.append({"entries": [(rid, [toks[t]], [0]) for rid, toks in reqs.items() if t < len(toks)], "end": []})
+        got = replay.run_steps(eng, steps)
+        assert len(got) == 40 + 57
+        replay.compare(got, cfg, weights, reqs, TOL["bfloat16"], f"decode, folded {folded}")
