@@ -163,7 +163,8 @@ class LLM:
                  ignore_eos: bool = False, sampling: SamplingParams | None = None, logprobs: bool = False,
                  priorities=None, stop=None) -> list:
         """prompts: a list of token-id lists (or strings, with a tokenizer).  One CompletionOutput each,
-        in order.  `sampling` overrides temperature / seed / ignore_eos / logprobs when given.
+        in order.  `sampling` overrides temperature / seed / ignore_eos / logprobs when given: one SamplingParams for
+        all prompts, or a list with one a prompt.
         priorities: one of PRIORITY_LOW / NORMAL / HIGH (0, 1, 2) a prompt; the higher is served first.
         stop: strings that end a request where its text first holds one of them (the text stops in front of it,
         the finish reason is `stop`); needs a tokenizer."""
@@ -210,10 +211,13 @@ class LLM:
         ids = []
         if priorities is not None and len(priorities) != len(prompts):
             raise ValueError("one priority a prompt")
+        each = isinstance(sampling, (list, tuple))
+        if each and len(sampling) != len(prompts):
+            raise ValueError("one SamplingParams a prompt (or one for all)")
         for i, p in enumerate(prompts):
             toks = self.tokenize(p) if isinstance(p, str) else list(p)
-            params = sampling or SamplingParams(temperature=temperature, seed=seed, ignore_eos=ignore_eos,
-                                                logprobs=logprobs)
+            params = (sampling[i] if each else sampling) or SamplingParams(temperature=temperature, seed=seed,
+                                                                            ignore_eos=ignore_eos, logprobs=logprobs)
             ids.append(sched.submit(toks, params, max_tokens, **({} if priorities is None else {"priority": priorities[i]})))
         return sched, ids
 

@@ -78,6 +78,22 @@ def test_temperature_sampling_with_portions_equals_plain_inverse_cdf(folders):
     assert alone.response_token_ids == outs[2].response_token_ids
 
 
+def test_sampling_parameters_of_their_own_for_every_prompt(folders):
+    """`sampling` as a list: every prompt is sampled by its own parameters, as if it had been generated alone."""
+    cfg, _ = read_folder(folders["B"])
+    prompts = [random_tokens(n, cfg["vocab_size"], 70 + n) for n in (9, 14, 5)]
+    params = [SamplingParams(temperature=0.0, ignore_eos=True), SamplingParams(temperature=0.9, top_p=0.8, seed=3, ignore_eos=True),
+              SamplingParams(temperature=0.7, top_k=5, seed=11, ignore_eos=True)]
+    llm = LLM(folders["B"], dtype="float32", page_size=TINY["B"][1], kv_cache_tokens=256, max_seq_len=64)
+    together = llm.generate(prompts, max_tokens=7, sampling=params)
+    for p, sp, got in zip(prompts, params, together):
+        alone = llm.generate([p], max_tokens=7, sampling=sp)[0]
+        assert got.response_token_ids == alone.response_token_ids and len(got.response_token_ids) == 7
+    assert together[0].response_token_ids != together[1].response_token_ids
+    with pytest.raises(ValueError):
+        llm.generate(prompts, max_tokens=2, sampling=params[:2])
+
+
 def test_generation_survives_a_pool_that_runs_out(folders):
     cfg, weights = read_folder(folders["A"])
     prompts = [random_tokens(10, cfg["vocab_size"], 60 + k) for k in range(4)]
