@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
     python bench.py --workload qwen3-8b-mixed | qwen3-32b-decode     (two further workloads)
+    python bench.py --generate                                       (the decode workload through LLM.generate)
 
 A step is one decode step of `batch` requests, each holding a `prompt`-token random prompt
 (prefilled by the engine itself before the clock starts) and growing by one token per step.
@@ -515,6 +516,45 @@ def first_token(args) -> int:
     return 0
 
 
+def generate_workload(args) -> int:
+    """The decode workload of the baseline's benchmark configuration as a user runs it: 1, 8 and 64 prompts of 2,048
+    uniform-random tokens, 256 tokens generated for each, through `LLM.generate` (scheduler, sampler, engine; greedy
+    and at temperature 0.8).  One JSON line each: generated tokens a second after the first token, the time to the
+    first token of the last prompt served, and the steps by kind."""
+    import torch
+
+    from arle_amd.config import Qwen3Config
+    from arle_amd.engine import Engine
+    from arle_amd.engine.api import LLM
+
+    config = Qwen3Config.from_dict(dict(QWEN3_4B, num_hidden_layers=args.layers))
+    prompt, new, most = args.prompt_len, 256, 64
+    longest = -(-(prompt + new + 1) // 64) * 64
+    engine = Engine.from_config("Qwen3ForCausalLM", config, seed=0, std=0.02, dtype="bfloat16", page_size=args.page_size,
+                                max_tokens=most * longest, max_slots=most, max_request_tokens=longest)
+    gen = torch.Generator().manual_seed(1234)
+    for temperature in (0.0, 0.8):
+        for n in (1, 8, most):
+            llm = LLM(engine, num_slots=most, max_seq_len=longest)
+            prompts = [torch.randint(0, config.vocab_size, (prompt,), generator=gen).tolist() for _ in range(n)]
+            for _ in range(3):      # the third run replays what the first two captured (a shape is captured when it repeats)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                outs = llm.generate(prompts, max_tokens=new, temperature=temperature, seed=3, ignore_eos=True)
+                torch.cuda.synchronize()
+                wall = time.perf_counter() - t0
+            ttft = max(o.ttft_s for o in outs)
+            made = sum(o.usage.completion_tokens for o in outs)
+            print(json.dumps({"metric": f"{n} prompt(s) of {prompt:,} tokens, {new} generated each, through LLM.generate "
+                                        f"(Qwen3-4B shape, temperature {temperature})",
+                              "value": round((made - n) / (wall - ttft), 1), "unit": "generated tok/s after the first token",
+                              "higher_is_better": True, "n_gpus": 1, "dtype": "bf16", "layers": args.layers,
+                              "wall_s": round(wall, 4), "ttft_ms": round(ttft * 1e3, 1),
+                              "ms_per_token_a_request": round(sum(o.tpot_s for o in outs) / n * 1e3, 3),
+                              "steps": llm.last_stats["steps"]}), flush=True)
+    return 0
+
+
 def tune_products(args) -> int:
     """Measure the table of `arle_amd.kernels.tune` for one model's widths and write it; one line a (product, row
     count) to stderr, and at the end what the table gains over the rules at every row count where they differ."""
@@ -687,13 +727,16 @@ def main() -> int:
     ap.add_argument("--ceilings", action="store_true",
                     help="measure what a kernel that only reads, and one that only multiplies, reach on this GPU, and exit")
     ap.add_argument("--prompt-len", type=int, default=PROMPT,
-                    help="tokens of the prefill that --prefill-only measures (the default run's is 2,048)")
+                    help="tokens of the prefill that --prefill-only measures and of the prompts of --generate (default 2,048)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiles of its kernels) and print that")
     ap.add_argument("--gaps", action="store_true",
                     help="decode steps that wait for their tokens against steps launched ahead: time a step, GPU busy and idle")
     ap.add_argument("--first-token", action="store_true",
                     help="time to the first token through LLM.generate, portions by the GPU's memory against portions of 512")
+    ap.add_argument("--generate", action="store_true",
+                    help="the decode workload as a user runs it: 1, 8 and 64 prompts of --prompt-len tokens, 256 generated each, "
+                         "through LLM.generate")
     ap.add_argument("--sweep", action="store_true",
                     help="further sizes of the Qwen3-4B shape (batch 16/32, 8k/32k context, 8,192-token prefill, portions "
                          "beside decoding requests), one JSON line each")
@@ -719,6 +762,8 @@ def main() -> int:
         return sweep(args)
     if args.first_token:
         return first_token(args)
+    if args.generate:
+        return generate_workload(args)
     if args.gaps:
         return step_gaps(args)
     if args.workload == "qwen3-4b" and args.batch is None:
