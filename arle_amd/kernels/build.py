@@ -36,7 +36,8 @@ SOURCES = {
     "ceilings": "ceilings.hip",
     "host": "host/runtime.cpp",
 }
-HEADERS = ("common.h", "attention_static.h")
+HEADERS = ("common.h", "attention_static.h", "attention_args.h", "attention_stream.h", "attention_portions.h",
+           "attention_portions_dma.h")
 HOST_LIBS = ("host",)   # plain C++: page pool, block tables, step packing
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared"]
 
