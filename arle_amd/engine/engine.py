@@ -178,10 +178,13 @@ class Engine:
 
     # -- the step -------------------------------------------------------------------------
     @torch.no_grad()
-    def step(self, entries) -> torch.Tensor:
+    def step(self, entries, borrow_logits: bool = False) -> torch.Tensor:
         """Run one packed step; returns float32 logits [wanted, vocab] on the GPU.
 
         Raises `OutOfPages` (nothing changed) if the cache cannot take all entries.
+        borrow_logits: the caller is done with the logits before it calls `step` again (everything that reads
+        them is queued on this stream by then, as the scheduler's sampling is), so a captured step may hand out
+        the buffer that its next replay writes instead of a copy of it.
         """
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         if not entries:
@@ -214,9 +217,9 @@ class Engine:
             saved_state = self.cache.snapshot_state([e.request for e in entries])
             self.cache.sync_tables()
             if decode_only:
-                logits = self._decode_step_graphed(entries, before)
+                logits = self._decode_step_graphed(entries, before, borrow_logits)
             elif shape_key is not None:
-                logits = self._step_graphed(shape_key, entries, before)
+                logits = self._step_graphed(shape_key, entries, before, borrow_logits)
             else:
                 logits = self.model.forward(batch, self.cache)
         except Exception:
@@ -230,7 +233,7 @@ class Engine:
         return logits
 
     # -- captured decode steps ----------------------------------------------------------------
-    def _decode_step_graphed(self, entries, before) -> torch.Tensor:
+    def _decode_step_graphed(self, entries, before, borrow: bool = False) -> torch.Tensor:
         """A step of single decoded tokens through a HIP graph captured for its number of rows.
 
         The graph computes the logits of every row; the wanted ones are picked afterwards.  What
@@ -267,7 +270,7 @@ class Engine:
                              self.spec.vocab_size, self.device, into=static)
             graph.replay()
             self.graph_replays += 1
-            logits = static_logits.clone()
+            logits = static_logits if borrow else static_logits.clone()
         self._graphs[key] = rec    # most recently used last
         wanted = [i for i, e in enumerate(entries) for _ in e.want]
         if wanted == list(range(rows)):
@@ -360,7 +363,7 @@ class Engine:
         self._shapes_seen.add(key)
         return key if seen else None
 
-    def _step_graphed(self, key, entries, before) -> torch.Tensor:
+    def _step_graphed(self, key, entries, before, borrow: bool = False) -> torch.Tensor:
         """A step whose shape repeats, through a HIP graph captured for that shape (see _repeated_shape).
 
         As for decode steps, what varies (token ids, positions, slots, wanted rows) travels in the graph's
@@ -388,6 +391,6 @@ class Engine:
             build_step_batch(entries, slot_of, length_before, self.spec.vocab_size, self.device, into=static)
             graph.replay()
             self.graph_replays += 1
-            logits = static_logits.clone()
+            logits = static_logits if borrow else static_logits.clone()
         self._graphs[key] = rec    # most recently used last
         return logits

@@ -37,6 +37,7 @@ runs two forwards, `Split`).
 from __future__ import annotations
 
 import ctypes
+import inspect
 
 import time
 from collections import deque
@@ -262,6 +263,8 @@ class Scheduler:
         self.cfg = config or SchedulerConfig()
         self.cfg.validate()
         self.engine = engine
+        # the logits of a step are sampled from before the next step is launched: a captured step need not copy them
+        self._step_options = {"borrow_logits": True} if "borrow_logits" in inspect.signature(engine.step).parameters else {}
         self.cache = engine.cache
         self.sampler = sampler
         self.seed = seed
@@ -437,7 +440,7 @@ class Scheduler:
             if completes:
                 sampled.append(r)
         try:
-            logits = self.engine.step(entries)
+            logits = self.engine.step(entries, **self._step_options)
         except OutOfPages:
             # planning said it fits; if the pool disagrees, nothing was changed: skip the portions
             if not plan.prefill:

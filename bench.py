@@ -291,7 +291,7 @@ def mixed_8b(args) -> int:
                 entries = [StepEntry(k, [before.feed(i)], [0]) for i, k in enumerate(keys)]
             last_piece = a + n == prompt
             entries.append(StepEntry(tag, toks[a:a + n], [n - 1] if last_piece else []))
-            chosen = sampler.choose(engine.step(entries), greedy[:decoders + (1 if last_piece else 0)])
+            chosen = sampler.choose(engine.step(entries, borrow_logits=True), greedy[:decoders + (1 if last_piece else 0)])
             if args.no_overlap:
                 state["last"] = chosen.tokens()[:decoders]
             else:
@@ -375,7 +375,7 @@ def decode_32b(args) -> int:
             entries = [StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])]
         else:
             entries = [StepEntry(k, [before.feed(i)], [0]) for i, k in enumerate(keys)]
-        chosen = sampler.choose(engine.step(entries), greedy)
+        chosen = sampler.choose(engine.step(entries, borrow_logits=True), greedy)
         if args.no_overlap:
             state["last"] = chosen.tokens()
         else:
@@ -447,7 +447,7 @@ def step_gaps(args) -> int:
                 entries = [StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])]
             else:
                 entries = [StepEntry(k, [before.feed(i)], [0]) for i, k in enumerate(keys)]
-            state["chosen"] = sampler.choose(engine.step(entries), rows)
+            state["chosen"] = sampler.choose(engine.step(entries, borrow_logits=True), rows)
             if before is not None:
                 state["last"] = before.tokens()
 
@@ -627,7 +627,7 @@ def sweep(args) -> int:
                 entries = [StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])]
             else:
                 entries = [StepEntry(k, [before.feed(i)], [0]) for i, k in enumerate(keys)]
-            state["chosen"] = sampler.choose(engine.step(entries), greedy_rows[:batch])
+            state["chosen"] = sampler.choose(engine.step(entries, borrow_logits=True), greedy_rows[:batch])
             if before is not None:
                 state["last"] = before.tokens()
 
@@ -853,7 +853,7 @@ def main() -> int:
                 entries = [StepEntry(k, [t], [0]) for k, t in zip(keys, state["last"])]
             else:
                 entries = [StepEntry(k, [before.feed(i)], [0]) for i, k in enumerate(keys)]
-            state["chosen"] = sampler.choose(engine.step(entries), greedy_rows[:batch])
+            state["chosen"] = sampler.choose(engine.step(entries, borrow_logits=True), greedy_rows[:batch])
             if before is not None:
                 state["last"] = before.tokens()                 # the step before: every token reaches the host
 

@@ -118,6 +118,33 @@ def test_captured_decode_steps_equal_eager_ones_on_every_replay(model, dtype):
         assert torch.equal(a[key], b[key]), f"graph replay differs from the eager step at {key}"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_borrowed_logits_are_the_copied_ones_until_the_next_step(model, dtype):
+    """`step(..., borrow_logits=True)` may hand out the buffer that a captured step writes: read before the next
+    step they are the bits that a step without it returns, replay after replay, and the next replay does write
+    the same memory (which is why only a caller that is done with them by then may ask for it)."""
+    from arle_amd.engine import StepEntry
+
+    name, d, cfg, _ = model
+    reqs = _requests(cfg, [33, 47], 700)
+    make = lambda: Engine.from_folder(d, dtype=dtype, page_size=TINY[name][1], max_tokens=192, max_slots=4)
+    copying, borrowing = make(), make()
+    for eng in (copying, borrowing):
+        for rid, toks in reqs.items():
+            eng.add_request(rid)
+            eng.step([StepEntry(rid, toks[:20], [])])
+    seen = []
+    for t in range(20, 33):
+        entries = [StepEntry(rid, [toks[t]], [0]) for rid, toks in reqs.items()]
+        want = copying.step(entries)
+        got = borrowing.step(entries, borrow_logits=True)
+        assert torch.equal(got, want), f"token {t}"
+        seen.append((got.data_ptr(), want.data_ptr()))
+    assert borrowing.graph_replays >= 10
+    assert len({a for a, _ in seen}) < len(seen), "replays of one captured step hand out one buffer"
+    assert len({b for _, b in seen[-3:]}) == 3 or len({b for _, b in seen}) > 1, "copies are tensors of their own"
+
+
 def test_weights_held_as_operand_tiles_give_the_same_bits(model):
     """The decode-friendly second copy of the projection weights changes where the few-rows kernels read
     from, not what they add in which order."""
