@@ -77,6 +77,28 @@ def test_mixed_with_page_reuse(model, dtype):
     assert eng.cache.free_pages()[0] == eng.cache.groups[0].pool.num_pages
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_random_schedules_with_page_reuse(model, dtype):
+    """Schedules drawn at random: three to nine requests of 2 to 140 tokens, one to four live at a time, portions of
+    up to 3 to 90 tokens beside single tokens, a decoded tail of 0 to 40 tokens, and a pool that holds just the
+    longest live requests (each rounded up to 64 tokens), so that pages go round."""
+    import random
+
+    name, d, cfg, weights = model
+    for seed in range(6):
+        rng = random.Random(1000 * seed + 17)
+        lengths = [rng.randint(2, 140) for _ in range(rng.randint(3, 9))]
+        reqs = {f"q{i}": random_tokens(n, cfg["vocab_size"], 5000 + 31 * seed + i) for i, n in enumerate(lengths)}
+        live = rng.randint(1, 4)
+        room = sum(-(-n // 64) * 64 for n in sorted(lengths)[-live:])
+        eng = _engine(model, dtype, room)
+        steps = replay.mixed(reqs, max_live=live, seed=seed, decode_tail=rng.randint(0, 40),
+                             max_portion=rng.choice([3, 9, 17, 40, 90]))
+        got = replay.run_steps(eng, steps)
+        replay.compare(got, cfg, weights, reqs, TOL[dtype], f"random schedule {seed}/{dtype}, lengths {lengths}, {live} live")
+        assert eng.cache.free_pages()[0] == eng.cache.groups[0].pool.num_pages
+
+
 def test_float32_is_bit_identical_across_cuttings(model):
     """The 32-bit path fixes the order of every reduction, so cutting changes no bit."""
     _, _, cfg, weights = model
