@@ -14,7 +14,8 @@ infer/src/scheduler/cuda/execution.rs:385-425,669-800):
 2. decode rows: every decoding request brings its last token.  If the pool cannot take one
    more token of each, the request with the fewest generated tokens (ties: the longest
    prompt) is preempted until it can (decode.rs:16-21,82-116); a lone request that still
-   does not fit finishes with `length`.
+   does not fit finishes with `length` (decode.rs:52-73), here only once no prompt that is still
+   being fed holds pages either (see below).
 3. prompt portions under the token budget min(max_num_batched_tokens - decode rows,
    max_prefill_tokens): per request min(remaining, chunked_prefill_size), also capped by
    long_prefill_token_threshold while rows are decoding; a portion that does not fit the
@@ -31,8 +32,11 @@ infer/src/scheduler/cuda/execution.rs:385-425,669-800):
 
 Kept differently on purpose: a preempted request keeps the tokens it has generated and
 feeds prompt + generated again when it re-enters (the reference drops them and generates
-anew); and decode rows and prompt portions always share one step (the reference's default
-runs two forwards, `Split`).
+anew); decode rows and prompt portions always share one step (the reference's default
+runs two forwards, `Split`); and before the only decoding request is cut short for want of a page, the
+prompts that are still being fed give theirs back, the one admitted last first: they have produced
+nothing yet and wait in front of the queue, where the reference ends the decoding request with `length`
+while they keep their pages.
 """
 from __future__ import annotations
 
@@ -404,6 +408,12 @@ class Scheduler:
         # pages run out while decoding: preempt until one more token of each fits
         while decode and not self.cache.can_append([(r.id, 1) for r in decode]):
             if len(decode) == 1:
+                # nobody else is decoding.  A prompt that is still being fed has produced nothing yet: the one
+                # admitted last gives its pages back and waits, before a request that is generating is cut short.
+                holders = [r for r in self.prefilling if r.phase == "prefilling" and self.cache.length(r.id) > 0]
+                if holders:
+                    self._preempt(holders[-1])
+                    continue
                 self._finish(decode.pop(), LENGTH)
                 break
             victim = retract_victim(decode)
@@ -535,8 +545,8 @@ class Scheduler:
         r.t_finish = time.perf_counter()
 
     def _preempt(self, r: Request) -> None:
-        """Give a decoding request's pages back and queue it again, at the front."""
-        self.decoding.remove(r)
+        """Give a request's pages back and queue it again, at the front."""
+        (self.decoding if r in self.decoding else self.prefilling).remove(r)
         self.engine.end_request(r.id)
         r.phase = "waiting"
         r.fed = 0

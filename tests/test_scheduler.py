@@ -230,6 +230,25 @@ def test_a_lone_request_that_cannot_grow_finishes_with_length():
     assert eng.cache.free_pages() == [4]
 
 
+def test_a_lone_decoding_request_takes_pages_back_from_a_prompt_that_is_still_being_fed():
+    # 8 pages of 4.  a (prompt 10, 12 to generate: 6 pages in the end) and b (prompt 18) enter together and are fed in
+    # portions of 4; once a decodes, its growth is set aside and b, 12 tokens in and holding 3 pages, waits.  When a
+    # needs its sixth page nothing is free and a is the only request that decodes: b, which has produced nothing,
+    # gives its pages back and goes to the front of the queue, and a is not cut short.
+    eng, s = make(num_pages=8, page_size=4, slots=2, chunked_prefill_size=4)
+    a = s.submit(prompt(10, 1), max_tokens=12)
+    b = s.submit(prompt(18, 2), max_tokens=3)
+    s.run_until_done()
+    ra, rb = s.finished[a], s.finished[b]
+    assert ra.generated == expected_output(prompt(10, 1), 12) and ra.finish_reason == LENGTH
+    assert rb.generated == expected_output(prompt(18, 2), 3) and rb.finish_reason == LENGTH
+    assert rb.preemptions == 1 and ra.preemptions == 0 and s.stats["preemptions"] == 1
+    assert eng.steps[2] == [(a, 2, [1]), (b, 4, [])] and eng.steps[14] == [(b, 4, [])]   # b is fed from its start again
+    assert s.stats["tokens_prefilled"] == 10 + 12 + 18
+    assert not s.has_work() and not eng.cache.slot_of and eng.cache.free_pages() == [8]
+    eng.cache.check()
+
+
 def test_config_is_validated():
     with pytest.raises(ValueError):
         SchedulerConfig(chunked_prefill_size=0).validate()
