@@ -344,7 +344,9 @@ __global__ __launch_bounds__(kPfWaves* kWave, 1) __attribute__((amdgpu_waves_per
       if (EXACT || v_d[j] >= 0) {
         u32x2 v = vstage[j];
         if (unwritten) {  // slots past the last token may hold anything, also NaN: zero them for the products
-          const int off = tile * kPfKeys + v_off[j];
+          // by the keys that were fetched: in front of a window of a few keys those are the window's first four,
+          // which may reach past the last token
+          const int off = min(max(tile * kPfKeys + v_off[j], kv_lo & ~3), (kv_hi - 1) & ~3);
           if (off + 0 >= kv_total) v.x &= 0xffff0000u;
           if (off + 1 >= kv_total) v.x &= 0x0000ffffu;
           if (off + 2 >= kv_total) v.y &= 0xffff0000u;

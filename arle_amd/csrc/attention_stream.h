@@ -403,18 +403,23 @@ __global__ __launch_bounds__(INWG ? kInWgWavesMax * kWave : kWave) void attn_mfm
     // the key registers are free again: fetch the next block's keys while this block goes on
     if (more) load_k(blk + 1, kcur);
 
-    // a key beyond what the request holds may carry stale bits: its value must be 0, not 0 * garbage
-    if (key_base + 32 > kv_total) {
+    // a slot beyond what the request holds may carry stale bits: its value must be 0, not 0 * garbage.  Such slots
+    // are fetched in the request's last block only, but not only by the lanes whose own keys they are: with a window
+    // of a few keys the lanes of keys in front of it hold the window's first four values instead, which may reach
+    // past the last token.  So a lane goes by the keys it fetched.  PREP: the new token's own slot is written behind
+    // the loop and stale until then; the lanes that hold it by right get it from registers below.
+    const int stale_from = PREP ? start : kv_total;
+    if (key_base + 32 > stale_from) {
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        const int key4 = key_base + 16 * t + 4 * g;
+        const int key4 = min(max(key_base + 16 * t + 4 * g, kv_lo & ~3), (kv_hi - 1) & ~3);  // as load_v fetched it
 #pragma unroll
         for (int dt = 0; dt < DTL; ++dt) {
           if (!EXACT && dt >= n_dt) continue;
-          if (key4 + 0 >= kv_total) vraw[dt][2 * t] &= 0xffff0000u;
-          if (key4 + 1 >= kv_total) vraw[dt][2 * t] &= 0x0000ffffu;
-          if (key4 + 2 >= kv_total) vraw[dt][2 * t + 1] &= 0xffff0000u;
-          if (key4 + 3 >= kv_total) vraw[dt][2 * t + 1] &= 0x0000ffffu;
+          if (key4 + 0 >= stale_from) vraw[dt][2 * t] &= 0xffff0000u;
+          if (key4 + 1 >= stale_from) vraw[dt][2 * t] &= 0x0000ffffu;
+          if (key4 + 2 >= stale_from) vraw[dt][2 * t + 1] &= 0xffff0000u;
+          if (key4 + 3 >= stale_from) vraw[dt][2 * t + 1] &= 0x0000ffffu;
         }
       }
     }

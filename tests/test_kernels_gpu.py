@@ -456,11 +456,15 @@ def test_kernels_refuse_what_they_were_not_written_for():
         ops.embed_gather(torch.zeros(4, 4, device=DEV), torch.zeros(2, dtype=torch.int64, device=DEV))
 
 
-def _mfma_case(nq, nkv, D, P, segs, window, splits, seed, portion_splits=None):
-    """segs: [(cached length before the step, rows in the step)].  Returns (got, want) [T, nq*D]."""
+def _mfma_case(nq, nkv, D, P, segs, window, splits, seed, portion_splits=None, stale_nan=False):
+    """segs: [(cached length before the step, rows in the step)].  Returns (got, want) [T, nq*D].
+    stale_nan: every slot that no request has written holds NaN."""
     dt = torch.bfloat16
     lengths = [a + b for a, b in segs]
     table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, seed)
+    if stale_nan:
+        k_pages.fill_(float("nan"))
+        v_pages.fill_(float("nan"))
     qs, wants, row0, seg_start = [], [], [0], []
     for s, (cached, n) in enumerate(segs):
         g = _g(seed + 1 + s)
@@ -512,6 +516,24 @@ def test_attention_mfma_portions_with_their_keys_cut_into_parts(nq, nkv, D, P, p
 @pytest.mark.parametrize("window", [0, 50])
 def test_attention_mfma_decoded_tokens_split_over_the_keys(nq, nkv, D, P, splits, window):
     got, want = _mfma_case(nq, nkv, D, P, [(299, 1), (0, 1), (31, 1), (32, 1), (95, 1)], window, splits, 80)
+    assert torch.isfinite(got).all()
+    assert _rel(got, want) < 8e-3
+
+
+@pytest.mark.parametrize("nq,nkv,D,P", [(16, 1, 128, 64), (8, 1, 128, 32), (16, 1, 80, 64), (32, 8, 128, 16), (6, 2, 32, 8), (8, 8, 64, 4)])
+@pytest.mark.parametrize("window", [1, 2, 3, 5])
+@pytest.mark.parametrize("splits", [None, 1, 6])
+def test_attention_mfma_windows_of_a_few_keys_beside_stale_slots(nq, nkv, D, P, window, splits):
+    """A window of a few keys at the end of requests whose lengths are no multiples of four, every unwritten slot
+    NaN: the values that a kernel fetches in place of the keys in front of the window are the window's first four,
+    which reach past the last token, and 0 * NaN is NaN.  Decoded tokens (all three kernels' stale-slot handling
+    goes by the keys fetched, not by the keys asked for), and portions beside them."""
+    got, want = _mfma_case(nq, nkv, D, P, [(294, 1), (309, 1), (400, 1), (518, 1), (141, 1), (2, 1), (0, 1)], window, splits, 95,
+                           stale_nan=True)
+    assert torch.isfinite(got).all()
+    assert _rel(got, want) < 8e-3
+    got, want = _mfma_case(nq, nkv, D, P, [(34, 11), (13, 2), (283, 28), (214, 1), (257, 1), (132, 1), (0, 70), (61, 130)], window,
+                           1 if splits is None else splits, 96, stale_nan=True)
     assert torch.isfinite(got).all()
     assert _rel(got, want) < 8e-3
 
@@ -654,7 +676,8 @@ def test_attention_portions_list_their_work_once_for_calls_that_name_the_same_st
 @pytest.mark.parametrize("n_parts,splits,window,w_dtype", [(1, 1, 0, torch.bfloat16), (4, None, 0, torch.float32),
                                                            (3, 5, 37, torch.bfloat16), (7, 64, 0, None),
                                                            (2, 3, 0, torch.bfloat16), (5, 2, 37, torch.float32), (1, 4, 0, None),
-                                                           (0, None, 0, torch.bfloat16), (0, 3, 37, torch.float32)])
+                                                           (0, None, 0, torch.bfloat16), (0, 3, 37, torch.float32),
+                                                           (2, 3, 2, torch.bfloat16), (0, 1, 3, torch.float32), (3, None, 1, None)])
 def test_decode_attention_with_the_preparation_folded_in(nq, nkv, D, rot, P, n_parts, splits, window, w_dtype):
     """A step of single decoded tokens from the float32 stack of its q|k|v projection: sum, per-head norm, rotation,
     cache write and attention in one kernel.  Requests whose new token is the first of all, the first or last of
