@@ -671,6 +671,9 @@ def test_attention_portions_list_their_work_once_for_calls_that_name_the_same_st
         lib.function("arle_attn_prefill_variant")(-1)
 
 
+PREP_CACHED = None    # other context lengths for the test below, when something else calls it
+
+
 @pytest.mark.parametrize("nq,nkv,D,rot,P", [(32, 8, 128, 128, 16), (8, 8, 64, 64, 8), (16, 1, 128, 64, 64), (6, 2, 64, 0, 4),
                                             (4, 4, 128, 0, 32), (12, 2, 128, 128, 128)])
 @pytest.mark.parametrize("n_parts,splits,window,w_dtype", [(1, 1, 0, torch.bfloat16), (4, None, 0, torch.float32),
@@ -685,7 +688,7 @@ def test_decode_attention_with_the_preparation_folded_in(nq, nkv, D, rot, P, n_p
     written yet (the new token's own slot among them).  Against the plain implementation, and against the two
     kernels that it replaces: the same cache to the last bit but one, and nothing else touched."""
     dt, eps, theta = torch.bfloat16, 1e-6, 1e4
-    cached = [0, 1, 31, 32, 63, P - 1, P, 700, 1029, 255]     # tokens a request holds before the step
+    cached = PREP_CACHED or [0, 1, 31, 32, 63, P - 1, P, 700, 1029, 255]     # tokens a request holds before the step
     lengths = [c + 1 for c in cached]
     T = len(cached)
     table, k_pages, v_pages = _paged_setup(lengths, nkv, D, P, dt, 500)
