@@ -554,7 +554,9 @@ def test_random_traffic_gives_the_same_tokens_with_and_without_steps_launched_ah
                         for j, i in ids.items()})
         if overlap:
             ahead = s.stats.get("steps_ahead", 0)
-    aborted = {j for j, r in results[1].items() if r[1] == ABORT}
+    # (with steps launched ahead a request's end is found out one iteration late, so an abort may still reach a
+    # request that the waiting run had just finished)
+    aborted = {j for j in results[1] if ABORT in (results[0][j][1], results[1][j][1])}
     for j in results[1]:
         if j in aborted:     # an abort drops the token that was on its way: a prefix of what the waiting run kept
             a, b = results[0][j][0], results[1][j][0]
