@@ -67,6 +67,13 @@ class Qwen3Config:
         for name in ("hidden_size", "intermediate_size", "num_hidden_layers", "vocab_size"):
             if getattr(self, name) <= 0:
                 raise ConfigError(f"{name} must be positive")
+        # a damaged file is refused here, not by a model description that never gets done: rows and columns are
+        # indexed with 32-bit integers, and the layers are written out one by one
+        for name in ("hidden_size", "intermediate_size", "vocab_size", "max_position_embeddings", "q_width", "kv_width"):
+            if getattr(self, name) > 2 ** 31 - 1:
+                raise ConfigError(f"{name} = {getattr(self, name)} is beyond what a 32-bit index reaches")
+        if self.num_hidden_layers > 65535:
+            raise ConfigError(f"num_hidden_layers = {self.num_hidden_layers}: more than 65,535 layers are not taken")
         if not self.rms_norm_eps >= 0.0:
             raise ConfigError("rms_norm_eps must be non-negative")
         if not self.rope_theta > 0.0:

@@ -56,14 +56,26 @@ class SafetensorsFile:
             header = json.loads(self._fh.read(hlen).decode("utf-8"))
         except (UnicodeDecodeError, json.JSONDecodeError) as exc:
             raise SafetensorsError(f"{path}: header is not valid JSON: {exc}") from exc
-        self.metadata = header.pop("__metadata__", {}) or {}
+        if not isinstance(header, dict):
+            raise SafetensorsError(f"{path}: the header is not a JSON object")
+        metadata = header.pop("__metadata__", None)
+        self.metadata = metadata if isinstance(metadata, dict) else {}
         self._data_start = 8 + hlen
         self._entries = {}
+        whole = lambda v: isinstance(v, int) and not isinstance(v, bool) and v >= 0
         for name, info in header.items():
+            # a damaged header is refused here, with the tensor's name, and not by whatever trips over it later
+            if not (isinstance(info, dict) and isinstance(info.get("dtype"), str) and isinstance(info.get("shape"), list)
+                    and all(whole(n) for n in info["shape"]) and isinstance(info.get("data_offsets"), list)
+                    and len(info["data_offsets"]) == 2 and all(whole(n) for n in info["data_offsets"])):
+                raise SafetensorsError(f"{path}: tensor '{name}': the header entry must hold a dtype, a shape of "
+                                       f"non-negative integers and two non-negative data_offsets, got {info!r}")
             dtype, shape, (begin, end) = info["dtype"], tuple(info["shape"]), info["data_offsets"]
             if dtype not in _DTYPES:
                 raise SafetensorsError(f"{path}: tensor '{name}' has unsupported dtype {dtype}")
-            count = int(np.prod(shape, dtype=np.int64)) if shape else 1
+            count = 1
+            for n in shape:     # exact integers: a shape whose product does not fit 64 bits must not wrap round
+                count *= n
             nbytes = count * np.dtype(_DTYPES[dtype][0]).itemsize
             if end - begin != nbytes or self._data_start + end > size:
                 raise SafetensorsError(

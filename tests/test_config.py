@@ -50,6 +50,9 @@ def test_every_key_is_required(missing):
     (dict(max_position_embeddings=0), "max_position_embeddings"),
     (dict(hidden_size="big"), "hidden_size"),
     (dict(tie_word_embeddings=1), "tie_word_embeddings"),
+    (dict(num_hidden_layers=10 ** 12), "num_hidden_layers"),      # a damaged file must not start a model of 10^12 layers
+    (dict(vocab_size=2 ** 31), "vocab_size"),
+    (dict(num_attention_heads=2 ** 26, num_key_value_heads=2 ** 26), "q_width"),
 ])
 def test_invalid_configs(patch, msg):
     with pytest.raises(ConfigError, match=msg):

@@ -12,6 +12,7 @@ from arle_amd.models import expected_checkpoint_tensors
 from arle_amd.models.qwen3 import qwen3_spec
 from arle_amd.weights import (SafetensorsFile, WeightsError, load_weights, write_random_model,
                               write_safetensors)
+from arle_amd.weights.safetensors_io import SafetensorsError
 from tiny import ARCH, TINY_A, TINY_B
 
 
@@ -59,6 +60,23 @@ def test_file_written_by_the_safetensors_package_is_read_by_the_own_reader(tmp_p
         got = f.read(name)
         assert tuple(shape) == tuple(t.shape) and got.dtype == t.dtype and torch.equal(got, t), name
     f.close()
+
+
+@pytest.mark.parametrize("entry", [None, 5, {}, {"dtype": "BF16", "shape": [2], "data_offsets": [0]},
+                                   {"dtype": "BF16", "shape": [2], "data_offsets": "ab"},
+                                   {"dtype": "BF16", "shape": [-2], "data_offsets": [0, 4]},
+                                   {"dtype": None, "shape": [2], "data_offsets": [0, 4]},
+                                   {"dtype": "BF16", "shape": [2 ** 40, 2 ** 40], "data_offsets": [0, 4]},
+                                   {"dtype": "BF16", "shape": [2], "data_offsets": [-4, 0]}])
+def test_a_damaged_header_entry_is_refused_with_the_tensors_name(tmp_path, entry):
+    """Whatever stands where a tensor's dtype, shape and offsets belong: the reader's own error, naming the tensor,
+    and not the exception of whatever tripped over it."""
+    path = str(tmp_path / "bad.safetensors")
+    header = json.dumps({"model.w": entry, "__metadata__": 5}).encode()
+    with open(path, "wb") as fh:
+        fh.write(struct.pack("<Q", len(header)) + header + b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="model.w"):
+        SafetensorsFile(path)
 
 
 def test_data_length_mismatch_names_the_tensor(tmp_path):
