@@ -108,8 +108,11 @@ def build_step_batch(entries, slot_of, length_of, vocab_size: int, device, into=
     for e in entries:
         staged += e.want
     try:
-        wide = np.array(staged, dtype=np.int64)
-    except (TypeError, ValueError):
+        wide = np.array(staged)
+        if wide.dtype.kind not in "iu":     # a float would be cut to an integer without a word, a bool read as 0 or 1
+            raise TypeError
+        wide = wide.astype(np.int64)
+    except (TypeError, ValueError, OverflowError):
         raise ValueError("token ids and wanted places are integers (a DeviceToken only as the one token of an "
                          "entry)") from None
     np.clip(wide, -1, 2**31 - 1, out=wide)     # what is out of range stays out of range
