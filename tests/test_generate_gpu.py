@@ -184,6 +184,27 @@ def test_trace_run_program(folders, tmp_path, dtype, tol):
     replay.compare(got, cfg, weights, reqs, tol, f"trace_run/{dtype}")
 
 
+@pytest.mark.parametrize("bad,what", [
+    ('{"step": 1, "entries": [{"id": "a", "tokens": [1, 99999], "want": [0]}], "end": []}', "outside the vocabulary"),
+    ('{"step": 1, "entries": [{"id": "a", "tokens": [1, 2], "want": [5]}], "end": []}', "wanted place"),
+    ('{"step": 1, "entries": [{"id": "b", "tokens": ' + str(list(range(200))) + ', "want": []}], "end": []}', "OutOfPages"),
+    ('{"step": 1, "entries": [{"id": "a", "tok', "JSONDecodeError"),
+    ('{"entries": [], "end": []}', "KeyError"),
+])
+def test_trace_run_ends_with_the_line_and_the_reason_when_a_step_cannot_be_run(folders, tmp_path, bad, what):
+    """A good step, then one that cannot be read or run: the good step's file is there, its `done` line too, the
+    program names the input line and the reason on stderr and ends with 1 (no `done` for the bad step)."""
+    good = '{"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [2]}], "end": []}'
+    out = str(tmp_path / "out")
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folders["B"], "--dtype", "float32",
+                        "--out", out, "--max-tokens", "64"], input=good + "\n" + bad + "\n", capture_output=True, text=True,
+                       timeout=300)
+    assert p.returncode == 1
+    assert p.stdout.split() == ["done", "0"] and os.path.exists(os.path.join(out, "0.f32"))
+    assert "input line 2" in p.stderr and what in p.stderr
+    assert not os.path.exists(os.path.join(out, "1.f32"))
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_many_requests_through_the_scheduler_with_and_without_captured_steps(folders, dtype):
     """Thirty requests of random lengths and budgets through few slots, small portions and a pool that runs out now
