@@ -91,7 +91,7 @@ def build_parser() -> argparse.ArgumentParser:
     return ap
 
 
-def main(argv=None) -> int:
+def _run(argv=None) -> int:
     args = build_parser().parse_args(argv)
     if args.command == "random-weights":
         from . import models  # noqa: F401
@@ -167,6 +167,21 @@ def main(argv=None) -> int:
           f"output {max(out.usage.completion_tokens - 1, 0) / decode_time:.1f} tok/s "
           f"({out.usage.completion_tokens} tokens, {out.finish_reason})", file=sys.stderr)
     return 0
+
+
+def main(argv=None) -> int:
+    """The command line; what the user can mend (a folder that is not a model, a damaged file, a prompt that does
+    not fit, a missing compiler) ends in one line `error: ...` and exit code 1, not in a traceback."""
+    from .cache.manager import NoFreeSlot
+    from .cache.pages import OutOfPages
+    from .engine.engine import EngineError
+    from .kernels.build import BuildError
+
+    try:
+        return _run(argv)
+    except (ValueError, OSError, EngineError, OutOfPages, NoFreeSlot, BuildError) as exc:
+        print(f"error: {exc}", file=sys.stderr)
+        return 1
 
 
 if __name__ == "__main__":

@@ -1,61 +1,26 @@
-"""The command line's options, without a GPU: names and meanings follow the reference's `arle` and `infer`
-(crates/cli/src/args.rs:188-302, infer/src/main.rs:26-236)."""
-import pytest
+"""The command line where no GPU is needed: the random-weights mode, and what it says about folders that are no model."""
+import json
+import os
 
-from arle_amd.cli import build_parser, main
-
-
-def test_global_options_and_run():
-    args = build_parser().parse_args(["--model-path", "/m", "--max-tokens", "auto", "--temperature", "0.7", "--no-cuda-graph",
-                                      "--num-slots", "8", "--chunked-prefill-size", "2048", "run", "--prompt-ids", "1, 2,3",
-                                      "--json"])
-    assert args.command == "run" and args.model_path == "/m" and args.max_tokens == 0 and args.temperature == 0.7
-    assert args.no_cuda_graph and not args.no_weight_tiles and args.num_slots == 8 and args.chunked_prefill_size == 2048
-    assert args.prompt_ids == "1, 2,3" and args.json
+from arle_amd.cli import main
+from tiny import TINY_A, ARCH
 
 
-def test_defaults_are_the_reference_library_defaults():
-    args = build_parser().parse_args(["--model-path", "/m", "run", "--prompt", "hi"])
-    # infer/src/main.rs:90-105: slots 4, 16384 tokens a step, the portion and the prompt tokens of a step left to be
-    # settled by the GPU's memory (infer/src/scheduler/types.rs:315-334); greedy (crates/cli/src/args.rs)
-    assert (args.num_slots, args.chunked_prefill_size, args.max_num_batched_tokens, args.max_prefill_tokens) == (4, None, 16384, None)
-    assert args.temperature == 0.0 and args.top_k == -1 and args.top_p == 1.0 and args.min_p == 0.0 and args.seed == 42
-    assert not args.no_cuda_graph and not args.no_weight_tiles and args.dtype == "bfloat16"
+def test_random_weights_mode_writes_a_model_folder(tmp_path, capsys):
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(dict(TINY_A, architectures=[ARCH])))
+    out = str(tmp_path / "model")
+    assert main(["random-weights", "--config", str(config), "--out", out, "--seed-weights", "3"]) == 0
+    assert capsys.readouterr().out.strip() == out
+    assert sorted(os.listdir(out)) == ["config.json", "model.safetensors"]
+    assert json.load(open(os.path.join(out, "config.json")))["hidden_size"] == TINY_A["hidden_size"]
 
 
-def test_bad_values_are_refused(capsys):
-    with pytest.raises(SystemExit):
-        build_parser().parse_args(["--max-tokens", "-3", "run", "--prompt", "x"])
-    with pytest.raises(SystemExit):
-        build_parser().parse_args(["--dtype", "float16", "run", "--prompt", "x"])
-    with pytest.raises(SystemExit):   # one source of the prompt only
-        build_parser().parse_args(["run", "--prompt", "x", "--stdin"])
-    assert main(["run", "--prompt", "x"]) == 2          # no model folder
-    assert "--model-path" in capsys.readouterr().err
-
-
-def test_stop_strings_are_found_in_list_order_and_their_length_is_held_back():
-    """The reading of infer/src/scheduler/cuda/request.rs:396-413 (the reference holds no vectors for it): the first
-    stop string of the list that the text holds decides, not the one that comes first in the text; empty ones do
-    not count; without a hit all but the longest stop string's bytes may go out, cut back to a whole character."""
-    from arle_amd.engine.api import check_stop_sequences
-
-    assert check_stop_sequences("one two three", ["three", "two"]) == (True, 8)
-    assert check_stop_sequences("one two three", ["", "two"]) == (True, 4)
-    assert check_stop_sequences("one two", ["three"]) == (False, 2)          # 7 - 5
-    assert check_stop_sequences("on", ["three"]) == (False, 0)
-    assert check_stop_sequences("one two", []) == (False, 7) and check_stop_sequences("one two", [""]) == (False, 7)
-    assert check_stop_sequences("aé", ["xy"]) == (False, 1)                 # 3 bytes - 2 falls inside the é: back to "a"
-    assert check_stop_sequences("ab\u00e9\u00e9", ["\u00e9x"]) == (False, 2)    # 6 bytes - 3: inside the first é
-
-
-def test_slots_left_to_the_engine_follow_what_the_cache_holds():
-    """--num-slots auto (the reference's flag left unset, infer/src/main.rs:782-855): as many requests of the longest
-    length as the cache holds, from 4 to 128."""
-    from arle_amd.cache.manager import slots_for_tokens
-
-    assert build_parser().parse_args(["--num-slots", "auto", "run", "--prompt", "x"]).num_slots is None
-    assert build_parser().parse_args(["--num-slots", "7", "run", "--prompt", "x"]).num_slots == 7
-    with pytest.raises(SystemExit):
-        build_parser().parse_args(["--num-slots", "0", "run", "--prompt", "x"])
-    assert [slots_for_tokens(t, 64) for t in (0, 128, 256, 2048, 64 * 128, 10 ** 9)] == [4, 4, 4, 32, 128, 128]
+def test_a_folder_that_is_no_model_ends_in_one_line_and_exit_code_1(tmp_path, capsys):
+    assert main(["--model-path", str(tmp_path / "nothing"), "run", "--prompt-ids", "1,2"]) == 1
+    err = capsys.readouterr().err.strip().splitlines()
+    assert len(err) == 1 and err[0].startswith("error: ") and "config.json" in err[0]
+    (tmp_path / "config.json").write_text(json.dumps(dict(TINY_A, architectures=[ARCH], num_hidden_layers=10 ** 12)))
+    assert main(["--model-path", str(tmp_path), "run", "--prompt-ids", "1,2"]) == 1
+    assert "num_hidden_layers" in capsys.readouterr().err
+    assert main(["run", "--prompt-ids", "1,2"]) == 2      # no model named at all: a usage error
